@@ -1,0 +1,241 @@
+/*
+ * pixienn_hip.h -- C ABI of the MI355X (gfx950) non-convolution layer kernels.
+ *
+ * Drop-in boundary for PixieNN's kernel entry points (the free functions the
+ * reference declares in its include/<Name>.cuh headers and calls from the layers
+ * under include/cuda/).
+ * Each function cites the reference interface it replaces as <file>:<lines>.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name starts with "host_";
+ *     tensors are fp32, NCHW, contiguous: index = ((n*C + c)*H + y)*W + x;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     no function synchronises the device, callers order work through the
+ *     stream (the reference's cudaDeviceSynchronize() calls are not kept);
+ *   - return value: PXH_OK (0); PXH_ERR_* (< 0) for a rejected call, nothing
+ *     was launched; > 0 is the hipError_t of a failed launch.
+ *     pxh_last_error() gives the message of the calling thread's last failure;
+ *   - buffers are caller owned.  Aliasing is only allowed where a function
+ *     says so ("in place").
+ */
+#ifndef PIXIENN_HIP_H
+#define PIXIENN_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PXH_OK 0
+#define PXH_ERR_INVALID_ARGUMENT (-1)
+#define PXH_ERR_UNSUPPORTED (-2)
+#define PXH_ERR_WORKSPACE (-3)
+
+/* include/ActivationTypes.h:19-30 (same numbering) */
+enum pxh_activation {
+    PXH_LEAKY = 0, PXH_LINEAR, PXH_LOGGY, PXH_LOGISTIC, PXH_MISH,
+    PXH_RELU, PXH_SOFTPLUS, PXH_SWISH, PXH_TANH
+};
+
+const char* pxh_last_error(void);
+/* library version, bumped when a signature changes */
+int pxh_abi_version(void);
+/* Host-only check hook: n / d through the multiply-high division the index maps use
+ * (n < 2^31, d >= 1).  No reference counterpart. */
+unsigned pxh_debug_fastdiv(unsigned n, unsigned d);
+
+/* ------------------------------------------------------------------------
+ * Conv-layer epilogue, forward.
+ * ---------------------------------------------------------------------- */
+
+/* BN-inference + activation in one pass:
+ *   y = act( ((x - rolling_mean[c]) / (sqrt(rolling_var[c]) + 1e-5)) * scale[c] + bias[c] )
+ * with the rounding sequence of the CPU layer (subtract, divide, scale, add
+ * each rounded to fp32).  pre_activation (nullable) receives the value before
+ * act.  In place allowed (y == x).
+ * Replaces, for an inferring ConvLayer/BatchNormLayer: cudnnBatchNormalizationForwardInference
+ * + preActivation_.copy + activate(), include/cuda/ConvLayer.h:284-307; CPU semantics
+ * src/BatchNorm.cpp:24-67 (training == false), include/ConvLayer.h:227-236. */
+int pxh_bn_infer_act_forward(const float* x, float* y, float* pre_activation,
+                             const float* rolling_mean, const float* rolling_var,
+                             const float* scale, const float* bias,
+                             int batch, int channels, int spatial, int activation, void* stream);
+
+/* bias + activation in one pass: y = act(x + bias[c]); pre_activation nullable; in place allowed.
+ * Replaces addBiasGpu (include/BiasKernels.cuh:21) + preActivation_.copy + activate()
+ * (include/Activation.cuh:26) for a ConvLayer without batch_normalize. */
+int pxh_bias_act_forward(const float* x, float* y, float* pre_activation, const float* bias,
+                         int batch, int channels, int spatial, int activation, void* stream);
+
+/* Bytes of device workspace the BN training entry points need for this shape. */
+size_t pxh_bn_workspace_bytes(int batch, int channels, int spatial);
+
+/* BN-training forward + activation:
+ *   mean[c], var[c] (population variance) over N*H*W; rolling = 0.99*rolling + 0.01*stat;
+ *   x_hat = (x - mean)/(sqrt(var) + 1e-5); pre = x_hat*scale + bias; y = act(pre).
+ * Outputs x_saved, x_norm, pre_activation are each nullable (not materialised when NULL);
+ * y == x is allowed when x_saved is NULL or distinct from x.
+ * workspace: pxh_bn_workspace_bytes() bytes, or NULL to use a per-device buffer the
+ * library allocates on first use and keeps.
+ * Replaces cudnnBatchNormalizationForwardTraining + the x_/preActivation_ copies + activate(),
+ * include/cuda/ConvLayer.h:284-307, include/cuda/BatchNormLayer.h:59-92; CPU semantics
+ * src/BatchNorm.cpp:47-66, src/CpuUtil.cpp:248-301. */
+int pxh_bn_train_act_forward(const float* x, float* y, float* pre_activation, float* x_saved,
+                             float* x_norm, float* mean, float* var, float* rolling_mean,
+                             float* rolling_var, const float* scale, const float* bias,
+                             int batch, int channels, int spatial, int activation,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/* Per-channel batch statistics only (first half of the above). */
+int pxh_bn_stats(const float* x, float* mean, float* var, int batch, int channels, int spatial,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Conv-layer epilogue, backward.
+ * ---------------------------------------------------------------------- */
+
+/* Activation gradient + BN backward:
+ *   d' = delta * act'(pre);  bias_updates[c] += sum d';  scale_updates[c] += sum d' * x_hat;
+ *   d'' = d' * scale[c];  mean_delta, var_delta as src/CpuUtil.cpp:303-327;
+ *   delta <- d''/sqrt(var+1e-5) + var_delta*2*(x-mean)/(N*HW) + mean_delta/(N*HW)   (in place)
+ * x is the saved conv output (x_saved of the forward).  pre_activation may be NULL: it is then
+ * recomputed from x exactly as the forward computed it.  mean_delta / var_delta are outputs
+ * (nullable).  workspace as for the forward.
+ * Replaces gradient() + cudnnBatchNormalizationBackward, include/cuda/ConvLayer.h:315-338;
+ * CPU semantics include/ConvLayer.h:244-252, src/BatchNorm.cpp:69-96. */
+int pxh_bn_act_backward(float* delta, const float* x, const float* pre_activation,
+                        const float* mean, const float* var, const float* scale, const float* bias,
+                        float* scale_updates, float* bias_updates, float* mean_delta, float* var_delta,
+                        int batch, int channels, int spatial, int activation,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* Activation gradient + bias backward for a ConvLayer without batch_normalize:
+ *   delta *= act'(pre) (in place);  bias_updates[c] += sum over N*HW of delta.
+ * Replaces gradient() (include/Activation.cuh:27) + backwardBiasGpu (include/BiasKernels.cuh:22). */
+int pxh_bias_act_backward(float* delta, const float* pre_activation, float* bias_updates,
+                          int batch, int channels, int spatial, int activation,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Stand-alone pieces with the reference's own signatures.
+ * ---------------------------------------------------------------------- */
+
+/* include/Activation.cuh:26-27 */
+int pxh_activate(int activation, float* x, size_t n, void* stream);
+int pxh_gradient(int activation, const float* x, size_t n, float* delta, void* stream);
+/* include/BiasKernels.cuh:21-22 (bias_updates accumulates) */
+int pxh_add_bias(float* output, const float* bias, int batch, int n, int size, void* stream);
+int pxh_backward_bias(float* bias_updates, const float* delta, int batch, int n, int size,
+                      void* workspace, size_t workspace_bytes, void* stream);
+/* include/CudaUtils.cuh:27-31 */
+int pxh_fill_f32(float* x, size_t n, float value, void* stream);
+int pxh_fill_i32(int* x, size_t n, int value, void* stream);
+int pxh_constrain(int n, float alpha, float* x, void* stream);
+int pxh_mul(int n, const float* x, float* y, void* stream);          /* y[i] = x[i]*y[i]; x == y allowed */
+/* cublasSaxpy as used for "grad += delta", include/cuda/YoloLayer.h:163, cuda/ShortcutLayer.h:49 */
+int pxh_axpy(size_t n, float alpha, const float* x, float* y, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Max-pool.  include/MaxPoolKernels.cuh:5-7, CPU semantics include/MaxPoolLayer.h:88-158.
+ * ---------------------------------------------------------------------- */
+
+/* Writes every element of out and indexes (no prior zero fill needed).  indexes hold the flat
+ * NCHW input index of the first strict maximum in row-major window order, or -1. */
+int pxh_maxpool_forward(const float* in, float* out, int* indexes, int batch, int channels,
+                        int ih, int iw, int oh, int ow, int kernel, int stride, int padding,
+                        void* stream);
+/* grad[indexes[i]] += delta[i] in ascending i order for every input cell, i.e. bit-identical to
+ * the sequential CPU loop also when windows overlap (stride < kernel).  No atomics. */
+int pxh_maxpool_backward(const float* delta, const int* indexes, float* grad, int batch, int channels,
+                         int ih, int iw, int oh, int ow, int kernel, int stride, int padding,
+                         void* stream);
+/* The reference's geometry-free signature (maxPoolBackwardGpu).  Float atomics: bit-exact only
+ * when no two outputs share an index (stride >= kernel). */
+int pxh_maxpool_backward_scatter(const float* delta, const int* indexes, float* grad, int size,
+                                 void* stream);
+
+/* ------------------------------------------------------------------------
+ * Upsample.  include/UpsampleKernels.cuh:21-22, CPU semantics include/UpsampleLayer.h:97-121.
+ * forward != 0: out[b,k,j,i] = scale * in[b,k,j/stride,i/stride]   (plain store, every element)
+ * forward == 0: acc[in] += scale * out[...] for the stride^2 covered cells in raster order.
+ * ---------------------------------------------------------------------- */
+int pxh_upsample(const float* in, int w, int h, int c, int batch, int stride, int forward,
+                 float scale, float* acc, float* out, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Shortcut.  include/ShortcutKernel.cuh:21-22, CPU semantics include/ShortcutLayer.h:84-141.
+ * ---------------------------------------------------------------------- */
+
+/* The reference's index-mapped blend: out[oi] = s1*out[oi] + s2*add[ai]. */
+int pxh_shortcut(int batch, int w1, int h1, int c1, const float* add, int w2, int h2, int c2,
+                 float s1, float s2, float* out, void* stream);
+/* Whole ShortcutLayer::forward in one pass (same-shape operands):
+ *   pre = alpha*input + beta*from_output; output = act(pre); pre_activation nullable. */
+int pxh_shortcut_forward(const float* input, const float* from_output, float* output,
+                         float* pre_activation, size_t n, float alpha, float beta, int activation,
+                         void* stream);
+/* Whole ShortcutLayer::backward in one pass:
+ *   delta *= act'(pre_activation) (in place; skipped for linear, pre_activation may then be NULL);
+ *   from_delta = 1*from_delta + beta*delta;  grad += alpha*delta (grad nullable). */
+int pxh_shortcut_backward(float* delta, const float* pre_activation, float* from_delta, float* grad,
+                          size_t n, float alpha, float beta, int activation, void* stream);
+
+/* ------------------------------------------------------------------------
+ * YOLO head.  include/YoloKernels.cuh:7-17, CPU semantics include/YoloLayer.h:164-239, 390-547.
+ * Layout: [batch][mask][5+classes][area]; entries 0..3 box, 4 objectness, 5.. classes.
+ * truths: [batch][max_truth][5] = x, y, w, h, class id (as float); truth_counts[batch].
+ * stats[12] (accumulated into, as the reference does): 0 sum IoU, 1 #IoU>.5, 2 #IoU>.75,
+ *   3 sum class prob, 4 sum obj at positives, 5 sum obj over all slots, 6 count, 7 class count;
+ *   8 box, 9 object, 10 no-object, 11 class sum of squared delta (overwritten).
+ * ---------------------------------------------------------------------- */
+
+/* yoloActivateGpu: logistic on entries 0, 1, 4.., copy of entries 2, 3.  In place allowed. */
+int pxh_yolo_activate(const float* input, float* output, int batch, int masks, int classes,
+                      int area, void* stream);
+
+/* yoloLossGpu with its argument list: region pass over every slot, then the host-assigned
+ * positive slots, then cost (sum of squared delta, ADDED to *cost) and loss components.
+ * delta must be zero on entry, as in the reference. */
+int pxh_yolo_loss(const float* output, float* delta, const float* truths, const int* truth_counts,
+                  int max_truth, const int* assigned_classes, const int* assigned_anchors,
+                  const float* assigned_boxes, const int* masks, const float* anchors,
+                  float* stats, float* cost, int batch, int mask_count, int anchor_count,
+                  int classes, int width, int height, int net_width, int net_height,
+                  float ignore_thresh, float truth_thresh, float coord_scale, float object_scale,
+                  float noobject_scale, float class_scale, void* workspace, size_t workspace_bytes,
+                  void* stream);
+
+size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int width, int height);
+
+/* Whole YoloLayer::forward of a loss-computing pass in one sweep over the head: decode, dense
+ * delta (every element written, no prior fill), positives assigned on the device from the
+ * truths with the CPU layer's rule (best anchor over all anchors, later truth overwrites),
+ * cost = sum(delta^2) (written to *cost, not divided by batch) and stats[12] (overwritten).
+ * host_masks[mask_count], host_anchors[2*anchor_count] are HOST int arrays (layer constants). */
+int pxh_yolo_forward_train(const float* input, float* output, float* delta, const float* truths,
+                           const int* truth_counts, int max_truth, const int* host_masks,
+                           const int* host_anchors, float* stats, float* cost, int batch,
+                           int mask_count, int anchor_count, int classes, int width, int height,
+                           int net_width, int net_height, float ignore_thresh, float truth_thresh,
+                           float coord_scale, float object_scale, float noobject_scale,
+                           float class_scale, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Adam.  include/Adam.cuh:21, include/cuda/Adam.h:49-90.
+ * ---------------------------------------------------------------------- */
+
+/* adamGpu: x += rate * (m/(1-b1^t)) / (sqrt(v/(1-b2^t)) + eps) */
+int pxh_adam(int n, float* x, const float* m, const float* v, float beta1, float beta2, float rate,
+             float eps, int t, void* stream);
+/* Whole Adam<CUDA>::update in one pass, same per-element operation order:
+ *   d *= 1/batch; if apply_decay d += -decay*w; m = b1*m + (1-b1)*d; v = b2*v + (1-b2)*d*d;
+ *   w += lr * (m/(1-b1^t)) / (sqrt(v/(1-b2^t)) + eps);  d = 0.
+ * (L2 decay folded into the update before the moments, as the reference does; not decoupled.) */
+int pxh_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch, int t, float lr,
+                    float beta1, float beta2, float eps, float decay, int apply_decay, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

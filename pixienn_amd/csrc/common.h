@@ -1,0 +1,177 @@
+// Shared host/device helpers for the gfx950 layer kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/pixienn_hip.h"
+
+namespace pxh {
+
+constexpr int kWave = 64;          // CDNA wavefront
+constexpr int kBlock = 256;        // 4 waves per workgroup
+constexpr int kUnroll = 4;         // float4 loads in flight per lane in streaming kernels
+constexpr int kChunk = kBlock * 4 * kUnroll;   // elements one workgroup streams: 4096
+
+// ---------------------------------------------------------------- errors
+void set_error(const char* fmt, ...);
+int fail_invalid(const char* fmt, ...);
+int check_launch(const char* what);
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---------------------------------------------------------------- workspace
+// Per-device scratch the library owns, grown on demand and kept until exit.
+void* library_workspace(size_t bytes);
+// Picks the caller's workspace when given (checking its size), else the library's.
+int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out);
+
+// ---------------------------------------------------------------- fast division
+// q = n / d for 0 <= n < 2^31 by a multiply-high and a shift (d >= 1).
+struct FastDiv {
+    uint32_t d, m, s;
+    FastDiv() : d(1), m(0), s(0) {}
+    explicit FastDiv(uint32_t div) : d(div)
+    {
+        s = 0;
+        while ((1ull << s) < div) ++s;
+        m = static_cast<uint32_t>(((1ull << 32) * ((1ull << s) - div)) / div + 1);
+    }
+    __host__ __device__ __forceinline__ uint32_t div(uint32_t n) const
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        uint32_t t = __umulhi(n, m);
+#else
+        uint32_t t = static_cast<uint32_t>((static_cast<uint64_t>(n) * m) >> 32);
+#endif
+        return (t + n) >> s;
+    }
+    __host__ __device__ __forceinline__ void divmod(uint32_t n, uint32_t& q, uint32_t& r) const
+    {
+        q = div(n);
+        r = n - q * d;
+    }
+};
+
+// ---------------------------------------------------------------- activations (device)
+// The arithmetic follows the CPU functors operation by operation (fp32, no contraction).
+__device__ __forceinline__ float softplus_apply(float x)
+{
+    if (x > 20.0f) return x;
+    if (x < -20.0f) return expf(x);
+    return logf(expf(x) + 1.0f);
+}
+
+__device__ __forceinline__ float softplus_grad(float x)
+{
+    if (x > 20.0f) return 1.0f;
+    if (x < -20.0f) return expf(x);
+    return 1.0f / (1.0f + expf(-x));
+}
+
+template<int ACT>
+__device__ __forceinline__ float act_apply(float x)
+{
+    if constexpr (ACT == PXH_LEAKY) return x > 0.0f ? x : 0.1f * x;
+    else if constexpr (ACT == PXH_LINEAR) return x;
+    else if constexpr (ACT == PXH_LOGGY) return 2.0f / (1.0f + expf(-x)) - 1.0f;
+    else if constexpr (ACT == PXH_LOGISTIC) return 1.0f / (1.0f + expf(-x));
+    else if constexpr (ACT == PXH_MISH) return x * tanhf(softplus_apply(x));
+    else if constexpr (ACT == PXH_RELU) return x > 0.0f ? x : 0.0f;
+    else if constexpr (ACT == PXH_SOFTPLUS) return softplus_apply(x);
+    else if constexpr (ACT == PXH_SWISH) return x / (1.0f + expf(-1.0f * x));
+    else return tanhf(x);
+}
+
+template<int ACT>
+__device__ __forceinline__ float act_grad(float x)
+{
+    if constexpr (ACT == PXH_LEAKY) return x > 0.0f ? 1.0f : 0.1f;
+    else if constexpr (ACT == PXH_LINEAR) return 1.0f;
+    else if constexpr (ACT == PXH_LOGGY) {
+        float y = (x + 1.0f) / 2.0f;
+        return 2.0f * (1.0f - y) * y;
+    } else if constexpr (ACT == PXH_LOGISTIC) {
+        float y = 1.0f / (1.0f + expf(-x));
+        return y * (1.0f - y);
+    } else if constexpr (ACT == PXH_MISH) {
+        float sp = softplus_apply(x);
+        float gsp = softplus_grad(x);
+        float tsp = tanhf(sp);
+        float gtsp = (1.0f - tsp * tsp) * gsp;
+        return x * gtsp + tsp;
+    } else if constexpr (ACT == PXH_RELU) return x > 0.0f ? 1.0f : 0.0f;
+    else if constexpr (ACT == PXH_SOFTPLUS) return softplus_grad(x);
+    else if constexpr (ACT == PXH_SWISH) {
+        float val = 1.0f / (1.0f + expf(-1.0f * x));
+        return x * val + 1.0f * val * (1.0f - x * val);
+    } else {
+        float y = tanhf(x);
+        return 1.0f - y * y;
+    }
+}
+
+// Calls f.template operator()<ACT>() for the runtime activation id; false if unknown.
+template<typename F>
+inline bool dispatch_activation(int act, F&& f)
+{
+    switch (act) {
+    case PXH_LEAKY: f.template operator()<PXH_LEAKY>(); return true;
+    case PXH_LINEAR: f.template operator()<PXH_LINEAR>(); return true;
+    case PXH_LOGGY: f.template operator()<PXH_LOGGY>(); return true;
+    case PXH_LOGISTIC: f.template operator()<PXH_LOGISTIC>(); return true;
+    case PXH_MISH: f.template operator()<PXH_MISH>(); return true;
+    case PXH_RELU: f.template operator()<PXH_RELU>(); return true;
+    case PXH_SOFTPLUS: f.template operator()<PXH_SOFTPLUS>(); return true;
+    case PXH_SWISH: f.template operator()<PXH_SWISH>(); return true;
+    case PXH_TANH: f.template operator()<PXH_TANH>(); return true;
+    default: return false;
+    }
+}
+
+// ---------------------------------------------------------------- reductions
+// Sum over the 64 lanes of a wavefront; every lane returns the total.
+__device__ __forceinline__ double wave_sum(double v)
+{
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// Sum over a kBlock-thread workgroup through LDS; result valid in thread 0.
+// `slots` is LDS of at least kBlock / kWave doubles per concurrently reduced value.
+__device__ __forceinline__ double block_sum(double v, double* slots)
+{
+    v = wave_sum(v);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) slots[wave] = v;
+    __syncthreads();
+    double total = 0.0;
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 0; w < kBlock / kWave; ++w) total += slots[w];
+    }
+    return total;
+}
+
+inline unsigned grid_for(size_t items, size_t per_block)
+{
+    return static_cast<unsigned>((items + per_block - 1) / per_block);
+}
+
+}  // namespace pxh

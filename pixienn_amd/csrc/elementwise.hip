@@ -1,0 +1,430 @@
+// Flat fp32 streaming kernels: activation, fill/clip/multiply/axpy helpers, shortcut, Adam.
+#include "stream.h"
+
+#include <cmath>
+
+namespace pxh {
+namespace {
+
+// ---------------------------------------------------------------- activation
+template<int ACT>
+struct ActivateOp {
+    float* x;
+    template<int V> struct Regs { Pack<V> x; };
+    template<int V> __device__ void load(size_t e, Regs<V>& r) const { r.x = ld<V>(x, e); }
+    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> o;
+#pragma unroll
+        for (int k = 0; k < V; ++k) o.v[k] = act_apply<ACT>(r.x.v[k]);
+        st<V>(x, e, o);
+    }
+};
+
+template<int ACT>
+struct GradientOp {
+    const float* x;
+    float* delta;
+    template<int V> struct Regs { Pack<V> x, d; };
+    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    {
+        r.x = ld<V>(x, e);
+        r.d = ld<V>(delta, e);
+    }
+    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> o;
+#pragma unroll
+        for (int k = 0; k < V; ++k) o.v[k] = r.d.v[k] * act_grad<ACT>(r.x.v[k]);
+        st<V>(delta, e, o);
+    }
+};
+
+// ---------------------------------------------------------------- helpers
+struct FillOp {
+    float* x;
+    float value;
+    template<int V> struct Regs {};
+    template<int V> __device__ void load(size_t, Regs<V>&) const {}
+    template<int V> __device__ void finish(size_t e, const Regs<V>&) const
+    {
+        Pack<V> o;
+#pragma unroll
+        for (int k = 0; k < V; ++k) o.v[k] = value;
+        st<V>(x, e, o);
+    }
+};
+
+struct ConstrainOp {
+    float* x;
+    float alpha;
+    template<int V> struct Regs { Pack<V> x; };
+    template<int V> __device__ void load(size_t e, Regs<V>& r) const { r.x = ld<V>(x, e); }
+    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> o;
+#pragma unroll
+        for (int k = 0; k < V; ++k) o.v[k] = fminf(alpha, fmaxf(-alpha, r.x.v[k]));
+        st<V>(x, e, o);
+    }
+};
+
+struct MulOp {
+    const float* x;
+    float* y;
+    template<int V> struct Regs { Pack<V> x, y; };
+    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    {
+        r.x = ld<V>(x, e);
+        r.y = ld<V>(y, e);
+    }
+    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> o;
+#pragma unroll
+        for (int k = 0; k < V; ++k) o.v[k] = r.x.v[k] * r.y.v[k];
+        st<V>(y, e, o);
+    }
+};
+
+struct AxpyOp {
+    const float* x;
+    float* y;
+    float alpha;
+    template<int V> struct Regs { Pack<V> x, y; };
+    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    {
+        r.x = ld<V>(x, e);
+        r.y = ld<V>(y, e);
+    }
+    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> o;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            const float p = alpha * r.x.v[k];
+            o.v[k] = r.y.v[k] + p;
+        }
+        st<V>(y, e, o);
+    }
+};
+
+// ---------------------------------------------------------------- shortcut
+// pre = alpha*in + beta*from (two products, one sum, each rounded); out = act(pre)
+template<int ACT>
+struct ShortcutForwardOp {
+    const float* in;
+    const float* from;
+    float* out;
+    float* pre;   // nullable
+    float alpha, beta;
+    template<int V> struct Regs { Pack<V> a, b; };
+    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    {
+        r.a = ld<V>(in, e);
+        r.b = ld<V>(from, e);
+    }
+    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> p, o;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            const float pa = alpha * r.a.v[k];
+            const float pb = beta * r.b.v[k];
+            p.v[k] = pa + pb;
+            o.v[k] = act_apply<ACT>(p.v[k]);
+        }
+        if (pre) st<V>(pre, e, p);
+        st<V>(out, e, o);
+    }
+};
+
+// delta *= act'(pre); from_delta = 1*from_delta + beta*delta; grad += alpha*delta
+template<int ACT>
+struct ShortcutBackwardOp {
+    float* delta;
+    const float* pre;
+    float* from_delta;
+    float* grad;   // nullable
+    float alpha, beta;
+    template<int V> struct Regs { Pack<V> d, p, f, g; };
+    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    {
+        r.d = ld<V>(delta, e);
+        if constexpr (ACT != PXH_LINEAR) r.p = ld<V>(pre, e);
+        r.f = ld<V>(from_delta, e);
+        if (grad) r.g = ld<V>(grad, e);
+    }
+    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> d = r.d, f, g;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            if constexpr (ACT != PXH_LINEAR) d.v[k] = d.v[k] * act_grad<ACT>(r.p.v[k]);
+            const float keep = 1.0f * r.f.v[k];
+            const float add = beta * d.v[k];
+            f.v[k] = keep + add;
+            if (grad) {
+                const float ga = alpha * d.v[k];
+                g.v[k] = r.g.v[k] + ga;
+            }
+        }
+        if constexpr (ACT != PXH_LINEAR) st<V>(delta, e, d);
+        st<V>(from_delta, e, f);
+        if (grad) st<V>(grad, e, g);
+    }
+};
+
+// The reference's index-mapped blend for operands of different shape.
+__global__ __launch_bounds__(kBlock) void shortcut_mapped_kernel(uint32_t size, FastDiv by_w, FastDiv by_h, FastDiv by_c,
+                                                                 int stride, int sample, int w1, int h1, int c1,
+                                                                 const float* add, int w2, int h2, int c2, float s1,
+                                                                 float s2, float* out)
+{
+    const uint32_t id = blockIdx.x * kBlock + threadIdx.x;
+    if (id >= size) return;
+    uint32_t rows, planes, i, j, k, b;
+    by_w.divmod(id, rows, i);
+    by_h.divmod(rows, planes, j);
+    by_c.divmod(planes, b, k);
+    const size_t oi = i * sample + static_cast<size_t>(w2) * (j * sample + static_cast<size_t>(h2) * (k + static_cast<size_t>(c2) * b));
+    const size_t ai = i * stride + static_cast<size_t>(w1) * (j * stride + static_cast<size_t>(h1) * (k + static_cast<size_t>(c1) * b));
+    const float po = s1 * out[oi];
+    const float pa = s2 * add[ai];
+    out[oi] = po + pa;
+}
+
+// ---------------------------------------------------------------- Adam
+// One fp32 rounding per BLAS call of the reference sequence (include/cuda/Adam.h:49-90).
+struct AdamUpdateOp {
+    float* w;
+    float* d;
+    float* m;
+    float* v;
+    float inv_batch, neg_decay, beta1, beta2, a1, a2, c1, c2, lr, eps;
+    int apply_decay;
+    template<int V> struct Regs { Pack<V> w, d, m, v; };
+    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    {
+        r.w = ld<V>(w, e);
+        r.d = ld<V>(d, e);
+        r.m = ld<V>(m, e);
+        r.v = ld<V>(v, e);
+    }
+    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> ow, om, ov, od;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            float g = r.d.v[k] * inv_batch;
+            if (apply_decay) {
+                const float l2 = neg_decay * r.w.v[k];
+                g = g + l2;
+            }
+            float mi = r.m.v[k] * beta1;
+            float vi = r.v.v[k] * beta2;
+            const float am = a1 * g;
+            mi = mi + am;
+            const float g2 = g * g;
+            const float av = a2 * g2;
+            vi = vi + av;
+            const float mhat = mi / c1;
+            const float vhat = vi / c2;
+            const float step = lr * mhat / (sqrtf(vhat) + eps);
+            ow.v[k] = r.w.v[k] + step;
+            om.v[k] = mi;
+            ov.v[k] = vi;
+            od.v[k] = 0.0f;
+        }
+        st<V>(w, e, ow);
+        st<V>(m, e, om);
+        st<V>(v, e, ov);
+        st<V>(d, e, od);
+    }
+};
+
+struct AdamStepOp {
+    float* x;
+    const float* m;
+    const float* v;
+    float c1, c2, rate, eps;
+    template<int V> struct Regs { Pack<V> x, m, v; };
+    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    {
+        r.x = ld<V>(x, e);
+        r.m = ld<V>(m, e);
+        r.v = ld<V>(v, e);
+    }
+    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> o;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            const float mhat = r.m.v[k] / c1;
+            const float vhat = r.v.v[k] / c2;
+            const float step = rate * mhat / (sqrtf(vhat) + eps);
+            o.v[k] = r.x.v[k] + step;
+        }
+        st<V>(x, e, o);
+    }
+};
+
+}  // namespace
+}  // namespace pxh
+
+using namespace pxh;
+
+extern "C" {
+
+int pxh_activate(int activation, float* x, size_t n, void* stream)
+{
+    if (!x && n) return fail_invalid("pxh_activate: null pointer");
+    int rc = PXH_OK;
+    const bool known = dispatch_activation(activation, [&]<int ACT>() {
+        if constexpr (ACT == PXH_LINEAR) return;
+        rc = launch_stream("pxh_activate", n, aligned16(x), ActivateOp<ACT>{ x }, as_stream(stream));
+    });
+    if (!known) return fail_invalid("pxh_activate: unknown activation %d", activation);
+    return rc;
+}
+
+int pxh_gradient(int activation, const float* x, size_t n, float* delta, void* stream)
+{
+    if ((!x || !delta) && n) return fail_invalid("pxh_gradient: null pointer");
+    int rc = PXH_OK;
+    const bool known = dispatch_activation(activation, [&]<int ACT>() {
+        if constexpr (ACT == PXH_LINEAR) return;
+        rc = launch_stream("pxh_gradient", n, aligned16(x) && aligned16(delta), GradientOp<ACT>{ x, delta },
+                           as_stream(stream));
+    });
+    if (!known) return fail_invalid("pxh_gradient: unknown activation %d", activation);
+    return rc;
+}
+
+int pxh_fill_f32(float* x, size_t n, float value, void* stream)
+{
+    if (!x && n) return fail_invalid("pxh_fill_f32: null pointer");
+    return launch_stream("pxh_fill_f32", n, aligned16(x), FillOp{ x, value }, as_stream(stream));
+}
+
+int pxh_fill_i32(int* x, size_t n, int value, void* stream)
+{
+    if (!x && n) return fail_invalid("pxh_fill_i32: null pointer");
+    float bits;
+    static_assert(sizeof(bits) == sizeof(value), "int and float must have the same size");
+    __builtin_memcpy(&bits, &value, sizeof(bits));
+    return launch_stream("pxh_fill_i32", n, aligned16(x), FillOp{ reinterpret_cast<float*>(x), bits },
+                         as_stream(stream));
+}
+
+int pxh_constrain(int n, float alpha, float* x, void* stream)
+{
+    if (n < 0 || (!x && n)) return fail_invalid("pxh_constrain: bad argument");
+    return launch_stream("pxh_constrain", static_cast<size_t>(n), aligned16(x), ConstrainOp{ x, alpha },
+                         as_stream(stream));
+}
+
+int pxh_mul(int n, const float* x, float* y, void* stream)
+{
+    if (n < 0 || ((!x || !y) && n)) return fail_invalid("pxh_mul: bad argument");
+    return launch_stream("pxh_mul", static_cast<size_t>(n), aligned16(x) && aligned16(y), MulOp{ x, y },
+                         as_stream(stream));
+}
+
+int pxh_axpy(size_t n, float alpha, const float* x, float* y, void* stream)
+{
+    if ((!x || !y) && n) return fail_invalid("pxh_axpy: null pointer");
+    return launch_stream("pxh_axpy", n, aligned16(x) && aligned16(y), AxpyOp{ x, y, alpha }, as_stream(stream));
+}
+
+int pxh_shortcut(int batch, int w1, int h1, int c1, const float* add, int w2, int h2, int c2, float s1, float s2,
+                 float* out, void* stream)
+{
+    if (!add || !out) return fail_invalid("pxh_shortcut: null pointer");
+    if (batch <= 0 || w1 <= 0 || h1 <= 0 || c1 <= 0 || w2 <= 0 || h2 <= 0 || c2 <= 0)
+        return fail_invalid("pxh_shortcut: dimensions must be positive");
+    int stride = w1 / w2; if (stride < 1) stride = 1;
+    int sample = w2 / w1; if (sample < 1) sample = 1;
+    // the CPU layer rejects these (PX_CHECK in ShortcutLayer::shortcut)
+    if (stride != h1 / h2) return fail_invalid("pxh_shortcut: stride must be equal in x and y direction");
+    if (sample != h2 / h1) return fail_invalid("pxh_shortcut: sample must be equal in x and y direction");
+    const int minw = w1 < w2 ? w1 : w2, minh = h1 < h2 ? h1 : h2, minc = c1 < c2 ? c1 : c2;
+    const unsigned long long size = 1ull * batch * minw * minh * minc;
+    if (size >= (1ull << 31)) {
+        set_error("pxh_shortcut: too many elements");
+        return PXH_ERR_UNSUPPORTED;
+    }
+    if (w1 == w2 && h1 == h2 && c1 == c2) {
+        // same shape: identity index maps, out = s1*out + s2*add as a flat stream
+        return launch_stream("pxh_shortcut", static_cast<size_t>(size), aligned16(add) && aligned16(out),
+                             ShortcutForwardOp<PXH_LINEAR>{ out, add, out, nullptr, s1, s2 }, as_stream(stream));
+    }
+    hipLaunchKernelGGL(shortcut_mapped_kernel, dim3(grid_for(size, kBlock)), dim3(kBlock), 0, as_stream(stream),
+                       static_cast<uint32_t>(size), FastDiv(minw), FastDiv(minh), FastDiv(minc), stride, sample, w1,
+                       h1, c1, add, w2, h2, c2, s1, s2, out);
+    return check_launch("pxh_shortcut");
+}
+
+int pxh_shortcut_forward(const float* input, const float* from_output, float* output, float* pre_activation,
+                         size_t n, float alpha, float beta, int activation, void* stream)
+{
+    if ((!input || !from_output || !output) && n) return fail_invalid("pxh_shortcut_forward: null pointer");
+    int rc = PXH_OK;
+    const bool vec = aligned16(input) && aligned16(from_output) && aligned16(output) && aligned16(pre_activation);
+    const bool known = dispatch_activation(activation, [&]<int ACT>() {
+        rc = launch_stream("pxh_shortcut_forward", n, vec,
+                           ShortcutForwardOp<ACT>{ input, from_output, output, pre_activation, alpha, beta },
+                           as_stream(stream));
+    });
+    if (!known) return fail_invalid("pxh_shortcut_forward: unknown activation %d", activation);
+    return rc;
+}
+
+int pxh_shortcut_backward(float* delta, const float* pre_activation, float* from_delta, float* grad, size_t n,
+                          float alpha, float beta, int activation, void* stream)
+{
+    if ((!delta || !from_delta) && n) return fail_invalid("pxh_shortcut_backward: null pointer");
+    if (activation != PXH_LINEAR && !pre_activation && n)
+        return fail_invalid("pxh_shortcut_backward: pre_activation is required for a non-linear activation");
+    int rc = PXH_OK;
+    const bool vec = aligned16(delta) && aligned16(pre_activation) && aligned16(from_delta) && aligned16(grad);
+    const bool known = dispatch_activation(activation, [&]<int ACT>() {
+        rc = launch_stream("pxh_shortcut_backward", n, vec,
+                           ShortcutBackwardOp<ACT>{ delta, pre_activation, from_delta, grad, alpha, beta },
+                           as_stream(stream));
+    });
+    if (!known) return fail_invalid("pxh_shortcut_backward: unknown activation %d", activation);
+    return rc;
+}
+
+int pxh_adam(int n, float* x, const float* m, const float* v, float beta1, float beta2, float rate, float eps, int t,
+             void* stream)
+{
+    if (n < 0 || ((!x || !m || !v) && n)) return fail_invalid("pxh_adam: bad argument");
+    // bias corrections formed on the host in fp32, as powf(beta, t)
+    const float c1 = 1.0f - powf(beta1, static_cast<float>(t));
+    const float c2 = 1.0f - powf(beta2, static_cast<float>(t));
+    return launch_stream("pxh_adam", static_cast<size_t>(n), aligned16(x) && aligned16(m) && aligned16(v),
+                         AdamStepOp{ x, m, v, c1, c2, rate, eps }, as_stream(stream));
+}
+
+int pxh_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch, int t, float lr, float beta1,
+                    float beta2, float eps, float decay, int apply_decay, void* stream)
+{
+    if ((!w || !d || !m || !v) && n) return fail_invalid("pxh_adam_update: null pointer");
+    if (batch <= 0) return fail_invalid("pxh_adam_update: batch must be positive");
+    if (t < 1) return fail_invalid("pxh_adam_update: t must be at least 1 (the update count is pre-incremented)");
+    AdamUpdateOp op;
+    op.w = w; op.d = d; op.m = m; op.v = v;
+    op.inv_batch = 1.0f / static_cast<float>(batch);
+    op.neg_decay = -decay;
+    op.beta1 = beta1; op.beta2 = beta2;
+    op.a1 = 1.0f - beta1; op.a2 = 1.0f - beta2;
+    op.c1 = 1.0f - powf(beta1, static_cast<float>(t));
+    op.c2 = 1.0f - powf(beta2, static_cast<float>(t));
+    op.lr = lr; op.eps = eps; op.apply_decay = apply_decay;
+    return launch_stream("pxh_adam_update", n, aligned16(w) && aligned16(d) && aligned16(m) && aligned16(v), op,
+                         as_stream(stream));
+}
+
+}

@@ -1,0 +1,374 @@
+// Max-pool (values + int32 argmax) and nearest upsample, forward and backward, for gfx950.
+// Index and copy work is bit-exact against the CPU layers; accumulation follows their order.
+#include "stream.h"
+
+#include <cfloat>
+
+namespace pxh {
+namespace {
+
+struct PoolGeom {
+    int ih, iw, oh, ow, kernel, stride, origin;   // origin = -padding / 2
+};
+
+// ------------------------------------------------------------------ max-pool, any geometry
+// One output per lane.  Taps in row-major order; the first in-bounds tap is taken, later taps
+// only when strictly greater (include/MaxPoolLayer.h:106-127 of the reference).
+__global__ __launch_bounds__(kBlock) void maxpool_fwd_generic_kernel(const float* in, float* out, int* indexes,
+                                                                     uint32_t total, PoolGeom g, FastDiv by_ow,
+                                                                     FastDiv by_oh)
+{
+    const uint32_t o = blockIdx.x * kBlock + threadIdx.x;
+    if (o >= total) return;
+    uint32_t rows, ox, plane, oy;
+    by_ow.divmod(o, rows, ox);
+    by_oh.divmod(rows, plane, oy);
+    float best = -FLT_MAX;
+    int best_at = -1;
+    for (int ky = 0; ky < g.kernel; ++ky) {
+        const int y = g.origin + static_cast<int>(oy) * g.stride + ky;
+        if (y < 0 || y >= g.ih) continue;
+        for (int kx = 0; kx < g.kernel; ++kx) {
+            const int x = g.origin + static_cast<int>(ox) * g.stride + kx;
+            if (x < 0 || x >= g.iw) continue;
+            const int at = x + g.iw * (y + g.ih * static_cast<int>(plane));
+            const float v = in[at];
+            if (best_at < 0 || v > best) {
+                best_at = at;
+                best = v;
+            }
+        }
+    }
+    out[o] = best;
+    indexes[o] = best_at;
+}
+
+// 2x2 / stride 2 windows that all lie inside the input: VX outputs per lane from two
+// (2*VX)-wide row loads, stored as VX-wide value and index vectors.
+template<int VX>
+__global__ __launch_bounds__(kBlock) void maxpool_fwd_2x2_kernel(const float* in, float* out, int* indexes,
+                                                                 uint32_t units, int iw, int ow, FastDiv by_owv,
+                                                                 FastDiv by_oh)
+{
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= units) return;
+    uint32_t rows, oxv, plane, oy;
+    by_owv.divmod(t, rows, oxv);
+    by_oh.divmod(rows, plane, oy);
+    const uint32_t ih = by_oh.d * 2;
+    const uint32_t ox = oxv * VX;
+    const uint32_t in0 = (plane * ih + 2 * oy) * iw + 2 * ox;   // < 2^31 checked by the host
+    const Pack<2 * VX> r0 = ld<2 * VX>(in, in0);
+    const Pack<2 * VX> r1 = ld<2 * VX>(in, in0 + iw);
+    Pack<VX> v;
+    IPack<VX> ix;
+#pragma unroll
+    for (int k = 0; k < VX; ++k) {
+        float best = r0.v[2 * k];
+        int at = in0 + 2 * k;
+        if (r0.v[2 * k + 1] > best) { best = r0.v[2 * k + 1]; at = in0 + 2 * k + 1; }
+        if (r1.v[2 * k] > best) { best = r1.v[2 * k]; at = in0 + iw + 2 * k; }
+        if (r1.v[2 * k + 1] > best) { best = r1.v[2 * k + 1]; at = in0 + iw + 2 * k + 1; }
+        v.v[k] = best;
+        ix.v[k] = at;
+    }
+    const uint32_t o = (plane * by_oh.d + oy) * ow + ox;
+    st<VX>(out, o, v);
+    sti<VX>(indexes, o, ix);
+}
+
+// Backward, any geometry: one input cell per lane gathers, in ascending output order, the
+// deltas of the windows whose recorded argmax is this cell.  Ascending output order is the
+// order in which the sequential CPU loop reaches this cell (include/MaxPoolLayer.h:150-156).
+__global__ __launch_bounds__(kBlock) void maxpool_bwd_generic_kernel(const float* delta, const int* indexes,
+                                                                     float* grad, uint32_t total, PoolGeom g,
+                                                                     FastDiv by_iw, FastDiv by_ih)
+{
+    const uint32_t cell = blockIdx.x * kBlock + threadIdx.x;
+    if (cell >= total) return;
+    uint32_t rows, x, plane, y;
+    by_iw.divmod(cell, rows, x);
+    by_ih.divmod(rows, plane, y);
+    // windows with origin + o*stride <= p <= origin + o*stride + kernel - 1
+    const int py = static_cast<int>(y) - g.origin, px = static_cast<int>(x) - g.origin;
+    int oy0 = py - g.kernel + 1;
+    oy0 = oy0 <= 0 ? 0 : (oy0 + g.stride - 1) / g.stride;
+    int ox0 = px - g.kernel + 1;
+    ox0 = ox0 <= 0 ? 0 : (ox0 + g.stride - 1) / g.stride;
+    const int oy1 = min(g.oh - 1, py >= 0 ? py / g.stride : -1);
+    const int ox1 = min(g.ow - 1, px >= 0 ? px / g.stride : -1);
+    float acc = grad[cell];
+    bool touched = false;
+    for (int oy = oy0; oy <= oy1; ++oy)
+        for (int ox = ox0; ox <= ox1; ++ox) {
+            const int o = ox + g.ow * (oy + g.oh * static_cast<int>(plane));
+            if (indexes[o] == static_cast<int>(cell)) {
+                acc += delta[o];
+                touched = true;
+            }
+        }
+    if (touched) grad[cell] = acc;
+}
+
+// Backward for the 2x2 / stride 2 in-bounds case: one window per output, VX windows per lane,
+// the two grad rows are updated as full vectors so the read-modify-write stays coalesced.
+template<int VX>
+__global__ __launch_bounds__(kBlock) void maxpool_bwd_2x2_kernel(const float* delta, const int* indexes, float* grad,
+                                                                 uint32_t units, int iw, int ow, FastDiv by_owv,
+                                                                 FastDiv by_oh)
+{
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= units) return;
+    uint32_t rows, oxv, plane, oy;
+    by_owv.divmod(t, rows, oxv);
+    by_oh.divmod(rows, plane, oy);
+    const uint32_t ih = by_oh.d * 2;
+    const uint32_t ox = oxv * VX;
+    const uint32_t in0 = (plane * ih + 2 * oy) * iw + 2 * ox;
+    const uint32_t o = (plane * by_oh.d + oy) * ow + ox;
+    const Pack<VX> d = ld<VX>(delta, o);
+    const IPack<VX> ix = ldi<VX>(indexes, o);
+    Pack<2 * VX> g0 = ld<2 * VX>(grad, in0);
+    Pack<2 * VX> g1 = ld<2 * VX>(grad, in0 + iw);
+#pragma unroll
+    for (int k = 0; k < VX; ++k) {
+        const int at = ix.v[k];
+        const int base = static_cast<int>(in0) + 2 * k;
+        if (at == base) g0.v[2 * k] += d.v[k];
+        else if (at == base + 1) g0.v[2 * k + 1] += d.v[k];
+        else if (at == base + iw) g1.v[2 * k] += d.v[k];
+        else if (at == base + iw + 1) g1.v[2 * k + 1] += d.v[k];
+    }
+    st<2 * VX>(grad, in0, g0);
+    st<2 * VX>(grad, in0 + iw, g1);
+}
+
+__global__ __launch_bounds__(kBlock) void maxpool_bwd_scatter_kernel(const float* delta, const int* indexes,
+                                                                     float* grad, int size)
+{
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= size) return;
+    const int at = indexes[i];
+    if (at >= 0) atomicAdd(grad + at, delta[i]);
+}
+
+// ------------------------------------------------------------------ upsample
+// stride 2: VX inputs per lane; forward writes the 2 x (2*VX) block, backward folds it into the
+// input cell as (((acc + s*o00) + s*o01) + s*o10) + s*o11, the raster order of the CPU loop.
+template<int VX, bool FORWARD>
+__global__ __launch_bounds__(kBlock) void upsample2_kernel(const float* in, float* acc, float* out, uint32_t units,
+                                                           int w, float scale, FastDiv by_wv, FastDiv by_h)
+{
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= units) return;
+    uint32_t rows, xv, plane, y;
+    by_wv.divmod(t, rows, xv);
+    by_h.divmod(rows, plane, y);
+    const uint32_t x = xv * VX;
+    const uint32_t ii = rows * w + x;                                   // rows = plane*h + y
+    const uint32_t ow = 2 * w;
+    const uint32_t oi = (2 * rows) * ow + 2 * x;                        // (plane*2h + 2y)*2w + 2x
+    if constexpr (FORWARD) {
+        const Pack<VX> v = ld<VX>(in, ii);
+        Pack<2 * VX> o;
+#pragma unroll
+        for (int k = 0; k < VX; ++k) {
+            const float s = scale * v.v[k];
+            o.v[2 * k] = s;
+            o.v[2 * k + 1] = s;
+        }
+        st<2 * VX>(out, oi, o);
+        st<2 * VX>(out, oi + ow, o);
+    } else {
+        Pack<VX> a = ld<VX>(acc, ii);
+        const Pack<2 * VX> r0 = ld<2 * VX>(out, oi);
+        const Pack<2 * VX> r1 = ld<2 * VX>(out, oi + ow);
+#pragma unroll
+        for (int k = 0; k < VX; ++k) {
+            float g = a.v[k];
+            float p = scale * r0.v[2 * k];
+            g = g + p;
+            p = scale * r0.v[2 * k + 1];
+            g = g + p;
+            p = scale * r1.v[2 * k];
+            g = g + p;
+            p = scale * r1.v[2 * k + 1];
+            g = g + p;
+            a.v[k] = g;
+        }
+        st<VX>(acc, ii, a);
+    }
+}
+
+// any stride: one input cell per lane
+template<bool FORWARD>
+__global__ __launch_bounds__(kBlock) void upsample_generic_kernel(const float* in, float* acc, float* out,
+                                                                  uint32_t total, int w, int stride, float scale,
+                                                                  FastDiv by_w)
+{
+    const uint32_t cell = blockIdx.x * kBlock + threadIdx.x;
+    if (cell >= total) return;
+    uint32_t rows, x;
+    by_w.divmod(cell, rows, x);
+    const size_t ow = static_cast<size_t>(w) * stride;
+    const size_t o0 = static_cast<size_t>(rows) * stride * ow + static_cast<size_t>(x) * stride;
+    if constexpr (FORWARD) {
+        const float s = scale * in[cell];
+        for (int dy = 0; dy < stride; ++dy)
+            for (int dx = 0; dx < stride; ++dx) out[o0 + dy * ow + dx] = s;
+    } else {
+        float g = acc[cell];
+        for (int dy = 0; dy < stride; ++dy)
+            for (int dx = 0; dx < stride; ++dx) {
+                const float p = scale * out[o0 + dy * ow + dx];
+                g = g + p;
+            }
+        acc[cell] = g;
+    }
+}
+
+int check_pool_args(const char* who, int batch, int channels, int ih, int iw, int oh, int ow, int kernel, int stride,
+                    int padding)
+{
+    if (batch <= 0 || channels <= 0 || ih <= 0 || iw <= 0 || oh <= 0 || ow <= 0)
+        return fail_invalid("%s: dimensions must be positive", who);
+    if (kernel <= 0) return fail_invalid("%s: MaxPool kernel must be positive", who);
+    if (stride <= 0) return fail_invalid("%s: MaxPool stride must be positive", who);
+    if (padding < 0) return fail_invalid("%s: MaxPool padding cannot be negative", who);
+    const unsigned long long in_total = 1ull * batch * channels * ih * iw;
+    const unsigned long long out_total = 1ull * batch * channels * oh * ow;
+    if (in_total >= (1ull << 31) || out_total >= (1ull << 31)) {
+        // the index tensor is int32: larger inputs cannot be represented by the layer at all
+        set_error("%s: tensors of 2^31 elements or more are not supported", who);
+        return PXH_ERR_UNSUPPORTED;
+    }
+    return PXH_OK;
+}
+
+// all windows 2x2, stride 2, inside the input
+bool is_2x2_inbounds(int ih, int iw, int oh, int ow, int kernel, int stride, int padding)
+{
+    return kernel == 2 && stride == 2 && padding <= 1 && ih % 2 == 0 && iw % 2 == 0 && oh == ih / 2 && ow == iw / 2;
+}
+
+}  // namespace
+}  // namespace pxh
+
+using namespace pxh;
+
+extern "C" {
+
+int pxh_maxpool_forward(const float* in, float* out, int* indexes, int batch, int channels, int ih, int iw, int oh,
+                        int ow, int kernel, int stride, int padding, void* stream)
+{
+    if (!in || !out || !indexes) return fail_invalid("pxh_maxpool_forward: null pointer");
+    int rc = check_pool_args("pxh_maxpool_forward", batch, channels, ih, iw, oh, ow, kernel, stride, padding);
+    if (rc) return rc;
+    hipStream_t s = as_stream(stream);
+    const uint32_t planes = static_cast<uint32_t>(batch) * channels;
+    const uint32_t total = planes * oh * ow;
+    if (is_2x2_inbounds(ih, iw, oh, ow, kernel, stride, padding) && aligned16(in) && aligned16(out) &&
+        aligned16(indexes)) {
+        if (iw % 8 == 0) {
+            const uint32_t units = total / 4;
+            hipLaunchKernelGGL((maxpool_fwd_2x2_kernel<4>), dim3(grid_for(units, kBlock)), dim3(kBlock), 0, s, in, out,
+                               indexes, units, iw, ow, FastDiv(ow / 4), FastDiv(oh));
+        } else if (iw % 4 == 0) {
+            const uint32_t units = total / 2;
+            hipLaunchKernelGGL((maxpool_fwd_2x2_kernel<2>), dim3(grid_for(units, kBlock)), dim3(kBlock), 0, s, in, out,
+                               indexes, units, iw, ow, FastDiv(ow / 2), FastDiv(oh));
+        } else {
+            hipLaunchKernelGGL((maxpool_fwd_2x2_kernel<1>), dim3(grid_for(total, kBlock)), dim3(kBlock), 0, s, in, out,
+                               indexes, total, iw, ow, FastDiv(ow), FastDiv(oh));
+        }
+        return check_launch("pxh_maxpool_forward");
+    }
+    const PoolGeom g{ ih, iw, oh, ow, kernel, stride, -padding / 2 };
+    hipLaunchKernelGGL(maxpool_fwd_generic_kernel, dim3(grid_for(total, kBlock)), dim3(kBlock), 0, s, in, out, indexes,
+                       total, g, FastDiv(ow), FastDiv(oh));
+    return check_launch("pxh_maxpool_forward");
+}
+
+int pxh_maxpool_backward(const float* delta, const int* indexes, float* grad, int batch, int channels, int ih, int iw,
+                         int oh, int ow, int kernel, int stride, int padding, void* stream)
+{
+    if (!delta || !indexes || !grad) return fail_invalid("pxh_maxpool_backward: null pointer");
+    int rc = check_pool_args("pxh_maxpool_backward", batch, channels, ih, iw, oh, ow, kernel, stride, padding);
+    if (rc) return rc;
+    hipStream_t s = as_stream(stream);
+    const uint32_t planes = static_cast<uint32_t>(batch) * channels;
+    const uint32_t out_total = planes * oh * ow;
+    if (is_2x2_inbounds(ih, iw, oh, ow, kernel, stride, padding) && aligned16(delta) && aligned16(indexes) &&
+        aligned16(grad)) {
+        if (iw % 8 == 0) {
+            const uint32_t units = out_total / 4;
+            hipLaunchKernelGGL((maxpool_bwd_2x2_kernel<4>), dim3(grid_for(units, kBlock)), dim3(kBlock), 0, s, delta,
+                               indexes, grad, units, iw, ow, FastDiv(ow / 4), FastDiv(oh));
+        } else if (iw % 4 == 0) {
+            const uint32_t units = out_total / 2;
+            hipLaunchKernelGGL((maxpool_bwd_2x2_kernel<2>), dim3(grid_for(units, kBlock)), dim3(kBlock), 0, s, delta,
+                               indexes, grad, units, iw, ow, FastDiv(ow / 2), FastDiv(oh));
+        } else {
+            hipLaunchKernelGGL((maxpool_bwd_2x2_kernel<1>), dim3(grid_for(out_total, kBlock)), dim3(kBlock), 0, s,
+                               delta, indexes, grad, out_total, iw, ow, FastDiv(ow), FastDiv(oh));
+        }
+        return check_launch("pxh_maxpool_backward");
+    }
+    const PoolGeom g{ ih, iw, oh, ow, kernel, stride, -padding / 2 };
+    const uint32_t in_total = planes * ih * iw;
+    hipLaunchKernelGGL(maxpool_bwd_generic_kernel, dim3(grid_for(in_total, kBlock)), dim3(kBlock), 0, s, delta,
+                       indexes, grad, in_total, g, FastDiv(iw), FastDiv(ih));
+    return check_launch("pxh_maxpool_backward");
+}
+
+int pxh_maxpool_backward_scatter(const float* delta, const int* indexes, float* grad, int size, void* stream)
+{
+    if (size < 0 || ((!delta || !indexes || !grad) && size)) return fail_invalid("pxh_maxpool_backward_scatter: bad argument");
+    if (size == 0) return PXH_OK;
+    hipLaunchKernelGGL(maxpool_bwd_scatter_kernel, dim3(grid_for(size, kBlock)), dim3(kBlock), 0, as_stream(stream),
+                       delta, indexes, grad, size);
+    return check_launch("pxh_maxpool_backward_scatter");
+}
+
+int pxh_upsample(const float* in, int w, int h, int c, int batch, int stride, int forward, float scale, float* acc,
+                 float* out, void* stream)
+{
+    if (w <= 0 || h <= 0 || c <= 0 || batch <= 0 || stride <= 0)
+        return fail_invalid("pxh_upsample: dimensions and stride must be positive");
+    if (!out || (forward && !in) || (!forward && !acc)) return fail_invalid("pxh_upsample: null pointer");
+    const unsigned long long out_total = 1ull * batch * c * h * w * stride * stride;
+    if (out_total >= (1ull << 31)) {
+        set_error("pxh_upsample: tensors of 2^31 elements or more are not supported");
+        return PXH_ERR_UNSUPPORTED;
+    }
+    hipStream_t s = as_stream(stream);
+    const uint32_t total = static_cast<uint32_t>(batch) * c * h * w;
+    const float* small = forward ? in : acc;
+    if (stride == 2 && aligned16(small) && aligned16(out)) {
+        // VX inputs per lane; the input vector needs 4*VX-byte alignment of every row start
+        const int vx = (w % 4 == 0) ? 4 : (w % 2 == 0 ? 2 : 1);
+        const uint32_t units = total / vx;
+        const dim3 grid(grid_for(units, kBlock));
+#define PXH_UPSAMPLE2(VX, FWD)                                                                              \
+        hipLaunchKernelGGL((upsample2_kernel<VX, FWD>), grid, dim3(kBlock), 0, s, in, acc, out, units, w, \
+                           scale, FastDiv(w / VX), FastDiv(h))
+        if (forward) {
+            if (vx == 4) PXH_UPSAMPLE2(4, true); else if (vx == 2) PXH_UPSAMPLE2(2, true); else PXH_UPSAMPLE2(1, true);
+        } else {
+            if (vx == 4) PXH_UPSAMPLE2(4, false); else if (vx == 2) PXH_UPSAMPLE2(2, false); else PXH_UPSAMPLE2(1, false);
+        }
+#undef PXH_UPSAMPLE2
+        return check_launch("pxh_upsample");
+    }
+    const dim3 grid(grid_for(total, kBlock));
+    if (forward) {
+        hipLaunchKernelGGL((upsample_generic_kernel<true>), grid, dim3(kBlock), 0, s, in, acc, out, total, w, stride,
+                           scale, FastDiv(w));
+    } else {
+        hipLaunchKernelGGL((upsample_generic_kernel<false>), grid, dim3(kBlock), 0, s, in, acc, out, total, w, stride,
+                           scale, FastDiv(w));
+    }
+    return check_launch("pxh_upsample");
+}
+
+}

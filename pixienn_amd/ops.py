@@ -1,0 +1,253 @@
+"""Torch-tensor front-end over the C ABI: argument checking and stream plumbing only.
+
+Every function launches on torch's current HIP stream and returns without synchronising.
+Tensors must be fp32 (int32 for indices), contiguous and on a HIP device.
+"""
+import numpy as np
+import torch
+
+from . import capi
+from .capi import PxError, act_id, call, ptr
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _chk(t, dtype=torch.float32, name="tensor"):
+    if t is None:
+        return
+    if not isinstance(t, torch.Tensor):
+        raise PxError("%s: torch.Tensor expected" % name)
+    if not t.is_cuda:
+        raise PxError("%s must live on the GPU (got %s); there is no CPU path" % (name, t.device))
+    if t.dtype != dtype:
+        raise PxError("%s must be %s (got %s)" % (name, dtype, t.dtype))
+    if not t.is_contiguous():
+        raise PxError("%s must be contiguous" % name)
+
+
+def _chk_all(*ts):
+    for t in ts:
+        _chk(t)
+
+
+def _nchw(x):
+    if x.dim() != 4:
+        raise PxError("NCHW tensor expected, got %d dims" % x.dim())
+    n, c, h, w = x.shape
+    return n, c, h * w
+
+
+# ---------------------------------------------------------------- epilogue forward
+def bn_infer_act_forward(x, y, rolling_mean, rolling_var, scale, bias, activation, pre_activation=None):
+    _chk_all(x, y, rolling_mean, rolling_var, scale, bias, pre_activation)
+    n, c, s = _nchw(x)
+    call("pxh_bn_infer_act_forward", ptr(x), ptr(y), ptr(pre_activation), ptr(rolling_mean), ptr(rolling_var),
+         ptr(scale), ptr(bias), n, c, s, act_id(activation), _stream())
+    return y
+
+
+def bias_act_forward(x, y, bias, activation, pre_activation=None):
+    _chk_all(x, y, bias, pre_activation)
+    n, c, s = _nchw(x)
+    call("pxh_bias_act_forward", ptr(x), ptr(y), ptr(pre_activation), ptr(bias), n, c, s, act_id(activation),
+         _stream())
+    return y
+
+
+def bn_workspace_bytes(batch, channels, spatial):
+    return int(capi.load().pxh_bn_workspace_bytes(batch, channels, spatial))
+
+
+def bn_train_act_forward(x, y, mean, var, rolling_mean, rolling_var, scale, bias, activation,
+                         pre_activation=None, x_saved=None, x_norm=None, workspace=None):
+    _chk_all(x, y, mean, var, rolling_mean, rolling_var, scale, bias, pre_activation, x_saved, x_norm)
+    n, c, s = _nchw(x)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("pxh_bn_train_act_forward", ptr(x), ptr(y), ptr(pre_activation), ptr(x_saved), ptr(x_norm), ptr(mean),
+         ptr(var), ptr(rolling_mean), ptr(rolling_var), ptr(scale), ptr(bias), n, c, s, act_id(activation),
+         ptr(workspace), wb, _stream())
+    return y
+
+
+def bn_stats(x, mean, var, workspace=None):
+    _chk_all(x, mean, var)
+    n, c, s = _nchw(x)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("pxh_bn_stats", ptr(x), ptr(mean), ptr(var), n, c, s, ptr(workspace), wb, _stream())
+
+
+# ---------------------------------------------------------------- epilogue backward
+def bn_act_backward(delta, x, mean, var, scale, bias, scale_updates, bias_updates, activation,
+                    pre_activation=None, mean_delta=None, var_delta=None, workspace=None):
+    _chk_all(delta, x, mean, var, scale, bias, scale_updates, bias_updates, pre_activation, mean_delta, var_delta)
+    n, c, s = _nchw(delta)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("pxh_bn_act_backward", ptr(delta), ptr(x), ptr(pre_activation), ptr(mean), ptr(var), ptr(scale), ptr(bias),
+         ptr(scale_updates), ptr(bias_updates), ptr(mean_delta), ptr(var_delta), n, c, s, act_id(activation),
+         ptr(workspace), wb, _stream())
+    return delta
+
+
+def bias_act_backward(delta, pre_activation, bias_updates, activation, workspace=None):
+    _chk_all(delta, pre_activation, bias_updates)
+    n, c, s = _nchw(delta)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("pxh_bias_act_backward", ptr(delta), ptr(pre_activation), ptr(bias_updates), n, c, s, act_id(activation),
+         ptr(workspace), wb, _stream())
+    return delta
+
+
+# ---------------------------------------------------------------- stand-alone pieces
+def activate(activation, x):
+    _chk(x)
+    call("pxh_activate", act_id(activation), ptr(x), x.numel(), _stream())
+    return x
+
+
+def gradient(activation, x, delta):
+    _chk_all(x, delta)
+    call("pxh_gradient", act_id(activation), ptr(x), x.numel(), ptr(delta), _stream())
+    return delta
+
+
+def add_bias(output, bias, batch, n, size):
+    _chk_all(output, bias)
+    call("pxh_add_bias", ptr(output), ptr(bias), batch, n, size, _stream())
+
+
+def backward_bias(bias_updates, delta, batch, n, size):
+    _chk_all(bias_updates, delta)
+    call("pxh_backward_bias", ptr(bias_updates), ptr(delta), batch, n, size, None, 0, _stream())
+
+
+def fill(x, value):
+    if x.dtype == torch.int32:
+        _chk(x, torch.int32)
+        call("pxh_fill_i32", ptr(x), x.numel(), int(value), _stream())
+    else:
+        _chk(x)
+        call("pxh_fill_f32", ptr(x), x.numel(), float(value), _stream())
+    return x
+
+
+def constrain(alpha, x):
+    _chk(x)
+    call("pxh_constrain", x.numel(), float(alpha), ptr(x), _stream())
+
+
+def mul(x, y):
+    _chk_all(x, y)
+    call("pxh_mul", x.numel(), ptr(x), ptr(y), _stream())
+
+
+def axpy(alpha, x, y):
+    _chk_all(x, y)
+    call("pxh_axpy", x.numel(), float(alpha), ptr(x), ptr(y), _stream())
+
+
+# ---------------------------------------------------------------- max-pool / upsample / shortcut
+def maxpool_out_dim(n, kernel, stride, padding):
+    """include/MaxPoolLayer.h:62-63 of the reference."""
+    return (n + padding - kernel) // stride + 1
+
+
+def maxpool_forward(x, out, indexes, kernel, stride, padding):
+    _chk_all(x, out)
+    _chk(indexes, torch.int32, "indexes")
+    n, c, ih, iw = x.shape
+    oh, ow = out.shape[2], out.shape[3]
+    call("pxh_maxpool_forward", ptr(x), ptr(out), ptr(indexes), n, c, ih, iw, oh, ow, kernel, stride, padding,
+         _stream())
+
+
+def maxpool_backward(delta, indexes, grad, kernel, stride, padding):
+    _chk_all(delta, grad)
+    _chk(indexes, torch.int32, "indexes")
+    n, c, ih, iw = grad.shape
+    oh, ow = delta.shape[2], delta.shape[3]
+    call("pxh_maxpool_backward", ptr(delta), ptr(indexes), ptr(grad), n, c, ih, iw, oh, ow, kernel, stride, padding,
+         _stream())
+
+
+def maxpool_backward_scatter(delta, indexes, grad):
+    _chk_all(delta, grad)
+    _chk(indexes, torch.int32, "indexes")
+    call("pxh_maxpool_backward_scatter", ptr(delta), ptr(indexes), ptr(grad), delta.numel(), _stream())
+
+
+def upsample_forward(x, out, stride=2, scale=1.0):
+    _chk_all(x, out)
+    n, c, h, w = x.shape
+    call("pxh_upsample", ptr(x), w, h, c, n, stride, 1, float(scale), None, ptr(out), _stream())
+
+
+def upsample_backward(delta, grad, stride=2, scale=1.0):
+    _chk_all(delta, grad)
+    n, c, h, w = grad.shape
+    call("pxh_upsample", None, w, h, c, n, stride, 0, float(scale), ptr(grad), ptr(delta), _stream())
+
+
+def shortcut(batch, w1, h1, c1, add, w2, h2, c2, s1, s2, out):
+    _chk_all(add, out)
+    call("pxh_shortcut", batch, w1, h1, c1, ptr(add), w2, h2, c2, float(s1), float(s2), ptr(out), _stream())
+
+
+def shortcut_forward(inp, from_output, output, activation="linear", alpha=1.0, beta=1.0, pre_activation=None):
+    _chk_all(inp, from_output, output, pre_activation)
+    call("pxh_shortcut_forward", ptr(inp), ptr(from_output), ptr(output), ptr(pre_activation), inp.numel(),
+         float(alpha), float(beta), act_id(activation), _stream())
+
+
+def shortcut_backward(delta, from_delta, grad=None, activation="linear", alpha=1.0, beta=1.0, pre_activation=None):
+    _chk_all(delta, from_delta, grad, pre_activation)
+    call("pxh_shortcut_backward", ptr(delta), ptr(pre_activation), ptr(from_delta), ptr(grad), delta.numel(),
+         float(alpha), float(beta), act_id(activation), _stream())
+
+
+# ---------------------------------------------------------------- YOLO head
+def yolo_activate(inp, out, batch, masks, classes, area):
+    _chk_all(inp, out)
+    call("pxh_yolo_activate", ptr(inp), ptr(out), batch, masks, classes, area, _stream())
+
+
+def yolo_forward_train(inp, out, delta, truths, truth_counts, max_truth, masks, anchors, stats, cost, batch, classes,
+                       width, height, net_width, net_height, ignore_thresh, truth_thresh, coord_scale=1.0,
+                       object_scale=1.0, noobject_scale=1.0, class_scale=1.0, workspace=None):
+    _chk_all(inp, out, delta, truths, stats, cost)
+    _chk(truth_counts, torch.int32, "truth_counts")
+    m = np.ascontiguousarray(masks, dtype=np.int32)
+    a = np.ascontiguousarray(anchors, dtype=np.int32)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("pxh_yolo_forward_train", ptr(inp), ptr(out), ptr(delta), ptr(truths), ptr(truth_counts), int(max_truth),
+         m.ctypes.data, a.ctypes.data, ptr(stats), ptr(cost), batch, len(m), len(a) // 2, classes, width, height,
+         net_width, net_height, float(ignore_thresh), float(truth_thresh), float(coord_scale), float(object_scale),
+         float(noobject_scale), float(class_scale), ptr(workspace), wb, _stream())
+
+
+def yolo_loss(output, delta, truths, truth_counts, max_truth, assigned_classes, assigned_anchors, assigned_boxes,
+              masks, anchors, stats, cost, batch, anchor_count, classes, width, height, net_width, net_height,
+              ignore_thresh, truth_thresh, coord_scale, object_scale, noobject_scale, class_scale):
+    _chk_all(output, delta, truths, assigned_boxes, anchors, stats, cost)
+    for t, nm in ((truth_counts, "truth_counts"), (assigned_classes, "assigned_classes"),
+                  (assigned_anchors, "assigned_anchors"), (masks, "masks")):
+        _chk(t, torch.int32, nm)
+    call("pxh_yolo_loss", ptr(output), ptr(delta), ptr(truths), ptr(truth_counts), int(max_truth),
+         ptr(assigned_classes), ptr(assigned_anchors), ptr(assigned_boxes), ptr(masks), ptr(anchors), ptr(stats),
+         ptr(cost), batch, masks.numel(), anchor_count, classes, width, height, net_width, net_height,
+         float(ignore_thresh), float(truth_thresh), float(coord_scale), float(object_scale), float(noobject_scale),
+         float(class_scale), None, 0, _stream())
+
+
+# ---------------------------------------------------------------- Adam
+def adam(x, m, v, beta1, beta2, rate, eps, t):
+    _chk_all(x, m, v)
+    call("pxh_adam", x.numel(), ptr(x), ptr(m), ptr(v), float(beta1), float(beta2), float(rate), float(eps), int(t),
+         _stream())
+
+
+def adam_update(w, d, m, v, batch, t, lr, beta1=0.9, beta2=0.999, eps=1e-8, decay=0.0, apply_decay=False):
+    _chk_all(w, d, m, v)
+    call("pxh_adam_update", w.numel(), ptr(w), ptr(d), ptr(m), ptr(v), int(batch), int(t), float(lr), float(beta1),
+         float(beta2), float(eps), float(decay), int(bool(apply_decay)), _stream())

@@ -1,0 +1,63 @@
+"""Layer shapes of the benchmark configurations and seeded synthetic inputs.
+
+Shapes follow the reference's model files (resources/models/yolov3.yml, yolov3-tiny.yml) and
+the synthetic shapes the baseline names.  Inputs come from numpy's counter-based Philox
+generator, so the same seed gives the same bits on every host.
+"""
+import numpy as np
+
+# (channels, height == width) of every BN'd conv output
+YOLOV3_TINY_CONV_SHAPES = [(16, 416), (32, 208), (64, 104), (128, 52), (256, 26), (512, 13), (1024, 13)]
+TINY_ANCHORS = [10, 14, 23, 27, 37, 58, 81, 82, 135, 169, 344, 319]
+TINY_MASKS = [[3, 4, 5], [0, 1, 2]]
+
+# YOLOv3 @608: distinct BN'd conv-output shapes (channels, size) and how many conv layers have each
+YOLOV3_BN_SHAPES = [(32, 608), (64, 304), (32, 304), (128, 152), (64, 152), (256, 76), (128, 76),
+                    (512, 38), (256, 38), (128, 38), (1024, 19), (512, 19), (256, 19)]
+# number of conv layers of yolov3.yml with each of those output shapes (72 BN'd convs in all)
+YOLOV3_BN_COUNTS = [1, 2, 1, 3, 2, 12, 11, 12, 11, 1, 8, 7, 1]
+# the three linear (bias only) 255-channel convs in front of the heads
+YOLOV3_HEAD_CONV_SHAPES = [(255, 19), (255, 38), (255, 76)]
+YOLOV3_SHORTCUT_SHAPES = [(64, 304, 1), (128, 152, 2), (256, 76, 8), (512, 38, 8), (1024, 19, 4)]
+YOLOV3_MAXPOOL_SHAPES = [(64, 304), (128, 152), (256, 76), (512, 38)]
+YOLOV3_UPSAMPLE_SHAPES = [(256, 19), (128, 38)]
+YOLOV3_HEAD_SIZES = [19, 38, 76]
+YOLOV3_ANCHORS = [10, 13, 16, 30, 33, 23, 30, 61, 62, 45, 59, 119, 116, 90, 156, 198, 373, 326]
+YOLOV3_MASKS = {19: [6, 7, 8], 38: [3, 4, 5], 76: [0, 1, 2]}
+YOLOV3_PARAMS = 61949149   # conv weights + biases + BN scales
+
+
+def rng(seed):
+    return np.random.Generator(np.random.Philox(key=int(seed)))
+
+
+def normal(seed, shape, mean=0.0, std=1.0):
+    return (rng(seed).standard_normal(shape, dtype=np.float32) * np.float32(std) + np.float32(mean)).astype(np.float32)
+
+
+def uniform(seed, shape, lo=0.0, hi=1.0):
+    return rng(seed).uniform(lo, hi, shape).astype(np.float32)
+
+
+def bn_params(seed, channels):
+    """gamma = 1, beta ~ N(0, 0.1), running mean ~ N(0, 0.1), running var ~ U(0.5, 1.5)."""
+    g = rng(seed)
+    scale = np.ones(channels, np.float32)
+    bias = (0.1 * g.standard_normal(channels)).astype(np.float32)
+    mean = (0.1 * g.standard_normal(channels)).astype(np.float32)
+    var = g.uniform(0.5, 1.5, channels).astype(np.float32)
+    return scale, bias, mean, var
+
+
+def yolo_truths(seed, batch, max_boxes=20, classes=80):
+    """1..max_boxes boxes per image: centres U(0,1), w/h log-uniform in [0.02, 0.9], class uniform.
+    Returns (truths[batch, max_boxes, 5], counts[batch])."""
+    g = rng(seed)
+    counts = g.integers(1, max_boxes + 1, batch).astype(np.int32)
+    truths = np.zeros((batch, max_boxes, 5), np.float32)
+    for b in range(batch):
+        k = int(counts[b])
+        truths[b, :k, 0:2] = g.uniform(0.0, 1.0, (k, 2))
+        truths[b, :k, 2:4] = np.exp(g.uniform(np.log(0.02), np.log(0.9), (k, 2)))
+        truths[b, :k, 4] = g.integers(0, classes, k)
+    return truths, counts

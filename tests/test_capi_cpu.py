@@ -1,0 +1,91 @@
+"""CPU-side checks of the C-ABI library: it loads, exports what include/pixienn_hip.h declares,
+and rejects bad calls before anything is launched.  No compute, no GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from pixienn_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "pixienn_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pxh_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    names = header_symbols()
+    assert len(names) >= 30
+    for n in names:
+        assert hasattr(lib, n), "missing export: " + n
+    # the Python binding covers the whole header, nothing more, nothing less
+    assert sorted(names) == capi.declared_symbols()
+
+
+def test_abi_version():
+    assert capi.load().pxh_abi_version() == 1
+
+
+def test_fastdiv_matches_integer_division():
+    lib = capi.load()
+    divisors = [1, 2, 3, 5, 7, 13, 19, 64, 85, 169, 255, 256, 361, 676, 1444, 4096, 5776, 92416, 369664, 2 ** 20 + 1,
+                2 ** 30 - 1]
+    for d in divisors:
+        for n in [0, 1, d - 1, d, d + 1, 2 * d - 1, 2 * d, 12345678, 2 ** 31 - 1, 2 ** 31 - d, 189267968]:
+            if 0 <= n < 2 ** 31:
+                assert lib.pxh_debug_fastdiv(n, d) == n // d, (n, d)
+    import random
+    r = random.Random(3)
+    for _ in range(20000):
+        d = r.randint(1, 2 ** 22)
+        n = r.randint(0, 2 ** 31 - 1)
+        assert lib.pxh_debug_fastdiv(n, d) == n // d, (n, d)
+
+
+def test_rejects_bad_arguments_without_launching():
+    inv = -1
+    # dummy non-null addresses: validation happens before any device access
+    p = 256
+    assert capi.call_raw("pxh_activate", 0, None, 5, None) == inv
+    assert capi.call_raw("pxh_activate", 99, p, 5, None) == inv
+    assert "unknown activation" in capi.last_error()
+    assert capi.call_raw("pxh_bn_infer_act_forward", p, p, None, p, p, p, p, 0, 3, 4, 0, None) == inv
+    assert capi.call_raw("pxh_bn_infer_act_forward", p, p, None, None, p, p, p, 1, 3, 4, 0, None) == inv
+    # the reference's maxpool constructor checks (include/MaxPoolLayer.h:57-59)
+    assert capi.call_raw("pxh_maxpool_forward", p, p, p, 1, 1, 4, 4, 2, 2, 0, 2, 1, None) == inv
+    assert "kernel must be positive" in capi.last_error()
+    assert capi.call_raw("pxh_maxpool_forward", p, p, p, 1, 1, 4, 4, 2, 2, 2, 0, 1, None) == inv
+    assert "stride must be positive" in capi.last_error()
+    assert capi.call_raw("pxh_maxpool_forward", p, p, p, 1, 1, 4, 4, 2, 2, 2, 2, -1, None) == inv
+    assert "padding cannot be negative" in capi.last_error()
+    # the reference's shortcut checks (include/ShortcutLayer.h:123-124)
+    assert capi.call_raw("pxh_shortcut", 1, 4, 4, 1, p, 2, 4, 1, 1.0, 1.0, p, None) == inv
+    assert "equal in x and y" in capi.last_error()
+    assert capi.call_raw("pxh_adam_update", 8, p, p, p, p, 0, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 0, None) == inv
+    assert capi.call_raw("pxh_adam_update", 8, p, p, p, p, 1, 0, 1e-3, 0.9, 0.999, 1e-8, 0.0, 0, None) == inv
+    # tensors of 2^31 elements or more are refused, not mis-indexed
+    assert capi.call_raw("pxh_bn_infer_act_forward", p, p, None, p, p, p, p, 1024, 1024, 4096, 0, None) == -2
+    with pytest.raises(capi.PxError):
+        capi.call("pxh_activate", 0, None, 5, None)
+
+
+def test_workspace_sizes():
+    lib = capi.load()
+    assert lib.pxh_bn_workspace_bytes(0, 1, 1) == 0
+    small = lib.pxh_bn_workspace_bytes(16, 256, 361)
+    big = lib.pxh_bn_workspace_bytes(16, 32, 608 * 608)
+    assert 0 < small < big < (1 << 24)
+    assert lib.pxh_yolo_workspace_bytes(64, 3, 80, 76, 76) == 64 * 3 * 23 * 13 * 8
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+    from pixienn_amd import ops
+    x = torch.zeros(1, 2, 4, 4)
+    with pytest.raises(capi.PxError):
+        ops.activate("leaky", x)

@@ -1,0 +1,262 @@
+"""GPU parity: conv-layer epilogue (BN inference/training + bias + activation, forward and
+backward) against the CPU checker on the same seeded inputs, through the C ABI.
+
+Tolerance (stated by the task for BN/activation): 1e-5 relative.  An element whose value is
+the difference of larger intermediates (x_hat*scale + bias cancelling, a sum of deltas) is
+bounded relative to those intermediates: that is the `floor` argument of assert_close.
+"""
+import numpy as np
+import pytest
+
+from pixienn_amd import workloads as wl
+from util import F, assert_bit_exact, assert_close, gpu, host, ulp_distance
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-5
+# loggy = 2*sigmoid(x) - 1 cancels against 1 near x = 0: its error is bounded relative to 1
+FLOOR = {"loggy": 1.0}
+ACTS = ["leaky", "linear", "loggy", "logistic", "mish", "relu", "softplus", "swish", "tanh"]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from pixienn_amd import ops as o
+    return o
+
+
+def bn_case(seed, N, C, HW, spread=1.0):
+    x = wl.normal(seed, (N, C, HW, 1), std=spread)
+    scale, bias, mean, var = wl.bn_params(seed + 1, C)
+    scale = (scale + 0.25 * wl.normal(seed + 2, C)).astype(F)
+    return x, scale, bias, mean, var
+
+
+# spatial sizes cover: 128-bit fast path, planes that are not a multiple of 4 (13x13, 19x19),
+# several planes per workgroup, planes below the fast-path limit, single elements
+SHAPES = [(2, 16, 416 * 416 // 16), (3, 32, 52 * 52), (4, 64, 26 * 26), (5, 7, 169), (3, 11, 361),
+          (2, 5, 28), (2, 5, 27), (3, 4, 1), (1, 1, 4097), (2, 3, 4096), (7, 2, 33)]
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_bn_infer_act_forward_matches_oracle(ops, oracle, act):
+    for si, (N, C, HW) in enumerate(SHAPES):
+        x, scale, bias, rmean, rvar = bn_case(100 + si, N, C, HW)
+        want = x.copy(); pre_want = np.empty_like(x)
+        oracle.conv_epilogue_forward(True, False, act, N, C, HW, 1, want, pre_want, np.zeros(C, F), np.zeros(C, F),
+                                     rmean.copy(), rvar.copy(), scale, bias, None, None)
+        gx = gpu(x); gy = gpu(np.zeros_like(x)); gpre = gpu(np.zeros_like(x))
+        ops.bn_infer_act_forward(gx, gy, gpu(rmean), gpu(rvar), gpu(scale), gpu(bias), act, pre_activation=gpre)
+        what = "%s %s" % (act, (N, C, HW))
+        # the pre-activation is a fixed sequence of exactly rounded fp32/fp64 operations
+        d = ulp_distance(host(gpre), pre_want)
+        assert d.max() <= 1 and (d > 0).mean() < 1e-4, (what, int(d.max()), float((d > 0).mean()))
+        assert_close(host(gy), want, RTOL, FLOOR.get(act, 1e-3), what)
+        if act in ("leaky", "linear", "relu"):
+            d = ulp_distance(host(gy), want)
+            assert d.max() <= 1 and (d > 0).mean() < 1e-4, what
+
+
+def test_bn_infer_in_place_and_unaligned(ops, oracle):
+    import torch
+    N, C, HW = 3, 6, 361
+    x, scale, bias, rmean, rvar = bn_case(200, N, C, HW)
+    want = x.copy()
+    oracle.conv_epilogue_forward(True, False, "leaky", N, C, HW, 1, want, None, np.zeros(C, F), np.zeros(C, F),
+                                 rmean.copy(), rvar.copy(), scale, bias, None, None)
+    gx = gpu(x)
+    ops.bn_infer_act_forward(gx, gx, gpu(rmean), gpu(rvar), gpu(scale), gpu(bias), "leaky")
+    assert_close(host(gx), want, RTOL, 1e-3, "in place")
+    # a view that starts 4 bytes into an allocation: not 16-byte aligned -> scalar kernel
+    buf = torch.zeros(x.size + 1, device="cuda")
+    view = buf[1:].view(N, C, HW, 1)
+    view.copy_(gpu(x))
+    out = torch.zeros(x.size + 1, device="cuda")[1:].view(N, C, HW, 1)
+    assert view.data_ptr() % 16 != 0
+    ops.bn_infer_act_forward(view, out, gpu(rmean), gpu(rvar), gpu(scale), gpu(bias), "leaky")
+    assert_close(host(out), want, RTOL, 1e-3, "unaligned")
+
+
+@pytest.mark.parametrize("act", ["linear", "leaky", "logistic"])
+def test_bias_act_forward_matches_oracle(ops, oracle, act):
+    for si, (N, C, HW) in enumerate([(2, 255, 169), (1, 255, 676), (3, 5, 27), (2, 18, 361)]):
+        x = wl.normal(300 + si, (N, C, HW, 1))
+        bias = wl.normal(310 + si, C, std=0.1)
+        want = x.copy(); pre_want = np.empty_like(x)
+        oracle.conv_epilogue_forward(False, False, act, N, C, HW, 1, want, pre_want, None, None, None, None, None,
+                                     bias, None, None)
+        gy = gpu(np.zeros_like(x)); gpre = gpu(np.zeros_like(x))
+        ops.bias_act_forward(gpu(x), gy, gpu(bias), act, pre_activation=gpre)
+        assert_bit_exact(host(gpre), pre_want, "bias pre " + act)
+        if act == "logistic":
+            assert_close(host(gy), want, RTOL, 1e-6, "bias " + act)
+        else:
+            assert_bit_exact(host(gy), want, "bias " + act)
+    # addBiasGpu signature
+    x = wl.normal(320, (2, 3, 50, 1)); bias = wl.normal(321, 3)
+    want = x.copy(); oracle.add_bias(want, bias, 2, 3, 50)
+    gx = gpu(x); ops.add_bias(gx, gpu(bias), 2, 3, 50)
+    assert_bit_exact(host(gx), want, "add_bias")
+
+
+TRAIN_SHAPES = [(4, 8, 52 * 52), (3, 16, 361), (16, 5, 169), (2, 3, 4096 + 512), (5, 2, 27), (2, 4, 1024 * 3 + 4),
+                (1, 3, 37)]
+
+
+@pytest.mark.parametrize("act", ["leaky", "mish", "linear"])
+def test_bn_train_forward_matches_oracle(ops, oracle, act):
+    for si, (N, C, HW) in enumerate(TRAIN_SHAPES):
+        x, scale, bias, rmean, rvar = bn_case(400 + si, N, C, HW, spread=1.5)
+        x += wl.normal(450 + si, (1, C, 1, 1), std=2.0)          # per-channel offsets
+        want = x.copy(); pre_w = np.empty_like(x); xs_w = np.empty_like(x); xn_w = np.empty_like(x)
+        mean_w = np.zeros(C, F); var_w = np.zeros(C, F); rm_w = rmean.copy(); rv_w = rvar.copy()
+        oracle.conv_epilogue_forward(True, True, act, N, C, HW, 1, want, pre_w, mean_w, var_w, rm_w, rv_w, scale,
+                                     bias, xs_w, xn_w)
+        gy, gpre, gxs, gxn = (gpu(np.zeros_like(x)) for _ in range(4))
+        gm, gv, grm, grv = gpu(np.zeros(C, F)), gpu(np.zeros(C, F)), gpu(rmean), gpu(rvar)
+        ops.bn_train_act_forward(gpu(x), gy, gm, gv, grm, grv, gpu(scale), gpu(bias), act, pre_activation=gpre,
+                                 x_saved=gxs, x_norm=gxn)
+        what = "%s %s" % (act, (N, C, HW))
+        assert_close(host(gm), mean_w, RTOL, 1.0, what + " mean")
+        assert_close(host(gv), var_w, RTOL, 1e-3, what + " var")
+        assert_close(host(grm), rm_w, RTOL, 1e-1, what + " rolling mean")
+        assert_close(host(grv), rv_w, RTOL, 1e-3, what + " rolling var")
+        assert_bit_exact(host(gxs), x, what + " x_saved")
+        # x_hat = (x - mean)/sigma cancels where x is near the mean: the bound is relative to
+        # the operands of that subtraction, (|mean| + sigma)/sigma per channel
+        sigma = np.sqrt(var_w.astype(np.float64))
+        fl = ((np.abs(mean_w) + sigma) / sigma).reshape(1, C, 1, 1)
+        assert_close(host(gxn), xn_w, RTOL, fl, what + " x_norm")
+        fl = fl * np.abs(scale).reshape(1, C, 1, 1) + np.abs(bias).reshape(1, C, 1, 1)
+        assert_close(host(gpre), pre_w, RTOL, fl, what + " pre")
+        assert_close(host(gy), want, RTOL, fl, what + " y")
+        # nullable outputs: same y without materialising the saved tensors
+        gy2 = gpu(np.zeros_like(x))
+        ops.bn_train_act_forward(gpu(x), gy2, gm, gv, gpu(rmean), gpu(rvar), gpu(scale), gpu(bias), act)
+        assert_bit_exact(host(gy2), host(gy), what + " nullable outputs")
+
+
+def test_bn_stats_beats_sequential_fp32_at_scale(ops, oracle):
+    """At 1.3 M elements per channel the reference's left-to-right fp32 sums have drifted from
+    the exact statistics by more than the kernel has: the kernel must sit at least as close
+    to the fp64-accumulated statistics as the fp32 checker does, and within 1e-5 of it."""
+    N, C, HW = 4, 3, 576 * 576
+    x = wl.normal(500, (N, C, HW, 1), std=1.3) + np.array([0.5, -3.0, 10.0], F).reshape(1, C, 1, 1)
+    x = x.astype(F)
+    m32 = np.zeros(C, F); v32 = np.zeros(C, F)
+    oracle.mean(x, N, C, HW, m32); oracle.variance(x, m32, N, C, HW, v32)
+    x64 = x.astype(np.float64)
+    m64 = x64.mean(axis=(0, 2, 3)); v64 = x64.var(axis=(0, 2, 3))
+    gm, gv = gpu(np.zeros(C, F)), gpu(np.zeros(C, F))
+    ops.bn_stats(gpu(x), gm, gv)
+    gm, gv = host(gm), host(gv)
+    assert np.all(np.abs(gm - m64) <= np.abs(m32 - m64) + 1e-7)
+    assert np.all(np.abs(gv - v64) <= np.abs(v32 - v64) + 1e-7 * v64)
+    assert_close(gm, m64, 2e-7, 1.0, "mean vs fp64")
+    assert_close(gv, v64, 1e-6, 1e-3, "var vs fp64")
+
+
+@pytest.mark.parametrize("act", ["leaky", "mish", "linear", "logistic"])
+@pytest.mark.parametrize("with_pre", [True, False])
+def test_bn_backward_matches_oracle(ops, oracle, act, with_pre):
+    for si, (N, C, HW) in enumerate(TRAIN_SHAPES):
+        x, scale, bias, rmean, rvar = bn_case(600 + si, N, C, HW, spread=1.5)
+        delta = wl.normal(650 + si, x.shape)
+        out = x.copy(); pre = np.empty_like(x); xs = np.empty_like(x); xn = np.empty_like(x)
+        mean = np.zeros(C, F); var = np.zeros(C, F)
+        oracle.conv_epilogue_forward(True, True, act, N, C, HW, 1, out, pre, mean, var, rmean.copy(), rvar.copy(),
+                                     scale, bias, xs, xn)
+        su0 = wl.normal(660 + si, C); bu0 = wl.normal(661 + si, C)
+        d_w = delta.copy(); su_w = su0.copy(); bu_w = bu0.copy(); md_w = np.zeros(C, F); vd_w = np.zeros(C, F)
+        oracle.conv_epilogue_backward(True, act, N, C, HW, 1, d_w, pre, mean, var, md_w, vd_w, scale, su_w, bu_w,
+                                      xs, xn)
+        gd = gpu(delta); gsu = gpu(su0); gbu = gpu(bu0); gmd = gpu(np.zeros(C, F)); gvd = gpu(np.zeros(C, F))
+        ops.bn_act_backward(gd, gpu(x), gpu(mean), gpu(var), gpu(scale), gpu(bias), gsu, gbu, act,
+                            pre_activation=gpu(pre) if with_pre else None, mean_delta=gmd, var_delta=gvd)
+        what = "%s pre=%s %s" % (act, with_pre, (N, C, HW))
+        count = N * HW
+        # per-channel sums: relative to the size of the summed terms (norm-wise bound)
+        sum_scale = np.sqrt(count)
+        assert_close(host(gbu) - bu0, bu_w - bu0, RTOL, sum_scale, what + " bias updates")
+        assert_close(host(gsu) - su0, su_w - su0, RTOL, sum_scale, what + " scale updates")
+        assert_close(host(gmd), md_w, RTOL, sum_scale, what + " mean delta")
+        assert_close(host(gvd), vd_w, RTOL, sum_scale, what + " var delta")
+        assert_close(host(gd), d_w, RTOL, 1e-1, what + " dx")
+
+
+@pytest.mark.parametrize("act", ["linear", "leaky", "logistic"])
+def test_bias_backward_matches_oracle(ops, oracle, act):
+    for si, (N, C, HW) in enumerate([(2, 255, 169), (3, 18, 361), (2, 4, 4096), (3, 5, 27)]):
+        pre = wl.normal(700 + si, (N, C, HW, 1))
+        delta = wl.normal(710 + si, pre.shape)
+        bu0 = wl.normal(720 + si, C)
+        d_w = delta.copy(); bu_w = bu0.copy()
+        oracle.conv_epilogue_backward(False, act, N, C, HW, 1, d_w, pre, None, None, None, None, None, None, bu_w,
+                                      None, None)
+        gd = gpu(delta); gbu = gpu(bu0)
+        ops.bias_act_backward(gd, gpu(pre), gbu, act)
+        if act == "logistic":
+            assert_close(host(gd), d_w, RTOL, 1e-6, "bias bwd delta")
+        else:
+            assert_bit_exact(host(gd), d_w, "bias bwd delta " + act)
+        assert_close(host(gbu) - bu0, bu_w - bu0, RTOL, np.sqrt(N * HW), "bias updates " + act)
+    # backwardBiasGpu known answer held by the reference (tests/src/blas.cpp:75-92)
+    gbu = gpu(np.array([0.25, -0.25, 1.0], F))
+    d = np.tile(np.repeat(np.array([1.0, -2.0, 0.5], F), 4), 2)
+    ops.backward_bias(gbu, gpu(d), 2, 3, 4)
+    assert host(gbu).tolist() == [8.25, -16.25, 5.0]
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_activation_kats_and_sweep(ops, oracle, kats, act):
+    for case in kats["activations"]["cases"]:
+        if case["name"] != act:
+            continue
+        x = np.array(case["input"], F)
+        if case["apply"] is not None:
+            got = host(ops.activate(act, gpu(x)))
+            assert np.allclose(got, case["apply"], rtol=4e-7, atol=1e-12), (act, got)
+        got = host(ops.gradient(act, gpu(x), gpu(np.array(case["delta"], F))))
+        assert np.allclose(got, case["gradient"], rtol=1e-5, atol=case.get("gradient_tol", 1e-7)), (act, got)
+    x = np.concatenate([np.linspace(-25, 25, 100001, dtype=F), wl.normal(800, 30001, std=2.0),
+                        np.array([0.0, -0.0, 20.0, -20.0, 20.000002, -20.000002, 60.0, -60.0], F)]).astype(F)
+    d = wl.normal(801, x.size)
+    want = oracle.activate(act, x.copy())
+    got = host(ops.activate(act, gpu(x)))
+    # Conditioning of the CPU formulas themselves: float(1 + e^x) inside softplus/mish carries an
+    # absolute error of an ulp of 1, scaled by |x| in mish; y*(1-y), 1-y*y and the swish
+    # derivative cancel against 1.  A 1-ulp difference between two libm expf/tanhf therefore
+    # shows as 3e-7 absolute (times |x| or |delta|), which the floors below express as 1e-5 of
+    # 0.03; everything else is held to 1e-5 of the value itself (floor 1e-6).
+    ax = np.maximum(1.0, np.abs(x.astype(np.float64)))
+    fl = {"loggy": 1.0, "softplus": 0.03 * ax, "mish": 0.03 * ax}.get(act, 1e-6)
+    assert_close(got, want, RTOL, fl, act + " apply sweep")
+    wantg = oracle.gradient(act, x, d.copy())
+    gotg = host(ops.gradient(act, gpu(x), gpu(d)))
+    flg = 1e-6 if act in ("leaky", "linear", "relu") else np.maximum(0.03 * np.abs(d.astype(np.float64)) * ax, 1e-6)
+    assert_close(gotg, wantg, RTOL, flg, act + " gradient sweep")
+    # odd length + unaligned start exercise the tail and scalar kernels
+    import torch
+    buf = torch.zeros(1003, device="cuda")
+    v = buf[3:]
+    v.copy_(gpu(x[:1000]))
+    ops.activate(act, v)
+    assert_close(host(v), want[:1000], RTOL, fl if np.isscalar(fl) else fl[:1000], act + " unaligned")
+
+
+def test_helper_kernels(ops, oracle):
+    import torch
+    x = wl.normal(900, 10007)
+    g = gpu(x.copy()); ops.constrain(0.5, g)
+    w = x.copy(); oracle.constrain(0.5, w)
+    assert_bit_exact(host(g), w, "constrain")
+    y = wl.normal(901, 10007)
+    gy = gpu(y.copy()); ops.mul(gpu(x), gy)
+    assert_bit_exact(host(gy), x * y, "mul")       # tests/src/vector.cpp:107-117 semantics: y = x*y
+    gy = gpu(y.copy()); ops.axpy(0.75, gpu(x), gy)
+    w = y.copy(); oracle.axpy(0.75, x, w)
+    assert_bit_exact(host(gy), w, "axpy")
+    f = torch.empty(1001, device="cuda"); ops.fill(f, 2.5)
+    assert bool((f == 2.5).all())
+    i = torch.empty(1001, device="cuda", dtype=torch.int32); ops.fill(i, -1)
+    assert bool((i == -1).all())

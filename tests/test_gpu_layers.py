@@ -1,0 +1,160 @@
+"""GPU parity: max-pool, upsample and shortcut, forward and backward, bit-exact against the CPU
+checker (values, int32 indices and accumulation order), through the C ABI."""
+import numpy as np
+import pytest
+
+from pixienn_amd import workloads as wl
+from util import F, assert_bit_exact, gpu, host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from pixienn_amd import ops as o
+    return o
+
+
+def run_maxpool(ops, oracle, x, kernel, stride, padding, seed):
+    import torch
+    N, C, H, W = x.shape
+    oh = oracle.maxpool_out_dim(H, kernel, stride, padding)
+    ow = oracle.maxpool_out_dim(W, kernel, stride, padding)
+    assert oh == ops.maxpool_out_dim(H, kernel, stride, padding)
+    out_w = np.zeros((N, C, oh, ow), F); idx_w = np.zeros((N, C, oh, ow), np.int32)
+    oracle.maxpool_forward(x, out_w, idx_w, N, C, H, W, oh, ow, kernel, stride, padding)
+    # poisoned outputs: the kernel must write every element itself
+    gout = torch.full((N, C, oh, ow), 123.0, device="cuda")
+    gidx = torch.full((N, C, oh, ow), -77, device="cuda", dtype=torch.int32)
+    ops.maxpool_forward(gpu(x), gout, gidx, kernel, stride, padding)
+    what = "maxpool %s k%d s%d p%d" % (x.shape, kernel, stride, padding)
+    assert_bit_exact(host(gout), out_w, what + " values")
+    assert_bit_exact(host(gidx), idx_w, what + " indexes")
+    delta = wl.normal(seed, out_w.shape)
+    grad0 = wl.normal(seed + 1, x.shape)
+    grad_w = grad0.copy()
+    oracle.maxpool_backward(delta, idx_w, grad_w)
+    ggrad = gpu(grad0)
+    ops.maxpool_backward(gpu(delta), gidx, ggrad, kernel, stride, padding)
+    assert_bit_exact(host(ggrad), grad_w, what + " backward")
+    return idx_w, delta, grad0, grad_w
+
+
+def test_maxpool_reference_kat(ops, kats):
+    import torch
+    c = kats["maxpool"]
+    x = gpu(np.array(c["input"], F).reshape(1, 1, 3, 3))
+    out = torch.zeros(1, 1, 3, 3, device="cuda"); idx = torch.full((1, 1, 3, 3), -1, device="cuda", dtype=torch.int32)
+    ops.maxpool_forward(x, out, idx, c["kernel"], c["stride"], c["padding"])
+    assert host(out).ravel().tolist() == c["expected_out"]
+    grad = torch.full((1, 1, 3, 3), c["grad_fill"], device="cuda")
+    ops.maxpool_backward(torch.full((1, 1, 3, 3), c["delta_fill"], device="cuda"), idx, grad, c["kernel"], c["stride"],
+                         c["padding"])
+    assert host(grad).ravel().tolist() == c["expected_grad"]
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 304, 304), (2, 4, 76, 76), (2, 5, 38, 38), (3, 4, 26, 26),
+                                   (1, 2, 416, 416), (2, 3, 6, 10), (2, 2, 20, 12)])
+def test_maxpool_2x2_stride2(ops, oracle, shape):
+    x = wl.normal(1000 + shape[2], shape)
+    run_maxpool(ops, oracle, x, 2, 2, 1, 1100)
+    run_maxpool(ops, oracle, x, 2, 2, 0, 1101)
+    # heavy ties: the first maximum in window order must win
+    xt = np.round(x).astype(F)
+    run_maxpool(ops, oracle, xt, 2, 2, 1, 1102)
+
+
+@pytest.mark.parametrize("geom", [(13, 13, 2, 1, 1), (13, 13, 3, 1, 2), (9, 11, 3, 2, 2), (7, 7, 2, 2, 1),
+                                  (8, 8, 3, 3, 0), (5, 9, 2, 1, 0), (6, 6, 4, 2, 3), (4, 4, 1, 1, 0), (5, 5, 2, 3, 1)])
+def test_maxpool_general_geometry(ops, oracle, geom):
+    H, W, k, s, p = geom
+    x = wl.normal(1200 + H * W + k, (2, 3, H, W))
+    run_maxpool(ops, oracle, x, k, s, p, 1300)
+    run_maxpool(ops, oracle, np.round(x).astype(F), k, s, p, 1301)
+
+
+def test_maxpool_special_values(ops, oracle):
+    x = wl.normal(1400, (1, 2, 8, 8))
+    x[0, 0, 0, 0] = np.nan          # first tap NaN: sticky
+    x[0, 0, 2, 3] = np.nan          # later tap NaN: never taken
+    x[0, 1, 4:6, 4:6] = [[0.0, -0.0], [-0.0, 0.0]]
+    x[0, 1, 0:2, 0:2] = -np.inf
+    x[0, 1, 6:8, 6:8] = np.finfo(np.float32).min
+    run_maxpool(ops, oracle, x, 2, 2, 1, 1401)
+    run_maxpool(ops, oracle, x, 2, 1, 1, 1402)
+
+
+def test_maxpool_scatter_signature(ops, oracle):
+    x = wl.normal(1500, (2, 3, 12, 12))
+    idx_w, delta, grad0, grad_w = run_maxpool(ops, oracle, x, 2, 2, 1, 1501)
+    g = gpu(grad0)
+    ops.maxpool_backward_scatter(gpu(delta), gpu(idx_w), g)
+    assert_bit_exact(host(g), grad_w, "scatter (unique indexes)")
+
+
+@pytest.mark.parametrize("shape,stride", [((2, 3, 19, 19), 2), ((2, 4, 38, 38), 2), ((2, 3, 13, 13), 2),
+                                          ((1, 2, 8, 12), 2), ((2, 2, 5, 6), 2), ((2, 2, 5, 7), 3), ((1, 3, 4, 4), 1),
+                                          ((2, 2, 6, 10), 4)])
+def test_upsample_forward_backward(ops, oracle, shape, stride):
+    import torch
+    N, C, H, W = shape
+    x = wl.normal(1600 + H, shape)
+    for scale in (1.0, 0.75):
+        out_w = np.zeros((N, C, H * stride, W * stride), F)
+        oracle.upsample(x, W, H, C, N, stride, True, scale, None, out_w)
+        gout = torch.full(out_w.shape, 55.0, device="cuda")     # no zero-fill needed
+        ops.upsample_forward(gpu(x), gout, stride, scale)
+        assert_bit_exact(host(gout), out_w, "upsample fwd %s s%d" % (shape, stride))
+        delta = wl.normal(1700 + W, out_w.shape)
+        grad0 = wl.normal(1701 + W, shape)
+        grad_w = grad0.copy()
+        oracle.upsample(None, W, H, C, N, stride, False, scale, grad_w, delta)
+        gg = gpu(grad0)
+        ops.upsample_backward(gpu(delta), gg, stride, scale)
+        assert_bit_exact(host(gg), grad_w, "upsample bwd %s s%d scale %g" % (shape, stride, scale))
+
+
+@pytest.mark.parametrize("act", ["linear", "leaky"])
+@pytest.mark.parametrize("shape", [(2, 8, 38, 38), (3, 5, 19, 19), (1, 1, 1, 3), (2, 3, 64, 64)])
+def test_shortcut_forward_backward(ops, oracle, shape, act):
+    import torch
+    N, C, H, W = shape
+    a = wl.normal(1800 + W, shape); b = wl.normal(1801 + W, shape)
+    for alpha, beta in ((1.0, 1.0), (0.5, 1.25)):
+        out_w = np.empty_like(a); pre_w = np.empty_like(a)
+        oracle.shortcut_forward(act, N, W, H, C, a, b, alpha, beta, out_w, pre_w)
+        gout = torch.full(shape, 9.0, device="cuda"); gpre = torch.full(shape, 9.0, device="cuda")
+        ops.shortcut_forward(gpu(a), gpu(b), gout, act, alpha, beta, pre_activation=gpre)
+        what = "shortcut %s %s a=%g b=%g" % (shape, act, alpha, beta)
+        assert_bit_exact(host(gout), out_w, what + " out")
+        assert_bit_exact(host(gpre), pre_w, what + " pre")
+        d0 = wl.normal(1810 + W, shape); fd0 = wl.normal(1811 + W, shape); g0 = wl.normal(1812 + W, shape)
+        d_w, fd_w, g_w = d0.copy(), fd0.copy(), g0.copy()
+        oracle.shortcut_backward(act, N, W, H, C, d_w, pre_w, fd_w, g_w, alpha, beta)
+        gd, gfd, gg = gpu(d0), gpu(fd0), gpu(g0)
+        ops.shortcut_backward(gd, gfd, gg, act, alpha, beta, pre_activation=gpre)
+        assert_bit_exact(host(gd), d_w, what + " delta")
+        assert_bit_exact(host(gfd), fd_w, what + " from delta")
+        assert_bit_exact(host(gg), g_w, what + " grad")
+        # first layer: grad == NULL
+        gd, gfd = gpu(d0), gpu(fd0)
+        ops.shortcut_backward(gd, gfd, None, act, alpha, beta, pre_activation=gpre)
+        assert_bit_exact(host(gfd), fd_w, what + " from delta (no grad)")
+
+
+def test_shortcut_reference_signature(ops, oracle):
+    """shortcutGpu's index-mapped blend, same shape and the shapes the CPU layer accepts."""
+    N, C, H, W = 2, 3, 6, 6
+    add = wl.normal(1900, (N, C, H, W)); out0 = wl.normal(1901, (N, C, H, W))
+    want = out0.copy()
+    assert oracle.shortcut(N, W, H, C, add, W, H, C, 0.5, 2.0, want) == 0
+    g = gpu(out0)
+    ops.shortcut(N, W, H, C, gpu(add), W, H, C, 0.5, 2.0, g)
+    assert_bit_exact(host(g), want, "shortcut same shape")
+    # fewer channels on one side (min over channels), identity spatial maps
+    add2 = wl.normal(1902, (N, 2, H, W))
+    want = out0.copy()
+    assert oracle.shortcut(N, W, H, 2, add2, W, H, C, 1.0, 1.0, want) == 0
+    g = gpu(out0)
+    ops.shortcut(N, W, H, 2, gpu(add2), W, H, C, 1.0, 1.0, g)
+    assert_bit_exact(host(g), want, "shortcut channel mismatch")
