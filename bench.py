@@ -1,0 +1,407 @@
+#!/usr/bin/env python3
+"""Benchmark of the non-convolution layer kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+A step is one pass of the headline workload: the fused BN-inference + bias + activation
+epilogue over every YOLOv3-tiny conv-output shape at batch 64, for leaky, mish and logistic
+(21 launches, 2.9 GB of tensors read and as much written).  W warm-up steps, then exactly K
+timed steps bracketed by device synchronisation; rank 0 prints ONE JSON line.
+
+value      algorithmic GB/s of the timed steps (8 bytes per element: read x, write y), inputs
+           resident in HBM before the timed region starts
+roofline   the leaky epilogue kernel: algorithmic bytes per launch / its mean launch duration
+           from HIP events recorded on the launch stream inside the timed region
+extras     the other kernels of the path (max-pool, upsample, shortcut, YOLO head, BN training
+           forward/backward, Adam) at the baseline's shapes, measured after the timed region
+           and reported in the same line, with the non-conv ms/batch of YOLOv3 at 608
+cpu_baseline  the CPU checker (a port of the reference's single-threaded CPU path) timed on a
+           bounded sample of the same workload on this host, one core
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+EPILOGUE_BATCH = 64
+EPILOGUE_ACTS = ["leaky", "mish", "logistic"]
+
+# HBM bytes per launch of the leaky epilogue kernel relative to its algorithmic bytes, from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/epilogue_leaky_pmc.txt); None = not measured
+EPILOGUE_TRAFFIC_RATIO = None
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-extras", action="store_true", help="skip the other kernels of the path")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--cpu-batch", type=int, default=64, help="images per shape in the CPU sample")
+    return ap.parse_args()
+
+
+class Timer:
+    """Mean duration of a launch sequence from HIP events on the current stream."""
+
+    def __init__(self, torch):
+        self.torch = torch
+
+    def time(self, fn, reps, warm=2, rotate=1):
+        """fn(i) launches one repetition using buffer set i % rotate.  Returns ms per repetition."""
+        t = self.torch
+        for i in range(warm):
+            fn(i % rotate)
+        t.cuda.synchronize()
+        start = t.cuda.Event(enable_timing=True)
+        stop = t.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(reps):
+            fn(i % rotate)
+        stop.record()
+        t.cuda.synchronize()
+        return start.elapsed_time(stop) / reps
+
+
+def rotation_for(bytes_per_set, llc_bytes=256 << 20, cap=8):
+    """Distinct buffer sets needed so that a set has left the 256 MB last-level cache before
+    it is touched again."""
+    n = int(llc_bytes * 2 // max(1, bytes_per_set)) + 1
+    return max(1, min(cap, n))
+
+
+def epilogue_workload(torch, wl):
+    """Resident tensors of the headline sweep: (channels, size, x, y, params) per shape."""
+    dev = torch.device("cuda:0")
+    shapes = []
+    gen = torch.Generator(device=dev)
+    for i, (c, s) in enumerate(wl.YOLOV3_TINY_CONV_SHAPES):
+        gen.manual_seed(3000 + i)
+        x = torch.randn((EPILOGUE_BATCH, c, s, s), device=dev, generator=gen)
+        y = torch.empty_like(x)
+        scale, bias, mean, var = (torch.from_numpy(a).to(dev) for a in wl.bn_params(2000 + i, c))
+        shapes.append(dict(c=c, s=s, x=x, y=y, scale=scale, bias=bias, mean=mean, var=var,
+                           elems=x.numel()))
+    return shapes
+
+
+def fold_weights(ops, shapes):
+    """What a layer does once after loading its weights: fold the per-channel constants."""
+    for sh in shapes:
+        sh["folded"] = ops.bn_fold(sh["mean"], sh["var"], sh["scale"], sh["bias"])
+
+
+def run_epilogue_step(ops, shapes, events=None, torch=None, raw=False):
+    """One pass of the sweep.  With `events`, one HIP-event pair brackets each activation's
+    group of 7 launches (an event between two kernels would add its own few microseconds to
+    every launch it brackets)."""
+    for act in EPILOGUE_ACTS:
+        if events is not None:
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            a.record()
+        for sh in shapes:
+            if raw:
+                ops.bn_infer_act_forward(sh["x"], sh["y"], sh["mean"], sh["var"], sh["scale"], sh["bias"], act)
+            else:
+                ops.bn_folded_act_forward(sh["x"], sh["y"], sh["folded"], act)
+        if events is not None:
+            b.record()
+            events.append((act, a, b))
+
+
+def measure_extras(torch, ops, wl, timer):
+    """The other kernels of the path at the baseline's shapes.  Returns (rows, ms_per_batch)."""
+    dev = torch.device("cuda:0")
+    rows = []
+
+    def add(name, shape, bytes_, ms, note=""):
+        gbs = bytes_ / (ms * 1e-3) / 1e9
+        rows.append(dict(kernel=name, shape=shape, MB=round(bytes_ / 1e6, 1), ms=round(ms, 4),
+                         GBps=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 3), note=note))
+        return ms
+
+    def randn(*shape):
+        return torch.randn(shape, device=dev)
+
+    N = 16
+    # ---- max-pool 2x2 s2 forward + backward (config 2)
+    for c, s in wl.YOLOV3_MAXPOOL_SHAPES:
+        e_in = N * c * s * s
+        e_out = e_in // 4
+        rot = rotation_for(4 * e_in + 8 * e_out)
+        xs = [randn(N, c, s, s) for _ in range(rot)]
+        outs = [torch.empty((N, c, s // 2, s // 2), device=dev) for _ in range(rot)]
+        idxs = [torch.empty((N, c, s // 2, s // 2), device=dev, dtype=torch.int32) for _ in range(rot)]
+        ms = timer.time(lambda i: ops.maxpool_forward(xs[i], outs[i], idxs[i], 2, 2, 1), 20, rotate=rot)
+        add("maxpool_fwd", "%dx%dx%d^2" % (N, c, s), 4 * e_in + 8 * e_out, ms, "4B/in + 8B/out")
+        deltas = [randn(N, c, s // 2, s // 2) for _ in range(rot)]
+        ms = timer.time(lambda i: ops.maxpool_backward(deltas[i], idxs[i], xs[i], 2, 2, 1), 20, rotate=rot)
+        add("maxpool_bwd", "%dx%dx%d^2" % (N, c, s), 8 * e_out + 8 * e_in, ms, "full-grad RMW: 8B/out + 8B/in")
+        del xs, outs, idxs, deltas
+    # ---- upsample x2 forward + backward
+    for c, s in wl.YOLOV3_UPSAMPLE_SHAPES:
+        e_in = N * c * s * s
+        e_out = 4 * e_in
+        rot = rotation_for(4 * e_in + 4 * e_out)
+        xs = [randn(N, c, s, s) for _ in range(rot)]
+        outs = [torch.empty((N, c, 2 * s, 2 * s), device=dev) for _ in range(rot)]
+        ms_f = timer.time(lambda i: ops.upsample_forward(xs[i], outs[i], 2, 1.0), 50, rotate=rot)
+        add("upsample_fwd", "%dx%dx%d^2" % (N, c, s), 4 * e_in + 4 * e_out, ms_f, "4B/in + 4B/out")
+        ms_b = timer.time(lambda i: ops.upsample_backward(outs[i], xs[i], 2, 1.0), 50, rotate=rot)
+        add("upsample_bwd", "%dx%dx%d^2" % (N, c, s), 4 * e_out + 8 * e_in, ms_b, "4B/out + 8B/in")
+        del xs, outs
+    # ---- shortcut forward + backward
+    shortcut_ms = {}
+    for c, s, count in wl.YOLOV3_SHORTCUT_SHAPES:
+        e = N * c * s * s
+        rot = rotation_for(12 * e)
+        a = [randn(N, c, s, s) for _ in range(rot)]
+        b = [randn(N, c, s, s) for _ in range(rot)]
+        o = [torch.empty((N, c, s, s), device=dev) for _ in range(rot)]
+        ms_f = timer.time(lambda i: ops.shortcut_forward(a[i], b[i], o[i], "linear"), 20, rotate=rot)
+        add("shortcut_fwd", "%dx%dx%d^2" % (N, c, s), 12 * e, ms_f, "12B/elem")
+        ms_b = timer.time(lambda i: ops.shortcut_backward(o[i], a[i], b[i], "linear"), 20, rotate=rot)
+        add("shortcut_bwd", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_b, "20B/elem")
+        shortcut_ms[(c, s)] = (ms_f, ms_b, count)
+        del a, b, o
+    # ---- YOLO head (config 3): batch 64
+    NB = 64
+    truths_np, counts_np = wl.yolo_truths(5100, NB)
+    truths = torch.from_numpy(truths_np).to(dev)
+    counts = torch.from_numpy(counts_np).to(dev)
+    stats = torch.zeros(12, device=dev)
+    cost = torch.zeros(1, device=dev)
+    head_ms = {}
+    for s in wl.YOLOV3_HEAD_SIZES:
+        e = NB * 255 * s * s
+        rot = rotation_for(12 * e)
+        xin = [2.0 * randn(NB, 255, s, s) for _ in range(rot)]
+        out = [torch.empty((NB, 255, s, s), device=dev) for _ in range(rot)]
+        dl = [torch.empty((NB, 255, s, s), device=dev) for _ in range(rot)]
+        ms_d = timer.time(lambda i: ops.yolo_activate(xin[i], out[i], NB, 3, 80, s * s), 20, rotate=rot)
+        add("yolo_decode", "%dx255x%d^2" % (NB, s), 8 * e, ms_d, "8B/elem")
+        ms_t = timer.time(lambda i: ops.yolo_forward_train(
+            xin[i], out[i], dl[i], truths, counts, truths.shape[1], wl.YOLOV3_MASKS[s], wl.YOLOV3_ANCHORS, stats,
+            cost, NB, 80, s, s, 608, 608, 0.7, 1.0, 1.0, 2.0, 0.1, 1.0), 20, rotate=rot)
+        add("yolo_decode+delta+cost", "%dx255x%d^2" % (NB, s), 12 * e, ms_t, "fused 12B/elem")
+        head_ms[s] = (ms_d, ms_t)
+        del xin, out, dl
+    # ---- BN training forward / backward (config 4): batch 16 @608, 13 shapes
+    bn_ms = {}
+    for (c, s), count in zip(wl.YOLOV3_BN_SHAPES, wl.YOLOV3_BN_COUNTS):
+        e = N * c * s * s
+        rot = rotation_for(12 * e, cap=4)
+        x = [randn(N, c, s, s) for _ in range(rot)]
+        y = [torch.empty((N, c, s, s), device=dev) for _ in range(rot)]
+        d = [randn(N, c, s, s) for _ in range(rot)]
+        scale, bias, rmean, rvar = (torch.from_numpy(a).to(dev) for a in wl.bn_params(2000 + c, c))
+        mean = torch.zeros(c, device=dev); var = torch.ones(c, device=dev)
+        su = torch.zeros(c, device=dev); bu = torch.zeros(c, device=dev)
+        ms_f = timer.time(lambda i: ops.bn_train_act_forward(x[i], y[i], mean, var, rmean, rvar, scale, bias, "leaky"),
+                          10, rotate=rot)
+        add("bn_train_fwd(leaky)", "%dx%dx%d^2" % (N, c, s), 12 * e, ms_f, "stats 4B + apply 8B per elem; x kept")
+        ms_b = timer.time(lambda i: ops.bn_act_backward(d[i], x[i], mean, var, scale, bias, su, bu, "leaky"),
+                          10, rotate=rot)
+        add("bn_bwd(leaky)", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_b, "sums 8B + dx 12B per elem; pre recomputed")
+        bn_ms[(c, s)] = (ms_f, ms_b, count)
+        del x, y, d
+    # ---- linear bias epilogue of the three head convs at batch 16
+    for c, s in wl.YOLOV3_HEAD_CONV_SHAPES:
+        e = N * c * s * s
+        x = randn(N, c, s, s)
+        bias = randn(c)
+        ms = timer.time(lambda i: ops.bias_act_forward(x, x, bias, "linear"), 20)
+        add("bias_fwd(linear)", "%dx%dx%d^2" % (N, c, s), 8 * e, ms, "in place, cache resident")
+        bn_ms[("head", s)] = (ms, 0.0, 1)
+    # ---- Adam (config 4): 61.9M parameters, 10 steps
+    P = wl.YOLOV3_PARAMS
+    w = 0.02 * randn(P); g = 1e-3 * randn(P)
+    m = torch.zeros(P, device=dev); v = torch.zeros(P, device=dev)
+    d = torch.empty(P, device=dev)
+    step = [0]
+
+    def adam_step(i):
+        step[0] += 1
+        d.copy_(g)                       # the update is consumed (zeroed) by each step
+        ops.adam_update(w, d, m, v, 16, min(step[0], 1000), 1e-3, 0.9, 0.999, 1e-8, 5e-4, True)
+
+    # time the copy separately and subtract it: only the Adam kernel is reported
+    ms_both = timer.time(adam_step, 10)
+    ms_copy = timer.time(lambda i: d.copy_(g), 10)
+    ms_adam = max(ms_both - ms_copy, 1e-6)
+    add("adam_update", "%d params" % P, 32 * P, ms_adam, "32B/param, L2 folded into the update")
+
+    # ---- non-conv ms per batch, YOLOv3 @608, batch 16, one training step:
+    # 72 BN'd conv epilogues fwd+bwd, 3 bias epilogues, 23 shortcuts fwd+bwd, 2 upsamples fwd+bwd,
+    # 3 heads (fused decode+delta) at batch 16 scaled from the batch-64 measurement, Adam
+    total = 0.0
+    for key, (f, b, count) in bn_ms.items():
+        total += (f + b) * count
+    for key, (f, b, count) in shortcut_ms.items():
+        total += (f + b) * count
+    for r in rows:
+        if r["kernel"].startswith("upsample"):
+            total += r["ms"]
+    for s, (ms_d, ms_t) in head_ms.items():
+        total += ms_t * N / NB
+    total += ms_adam
+    return rows, total
+
+
+def cpu_baseline(wl, batch):
+    """The CPU checker on `batch` images per shape of the same sweep, one core."""
+    import numpy as np
+    import oracle
+    oracle.lib()
+    F = np.float32
+    elems = 0
+    t_total = 0.0
+    for i, (c, s) in enumerate(wl.YOLOV3_TINY_CONV_SHAPES):
+        x = wl.normal(3000 + i, (batch, c, s, s))
+        scale, bias, mean, var = wl.bn_params(2000 + i, c)
+        for act in EPILOGUE_ACTS:
+            y = x.copy()
+            t0 = time.perf_counter()
+            oracle.conv_epilogue_forward(True, False, act, batch, c, s, s, y, None, np.zeros(c, F), np.zeros(c, F),
+                                         mean, var, scale, bias, None, None)
+            t_total += time.perf_counter() - t0
+            elems += x.size
+    return dict(value=round(8.0 * elems / t_total / 1e9, 3), unit="GB/s", cores=1, kind="port",
+                sample="same 7 shapes x 3 activations at batch %d (%.1f M elements, %.1f s)"
+                       % (batch, elems / 1e6, t_total),
+                host_cpus=os.cpu_count())
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one GPU: this path has no multi-GPU part (every kernel is independent per image "
+            "and per channel); run with --gpus 1")
+        sys.exit(2)
+    import torch
+    from pixienn_amd import capi, ops, workloads as wl
+    capi.load()      # fails loudly when the HIP library is missing
+    assert torch.cuda.is_available(), "no GPU visible"
+    torch.cuda.set_device(0)
+    timer = Timer(torch)
+
+    shapes = epilogue_workload(torch, wl)
+    fold_weights(ops, shapes)
+    elems_sweep = sum(sh["elems"] for sh in shapes)
+    elems_step = elems_sweep * len(EPILOGUE_ACTS)
+    bytes_step = 8.0 * elems_step
+
+    for _ in range(args.warmup):
+        run_epilogue_step(ops, shapes)
+    torch.cuda.synchronize()
+    events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_epilogue_step(ops, shapes, events, torch)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = bytes_step / (ms_per_step * 1e-3) / 1e9
+
+    # per-activation kernel figures from the event pairs of the timed region
+    group_ms = {}
+    for act, a, b in events:
+        group_ms.setdefault(act, []).append(a.elapsed_time(b))
+    per_act = {}
+    for act, v in group_ms.items():
+        ms = sum(v) / len(v)
+        per_act[act] = dict(ms_per_sweep=round(ms, 4), GBps=round(8.0 * elems_sweep / (ms * 1e-3) / 1e9, 1))
+        log("epilogue %-9s sweep of %d shapes: %8.4f ms %8.1f GB/s" % (act, len(shapes), ms, per_act[act]["GBps"]))
+    launches = len(shapes)
+    leaky_ms = sum(group_ms["leaky"]) / len(group_ms["leaky"])
+    achieved = 8.0 * elems_sweep / (leaky_ms * 1e-3) / 1e9
+    bytes_per_launch = 8.0 * elems_sweep / launches
+    roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=round(achieved / HBM_PEAK_GBS, 4),
+                    traffic=None if EPILOGUE_TRAFFIC_RATIO is None else round(EPILOGUE_TRAFFIC_RATIO * bytes_per_launch),
+                    kernel="epilogue_fwd_kernel<PXH_LEAKY, true, *>",
+                    bytes_per_launch=round(bytes_per_launch),
+                    mean_launch_ms=round(leaky_ms / launches, 5))
+
+    # the same step through the two-launch entry point that folds the constants on every call
+    for _ in range(2):
+        run_epilogue_step(ops, shapes, raw=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_epilogue_step(ops, shapes, raw=True)
+    torch.cuda.synchronize()
+    value_raw = bytes_step / ((time.perf_counter() - t0) / args.steps) / 1e9
+    log("whole sweep: %.1f GB/s with folded constants, %.1f GB/s folding on every call" % (value, value_raw))
+
+    # per shape, each measured alone over rotating buffers (HIP events around 20 launches)
+    per_shape = []
+    if not args.no_extras:
+        for sh in shapes:
+            rot = rotation_for(8 * sh["elems"], cap=3)
+            xs = [sh["x"]] + [torch.randn_like(sh["x"]) for _ in range(rot - 1)]
+            ys = [sh["y"]] + [torch.empty_like(sh["y"]) for _ in range(rot - 1)]
+            for act in EPILOGUE_ACTS:
+                ms = timer.time(lambda i: ops.bn_folded_act_forward(xs[i], ys[i], sh["folded"], act), 20, rotate=rot)
+                r = dict(act=act, shape="%dx%dx%d^2" % (EPILOGUE_BATCH, sh["c"], sh["s"]), ms=round(ms, 4),
+                         GBps=round(8.0 * sh["elems"] / (ms * 1e-3) / 1e9, 1))
+                per_shape.append(r)
+                log("epilogue %-9s %-16s %8.4f ms %8.1f GB/s" % (r["act"], r["shape"], r["ms"], r["GBps"]))
+            del xs, ys
+
+    extras, ms_batch = (None, None)
+    if not args.no_extras:
+        extras, ms_batch = measure_extras(torch, ops, wl, timer)
+        for r in extras:
+            log("%-24s %-18s %9.1f MB %8.4f ms %8.1f GB/s  %4.1f%%  %s"
+                % (r["kernel"], r["shape"], r["MB"], r["ms"], r["GBps"], 100 * r["frac"], r["note"]))
+        log("non-conv ms/batch, YOLOv3 @608, batch 16, training step: %.3f" % ms_batch)
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(wl, args.cpu_batch)
+        log("cpu baseline:", cpu)
+
+    line = {
+        "metric": "fused BN+act epilogue GB/s (% of HBM peak); non-conv ms/batch YOLOv3 608",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: fused BN-inference+bias+activation epilogue sweep, NCHW fp32, N=64, "
+                               "7 YOLOv3-tiny conv-output shapes x {leaky, mish, logistic}; per-channel constants "
+                               "folded once before the timed region, as a layer does after loading its weights",
+                   "bytes_per_step": int(bytes_step), "launches_per_step": len(shapes) * len(EPILOGUE_ACTS),
+                   "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "noconv_ms_per_batch_yolov3_608": None if ms_batch is None else round(ms_batch, 3),
+        "value_folding_every_call": round(value_raw, 1),
+        "per_activation": per_act,
+        "per_shape": per_shape,
+        "extras": extras,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

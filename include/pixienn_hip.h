@@ -54,13 +54,27 @@ unsigned pxh_debug_fastdiv(unsigned n, unsigned d);
  * with the rounding sequence of the CPU layer (subtract, divide, scale, add
  * each rounded to fp32).  pre_activation (nullable) receives the value before
  * act.  In place allowed (y == x).
+ * Two launches: the per-channel constants are folded into `workspace`
+ * (pxh_bn_folded_bytes(channels) bytes, or NULL for the library's per-device buffer), then the
+ * tensor is streamed once.
  * Replaces, for an inferring ConvLayer/BatchNormLayer: cudnnBatchNormalizationForwardInference
  * + preActivation_.copy + activate(), include/cuda/ConvLayer.h:284-307; CPU semantics
  * src/BatchNorm.cpp:24-67 (training == false), include/ConvLayer.h:227-236. */
 int pxh_bn_infer_act_forward(const float* x, float* y, float* pre_activation,
                              const float* rolling_mean, const float* rolling_var,
                              const float* scale, const float* bias,
-                             int batch, int channels, int spatial, int activation, void* stream);
+                             int batch, int channels, int spatial, int activation,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same, split for a layer whose weights do not change between calls: fold once (after
+ * loading or updating the weights), then every forward is the single streaming launch.
+ * `folded` is a caller-owned, 16-byte aligned device buffer of pxh_bn_folded_bytes(channels).
+ * No counterpart in the reference, whose cuDNN call re-derives the constants on every forward. */
+size_t pxh_bn_folded_bytes(int channels);
+int pxh_bn_fold(const float* rolling_mean, const float* rolling_var, const float* scale,
+                const float* bias, int channels, void* folded, void* stream);
+int pxh_bn_folded_act_forward(const float* x, float* y, float* pre_activation, const void* folded,
+                              int batch, int channels, int spatial, int activation, void* stream);
 
 /* bias + activation in one pass: y = act(x + bias[c]); pre_activation nullable; in place allowed.
  * Replaces addBiasGpu (include/BiasKernels.cuh:21) + preActivation_.copy + activate()

@@ -20,7 +20,9 @@ Z = ctypes.c_size_t
 
 # name -> argument types (every function returns int unless listed in _OTHER_RETURNS)
 SIGNATURES = {
-    "pxh_bn_infer_act_forward": [P, P, P, P, P, P, P, I, I, I, I, P],
+    "pxh_bn_infer_act_forward": [P, P, P, P, P, P, P, I, I, I, I, P, Z, P],
+    "pxh_bn_fold": [P, P, P, P, I, P, P],
+    "pxh_bn_folded_act_forward": [P, P, P, P, I, I, I, I, P],
     "pxh_bias_act_forward": [P, P, P, P, I, I, I, I, P],
     "pxh_bn_train_act_forward": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, P, Z, P],
     "pxh_bn_stats": [P, P, P, I, I, I, P, Z, P],
@@ -52,6 +54,7 @@ _OTHER_RETURNS = {
     "pxh_last_error": (ctypes.c_char_p, []),
     "pxh_abi_version": (I, []),
     "pxh_bn_workspace_bytes": (Z, [I, I, I]),
+    "pxh_bn_folded_bytes": (Z, [I]),
     "pxh_yolo_workspace_bytes": (Z, [I, I, I, I, I]),
     "pxh_debug_fastdiv": (ctypes.c_uint, [ctypes.c_uint, ctypes.c_uint]),
 }

@@ -14,8 +14,6 @@ namespace pxh {
 
 constexpr int kWave = 64;          // CDNA wavefront
 constexpr int kBlock = 256;        // 4 waves per workgroup
-constexpr int kUnroll = 4;         // float4 loads in flight per lane in streaming kernels
-constexpr int kChunk = kBlock * 4 * kUnroll;   // elements one workgroup streams: 4096
 
 // ---------------------------------------------------------------- errors
 void set_error(const char* fmt, ...);
@@ -75,6 +73,40 @@ __device__ __forceinline__ float softplus_grad(float x)
     return 1.0f / (1.0f + expf(-x));
 }
 
+// tanh(softplus(x)) for |x| <= 20.  The CPU functor evaluates tanhf(logf(u)) with
+// u = float(expf(x) + 1); tanh(log u) = (u*u - 1)/(u*u + 1) exactly, and (u - 1) is exact in
+// fp32, so the same rounded u gives the same value to a few ulp with one exp and one division
+// instead of exp + log + tanh.
+__device__ __forceinline__ float tanh_softplus_mid(float x)
+{
+    const float u = expf(x) + 1.0f;
+    const float num = (u - 1.0f) * (u + 1.0f);
+    const float den = u * u + 1.0f;
+    return num / den;
+}
+
+__device__ __forceinline__ float mish_apply(float x)
+{
+    if (x > 20.0f) return x;                 // tanhf(x) is 1.0f here
+    if (x < -20.0f) return x * expf(x);      // tanhf(s) is s for s < 2.1e-9
+    return x * tanh_softplus_mid(x);
+}
+
+__device__ __forceinline__ float mish_grad(float x)
+{
+    if (x > 20.0f) return 1.0f;              // (1 - 1*1)*1*x + 1
+    float tsp, gsp;
+    if (x < -20.0f) {
+        tsp = expf(x);
+        gsp = tsp;
+    } else {
+        tsp = tanh_softplus_mid(x);
+        gsp = 1.0f / (1.0f + expf(-x));
+    }
+    const float gtsp = (1.0f - tsp * tsp) * gsp;
+    return x * gtsp + tsp;
+}
+
 template<int ACT>
 __device__ __forceinline__ float act_apply(float x)
 {
@@ -82,7 +114,7 @@ __device__ __forceinline__ float act_apply(float x)
     else if constexpr (ACT == PXH_LINEAR) return x;
     else if constexpr (ACT == PXH_LOGGY) return 2.0f / (1.0f + expf(-x)) - 1.0f;
     else if constexpr (ACT == PXH_LOGISTIC) return 1.0f / (1.0f + expf(-x));
-    else if constexpr (ACT == PXH_MISH) return x * tanhf(softplus_apply(x));
+    else if constexpr (ACT == PXH_MISH) return mish_apply(x);
     else if constexpr (ACT == PXH_RELU) return x > 0.0f ? x : 0.0f;
     else if constexpr (ACT == PXH_SOFTPLUS) return softplus_apply(x);
     else if constexpr (ACT == PXH_SWISH) return x / (1.0f + expf(-1.0f * x));
@@ -101,11 +133,7 @@ __device__ __forceinline__ float act_grad(float x)
         float y = 1.0f / (1.0f + expf(-x));
         return y * (1.0f - y);
     } else if constexpr (ACT == PXH_MISH) {
-        float sp = softplus_apply(x);
-        float gsp = softplus_grad(x);
-        float tsp = tanhf(sp);
-        float gtsp = (1.0f - tsp * tsp) * gsp;
-        return x * gtsp + tsp;
+        return mish_grad(x);
     } else if constexpr (ACT == PXH_RELU) return x > 0.0f ? 1.0f : 0.0f;
     else if constexpr (ACT == PXH_SOFTPLUS) return softplus_grad(x);
     else if constexpr (ACT == PXH_SWISH) {

@@ -11,13 +11,13 @@ template<int ACT>
 struct ActivateOp {
     float* x;
     template<int V> struct Regs { Pack<V> x; };
-    template<int V> __device__ void load(size_t e, Regs<V>& r) const { r.x = ld<V>(x, e); }
-    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const { r.x = ld<V, NT>(x, e); }
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
         Pack<V> o;
 #pragma unroll
         for (int k = 0; k < V; ++k) o.v[k] = act_apply<ACT>(r.x.v[k]);
-        st<V>(x, e, o);
+        st<V, NT>(x, e, o);
     }
 };
 
@@ -26,17 +26,17 @@ struct GradientOp {
     const float* x;
     float* delta;
     template<int V> struct Regs { Pack<V> x, d; };
-    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
     {
-        r.x = ld<V>(x, e);
-        r.d = ld<V>(delta, e);
+        r.x = ld<V, NT>(x, e);
+        r.d = ld<V, NT>(delta, e);
     }
-    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
         Pack<V> o;
 #pragma unroll
         for (int k = 0; k < V; ++k) o.v[k] = r.d.v[k] * act_grad<ACT>(r.x.v[k]);
-        st<V>(delta, e, o);
+        st<V, NT>(delta, e, o);
     }
 };
 
@@ -45,13 +45,13 @@ struct FillOp {
     float* x;
     float value;
     template<int V> struct Regs {};
-    template<int V> __device__ void load(size_t, Regs<V>&) const {}
-    template<int V> __device__ void finish(size_t e, const Regs<V>&) const
+    template<int V, bool NT> __device__ void load(size_t, Regs<V>&) const {}
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>&) const
     {
         Pack<V> o;
 #pragma unroll
         for (int k = 0; k < V; ++k) o.v[k] = value;
-        st<V>(x, e, o);
+        st<V, NT>(x, e, o);
     }
 };
 
@@ -59,13 +59,13 @@ struct ConstrainOp {
     float* x;
     float alpha;
     template<int V> struct Regs { Pack<V> x; };
-    template<int V> __device__ void load(size_t e, Regs<V>& r) const { r.x = ld<V>(x, e); }
-    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const { r.x = ld<V, NT>(x, e); }
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
         Pack<V> o;
 #pragma unroll
         for (int k = 0; k < V; ++k) o.v[k] = fminf(alpha, fmaxf(-alpha, r.x.v[k]));
-        st<V>(x, e, o);
+        st<V, NT>(x, e, o);
     }
 };
 
@@ -73,17 +73,17 @@ struct MulOp {
     const float* x;
     float* y;
     template<int V> struct Regs { Pack<V> x, y; };
-    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
     {
-        r.x = ld<V>(x, e);
-        r.y = ld<V>(y, e);
+        r.x = ld<V, NT>(x, e);
+        r.y = ld<V, NT>(y, e);
     }
-    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
         Pack<V> o;
 #pragma unroll
         for (int k = 0; k < V; ++k) o.v[k] = r.x.v[k] * r.y.v[k];
-        st<V>(y, e, o);
+        st<V, NT>(y, e, o);
     }
 };
 
@@ -92,12 +92,12 @@ struct AxpyOp {
     float* y;
     float alpha;
     template<int V> struct Regs { Pack<V> x, y; };
-    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
     {
-        r.x = ld<V>(x, e);
-        r.y = ld<V>(y, e);
+        r.x = ld<V, NT>(x, e);
+        r.y = ld<V, NT>(y, e);
     }
-    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
         Pack<V> o;
 #pragma unroll
@@ -105,7 +105,7 @@ struct AxpyOp {
             const float p = alpha * r.x.v[k];
             o.v[k] = r.y.v[k] + p;
         }
-        st<V>(y, e, o);
+        st<V, NT>(y, e, o);
     }
 };
 
@@ -119,12 +119,12 @@ struct ShortcutForwardOp {
     float* pre;   // nullable
     float alpha, beta;
     template<int V> struct Regs { Pack<V> a, b; };
-    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
     {
-        r.a = ld<V>(in, e);
-        r.b = ld<V>(from, e);
+        r.a = ld<V, NT>(in, e);
+        r.b = ld<V, NT>(from, e);
     }
-    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
         Pack<V> p, o;
 #pragma unroll
@@ -134,8 +134,8 @@ struct ShortcutForwardOp {
             p.v[k] = pa + pb;
             o.v[k] = act_apply<ACT>(p.v[k]);
         }
-        if (pre) st<V>(pre, e, p);
-        st<V>(out, e, o);
+        if (pre) st<V, NT>(pre, e, p);
+        st<V, NT>(out, e, o);
     }
 };
 
@@ -148,14 +148,14 @@ struct ShortcutBackwardOp {
     float* grad;   // nullable
     float alpha, beta;
     template<int V> struct Regs { Pack<V> d, p, f, g; };
-    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
     {
-        r.d = ld<V>(delta, e);
-        if constexpr (ACT != PXH_LINEAR) r.p = ld<V>(pre, e);
-        r.f = ld<V>(from_delta, e);
-        if (grad) r.g = ld<V>(grad, e);
+        r.d = ld<V, NT>(delta, e);
+        if constexpr (ACT != PXH_LINEAR) r.p = ld<V, NT>(pre, e);
+        r.f = ld<V, NT>(from_delta, e);
+        if (grad) r.g = ld<V, NT>(grad, e);
     }
-    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
         Pack<V> d = r.d, f, g;
 #pragma unroll
@@ -169,9 +169,9 @@ struct ShortcutBackwardOp {
                 g.v[k] = r.g.v[k] + ga;
             }
         }
-        if constexpr (ACT != PXH_LINEAR) st<V>(delta, e, d);
-        st<V>(from_delta, e, f);
-        if (grad) st<V>(grad, e, g);
+        if constexpr (ACT != PXH_LINEAR) st<V, NT>(delta, e, d);
+        st<V, NT>(from_delta, e, f);
+        if (grad) st<V, NT>(grad, e, g);
     }
 };
 
@@ -204,14 +204,14 @@ struct AdamUpdateOp {
     float inv_batch, neg_decay, beta1, beta2, a1, a2, c1, c2, lr, eps;
     int apply_decay;
     template<int V> struct Regs { Pack<V> w, d, m, v; };
-    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
     {
-        r.w = ld<V>(w, e);
-        r.d = ld<V>(d, e);
-        r.m = ld<V>(m, e);
-        r.v = ld<V>(v, e);
+        r.w = ld<V, NT>(w, e);
+        r.d = ld<V, NT>(d, e);
+        r.m = ld<V, NT>(m, e);
+        r.v = ld<V, NT>(v, e);
     }
-    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
         Pack<V> ow, om, ov, od;
 #pragma unroll
@@ -236,10 +236,10 @@ struct AdamUpdateOp {
             ov.v[k] = vi;
             od.v[k] = 0.0f;
         }
-        st<V>(w, e, ow);
-        st<V>(m, e, om);
-        st<V>(v, e, ov);
-        st<V>(d, e, od);
+        st<V, NT>(w, e, ow);
+        st<V, NT>(m, e, om);
+        st<V, NT>(v, e, ov);
+        st<V, NT>(d, e, od);
     }
 };
 
@@ -249,13 +249,13 @@ struct AdamStepOp {
     const float* v;
     float c1, c2, rate, eps;
     template<int V> struct Regs { Pack<V> x, m, v; };
-    template<int V> __device__ void load(size_t e, Regs<V>& r) const
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
     {
-        r.x = ld<V>(x, e);
-        r.m = ld<V>(m, e);
-        r.v = ld<V>(v, e);
+        r.x = ld<V, NT>(x, e);
+        r.m = ld<V, NT>(m, e);
+        r.v = ld<V, NT>(v, e);
     }
-    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
         Pack<V> o;
 #pragma unroll
@@ -265,7 +265,7 @@ struct AdamStepOp {
             const float step = rate * mhat / (sqrtf(vhat) + eps);
             o.v[k] = r.x.v[k] + step;
         }
-        st<V>(x, e, o);
+        st<V, NT>(x, e, o);
     }
 };
 
@@ -282,7 +282,7 @@ int pxh_activate(int activation, float* x, size_t n, void* stream)
     int rc = PXH_OK;
     const bool known = dispatch_activation(activation, [&]<int ACT>() {
         if constexpr (ACT == PXH_LINEAR) return;
-        rc = launch_stream("pxh_activate", n, aligned16(x), ActivateOp<ACT>{ x }, as_stream(stream));
+        rc = launch_stream("pxh_activate", n, aligned16(x), 8, ActivateOp<ACT>{ x }, as_stream(stream));
     });
     if (!known) return fail_invalid("pxh_activate: unknown activation %d", activation);
     return rc;
@@ -294,7 +294,7 @@ int pxh_gradient(int activation, const float* x, size_t n, float* delta, void* s
     int rc = PXH_OK;
     const bool known = dispatch_activation(activation, [&]<int ACT>() {
         if constexpr (ACT == PXH_LINEAR) return;
-        rc = launch_stream("pxh_gradient", n, aligned16(x) && aligned16(delta), GradientOp<ACT>{ x, delta },
+        rc = launch_stream("pxh_gradient", n, aligned16(x) && aligned16(delta), 12, GradientOp<ACT>{ x, delta },
                            as_stream(stream));
     });
     if (!known) return fail_invalid("pxh_gradient: unknown activation %d", activation);
@@ -304,7 +304,7 @@ int pxh_gradient(int activation, const float* x, size_t n, float* delta, void* s
 int pxh_fill_f32(float* x, size_t n, float value, void* stream)
 {
     if (!x && n) return fail_invalid("pxh_fill_f32: null pointer");
-    return launch_stream("pxh_fill_f32", n, aligned16(x), FillOp{ x, value }, as_stream(stream));
+    return launch_stream("pxh_fill_f32", n, aligned16(x), 4, FillOp{ x, value }, as_stream(stream));
 }
 
 int pxh_fill_i32(int* x, size_t n, int value, void* stream)
@@ -313,28 +313,28 @@ int pxh_fill_i32(int* x, size_t n, int value, void* stream)
     float bits;
     static_assert(sizeof(bits) == sizeof(value), "int and float must have the same size");
     __builtin_memcpy(&bits, &value, sizeof(bits));
-    return launch_stream("pxh_fill_i32", n, aligned16(x), FillOp{ reinterpret_cast<float*>(x), bits },
+    return launch_stream("pxh_fill_i32", n, aligned16(x), 4, FillOp{ reinterpret_cast<float*>(x), bits },
                          as_stream(stream));
 }
 
 int pxh_constrain(int n, float alpha, float* x, void* stream)
 {
     if (n < 0 || (!x && n)) return fail_invalid("pxh_constrain: bad argument");
-    return launch_stream("pxh_constrain", static_cast<size_t>(n), aligned16(x), ConstrainOp{ x, alpha },
+    return launch_stream("pxh_constrain", static_cast<size_t>(n), aligned16(x), 8, ConstrainOp{ x, alpha },
                          as_stream(stream));
 }
 
 int pxh_mul(int n, const float* x, float* y, void* stream)
 {
     if (n < 0 || ((!x || !y) && n)) return fail_invalid("pxh_mul: bad argument");
-    return launch_stream("pxh_mul", static_cast<size_t>(n), aligned16(x) && aligned16(y), MulOp{ x, y },
+    return launch_stream("pxh_mul", static_cast<size_t>(n), aligned16(x) && aligned16(y), 12, MulOp{ x, y },
                          as_stream(stream));
 }
 
 int pxh_axpy(size_t n, float alpha, const float* x, float* y, void* stream)
 {
     if ((!x || !y) && n) return fail_invalid("pxh_axpy: null pointer");
-    return launch_stream("pxh_axpy", n, aligned16(x) && aligned16(y), AxpyOp{ x, y, alpha }, as_stream(stream));
+    return launch_stream("pxh_axpy", n, aligned16(x) && aligned16(y), 12, AxpyOp{ x, y, alpha }, as_stream(stream));
 }
 
 int pxh_shortcut(int batch, int w1, int h1, int c1, const float* add, int w2, int h2, int c2, float s1, float s2,
@@ -356,7 +356,7 @@ int pxh_shortcut(int batch, int w1, int h1, int c1, const float* add, int w2, in
     }
     if (w1 == w2 && h1 == h2 && c1 == c2) {
         // same shape: identity index maps, out = s1*out + s2*add as a flat stream
-        return launch_stream("pxh_shortcut", static_cast<size_t>(size), aligned16(add) && aligned16(out),
+        return launch_stream("pxh_shortcut", static_cast<size_t>(size), aligned16(add) && aligned16(out), 12,
                              ShortcutForwardOp<PXH_LINEAR>{ out, add, out, nullptr, s1, s2 }, as_stream(stream));
     }
     hipLaunchKernelGGL(shortcut_mapped_kernel, dim3(grid_for(size, kBlock)), dim3(kBlock), 0, as_stream(stream),
@@ -372,7 +372,7 @@ int pxh_shortcut_forward(const float* input, const float* from_output, float* ou
     int rc = PXH_OK;
     const bool vec = aligned16(input) && aligned16(from_output) && aligned16(output) && aligned16(pre_activation);
     const bool known = dispatch_activation(activation, [&]<int ACT>() {
-        rc = launch_stream("pxh_shortcut_forward", n, vec,
+        rc = launch_stream("pxh_shortcut_forward", n, vec, pre_activation ? 16 : 12,
                            ShortcutForwardOp<ACT>{ input, from_output, output, pre_activation, alpha, beta },
                            as_stream(stream));
     });
@@ -389,7 +389,7 @@ int pxh_shortcut_backward(float* delta, const float* pre_activation, float* from
     int rc = PXH_OK;
     const bool vec = aligned16(delta) && aligned16(pre_activation) && aligned16(from_delta) && aligned16(grad);
     const bool known = dispatch_activation(activation, [&]<int ACT>() {
-        rc = launch_stream("pxh_shortcut_backward", n, vec,
+        rc = launch_stream("pxh_shortcut_backward", n, vec, grad ? 20 : 12,
                            ShortcutBackwardOp<ACT>{ delta, pre_activation, from_delta, grad, alpha, beta },
                            as_stream(stream));
     });
@@ -404,7 +404,7 @@ int pxh_adam(int n, float* x, const float* m, const float* v, float beta1, float
     // bias corrections formed on the host in fp32, as powf(beta, t)
     const float c1 = 1.0f - powf(beta1, static_cast<float>(t));
     const float c2 = 1.0f - powf(beta2, static_cast<float>(t));
-    return launch_stream("pxh_adam", static_cast<size_t>(n), aligned16(x) && aligned16(m) && aligned16(v),
+    return launch_stream("pxh_adam", static_cast<size_t>(n), aligned16(x) && aligned16(m) && aligned16(v), 16,
                          AdamStepOp{ x, m, v, c1, c2, rate, eps }, as_stream(stream));
 }
 
@@ -423,7 +423,7 @@ int pxh_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch,
     op.c1 = 1.0f - powf(beta1, static_cast<float>(t));
     op.c2 = 1.0f - powf(beta2, static_cast<float>(t));
     op.lr = lr; op.eps = eps; op.apply_decay = apply_decay;
-    return launch_stream("pxh_adam_update", n, aligned16(w) && aligned16(d) && aligned16(m) && aligned16(v), op,
+    return launch_stream("pxh_adam_update", n, aligned16(w) && aligned16(d) && aligned16(m) && aligned16(v), 32, op,
                          as_stream(stream));
 }
 

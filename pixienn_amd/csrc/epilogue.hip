@@ -4,32 +4,53 @@
 // Numerics follow the CPU layer (src/BatchNorm.cpp, src/CpuUtil.cpp:248-342 of the reference):
 //   x_hat = float( double(x - mean) / (sqrt(double(var)) + 1e-5f) )     eps OUTSIDE the root
 //   pre   = float(float(x_hat * scale) + bias)                           two fp32 roundings
-// The quotient is formed as double(x - mean) * (1 / denominator): the double product rounds to
-// the same float as the double quotient except in ~1e-8 of cases.
+// The per-channel reciprocal R = 1 / (sqrt(double(var)) + eps) is formed once per channel in
+// fp64 and kept as two floats (hi + lo); x_hat = fma(t, hi, t * lo) then rounds t * R once, which
+// equals the rounded double quotient except in about 1e-7 of the elements (1 ulp there).
 #include "stream.h"
 
 namespace pxh {
 namespace {
 
 constexpr float kEps = .00001f;
-constexpr int kTable = 160;               // per-workgroup plane table entries
-constexpr int kMinSpatialFast = 28;       // kChunk / 28 + 2 <= kTable
 
-struct PlaneCoef {
-    double rdenom;   // 1 / (sqrt(var) + eps)
-    float mean, scale, bias, pad;
+// Folded per-channel constants of the forward pass (32 bytes: two 128-bit loads).
+struct __attribute__((aligned(16))) FoldCoef {
+    float mean, r_hi, r_lo, scale;
+    float bias, pad0, pad1, pad2;
 };
 
-__device__ __forceinline__ PlaneCoef make_coef(const float* mean, const float* var, const float* scale,
-                                               const float* bias, uint32_t c)
+__device__ __forceinline__ FoldCoef make_coef(float mean, float var, float scale, float bias)
 {
-    PlaneCoef k;
-    k.mean = mean[c];
-    k.scale = scale[c];
-    k.bias = bias[c];
-    k.pad = 0.0f;
-    k.rdenom = 1.0 / (sqrt(static_cast<double>(var[c])) + static_cast<double>(kEps));
+    const double r = 1.0 / (sqrt(static_cast<double>(var)) + static_cast<double>(kEps));
+    FoldCoef k;
+    k.mean = mean;
+    k.r_hi = static_cast<float>(r);
+    k.r_lo = static_cast<float>(r - static_cast<double>(k.r_hi));
+    k.scale = scale;
+    k.bias = bias;
+    k.pad0 = k.pad1 = k.pad2 = 0.0f;
     return k;
+}
+
+__device__ __forceinline__ float normalize(float x, const FoldCoef& k)
+{
+    const float t = x - k.mean;
+    return fmaf(t, k.r_hi, t * k.r_lo);
+}
+
+// pre-activation from x_hat: scale then bias, each rounded
+__device__ __forceinline__ float affine(float xn, const FoldCoef& k)
+{
+    const float s = xn * k.scale;
+    return s + k.bias;
+}
+
+__global__ __launch_bounds__(kBlock) void bn_fold_kernel(const float* mean, const float* var, const float* scale,
+                                                         const float* bias, int channels, FoldCoef* table)
+{
+    const int c = blockIdx.x * kBlock + threadIdx.x;
+    if (c < channels) table[c] = make_coef(mean[c], var[c], scale[c], bias[c]);
 }
 
 struct EpilogueArgs {
@@ -38,122 +59,109 @@ struct EpilogueArgs {
     float* pre;        // nullable
     float* x_saved;    // nullable
     float* x_norm;     // nullable
-    const float* mean;
-    const float* var;
-    const float* scale;
-    const float* bias;
+    const FoldCoef* table;   // BN
+    const float* bias;       // bias only
     FastDiv by_spatial;
     FastDiv by_channels;
     uint32_t total;
 };
 
-template<int ACT, bool BN>
-__device__ __forceinline__ float epilogue_value(float x, const PlaneCoef& k, float& xn)
+template<bool BN>
+__device__ __forceinline__ FoldCoef fetch_coef(const EpilogueArgs& a, uint32_t c)
 {
-    float pre;
     if constexpr (BN) {
-        const float t = x - k.mean;
-        xn = static_cast<float>(static_cast<double>(t) * k.rdenom);
-        const float s = xn * k.scale;
-        pre = s + k.bias;
+        return a.table[c];
+    } else {
+        FoldCoef k;
+        k.bias = a.bias[c];
+        return k;
+    }
+}
+
+template<bool BN>
+__device__ __forceinline__ float pre_value(float x, const FoldCoef& k, float& xn)
+{
+    if constexpr (BN) {
+        xn = normalize(x, k);
+        return affine(xn, k);
     } else {
         xn = 0.0f;
-        pre = x + k.bias;
+        return x + k.bias;
     }
-    return pre;
 }
 
-// One workgroup streams kChunk consecutive elements; the (few) planes it touches get their
-// per-channel constants computed once into LDS while the loads are in flight.
-template<int ACT, bool BN>
+// One 128-bit vector per lane over the flat tensor.  A lane finds its plane with one
+// multiply-high division and loads that channel's folded constants (a 32-byte, cache-resident
+// broadcast); the rare vector that straddles two planes loads the next channel's as well.
+template<int ACT, bool BN, bool NT>
 __global__ __launch_bounds__(kBlock) void epilogue_fwd_kernel(EpilogueArgs a)
 {
-    __shared__ PlaneCoef tab[kTable];
-    const uint32_t chunk0 = blockIdx.x * static_cast<uint32_t>(kChunk);
+    const uint32_t e = (blockIdx.x * static_cast<uint32_t>(kBlock) + threadIdx.x) * 4;
+    if (e >= a.total) return;
+    const bool full = e + 3 < a.total;
+    Pack<4> xin;
+    if (full) {
+        xin = ld<4, NT>(a.x, e);
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) xin.v[k] = (e + k < a.total) ? a.x[e + k] : 0.0f;
+    }
     const uint32_t hw = a.by_spatial.d;
-    uint32_t first_plane, rem0;
-    a.by_spatial.divmod(chunk0, first_plane, rem0);
-
-    Pack<4> xin[kUnroll];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        const uint32_t e = chunk0 + (u * kBlock + threadIdx.x) * 4;
-        if (e + 3 < a.total) {
-            xin[u] = ld<4>(a.x, e);
-        } else {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) xin[u].v[k] = (e + k < a.total) ? a.x[e + k] : 0.0f;
-        }
-    }
-
-    const uint32_t chunk_end = min(chunk0 + static_cast<uint32_t>(kChunk), a.total);
-    const uint32_t nplanes = a.by_spatial.div(chunk_end - 1) - first_plane + 1;
-    if (threadIdx.x < nplanes) {
-        uint32_t q, c;
-        a.by_channels.divmod(first_plane + threadIdx.x, q, c);
-        PlaneCoef k;
-        if constexpr (BN) {
-            k = make_coef(a.mean, a.var, a.scale, a.bias, c);
-        } else {
-            k.rdenom = 0.0;
-            k.mean = 0.0f;
-            k.scale = 1.0f;
-            k.bias = a.bias[c];
-            k.pad = 0.0f;
-        }
-        tab[threadIdx.x] = k;
-    }
-    __syncthreads();
-
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        const uint32_t l = (u * kBlock + threadIdx.x) * 4;
-        const uint32_t e = chunk0 + l;
-        if (e >= a.total) continue;
-        uint32_t lp, r;
-        a.by_spatial.divmod(rem0 + l, lp, r);
-        Pack<4> yo, po, no;
-        PlaneCoef k = tab[lp];
+    uint32_t plane, r, q, c;
+    a.by_spatial.divmod(e, plane, r);
+    a.by_channels.divmod(plane, q, c);
+    const FoldCoef k0 = fetch_coef<BN>(a, c);
+    Pack<4> yo, po, no;
+    if (r + 3 < hw) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            if (r + j == hw) k = tab[lp + 1];
-            po.v[j] = epilogue_value<ACT, BN>(xin[u].v[j], k, no.v[j]);
+            po.v[j] = pre_value<BN>(xin.v[j], k0, no.v[j]);
             yo.v[j] = act_apply<ACT>(po.v[j]);
         }
-        if (e + 3 < a.total) {
-            if (a.x_saved) st<4>(a.x_saved, e, xin[u]);
-            if (BN && a.x_norm) st<4>(a.x_norm, e, no);
-            if (a.pre) st<4>(a.pre, e, po);
-            st<4>(a.y, e, yo);
-        } else {
-            for (int j = 0; j < 4 && e + j < a.total; ++j) {
-                if (a.x_saved) a.x_saved[e + j] = xin[u].v[j];
-                if (BN && a.x_norm) a.x_norm[e + j] = no.v[j];
-                if (a.pre) a.pre[e + j] = po.v[j];
-                a.y[e + j] = yo.v[j];
+    } else {
+        // crosses into the next plane(s): walk element by element
+        FoldCoef k = k0;
+        uint32_t rr = r, cc = c;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (rr == hw) {
+                rr = 0;
+                cc = cc + 1 == a.by_channels.d ? 0 : cc + 1;
+                k = fetch_coef<BN>(a, cc);
             }
+            po.v[j] = pre_value<BN>(xin.v[j], k, no.v[j]);
+            yo.v[j] = act_apply<ACT>(po.v[j]);
+            ++rr;
+        }
+    }
+    if (full) {
+        if (a.x_saved) st<4, NT>(a.x_saved, e, xin);
+        if (BN && a.x_norm) st<4, NT>(a.x_norm, e, no);
+        if (a.pre) st<4, NT>(a.pre, e, po);
+        st<4, NT>(a.y, e, yo);
+    } else {
+        for (int j = 0; j < 4 && e + j < a.total; ++j) {
+            if (a.x_saved) a.x_saved[e + j] = xin.v[j];
+            if (BN && a.x_norm) a.x_norm[e + j] = no.v[j];
+            if (a.pre) a.pre[e + j] = po.v[j];
+            a.y[e + j] = yo.v[j];
         }
     }
 }
 
-// Any shape, any alignment: one element per lane, constants recomputed per element.
+// Pointers that are not 16-byte aligned: one element per lane.
 template<int ACT, bool BN>
-__global__ __launch_bounds__(kBlock) void epilogue_fwd_generic_kernel(EpilogueArgs a)
+__global__ __launch_bounds__(kBlock) void epilogue_fwd_scalar_kernel(EpilogueArgs a)
 {
     const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
     if (e >= a.total) return;
     uint32_t plane, r, q, c;
     a.by_spatial.divmod(e, plane, r);
     a.by_channels.divmod(plane, q, c);
-    PlaneCoef k;
-    if constexpr (BN) {
-        k = make_coef(a.mean, a.var, a.scale, a.bias, c);
-    } else {
-        k.bias = a.bias[c];
-    }
+    const FoldCoef k = fetch_coef<BN>(a, c);
     const float x = a.x[e];
     float xn;
-    const float pre = epilogue_value<ACT, BN>(x, k, xn);
+    const float pre = pre_value<BN>(x, k, xn);
     if (a.x_saved) a.x_saved[e] = x;
     if (BN && a.x_norm) a.x_norm[e] = xn;
     if (a.pre) a.pre[e] = pre;
@@ -175,16 +183,21 @@ int check_shape(const char* who, int batch, int channels, int spatial, uint32_t*
 }
 
 template<bool BN>
-int launch_epilogue_fwd(const char* who, EpilogueArgs a, int spatial, int activation, hipStream_t stream)
+int launch_epilogue_fwd(const char* who, EpilogueArgs a, int activation, hipStream_t stream)
 {
-    const bool fast = spatial >= kMinSpatialFast && aligned16(a.x) && aligned16(a.y) && aligned16(a.pre) &&
-                      aligned16(a.x_saved) && aligned16(a.x_norm);
+    // the walk across a plane boundary handles any plane size, including single elements
+    const bool vec = aligned16(a.x) && aligned16(a.y) && aligned16(a.pre) && aligned16(a.x_saved) &&
+                     aligned16(a.x_norm);
+    // bytes this launch moves: x in, y out, plus each materialised extra output
+    const size_t streams = 2 + (a.pre ? 1 : 0) + (a.x_saved ? 1 : 0) + (a.x_norm ? 1 : 0);
+    const bool nt = static_cast<size_t>(a.total) * 4 * streams >= kStreamingBytes;
     const bool known = dispatch_activation(activation, [&]<int ACT>() {
-        if (fast) {
-            hipLaunchKernelGGL((epilogue_fwd_kernel<ACT, BN>), dim3(grid_for(a.total, kChunk)), dim3(kBlock), 0,
-                               stream, a);
+        if (vec) {
+            const dim3 grid(grid_for(a.total, static_cast<size_t>(kBlock) * 4));
+            if (nt) hipLaunchKernelGGL((epilogue_fwd_kernel<ACT, BN, true>), grid, dim3(kBlock), 0, stream, a);
+            else hipLaunchKernelGGL((epilogue_fwd_kernel<ACT, BN, false>), grid, dim3(kBlock), 0, stream, a);
         } else {
-            hipLaunchKernelGGL((epilogue_fwd_generic_kernel<ACT, BN>), dim3(grid_for(a.total, kBlock)),
+            hipLaunchKernelGGL((epilogue_fwd_scalar_kernel<ACT, BN>), dim3(grid_for(a.total, kBlock)),
                                dim3(kBlock), 0, stream, a);
         }
     });
@@ -201,23 +214,9 @@ int launch_epilogue_fwd(const char* who, EpilogueArgs a, int spatial, int activa
 // segment in fp32, carry across segments in double; the workgroup's pair of sums goes to
 // partial[c][j] and a second kernel adds the partials of a channel in a fixed order.
 // ------------------------------------------------------------------------------------------
-constexpr int kSeg = kWave * 4 * kUnroll;   // 1024 floats
+constexpr int kSegLoads = 4;                  // 128-bit loads in flight per lane
+constexpr int kSeg = kWave * 4 * kSegLoads;   // 1024 floats
 constexpr int kItemsPerBlock = 16;
-
-struct ReducePlan {
-    int parts;    // segments per plane
-    int items;    // batch * parts
-    int blocks;   // workgroups per channel
-};
-
-ReducePlan make_plan(int batch, int spatial)
-{
-    ReducePlan p;
-    p.parts = (spatial + kSeg - 1) / kSeg;
-    p.items = batch * p.parts;
-    p.blocks = (p.items + kItemsPerBlock - 1) / kItemsPerBlock;
-    return p;
-}
 
 struct ReduceGeom {
     int channels, spatial, parts, items, blocks;
@@ -227,21 +226,20 @@ struct ReduceGeom {
 
 ReduceGeom make_geom(int batch, int channels, int spatial)
 {
-    ReducePlan p = make_plan(batch, spatial);
     ReduceGeom g;
     g.channels = channels;
     g.spatial = spatial;
-    g.parts = p.parts;
-    g.items = p.items;
-    g.blocks = p.blocks;
-    g.by_parts = FastDiv(static_cast<uint32_t>(p.parts));
-    g.by_blocks = FastDiv(static_cast<uint32_t>(p.blocks));
+    g.parts = (spatial + kSeg - 1) / kSeg;
+    g.items = batch * g.parts;
+    g.blocks = (g.items + kItemsPerBlock - 1) / kItemsPerBlock;
+    g.by_parts = FastDiv(static_cast<uint32_t>(g.parts));
+    g.by_blocks = FastDiv(static_cast<uint32_t>(g.blocks));
     return g;
 }
 
-// Visits every element of this workgroup's items: f(value_index, lane_local_count) is called as
-// body(offset_in_tensor) for V consecutive floats.  Returns through the functor's own state.
-template<int V, typename Body>
+// Calls body(base, seg0, seg1, lane) for every item of workgroup (c, j): `base` is the offset of
+// the item's plane, [seg0, seg1) its segment inside the plane.
+template<typename Body>
 __device__ __forceinline__ void for_each_item(const ReduceGeom& g, uint32_t c, uint32_t j, Body&& body)
 {
     const int lane = threadIdx.x & (kWave - 1);
@@ -259,7 +257,7 @@ __device__ __forceinline__ void for_each_item(const ReduceGeom& g, uint32_t c, u
 }
 
 // ---- statistics: S1 = sum(x - K), S2 = sum((x - K)^2), K = first element of the channel ----
-template<int V>
+template<int V, bool NT>
 __global__ __launch_bounds__(kBlock) void bn_stats_partial_kernel(const float* x, ReduceGeom g, double2* partial)
 {
     __shared__ double slots[2][kBlock / kWave];
@@ -267,13 +265,13 @@ __global__ __launch_bounds__(kBlock) void bn_stats_partial_kernel(const float* x
     g.by_blocks.divmod(blockIdx.x, c, j);
     const float shift = x[static_cast<size_t>(c) * g.spatial];
     double s1 = 0.0, s2 = 0.0;
-    for_each_item<V>(g, c, j, [&](size_t base, int seg0, int seg1, int lane) {
+    for_each_item(g, c, j, [&](size_t base, int seg0, int seg1, int lane) {
         constexpr int kLoads = kSeg / (kWave * V);
         Pack<V> v[kLoads];
 #pragma unroll
         for (int u = 0; u < kLoads; ++u) {
             const int off = seg0 + (u * kWave + lane) * V;
-            if (off < seg1) v[u] = ld<V>(x, base + off);
+            if (off < seg1) v[u] = ld<V, NT>(x, base + off);
         }
         float a1 = 0.0f, a2 = 0.0f;
 #pragma unroll
@@ -296,10 +294,13 @@ __global__ __launch_bounds__(kBlock) void bn_stats_partial_kernel(const float* x
     if (threadIdx.x == 0) partial[blockIdx.x] = make_double2(t1, t2);
 }
 
-// One wavefront per channel adds the channel's partials and finishes mean / variance.
+// One wavefront per channel adds the channel's partials, finishes mean / variance, updates the
+// rolling statistics and (when asked) folds the constants the apply pass needs.
 __global__ __launch_bounds__(kBlock) void bn_stats_finish_kernel(const float* x, const double2* partial, int channels,
                                                                  int spatial, int blocks, double count, float* mean,
-                                                                 float* var, float* rolling_mean, float* rolling_var)
+                                                                 float* var, float* rolling_mean, float* rolling_var,
+                                                                 const float* scale, const float* bias,
+                                                                 FoldCoef* table)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const int c = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
@@ -328,6 +329,7 @@ __global__ __launch_bounds__(kBlock) void bn_stats_finish_kernel(const float* x,
             r = 0.99f * rolling_var[c];
             rolling_var[c] = r + .01f * fv;
         }
+        if (table) table[c] = make_coef(fm, fv, scale[c], bias[c]);
     }
 }
 
@@ -342,27 +344,27 @@ struct BackwardArgs {
     const float* bias;
 };
 
-template<int ACT, bool BN, bool WRITE, int V>
+template<int ACT, bool BN, bool WRITE, int V, bool NT>
 __global__ __launch_bounds__(kBlock) void bwd_partial_kernel(BackwardArgs a, ReduceGeom g, double2* partial)
 {
     __shared__ double slots[2][kBlock / kWave];
     uint32_t c, j;
     g.by_blocks.divmod(blockIdx.x, c, j);
-    PlaneCoef k;
-    if constexpr (BN) k = make_coef(a.mean, a.var, a.scale, a.bias, c);
+    FoldCoef k;
+    if constexpr (BN) k = make_coef(a.mean[c], a.var[c], a.scale[c], a.bias[c]);
     const bool recompute = BN && a.pre == nullptr;
     double sa = 0.0, sb = 0.0;
-    for_each_item<V>(g, c, j, [&](size_t base, int seg0, int seg1, int lane) {
+    for_each_item(g, c, j, [&](size_t base, int seg0, int seg1, int lane) {
         constexpr int kLoads = kSeg / (kWave * V);
         Pack<V> d[kLoads], xv[kLoads], pv[kLoads];
 #pragma unroll
         for (int u = 0; u < kLoads; ++u) {
             const int off = seg0 + (u * kWave + lane) * V;
             if (off < seg1) {
-                d[u] = ld<V>(a.delta, base + off);
-                if constexpr (BN) xv[u] = ld<V>(a.x, base + off);
+                d[u] = ld<V, NT>(a.delta, base + off);
+                if constexpr (BN) xv[u] = ld<V, NT>(a.x, base + off);
                 if constexpr (ACT != PXH_LINEAR) {
-                    if (!recompute) pv[u] = ld<V>(a.pre, base + off);
+                    if (!recompute) pv[u] = ld<V, NT>(a.pre, base + off);
                 }
             }
         }
@@ -376,19 +378,15 @@ __global__ __launch_bounds__(kBlock) void bwd_partial_kernel(BackwardArgs a, Red
                     float dv = d[u].v[q];
                     if constexpr (ACT != PXH_LINEAR) {
                         float pre;
-                        if (recompute) {
-                            float xn;
-                            pre = epilogue_value<ACT, true>(xv[u].v[q], k, xn);
-                        } else {
-                            pre = pv[u].v[q];
-                        }
+                        if (recompute) pre = affine(normalize(xv[u].v[q], k), k);
+                        else pre = pv[u].v[q];
                         dv = dv * act_grad<ACT>(pre);
                         d[u].v[q] = dv;
                     }
                     fa += dv;
                     if constexpr (BN) fb += dv * (xv[u].v[q] - k.mean);
                 }
-                if constexpr (WRITE && ACT != PXH_LINEAR) st<V>(a.delta, base + off, d[u]);
+                if constexpr (WRITE && ACT != PXH_LINEAR) st<V, NT>(a.delta, base + off, d[u]);
             }
         }
         sa += static_cast<double>(fa);
@@ -399,18 +397,21 @@ __global__ __launch_bounds__(kBlock) void bwd_partial_kernel(BackwardArgs a, Red
     if (threadIdx.x == 0) partial[blockIdx.x] = make_double2(ta, tb);
 }
 
-// Per-channel constants of the dx pass, produced by the finish kernel.
-struct BackwardCoef {
+// Per-channel constants of the dx pass, produced by the finish kernel (64 bytes).
+struct __attribute__((aligned(16))) DxCoef {
+    FoldCoef f;
     double rroot;     // 1 / sqrt(float(var + eps))
     double c2;        // var_delta * 2 / count
     double md_term;   // float(mean_delta / float(count))
+    double pad;
 };
 
 template<bool BN>
 __global__ __launch_bounds__(kBlock) void bwd_finish_kernel(const double2* partial, int channels, int blocks, int count,
-                                                            const float* var, const float* scale,
-                                                            float* scale_updates, float* bias_updates,
-                                                            float* mean_delta, float* var_delta, BackwardCoef* coef)
+                                                            const float* mean, const float* var, const float* scale,
+                                                            const float* bias, float* scale_updates,
+                                                            float* bias_updates, float* mean_delta, float* var_delta,
+                                                            DxCoef* coef)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const int c = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
@@ -439,10 +440,12 @@ __global__ __launch_bounds__(kBlock) void bwd_finish_kernel(const double2* parti
             const float vd = sum_ddx * (-.5f * powf(ve, -3.0f / 2.0f));
             if (mean_delta) mean_delta[c] = md;
             if (var_delta) var_delta[c] = vd;
-            BackwardCoef k;
+            DxCoef k;
+            k.f = make_coef(mean[c], v, s, bias[c]);
             k.rroot = 1.0 / sqrt(static_cast<double>(ve));
             k.c2 = static_cast<double>(vd) * 2. / static_cast<double>(count);
             k.md_term = static_cast<double>(md / static_cast<float>(count));
+            k.pad = 0.0;
             coef[c] = k;
         }
     }
@@ -452,19 +455,10 @@ struct DxArgs {
     float* delta;
     const float* x;
     const float* pre;   // nullable: recomputed
-    const float* mean;
-    const float* var;
-    const float* scale;
-    const float* bias;
-    const BackwardCoef* coef;
+    const DxCoef* coef;
     FastDiv by_spatial;
     FastDiv by_channels;
     uint32_t total;
-};
-
-struct DxCoef {
-    PlaneCoef f;
-    BackwardCoef b;
 };
 
 template<int ACT>
@@ -472,133 +466,121 @@ __device__ __forceinline__ float dx_value(float d, float x, float pre_in, bool r
 {
     if constexpr (ACT != PXH_LINEAR) {
         float pre = pre_in;
-        if (recompute) {
-            float xn;
-            pre = epilogue_value<ACT, true>(x, k.f, xn);
-        }
+        if (recompute) pre = affine(normalize(x, k.f), k.f);
         d = d * act_grad<ACT>(pre);
     }
     const float dd = d * k.f.scale;
     const float xm = x - k.f.mean;
     // src/CpuUtil.cpp:336-338 evaluated in double, stored as float
-    const double v = static_cast<double>(dd) * k.b.rroot + k.b.c2 * static_cast<double>(xm) + k.b.md_term;
+    const double v = static_cast<double>(dd) * k.rroot + k.c2 * static_cast<double>(xm) + k.md_term;
     return static_cast<float>(v);
 }
 
-template<int ACT>
+template<int ACT, bool NT>
 __global__ __launch_bounds__(kBlock) void bn_dx_kernel(DxArgs a)
 {
-    __shared__ DxCoef tab[kTable];
-    const uint32_t chunk0 = blockIdx.x * static_cast<uint32_t>(kChunk);
-    const uint32_t hw = a.by_spatial.d;
-    uint32_t first_plane, rem0;
-    a.by_spatial.divmod(chunk0, first_plane, rem0);
+    const uint32_t e = (blockIdx.x * static_cast<uint32_t>(kBlock) + threadIdx.x) * 4;
+    if (e >= a.total) return;
+    const bool full = e + 3 < a.total;
     const bool recompute = a.pre == nullptr;
-
-    Pack<4> din[kUnroll], xin[kUnroll], pin[kUnroll];
+    Pack<4> din, xin, pin;
+    if (full) {
+        din = ld<4, NT>(a.delta, e);
+        xin = ld<4, NT>(a.x, e);
+        if (ACT != PXH_LINEAR && !recompute) pin = ld<4, NT>(a.pre, e);
+    } else {
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        const uint32_t e = chunk0 + (u * kBlock + threadIdx.x) * 4;
-        if (e + 3 < a.total) {
-            din[u] = ld<4>(a.delta, e);
-            xin[u] = ld<4>(a.x, e);
-            if (ACT != PXH_LINEAR && !recompute) pin[u] = ld<4>(a.pre, e);
-        } else {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const bool ok = e + k < a.total;
-                din[u].v[k] = ok ? a.delta[e + k] : 0.0f;
-                xin[u].v[k] = ok ? a.x[e + k] : 0.0f;
-                pin[u].v[k] = (ok && ACT != PXH_LINEAR && !recompute) ? a.pre[e + k] : 0.0f;
-            }
+        for (int k = 0; k < 4; ++k) {
+            const bool ok = e + k < a.total;
+            din.v[k] = ok ? a.delta[e + k] : 0.0f;
+            xin.v[k] = ok ? a.x[e + k] : 0.0f;
+            pin.v[k] = (ok && ACT != PXH_LINEAR && !recompute) ? a.pre[e + k] : 0.0f;
         }
     }
-
-    const uint32_t chunk_end = min(chunk0 + static_cast<uint32_t>(kChunk), a.total);
-    const uint32_t nplanes = a.by_spatial.div(chunk_end - 1) - first_plane + 1;
-    if (threadIdx.x < nplanes) {
-        uint32_t q, c;
-        a.by_channels.divmod(first_plane + threadIdx.x, q, c);
-        DxCoef k;
-        k.f = make_coef(a.mean, a.var, a.scale, a.bias, c);
-        k.b = a.coef[c];
-        tab[threadIdx.x] = k;
-    }
-    __syncthreads();
-
+    const uint32_t hw = a.by_spatial.d;
+    uint32_t plane, r, q, c;
+    a.by_spatial.divmod(e, plane, r);
+    a.by_channels.divmod(plane, q, c);
+    Pack<4> out;
+    if (r + 3 < hw) {
+        const DxCoef k = a.coef[c];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        const uint32_t l = (u * kBlock + threadIdx.x) * 4;
-        const uint32_t e = chunk0 + l;
-        if (e >= a.total) continue;
-        uint32_t lp, r;
-        a.by_spatial.divmod(rem0 + l, lp, r);
-        Pack<4> out;
-        if (r + 3 < hw) {
-            const DxCoef k = tab[lp];
+        for (int j = 0; j < 4; ++j) out.v[j] = dx_value<ACT>(din.v[j], xin.v[j], pin.v[j], recompute, k);
+    } else {
+        uint32_t rr = r, cc = c;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) out.v[j] = dx_value<ACT>(din[u].v[j], xin[u].v[j], pin[u].v[j], recompute, k);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const DxCoef k = tab[lp + (r + j >= hw ? 1 : 0)];
-                out.v[j] = dx_value<ACT>(din[u].v[j], xin[u].v[j], pin[u].v[j], recompute, k);
+        for (int j = 0; j < 4; ++j) {
+            if (rr == hw) {
+                rr = 0;
+                cc = cc + 1 == a.by_channels.d ? 0 : cc + 1;
             }
+            out.v[j] = dx_value<ACT>(din.v[j], xin.v[j], pin.v[j], recompute, a.coef[cc]);
+            ++rr;
         }
-        if (e + 3 < a.total) {
-            st<4>(a.delta, e, out);
-        } else {
-            for (int j = 0; j < 4 && e + j < a.total; ++j) a.delta[e + j] = out.v[j];
-        }
+    }
+    if (full) {
+        st<4, NT>(a.delta, e, out);
+    } else {
+        for (int j = 0; j < 4 && e + j < a.total; ++j) a.delta[e + j] = out.v[j];
     }
 }
 
 template<int ACT>
-__global__ __launch_bounds__(kBlock) void bn_dx_generic_kernel(DxArgs a)
+__global__ __launch_bounds__(kBlock) void bn_dx_scalar_kernel(DxArgs a)
 {
     const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
     if (e >= a.total) return;
     uint32_t plane, r, q, c;
     a.by_spatial.divmod(e, plane, r);
     a.by_channels.divmod(plane, q, c);
-    DxCoef k;
-    k.f = make_coef(a.mean, a.var, a.scale, a.bias, c);
-    k.b = a.coef[c];
     const bool recompute = a.pre == nullptr;
     const float pre = (ACT != PXH_LINEAR && !recompute) ? a.pre[e] : 0.0f;
-    a.delta[e] = dx_value<ACT>(a.delta[e], a.x[e], pre, recompute, k);
+    a.delta[e] = dx_value<ACT>(a.delta[e], a.x[e], pre, recompute, a.coef[c]);
 }
 
+// workspace: [partial sums][per-channel constants]
 size_t partial_bytes(int batch, int channels, int spatial)
 {
-    const ReducePlan p = make_plan(batch, spatial);
-    return static_cast<size_t>(channels) * p.blocks * sizeof(double2);
+    const ReduceGeom g = make_geom(batch, channels, spatial);
+    const size_t b = static_cast<size_t>(channels) * g.blocks * sizeof(double2);
+    return (b + 255) & ~static_cast<size_t>(255);
 }
 
 size_t workspace_bytes(int batch, int channels, int spatial)
 {
-    // partial sums, then the per-channel constants of the dx pass
-    size_t b = partial_bytes(batch, channels, spatial);
-    b = (b + 255) & ~static_cast<size_t>(255);
-    return b + static_cast<size_t>(channels) * sizeof(BackwardCoef);
+    return partial_bytes(batch, channels, spatial) + static_cast<size_t>(channels) * sizeof(DxCoef);
 }
 
-int launch_stats(const float* x, float* mean, float* var, float* rolling_mean, float* rolling_var, int batch,
-                 int channels, int spatial, void* ws, hipStream_t stream)
+void* coef_region(void* ws, int batch, int channels, int spatial)
+{
+    return static_cast<char*>(ws) + partial_bytes(batch, channels, spatial);
+}
+
+// A tensor this large cannot stay in the last-level cache between two passes over it.
+bool streams_past_cache(uint32_t total, int tensors)
+{
+    return static_cast<size_t>(total) * 4 * tensors >= kStreamingBytes;
+}
+
+int launch_stats(const float* x, float* mean, float* var, float* rolling_mean, float* rolling_var, const float* scale,
+                 const float* bias, FoldCoef* table, int batch, int channels, int spatial, uint32_t total, void* ws,
+                 hipStream_t stream)
 {
     const ReduceGeom g = make_geom(batch, channels, spatial);
     double2* partial = static_cast<double2*>(ws);
     const dim3 grid(static_cast<unsigned>(channels) * g.blocks);
+    const bool nt = streams_past_cache(total, 1);
     if (spatial % 4 == 0 && aligned16(x)) {
-        hipLaunchKernelGGL((bn_stats_partial_kernel<4>), grid, dim3(kBlock), 0, stream, x, g, partial);
+        if (nt) hipLaunchKernelGGL((bn_stats_partial_kernel<4, true>), grid, dim3(kBlock), 0, stream, x, g, partial);
+        else hipLaunchKernelGGL((bn_stats_partial_kernel<4, false>), grid, dim3(kBlock), 0, stream, x, g, partial);
     } else {
-        hipLaunchKernelGGL((bn_stats_partial_kernel<1>), grid, dim3(kBlock), 0, stream, x, g, partial);
+        hipLaunchKernelGGL((bn_stats_partial_kernel<1, false>), grid, dim3(kBlock), 0, stream, x, g, partial);
     }
     int rc = check_launch("bn_stats_partial");
     if (rc) return rc;
     hipLaunchKernelGGL(bn_stats_finish_kernel, dim3(grid_for(channels, kBlock / kWave)), dim3(kBlock), 0, stream, x,
                        partial, channels, spatial, g.blocks, static_cast<double>(batch) * spatial, mean, var,
-                       rolling_mean, rolling_var);
+                       rolling_mean, rolling_var, scale, bias, table);
     return check_launch("bn_stats_finish");
 }
 
@@ -609,19 +591,58 @@ using namespace pxh;
 
 extern "C" {
 
+size_t pxh_bn_workspace_bytes(int batch, int channels, int spatial)
+{
+    if (batch <= 0 || channels <= 0 || spatial <= 0) return 0;
+    return workspace_bytes(batch, channels, spatial);
+}
+
+size_t pxh_bn_folded_bytes(int channels)
+{
+    return channels > 0 ? static_cast<size_t>(channels) * sizeof(FoldCoef) : 0;
+}
+
+int pxh_bn_fold(const float* rolling_mean, const float* rolling_var, const float* scale, const float* bias,
+                int channels, void* folded, void* stream)
+{
+    if (!rolling_mean || !rolling_var || !scale || !bias || !folded) return fail_invalid("pxh_bn_fold: null pointer");
+    if (channels <= 0) return fail_invalid("pxh_bn_fold: channels must be positive");
+    if (!aligned16(folded)) return fail_invalid("pxh_bn_fold: folded must be 16-byte aligned");
+    hipLaunchKernelGGL(bn_fold_kernel, dim3(grid_for(channels, kBlock)), dim3(kBlock), 0, as_stream(stream),
+                       rolling_mean, rolling_var, scale, bias, channels, static_cast<FoldCoef*>(folded));
+    return check_launch("pxh_bn_fold");
+}
+
+int pxh_bn_folded_act_forward(const float* x, float* y, float* pre_activation, const void* folded, int batch,
+                              int channels, int spatial, int activation, void* stream)
+{
+    if (!x || !y || !folded) return fail_invalid("pxh_bn_folded_act_forward: null pointer");
+    if (!aligned16(folded)) return fail_invalid("pxh_bn_folded_act_forward: folded must be 16-byte aligned");
+    EpilogueArgs a{};
+    int rc = check_shape("pxh_bn_folded_act_forward", batch, channels, spatial, &a.total);
+    if (rc) return rc;
+    a.x = x; a.y = y; a.pre = pre_activation;
+    a.table = static_cast<const FoldCoef*>(folded);
+    a.by_spatial = FastDiv(spatial); a.by_channels = FastDiv(channels);
+    return launch_epilogue_fwd<true>("pxh_bn_folded_act_forward", a, activation, as_stream(stream));
+}
+
 int pxh_bn_infer_act_forward(const float* x, float* y, float* pre_activation, const float* rolling_mean,
                              const float* rolling_var, const float* scale, const float* bias, int batch,
-                             int channels, int spatial, int activation, void* stream)
+                             int channels, int spatial, int activation, void* workspace,
+                             size_t workspace_bytes_given, void* stream)
 {
     if (!x || !y || !rolling_mean || !rolling_var || !scale || !bias)
         return fail_invalid("pxh_bn_infer_act_forward: null pointer");
-    EpilogueArgs a{};
-    int rc = check_shape("pxh_bn_infer_act_forward", batch, channels, spatial, &a.total);
+    uint32_t total;
+    int rc = check_shape("pxh_bn_infer_act_forward", batch, channels, spatial, &total);
     if (rc) return rc;
-    a.x = x; a.y = y; a.pre = pre_activation; a.x_saved = nullptr; a.x_norm = nullptr;
-    a.mean = rolling_mean; a.var = rolling_var; a.scale = scale; a.bias = bias;
-    a.by_spatial = FastDiv(spatial); a.by_channels = FastDiv(channels);
-    return launch_epilogue_fwd<true>("pxh_bn_infer_act_forward", a, spatial, activation, as_stream(stream));
+    void* ws;
+    rc = resolve_workspace(workspace, workspace_bytes_given, pxh_bn_folded_bytes(channels), &ws);
+    if (rc) return rc;
+    rc = pxh_bn_fold(rolling_mean, rolling_var, scale, bias, channels, ws, stream);
+    if (rc) return rc;
+    return pxh_bn_folded_act_forward(x, y, pre_activation, ws, batch, channels, spatial, activation, stream);
 }
 
 int pxh_bias_act_forward(const float* x, float* y, float* pre_activation, const float* bias, int batch,
@@ -633,18 +654,12 @@ int pxh_bias_act_forward(const float* x, float* y, float* pre_activation, const 
     if (rc) return rc;
     a.x = x; a.y = y; a.pre = pre_activation; a.bias = bias;
     a.by_spatial = FastDiv(spatial); a.by_channels = FastDiv(channels);
-    return launch_epilogue_fwd<false>("pxh_bias_act_forward", a, spatial, activation, as_stream(stream));
+    return launch_epilogue_fwd<false>("pxh_bias_act_forward", a, activation, as_stream(stream));
 }
 
 int pxh_add_bias(float* output, const float* bias, int batch, int n, int size, void* stream)
 {
     return pxh_bias_act_forward(output, output, nullptr, bias, batch, n, size, PXH_LINEAR, stream);
-}
-
-size_t pxh_bn_workspace_bytes(int batch, int channels, int spatial)
-{
-    if (batch <= 0 || channels <= 0 || spatial <= 0) return 0;
-    return workspace_bytes(batch, channels, spatial);
 }
 
 int pxh_bn_stats(const float* x, float* mean, float* var, int batch, int channels, int spatial, void* workspace,
@@ -657,7 +672,8 @@ int pxh_bn_stats(const float* x, float* mean, float* var, int batch, int channel
     void* ws;
     rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws);
     if (rc) return rc;
-    return launch_stats(x, mean, var, nullptr, nullptr, batch, channels, spatial, ws, as_stream(stream));
+    return launch_stats(x, mean, var, nullptr, nullptr, nullptr, nullptr, nullptr, batch, channels, spatial, total,
+                        ws, as_stream(stream));
 }
 
 int pxh_bn_train_act_forward(const float* x, float* y, float* pre_activation, float* x_saved, float* x_norm,
@@ -675,12 +691,14 @@ int pxh_bn_train_act_forward(const float* x, float* y, float* pre_activation, fl
     rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws);
     if (rc) return rc;
     hipStream_t s = as_stream(stream);
-    rc = launch_stats(x, mean, var, rolling_mean, rolling_var, batch, channels, spatial, ws, s);
+    FoldCoef* table = static_cast<FoldCoef*>(coef_region(ws, batch, channels, spatial));
+    rc = launch_stats(x, mean, var, rolling_mean, rolling_var, scale, bias, table, batch, channels, spatial, a.total,
+                      ws, s);
     if (rc) return rc;
     a.x = x; a.y = y; a.pre = pre_activation; a.x_saved = x_saved; a.x_norm = x_norm;
-    a.mean = mean; a.var = var; a.scale = scale; a.bias = bias;
+    a.table = table;
     a.by_spatial = FastDiv(spatial); a.by_channels = FastDiv(channels);
-    return launch_epilogue_fwd<true>("pxh_bn_train_act_forward", a, spatial, activation, s);
+    return launch_epilogue_fwd<true>("pxh_bn_train_act_forward", a, activation, s);
 }
 
 int pxh_bn_act_backward(float* delta, const float* x, const float* pre_activation, const float* mean,
@@ -699,37 +717,43 @@ int pxh_bn_act_backward(float* delta, const float* x, const float* pre_activatio
     hipStream_t s = as_stream(stream);
     const ReduceGeom g = make_geom(batch, channels, spatial);
     double2* partial = static_cast<double2*>(ws);
-    size_t off = (partial_bytes(batch, channels, spatial) + 255) & ~static_cast<size_t>(255);
-    BackwardCoef* coef = reinterpret_cast<BackwardCoef*>(static_cast<char*>(ws) + off);
+    DxCoef* coef = static_cast<DxCoef*>(coef_region(ws, batch, channels, spatial));
 
     BackwardArgs b{ delta, x, pre_activation, mean, var, scale, bias };
     const bool vec = spatial % 4 == 0 && aligned16(delta) && aligned16(x) && aligned16(pre_activation);
+    const int tensors = pre_activation ? 3 : 2;
+    const bool nt = vec && streams_past_cache(total, tensors);
     const dim3 grid(static_cast<unsigned>(channels) * g.blocks);
     const bool known = dispatch_activation(activation, [&]<int ACT>() {
-        if (vec) {
-            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 4>), grid, dim3(kBlock), 0, s, b, g, partial);
+        if (nt) {
+            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 4, true>), grid, dim3(kBlock), 0, s, b, g, partial);
+        } else if (vec) {
+            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 4, false>), grid, dim3(kBlock), 0, s, b, g, partial);
         } else {
-            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 1>), grid, dim3(kBlock), 0, s, b, g, partial);
+            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 1, false>), grid, dim3(kBlock), 0, s, b, g, partial);
         }
     });
     if (!known) return fail_invalid("pxh_bn_act_backward: unknown activation %d", activation);
     rc = check_launch("bn_backward_partial");
     if (rc) return rc;
     hipLaunchKernelGGL((bwd_finish_kernel<true>), dim3(grid_for(channels, kBlock / kWave)), dim3(kBlock), 0, s, partial,
-                       channels, g.blocks, batch * spatial, var, scale, scale_updates, bias_updates, mean_delta,
-                       var_delta, coef);
+                       channels, g.blocks, batch * spatial, mean, var, scale, bias, scale_updates, bias_updates,
+                       mean_delta, var_delta, coef);
     rc = check_launch("bn_backward_finish");
     if (rc) return rc;
 
     DxArgs d{};
-    d.delta = delta; d.x = x; d.pre = pre_activation; d.mean = mean; d.var = var; d.scale = scale; d.bias = bias;
-    d.coef = coef; d.by_spatial = FastDiv(spatial); d.by_channels = FastDiv(channels); d.total = total;
-    const bool fast = spatial >= kMinSpatialFast && aligned16(delta) && aligned16(x) && aligned16(pre_activation);
+    d.delta = delta; d.x = x; d.pre = pre_activation; d.coef = coef;
+    d.by_spatial = FastDiv(spatial); d.by_channels = FastDiv(channels); d.total = total;
+    const bool dx_vec = aligned16(delta) && aligned16(x) && aligned16(pre_activation);
+    const bool dx_nt = streams_past_cache(total, tensors + 1);
     dispatch_activation(activation, [&]<int ACT>() {
-        if (fast) {
-            hipLaunchKernelGGL((bn_dx_kernel<ACT>), dim3(grid_for(total, kChunk)), dim3(kBlock), 0, s, d);
+        if (dx_vec) {
+            const dim3 dx_grid(grid_for(total, static_cast<size_t>(kBlock) * 4));
+            if (dx_nt) hipLaunchKernelGGL((bn_dx_kernel<ACT, true>), dx_grid, dim3(kBlock), 0, s, d);
+            else hipLaunchKernelGGL((bn_dx_kernel<ACT, false>), dx_grid, dim3(kBlock), 0, s, d);
         } else {
-            hipLaunchKernelGGL((bn_dx_generic_kernel<ACT>), dim3(grid_for(total, kBlock)), dim3(kBlock), 0, s, d);
+            hipLaunchKernelGGL((bn_dx_scalar_kernel<ACT>), dim3(grid_for(total, kBlock)), dim3(kBlock), 0, s, d);
         }
     });
     return check_launch("bn_backward_dx");
@@ -755,17 +779,17 @@ int pxh_bias_act_backward(float* delta, const float* pre_activation, float* bias
     const dim3 grid(static_cast<unsigned>(channels) * g.blocks);
     const bool known = dispatch_activation(activation, [&]<int ACT>() {
         if (vec) {
-            hipLaunchKernelGGL((bwd_partial_kernel<ACT, false, true, 4>), grid, dim3(kBlock), 0, s, b, g, partial);
+            hipLaunchKernelGGL((bwd_partial_kernel<ACT, false, true, 4, false>), grid, dim3(kBlock), 0, s, b, g, partial);
         } else {
-            hipLaunchKernelGGL((bwd_partial_kernel<ACT, false, true, 1>), grid, dim3(kBlock), 0, s, b, g, partial);
+            hipLaunchKernelGGL((bwd_partial_kernel<ACT, false, true, 1, false>), grid, dim3(kBlock), 0, s, b, g, partial);
         }
     });
     if (!known) return fail_invalid("pxh_bias_act_backward: unknown activation %d", activation);
     rc = check_launch("bias_backward_partial");
     if (rc) return rc;
     hipLaunchKernelGGL((bwd_finish_kernel<false>), dim3(grid_for(channels, kBlock / kWave)), dim3(kBlock), 0, s,
-                       partial, channels, g.blocks, batch * spatial, nullptr, nullptr, nullptr, bias_updates, nullptr,
-                       nullptr, nullptr);
+                       partial, channels, g.blocks, batch * spatial, nullptr, nullptr, nullptr, nullptr, nullptr,
+                       bias_updates, nullptr, nullptr, nullptr);
     return check_launch("bias_backward_finish");
 }
 

@@ -57,8 +57,8 @@ struct YoloActivateOp {
     FastDiv by_area;
     FastDiv by_entries;
     template<int V> struct Regs { Pack<V> x; };
-    template<int V> __device__ void load(size_t e, Regs<V>& r) const { r.x = ld<V>(in, e); }
-    template<int V> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const { r.x = ld<V, NT>(in, e); }
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
         uint32_t plane, off, q, entry;
         by_area.divmod(static_cast<uint32_t>(e), plane, off);
@@ -73,7 +73,7 @@ struct YoloActivateOp {
             const float x = r.x.v[k];
             o.v[k] = (entry < 2 || entry >= 4) ? 1.0f / (1.0f + expf(-x)) : x;
         }
-        st<V>(out, e, o);
+        st<V, NT>(out, e, o);
     }
 };
 
@@ -432,7 +432,7 @@ int pxh_yolo_activate(const float* input, float* output, int batch, int masks, i
     YoloActivateOp op{ input, output, FastDiv(area), FastDiv(classes + 5) };
     // the 128-bit path steps a row boundary at most once per vector: needs area >= 4
     const bool vec = area >= 4 && aligned16(input) && aligned16(output);
-    return launch_stream("pxh_yolo_activate", static_cast<size_t>(total), vec, op, as_stream(stream));
+    return launch_stream("pxh_yolo_activate", static_cast<size_t>(total), vec, 8, op, as_stream(stream));
 }
 
 size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int width, int height)

@@ -40,11 +40,33 @@ def _nchw(x):
 
 
 # ---------------------------------------------------------------- epilogue forward
-def bn_infer_act_forward(x, y, rolling_mean, rolling_var, scale, bias, activation, pre_activation=None):
+def bn_infer_act_forward(x, y, rolling_mean, rolling_var, scale, bias, activation, pre_activation=None,
+                         workspace=None):
     _chk_all(x, y, rolling_mean, rolling_var, scale, bias, pre_activation)
     n, c, s = _nchw(x)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
     call("pxh_bn_infer_act_forward", ptr(x), ptr(y), ptr(pre_activation), ptr(rolling_mean), ptr(rolling_var),
-         ptr(scale), ptr(bias), n, c, s, act_id(activation), _stream())
+         ptr(scale), ptr(bias), n, c, s, act_id(activation), ptr(workspace), wb, _stream())
+    return y
+
+
+def bn_fold(rolling_mean, rolling_var, scale, bias, folded=None):
+    """Folds the per-channel inference constants; returns the folded buffer."""
+    _chk_all(rolling_mean, rolling_var, scale, bias)
+    c = rolling_mean.numel()
+    if folded is None:
+        folded = torch.empty(int(capi.load().pxh_bn_folded_bytes(c)) // 4, device=rolling_mean.device,
+                             dtype=torch.float32)
+    _chk(folded)
+    call("pxh_bn_fold", ptr(rolling_mean), ptr(rolling_var), ptr(scale), ptr(bias), c, ptr(folded), _stream())
+    return folded
+
+
+def bn_folded_act_forward(x, y, folded, activation, pre_activation=None):
+    _chk_all(x, y, folded, pre_activation)
+    n, c, s = _nchw(x)
+    call("pxh_bn_folded_act_forward", ptr(x), ptr(y), ptr(pre_activation), ptr(folded), n, c, s,
+         act_id(activation), _stream())
     return y
 
 

@@ -54,8 +54,8 @@ def test_rejects_bad_arguments_without_launching():
     assert capi.call_raw("pxh_activate", 0, None, 5, None) == inv
     assert capi.call_raw("pxh_activate", 99, p, 5, None) == inv
     assert "unknown activation" in capi.last_error()
-    assert capi.call_raw("pxh_bn_infer_act_forward", p, p, None, p, p, p, p, 0, 3, 4, 0, None) == inv
-    assert capi.call_raw("pxh_bn_infer_act_forward", p, p, None, None, p, p, p, 1, 3, 4, 0, None) == inv
+    assert capi.call_raw("pxh_bn_infer_act_forward", p, p, None, p, p, p, p, 0, 3, 4, 0, None, 0, None) == inv
+    assert capi.call_raw("pxh_bn_infer_act_forward", p, p, None, None, p, p, p, 1, 3, 4, 0, None, 0, None) == inv
     # the reference's maxpool constructor checks (include/MaxPoolLayer.h:57-59)
     assert capi.call_raw("pxh_maxpool_forward", p, p, p, 1, 1, 4, 4, 2, 2, 0, 2, 1, None) == inv
     assert "kernel must be positive" in capi.last_error()
@@ -69,7 +69,7 @@ def test_rejects_bad_arguments_without_launching():
     assert capi.call_raw("pxh_adam_update", 8, p, p, p, p, 0, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 0, None) == inv
     assert capi.call_raw("pxh_adam_update", 8, p, p, p, p, 1, 0, 1e-3, 0.9, 0.999, 1e-8, 0.0, 0, None) == inv
     # tensors of 2^31 elements or more are refused, not mis-indexed
-    assert capi.call_raw("pxh_bn_infer_act_forward", p, p, None, p, p, p, p, 1024, 1024, 4096, 0, None) == -2
+    assert capi.call_raw("pxh_bn_infer_act_forward", p, p, None, p, p, p, p, 1024, 1024, 4096, 0, None, 0, None) == -2
     with pytest.raises(capi.PxError):
         capi.call("pxh_activate", 0, None, 5, None)
 
@@ -81,6 +81,7 @@ def test_workspace_sizes():
     big = lib.pxh_bn_workspace_bytes(16, 32, 608 * 608)
     assert 0 < small < big < (1 << 24)
     assert lib.pxh_yolo_workspace_bytes(64, 3, 80, 76, 76) == 64 * 3 * 23 * 13 * 8
+    assert lib.pxh_bn_folded_bytes(1024) == 1024 * 32 and lib.pxh_bn_folded_bytes(0) == 0
 
 
 def test_ops_refuse_cpu_tensors():

@@ -33,9 +33,10 @@ def bn_case(seed, N, C, HW, spread=1.0):
 
 
 # spatial sizes cover: 128-bit fast path, planes that are not a multiple of 4 (13x13, 19x19),
-# several planes per workgroup, planes below the fast-path limit, single elements
+# several planes per wavefront, planes below the fast-path limit (8), single elements
 SHAPES = [(2, 16, 416 * 416 // 16), (3, 32, 52 * 52), (4, 64, 26 * 26), (5, 7, 169), (3, 11, 361),
-          (2, 5, 28), (2, 5, 27), (3, 4, 1), (1, 1, 4097), (2, 3, 4096), (7, 2, 33)]
+          (2, 5, 28), (2, 5, 27), (3, 4, 1), (1, 1, 4097), (2, 3, 4096), (7, 2, 33), (3, 5, 8), (2, 3, 9), (4, 3, 7),
+          (5, 67, 11)]
 
 
 @pytest.mark.parametrize("act", ACTS)
@@ -55,6 +56,26 @@ def test_bn_infer_act_forward_matches_oracle(ops, oracle, act):
         if act in ("leaky", "linear", "relu"):
             d = ulp_distance(host(gy), want)
             assert d.max() <= 1 and (d > 0).mean() < 1e-4, what
+
+
+def test_bn_folded_matches_two_launch_entry(ops):
+    """Folding once and streaming is the same arithmetic as the entry point that folds per call."""
+    N, C, HW = 3, 19, 361
+    x, scale, bias, rmean, rvar = bn_case(150, N, C, HW)
+    a = gpu(np.zeros_like(x)); b = gpu(np.zeros_like(x))
+    ops.bn_infer_act_forward(gpu(x), a, gpu(rmean), gpu(rvar), gpu(scale), gpu(bias), "mish")
+    folded = ops.bn_fold(gpu(rmean), gpu(rvar), gpu(scale), gpu(bias))
+    ops.bn_folded_act_forward(gpu(x), b, folded, "mish")
+    assert_bit_exact(host(a), host(b), "folded vs per-call fold")
+    # caller-provided workspace for the per-call fold
+    import torch
+    ws = torch.empty(C * 8, device="cuda")
+    c = gpu(np.zeros_like(x))
+    ops.bn_infer_act_forward(gpu(x), c, gpu(rmean), gpu(rvar), gpu(scale), gpu(bias), "mish", workspace=ws)
+    assert_bit_exact(host(c), host(b), "caller workspace")
+    from pixienn_amd.capi import PxError
+    with pytest.raises(PxError):
+        ops.bn_infer_act_forward(gpu(x), c, gpu(rmean), gpu(rvar), gpu(scale), gpu(bias), "mish", workspace=ws[:8])
 
 
 def test_bn_infer_in_place_and_unaligned(ops, oracle):
@@ -100,7 +121,7 @@ def test_bias_act_forward_matches_oracle(ops, oracle, act):
 
 
 TRAIN_SHAPES = [(4, 8, 52 * 52), (3, 16, 361), (16, 5, 169), (2, 3, 4096 + 512), (5, 2, 27), (2, 4, 1024 * 3 + 4),
-                (1, 3, 37)]
+                (1, 3, 37), (6, 9, 8), (3, 5, 7)]
 
 
 @pytest.mark.parametrize("act", ["leaky", "mish", "linear"])
