@@ -220,7 +220,8 @@ int pxh_yolo_loss(const float* output, float* delta, const float* truths, const 
                   float noobject_scale, float class_scale, void* workspace, size_t workspace_bytes,
                   void* stream);
 
-size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int width, int height);
+size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int width, int height,
+                                int max_truth);
 
 /* Whole YoloLayer::forward of a loss-computing pass in one sweep over the head: decode, dense
  * delta (every element written, no prior fill), positives assigned on the device from the

@@ -55,7 +55,7 @@ _OTHER_RETURNS = {
     "pxh_abi_version": (I, []),
     "pxh_bn_workspace_bytes": (Z, [I, I, I]),
     "pxh_bn_folded_bytes": (Z, [I]),
-    "pxh_yolo_workspace_bytes": (Z, [I, I, I, I, I]),
+    "pxh_yolo_workspace_bytes": (Z, [I, I, I, I, I, I]),
     "pxh_debug_fastdiv": (ctypes.c_uint, [ctypes.c_uint, ctypes.c_uint]),
 }
 
