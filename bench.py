@@ -32,9 +32,10 @@ HBM_PEAK_GBS = 8000.0
 EPILOGUE_BATCH = 64
 EPILOGUE_ACTS = ["leaky", "mish", "logistic"]
 
-# HBM bytes per launch of the leaky epilogue kernel relative to its algorithmic bytes, from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/epilogue_leaky_pmc.txt); None = not measured
-EPILOGUE_TRAFFIC_RATIO = None
+# HBM bytes per launch of the leaky epilogue kernel relative to its algorithmic bytes, from two
+# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of this script, each scaled by what the counter
+# reads for the 2 x 512 MiB plain copy below (profiles/epilogue_sweep_hbm_traffic.txt)
+EPILOGUE_TRAFFIC_RATIO = 0.9998
 
 
 def log(*a):
@@ -44,8 +45,8 @@ def log(*a):
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip the other kernels of the path")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-batch", type=int, default=64, help="images per shape in the CPU sample")
@@ -136,6 +137,23 @@ def measure_extras(torch, ops, wl, timer):
         return torch.randn(shape, device=dev)
 
     N = 16
+    # ---- route concat of YOLOv3 @608: 256x38^2 (upsampled) ++ 512x38^2, and 128x76^2 ++ 256x76^2
+    for (c1, c2, s) in [(256, 512, 38), (128, 256, 76)]:
+        a = randn(N, c1, s, s); b = randn(N, c2, s, s)
+        r = torch.empty((N, c1 + c2, s, s), device=dev)
+
+        def concat(i):
+            ops.route_forward(a, r, 0)
+            ops.route_forward(b, r, c1 * s * s)
+
+        def split(i):
+            ops.route_backward(r, a, 0)
+            ops.route_backward(r, b, c1 * s * s)
+
+        e = N * (c1 + c2) * s * s
+        add("route_fwd", "%dx(%d+%d)x%d^2" % (N, c1, c2, s), 8 * e, timer.time(concat, 20), "2 launches, 8B/elem")
+        add("route_bwd", "%dx(%d+%d)x%d^2" % (N, c1, c2, s), 12 * e, timer.time(split, 20), "2 launches, 12B/elem")
+        del a, b, r
     # ---- max-pool 2x2 s2 forward + backward (config 2)
     for c, s in wl.YOLOV3_MAXPOOL_SHAPES:
         e_in = N * c * s * s
@@ -244,20 +262,33 @@ def measure_extras(torch, ops, wl, timer):
     add("adam_update", "%d params" % P, 32 * P, ms_adam, "32B/param, L2 folded into the update")
 
     # ---- non-conv ms per batch, YOLOv3 @608, batch 16, one training step:
-    # 72 BN'd conv epilogues fwd+bwd, 3 bias epilogues, 23 shortcuts fwd+bwd, 2 upsamples fwd+bwd,
-    # 3 heads (fused decode+delta) at batch 16 scaled from the batch-64 measurement, Adam
+    # 72 BN'd conv epilogues fwd+bwd, 3 bias epilogues, 23 shortcuts fwd+bwd, 2 upsamples and 2 route
+    # concats fwd+bwd, the four max-pools of the data-movement configuration fwd+bwd, 3 heads (fused
+    # decode+delta) at batch 16 scaled from the batch-64 measurement, Adam
     total = 0.0
     for key, (f, b, count) in bn_ms.items():
         total += (f + b) * count
     for key, (f, b, count) in shortcut_ms.items():
         total += (f + b) * count
     for r in rows:
-        if r["kernel"].startswith("upsample"):
+        if r["kernel"].startswith(("upsample", "maxpool", "route_fwd", "route_bwd")):
             total += r["ms"]
     for s, (ms_d, ms_t) in head_ms.items():
         total += ms_t * N / NB
     total += ms_adam
     return rows, total
+
+
+def calibration_copy(torch, ops, timer):
+    """A plain copy of known size (512 MiB read, 512 MiB written) through the route kernel: the
+    launch the hardware traffic counters are scaled by, and the practical ceiling of this HBM."""
+    n = 128 << 20
+    src = torch.randn((1, n), device="cuda:0")
+    dst = torch.empty_like(src)
+    ms = timer.time(lambda i: ops.route_forward(src, dst, 0), 10)
+    gbs = 8.0 * n / (ms * 1e-3) / 1e9
+    return dict(kernel="stream_kernel<4, true, RouteOp<false>>", elems=n, bytes=8 * n, ms=round(ms, 4),
+                GBps=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 3))
 
 
 def cpu_baseline(wl, batch):
@@ -361,6 +392,9 @@ def main():
                 log("epilogue %-9s %-16s %8.4f ms %8.1f GB/s" % (r["act"], r["shape"], r["ms"], r["GBps"]))
             del xs, ys
 
+    copy_row = calibration_copy(torch, ops, timer)
+    log("plain copy of 2 x 512 MiB: %.4f ms %.1f GB/s" % (copy_row["ms"], copy_row["GBps"]))
+
     extras, ms_batch = (None, None)
     if not args.no_extras:
         extras, ms_batch = measure_extras(torch, ops, wl, timer)
@@ -396,6 +430,7 @@ def main():
         "cpu_baseline": cpu,
         "noconv_ms_per_batch_yolov3_608": None if ms_batch is None else round(ms_batch, 3),
         "value_folding_every_call": round(value_raw, 1),
+        "plain_copy": copy_row,
         "per_activation": per_act,
         "per_shape": per_shape,
         "extras": extras,

@@ -151,6 +151,19 @@ int pxh_mul(int n, const float* x, float* y, void* stream);          /* y[i] = x
 int pxh_axpy(size_t n, float alpha, const float* x, float* y, void* stream);
 
 /* ------------------------------------------------------------------------
+ * Route (channel concatenation).  CPU semantics include/RouteLayer.h:91-137 (cblas_scopy /
+ * cblas_saxpy per image), device path include/cuda/RouteLayer.h:23-71 (one cudaMemcpy or
+ * cublasSaxpy per image and source layer; here one launch per source layer).
+ * Image b of the source layer (layer_outputs floats, packed) corresponds to
+ * route + b*route_outputs + offset.  forward copies the layer's output into the route's output;
+ * backward adds the route's delta slice into the layer's delta.  batch*route_outputs < 2^31.
+ * ---------------------------------------------------------------------- */
+int pxh_route_forward(const float* layer_output, float* route_output, int batch, int layer_outputs,
+                      int route_outputs, int offset, void* stream);
+int pxh_route_backward(const float* route_delta, float* layer_delta, int batch, int layer_outputs,
+                       int route_outputs, int offset, void* stream);
+
+/* ------------------------------------------------------------------------
  * Max-pool.  include/MaxPoolKernels.cuh:5-7, CPU semantics include/MaxPoolLayer.h:88-158.
  * ---------------------------------------------------------------------- */
 

@@ -232,6 +232,18 @@ def axpy(alpha, x, y):
     lib().pxo_axpy(_c_size(x.size), _c_float(alpha), _f(x), _f(y))
 
 
+def route_forward(layer_output, route_output, offset):
+    batch = layer_output.shape[0]
+    lib().pxo_route_forward(_f(layer_output), _f(route_output), batch, layer_output.size // batch,
+                            route_output.size // batch, int(offset))
+
+
+def route_backward(route_delta, layer_delta, offset):
+    batch = layer_delta.shape[0]
+    lib().pxo_route_backward(_f(route_delta), _f(layer_delta), batch, layer_delta.size // batch,
+                             route_delta.size // batch, int(offset))
+
+
 # ---------------- boxes / YOLO ----------------
 def _box(b):
     return (ctypes.c_float * 4)(*[float(v) for v in b])

@@ -607,6 +607,26 @@ void pxo_axpy(size_t n, float alpha, const float* x, float* y)
     for (size_t i = 0; i < n; ++i) y[i] = y[i] + alpha * x[i];
 }
 
+/* include/RouteLayer.h:91-113: cblas_scopy of each image of one source layer into its slice */
+void pxo_route_forward(const float* layer_output, float* route_output, int batch, int layer_outputs,
+                       int route_outputs, int offset)
+{
+    for (int b = 0; b < batch; ++b) {
+        const float* in = layer_output + (size_t) b * layer_outputs;
+        float* out = route_output + (size_t) b * route_outputs + offset;
+        for (int i = 0; i < layer_outputs; ++i) out[i] = in[i];
+    }
+}
+
+/* include/RouteLayer.h:115-137: cblas_saxpy(alpha = 1) of each slice into the source layer's delta */
+void pxo_route_backward(const float* route_delta, float* layer_delta, int batch, int layer_outputs,
+                        int route_outputs, int offset)
+{
+    for (int b = 0; b < batch; ++b)
+        pxo_axpy((size_t) layer_outputs, 1.0f, route_delta + (size_t) b * route_outputs + offset,
+                 layer_delta + (size_t) b * layer_outputs);
+}
+
 /* ------------------------------------------------------------------ */
 /* boxes -- src/DarkBox.cpp:84-151                                     */
 /* ------------------------------------------------------------------ */

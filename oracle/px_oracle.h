@@ -128,6 +128,13 @@ int pxo_yolo_build_targets(const pxo_yolo_cfg* cfg, const float* truths, int cou
                            int* classes, int* anchors, float* boxes);
 void pxo_axpy(size_t n, float alpha, const float* x, float* y);
 
+/* ---- route (channel concat): include/RouteLayer.h:91-137.  Parity pinned by construction only:
+ * a copy and an alpha = 1 saxpy per image; the reference holds no test for this layer. ---- */
+void pxo_route_forward(const float* layer_output, float* route_output, int batch, int layer_outputs,
+                       int route_outputs, int offset);
+void pxo_route_backward(const float* route_delta, float* layer_delta, int batch, int layer_outputs,
+                        int route_outputs, int offset);
+
 /* ---- Adam: include/cuda/Adam.h:49-90 + src/Adam.cu:26-37 ---- */
 void pxo_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch, int t, float lr,
                      float beta1, float beta2, float eps, float decay, int apply_decay);

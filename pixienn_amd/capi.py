@@ -37,6 +37,8 @@ SIGNATURES = {
     "pxh_constrain": [I, F, P, P],
     "pxh_mul": [I, P, P, P],
     "pxh_axpy": [Z, F, P, P, P],
+    "pxh_route_forward": [P, P, I, I, I, I, P],
+    "pxh_route_backward": [P, P, I, I, I, I, P],
     "pxh_maxpool_forward": [P, P, P, I, I, I, I, I, I, I, I, I, P],
     "pxh_maxpool_backward": [P, P, P, I, I, I, I, I, I, I, I, I, P],
     "pxh_maxpool_backward_scatter": [P, P, P, I, P],

@@ -109,6 +109,63 @@ struct AxpyOp {
     }
 };
 
+// ---------------------------------------------------------------- route (channel concat)
+// One source layer of a concatenation: image b of the layer (layer_outputs floats, packed) sits
+// at route + b*route_outputs + offset.  FORWARD copies layer -> route; BACKWARD adds the route
+// slice into the layer's delta (x + y, one rounding, like saxpy with alpha = 1).
+template<bool BACKWARD>
+struct RouteOp {
+    const float* src;      // forward: layer output; backward: route delta
+    float* dst;            // forward: route output; backward: layer delta
+    FastDiv by_image;      // layer_outputs
+    uint32_t route_outputs, offset;
+    template<int V> struct Regs { Pack<V> a, b; };
+    __device__ __forceinline__ size_t concat_index(size_t e) const
+    {
+        uint32_t image, within;
+        by_image.divmod(static_cast<uint32_t>(e), image, within);
+        return static_cast<size_t>(image) * route_outputs + offset + within;
+    }
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
+    {
+        if constexpr (BACKWARD) {
+            r.a = ld<V, NT>(src, concat_index(e));
+            r.b = ld<V, NT>(dst, e);
+        } else {
+            r.a = ld<V, NT>(src, e);
+        }
+    }
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        if constexpr (BACKWARD) {
+            Pack<V> o;
+#pragma unroll
+            for (int k = 0; k < V; ++k) o.v[k] = r.b.v[k] + r.a.v[k];
+            st<V, NT>(dst, e, o);
+        } else {
+            st<V, NT>(dst, concat_index(e), r.a);
+        }
+    }
+};
+
+int check_route(const char* who, const void* a, const void* b, int batch, int layer_outputs, int route_outputs,
+                int offset)
+{
+    if (batch < 0 || layer_outputs < 0 || route_outputs < 0 || offset < 0)
+        return fail_invalid("%s: negative size", who);
+    if (static_cast<int64_t>(offset) + layer_outputs > route_outputs)
+        return fail_invalid("%s: slice [%d, %d) exceeds the %d outputs of the route", who, offset,
+                            offset + layer_outputs, route_outputs);
+    const int64_t n = static_cast<int64_t>(batch) * layer_outputs;
+    if ((!a || !b) && n) return fail_invalid("%s: null pointer", who);
+    if (n >= (int64_t(1) << 31) || static_cast<int64_t>(batch) * route_outputs >= (int64_t(1) << 31))
+    {
+        set_error("%s: tensors of 2^31 elements or more are not supported", who);
+        return PXH_ERR_UNSUPPORTED;
+    }
+    return PXH_OK;
+}
+
 // ---------------------------------------------------------------- shortcut
 // pre = alpha*in + beta*from (two products, one sum, each rounded); out = act(pre)
 template<int ACT>
@@ -335,6 +392,36 @@ int pxh_axpy(size_t n, float alpha, const float* x, float* y, void* stream)
 {
     if ((!x || !y) && n) return fail_invalid("pxh_axpy: null pointer");
     return launch_stream("pxh_axpy", n, aligned16(x) && aligned16(y), 12, AxpyOp{ x, y, alpha }, as_stream(stream));
+}
+
+int pxh_route_forward(const float* layer_output, float* route_output, int batch, int layer_outputs,
+                      int route_outputs, int offset, void* stream)
+{
+    int rc = check_route("pxh_route_forward", layer_output, route_output, batch, layer_outputs, route_outputs, offset);
+    if (rc) return rc;
+    const size_t n = static_cast<size_t>(batch) * layer_outputs;
+    if (n == 0) return PXH_OK;
+    const bool vec = aligned16(layer_output) && aligned16(route_output) && layer_outputs % 4 == 0 &&
+                     route_outputs % 4 == 0 && offset % 4 == 0;
+    return launch_stream("pxh_route_forward", n, vec, 8,
+                         RouteOp<false>{ layer_output, route_output, FastDiv(layer_outputs),
+                                         static_cast<uint32_t>(route_outputs), static_cast<uint32_t>(offset) },
+                         as_stream(stream));
+}
+
+int pxh_route_backward(const float* route_delta, float* layer_delta, int batch, int layer_outputs,
+                       int route_outputs, int offset, void* stream)
+{
+    int rc = check_route("pxh_route_backward", route_delta, layer_delta, batch, layer_outputs, route_outputs, offset);
+    if (rc) return rc;
+    const size_t n = static_cast<size_t>(batch) * layer_outputs;
+    if (n == 0) return PXH_OK;
+    const bool vec = aligned16(route_delta) && aligned16(layer_delta) && layer_outputs % 4 == 0 &&
+                     route_outputs % 4 == 0 && offset % 4 == 0;
+    return launch_stream("pxh_route_backward", n, vec, 12,
+                         RouteOp<true>{ route_delta, layer_delta, FastDiv(layer_outputs),
+                                        static_cast<uint32_t>(route_outputs), static_cast<uint32_t>(offset) },
+                         as_stream(stream));
 }
 
 int pxh_shortcut(int batch, int w1, int h1, int c1, const float* add, int w2, int h2, int c2, float s1, float s2,

@@ -169,6 +169,23 @@ def axpy(alpha, x, y):
     call("pxh_axpy", x.numel(), float(alpha), ptr(x), ptr(y), _stream())
 
 
+def route_forward(layer_output, route_output, offset):
+    """Copies one source layer into its slice of a concatenation (include/RouteLayer.h:91-113).
+    layer_output [N, ...] packed; route_output [N, ...]; offset in floats within a route image."""
+    _chk_all(layer_output, route_output)
+    batch = layer_output.shape[0]
+    call("pxh_route_forward", ptr(layer_output), ptr(route_output), batch, layer_output.numel() // max(1, batch),
+         route_output.numel() // max(1, batch), int(offset), _stream())
+
+
+def route_backward(route_delta, layer_delta, offset):
+    """layer_delta += the layer's slice of route_delta (include/RouteLayer.h:115-137)."""
+    _chk_all(route_delta, layer_delta)
+    batch = layer_delta.shape[0]
+    call("pxh_route_backward", ptr(route_delta), ptr(layer_delta), batch, layer_delta.numel() // max(1, batch),
+         route_delta.numel() // max(1, batch), int(offset), _stream())
+
+
 # ---------------------------------------------------------------- max-pool / upsample / shortcut
 def maxpool_out_dim(n, kernel, stride, padding):
     """include/MaxPoolLayer.h:62-63 of the reference."""

@@ -158,3 +158,41 @@ def test_shortcut_reference_signature(ops, oracle):
     g = gpu(out0)
     ops.shortcut(N, W, H, 2, gpu(add2), W, H, C, 1.0, 1.0, g)
     assert_bit_exact(host(g), want, "shortcut channel mismatch")
+
+
+# route: YOLOv3-tiny concatenates 128x26^2 (upsampled) with 256x26^2; odd sizes take the scalar path
+@pytest.mark.parametrize("layers", [[(128, 26), (256, 26)], [(3, 5), (2, 5), (7, 5)], [(256, 38), (512, 38)], [(1, 1)]])
+def test_route_forward_backward(ops, oracle, layers):
+    import torch
+    N = 3
+    outs = [wl.normal(8100 + i, (N, c, s, s)) for i, (c, s) in enumerate(layers)]
+    per_image = [o[0].size for o in outs]
+    total = sum(per_image)
+    want = np.full((N, total), -5.0, F)
+    got = torch.full((N, total), -5.0, device="cuda")
+    offset = 0
+    for o, size in zip(outs, per_image):
+        oracle.route_forward(o, want, offset)
+        ops.route_forward(gpu(o), got, offset)
+        offset += size
+    assert_bit_exact(host(got), want, "route forward %s" % (layers,))
+    assert not (want == -5.0).any()
+    route_delta = wl.normal(8200, (N, total))
+    offset = 0
+    for i, (o, size) in enumerate(zip(outs, per_image)):
+        d0 = wl.normal(8300 + i, o.shape)
+        d_w = d0.copy()
+        oracle.route_backward(route_delta, d_w, offset)
+        d_g = gpu(d0)
+        ops.route_backward(gpu(route_delta), d_g, offset)
+        assert_bit_exact(host(d_g), d_w, "route backward %s layer %d" % (layers, i))
+        offset += size
+
+
+def test_route_rejects_slice_outside_route(ops):
+    import torch
+    from pixienn_amd import capi
+    a = torch.zeros(2, 8, device="cuda")
+    r = torch.zeros(2, 12, device="cuda")
+    with pytest.raises(capi.PxError):
+        ops.route_forward(a, r, 8)
