@@ -22,6 +22,8 @@
  *   upsample         parity unpinned by reference tests; closed form
  *                    (index copy), torch nearest interpolate, brute force
  *   shortcut         parity unpinned by reference tests; closed form a+b
+ *   route            parity unpinned by reference tests; closed form (copy,
+ *                    x + y per element)
  *   boxes / IoU      reference known-answer tests (tests/src/darkbox.cpp)
  *   YOLO head        reference known-answer tests (tests/src/yolo_cpu.cpp,
  *                    tests/src/yolo_cuda.cpp kernel-level vectors)

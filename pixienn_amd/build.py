@@ -53,5 +53,25 @@ def build_library(verbose=True):
     return LIB
 
 
+def build_host(verbose=True):
+    """Compiles the C++ layer interface (host/pixienn/*.h, header-only) as a translation unit of
+    its own: the check that it builds against the C ABI alone."""
+    host = os.path.join(PKG, "host")
+    probe = os.path.join(OBJ, "host_headers.cpp")
+    os.makedirs(OBJ, exist_ok=True)
+    with open(probe, "w") as f:
+        f.write('#include "pixienn/Layers.h"\nint pixienn_host_headers_compile() { return PXH_OK; }\n')
+    obj = os.path.join(OBJ, "host_headers.o")
+    cmd = [hipcc(), "-std=c++20", "-O1", "-Wall", "-Wextra", "-Wno-unused-parameter", "-I" + os.path.join(ROOT, "include"),
+           "-I" + host, "-c", probe, "-o", obj]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("host headers do not compile:\n" + proc.stderr)
+    if verbose and proc.stderr.strip():
+        print(proc.stderr, file=sys.stderr)
+    return obj
+
+
 if __name__ == "__main__":
     print(build_library())
+    print(build_host())

@@ -1,0 +1,231 @@
+// Layer interface of the MI355X kernels: the forward / backward / update / output / delta surface
+// of the engine's layers (reference: include/Layer.h:43-62) over the C ABI in pixienn_hip.h.
+//
+// What differs from the reference, on purpose:
+//   - properties come from a small key -> value map instead of a YAML node, with the reference's
+//     property names and defaults;
+//   - the model a layer belongs to is reduced to a Context: stream, training flag, network input
+//     size, class count, ground truth of the current batch and the optimiser settings;
+//   - Layer::forward does not zero-fill output_: every kernel here writes each output element.
+//     delta_ is still cleared when training, because backward passes accumulate into it.
+#pragma once
+
+#include <algorithm>
+#include <cmath>
+#include <map>
+#include <memory>
+#include <string>
+#include <variant>
+#include <vector>
+
+#include "DeviceVector.h"
+
+namespace px::hip {
+
+// ---------------------------------------------------------------- properties
+class Properties
+{
+public:
+    using Value = std::variant<int, float, bool, std::string, std::vector<int>>;
+
+    Properties() = default;
+    Properties(std::initializer_list<std::pair<const std::string, Value>> init) : values_(init) {}
+
+    Properties& set(const std::string& name, Value value)
+    {
+        values_[name] = std::move(value);
+        return *this;
+    }
+
+    bool has(const std::string& name) const { return values_.count(name) != 0; }
+
+    // Required property: throws when absent (reference: Layer<D>::property, include/Layer.h:240-250).
+    template<typename T>
+    T get(const std::string& name) const
+    {
+        auto it = values_.find(name);
+        PX_CHECK(it != values_.end(), "Layer has no property named \"" + name + "\".");
+        return convert<T>(it->second, name);
+    }
+
+    template<typename T>
+    T get(const std::string& name, const T& def) const
+    {
+        auto it = values_.find(name);
+        return it == values_.end() ? def : convert<T>(it->second, name);
+    }
+
+private:
+    template<typename T>
+    static T convert(const Value& v, const std::string& name)
+    {
+        if (const T* p = std::get_if<T>(&v)) return *p;
+        if constexpr (std::is_same_v<T, float>) {
+            if (const int* i = std::get_if<int>(&v)) return static_cast<float>(*i);
+        }
+        if constexpr (std::is_same_v<T, bool>) {
+            if (const int* i = std::get_if<int>(&v)) return *i != 0;
+        }
+        throw Error(__FILE__, __LINE__, __func__, "property \"" + name + "\" has another type");
+    }
+
+    std::map<std::string, Value> values_;
+};
+
+// ---------------------------------------------------------------- ground truth
+// One labelled box, relative to the image (reference: GroundTruth, include/GroundTruth.h).
+struct GroundTruth
+{
+    float x, y, w, h;
+    int classId;
+};
+
+using GroundTruthVec = std::vector<GroundTruth>;
+
+// ---------------------------------------------------------------- context
+// The part of the owning model the layers read.
+class Context
+{
+public:
+    hipStream_t stream = nullptr;
+    bool training = false;
+    int width = 0, height = 0;      // network input size
+    int classes = 0;
+
+    // optimiser (reference: Model<D>::adam*, learningRate, decay, include/Model.h)
+    float learningRate = 1e-3f, decay = 5e-4f;
+    float adamBeta1 = 0.9f, adamBeta2 = 0.999f, adamEpsilon = 1e-8f;
+    int timeStep = 1;               // Adam's t
+    int updateBatch = 1;            // images a parameter update averages over (batch * subdivisions)
+
+    // Uploads the ground truth of the current batch: [batch][maxTruth][5] floats + counts.
+    void setGroundTruth(const std::vector<GroundTruthVec>& batchTruth)
+    {
+        const auto batch = batchTruth.size();
+        std::size_t most = 1;
+        for (const auto& image: batchTruth) most = std::max(most, image.size());
+        std::vector<float> packed(batch * most * 5, 0.0f);
+        std::vector<int> counts(batch, 0);
+        for (std::size_t b = 0; b < batch; ++b) {
+            counts[b] = static_cast<int>(batchTruth[b].size());
+            for (std::size_t t = 0; t < batchTruth[b].size(); ++t) {
+                const auto& g = batchTruth[b][t];
+                float* p = &packed[(b * most + t) * 5];
+                p[0] = g.x; p[1] = g.y; p[2] = g.w; p[3] = g.h; p[4] = static_cast<float>(g.classId);
+            }
+        }
+        if (truths_.size() != packed.size()) truths_ = FloatVector(packed.size());
+        if (truthCounts_.size() != counts.size()) truthCounts_ = IntVector(counts.size());
+        truths_.copyHost(packed);
+        truthCounts_.copyHost(counts);
+        maxTruth_ = static_cast<int>(most);
+    }
+
+    const FloatVector& truths() const noexcept { return truths_; }
+    const IntVector& truthCounts() const noexcept { return truthCounts_; }
+    int maxTruth() const noexcept { return maxTruth_; }
+
+private:
+    FloatVector truths_;
+    IntVector truthCounts_;
+    int maxTruth_ = 0;
+};
+
+// ---------------------------------------------------------------- layer
+class Layer
+{
+public:
+    using V = FloatVector;
+    using Ptr = std::shared_ptr<Layer>;
+
+    Layer(Context& context, const Properties& props) : context_(context), props_(props)
+    {
+        batch_ = props.get<int>("batch", 1);
+        channels_ = props.get<int>("channels", 3);
+        height_ = props.get<int>("height", 0);
+        width_ = props.get<int>("width", 0);
+        index_ = props.get<int>("index", 0);
+        inputs_ = props.get<int>("inputs", channels_ * height_ * width_);
+        PX_CHECK(batch_ > 0 && channels_ > 0 && height_ >= 0 && width_ >= 0, "layer dimensions must be positive");
+    }
+
+    virtual ~Layer() = default;
+
+    // Clears the per-pass state.  Derived classes call it first, as in the reference
+    // (include/Layer.h:377-383), then write output_.
+    virtual void forward(const V& /*input*/)
+    {
+        if (training() && !delta_.empty()) delta_.fill(0.0f, stream());
+        cost_ = 0.0f;
+    }
+
+    // delta_ holds dL/d(output) on entry; a layer turns it into dL/d(input) and ACCUMULATES that
+    // into *grad (nullptr for the first layer).
+    virtual void backward(const V& /*input*/, V* /*grad*/)
+    {
+        if (gradientClipping_) PX_HIP_CHECK(pxh_constrain(static_cast<int>(delta_.size()), gradientClipValue_,
+                                                          delta_.data(), stream()));
+    }
+
+    virtual void update() {}
+
+    virtual bool hasCost() const noexcept { return false; }
+    float cost() const noexcept { return cost_; }
+
+    int batch() const noexcept { return batch_; }
+    int channels() const noexcept { return channels_; }
+    int height() const noexcept { return height_; }
+    int width() const noexcept { return width_; }
+    int index() const noexcept { return index_; }
+    int inputs() const noexcept { return inputs_; }
+    int outChannels() const noexcept { return outChannels_; }
+    int outHeight() const noexcept { return outHeight_; }
+    int outWidth() const noexcept { return outWidth_; }
+    int outputs() const noexcept { return outputs_; }
+
+    const V& output() const noexcept { return output_; }
+    V& delta() noexcept { return delta_; }
+
+    void setGradientClipping(bool on, float value) { gradientClipping_ = on; gradientClipValue_ = value; }
+
+protected:
+    // Sets the output shape and allocates output_ (and delta_, which inference never touches,
+    // only when the context trains).
+    void setOutput(int channels, int height, int width)
+    {
+        outChannels_ = channels;
+        outHeight_ = height;
+        outWidth_ = width;
+        outputs_ = channels * height * width;
+        const auto n = static_cast<std::size_t>(batch_) * outputs_;
+        PX_CHECK(n < (std::size_t(1) << 31), "tensors of 2^31 elements or more are not supported");
+        output_ = V(n);
+        if (context_.training) delta_ = V(n);
+    }
+
+    void checkInput(const V& input, const char* who) const
+    {
+        PX_CHECK(input.size() == static_cast<std::size_t>(batch_) * inputs_,
+                 std::string(who) + ": input size does not match batch * inputs");
+    }
+
+    Context& context() noexcept { return context_; }
+    const Context& context() const noexcept { return context_; }
+    const Properties& properties() const noexcept { return props_; }
+    hipStream_t stream() const noexcept { return context_.stream; }
+    bool training() const noexcept { return context_.training; }
+    bool inferring() const noexcept { return !context_.training; }
+
+    V output_, delta_;
+    float cost_ = 0.0f;
+
+private:
+    Context& context_;
+    Properties props_;
+    int batch_, channels_, height_, width_, index_, inputs_;
+    int outChannels_ = 0, outHeight_ = 0, outWidth_ = 0, outputs_ = 0;
+    bool gradientClipping_ = false;
+    float gradientClipValue_ = 1.0f;
+};
+
+}   // px::hip

@@ -1,0 +1,462 @@
+// The layers whose device work is the MI355X non-convolution kernels: conv epilogue (batch norm /
+// bias + activation), batch norm, max-pool, upsample, shortcut, route and the YOLO head.
+// Each class keeps the reference layer's properties, shape rules and error checks and issues the
+// fused C-ABI calls where the reference issues several library calls and copies.
+#pragma once
+
+#include <functional>
+
+#include "Adam.h"
+
+namespace px::hip {
+
+// reference: include/ActivationTypes.h:19-30 and the name table in src/Activation.cpp
+inline int activationFromName(const std::string& name)
+{
+    static const std::map<std::string, int> table = {
+            { "leaky", PXH_LEAKY }, { "linear", PXH_LINEAR }, { "loggy", PXH_LOGGY },
+            { "logistic", PXH_LOGISTIC }, { "mish", PXH_MISH }, { "relu", PXH_RELU },
+            { "softplus", PXH_SOFTPLUS }, { "swish", PXH_SWISH }, { "tanh", PXH_TANH } };
+    auto it = table.find(name);
+    PX_CHECK(it != table.end(), "unknown activation \"" + name + "\"");
+    return it->second;
+}
+
+// ---------------------------------------------------------------- conv epilogue
+// Everything a ConvLayer does after its GEMM and before its weight gradients
+// (reference: include/cuda/ConvLayer.h:284-307 forward, 315-338 backward, 388-413 update).
+// The convolution itself is delegated: `convolve` writes the raw conv result for an input, and
+// `convolveBackward` turns dL/d(conv result) into weight updates and dL/d(input).  Without them
+// the layer treats its input as the conv result (the form the kernels are measured in).
+class ConvLayer : public Layer
+{
+public:
+    using Convolve = std::function<void(const V& input, V& result)>;
+    using ConvolveBackward = std::function<void(const V& input, const V& delta, V* grad)>;
+
+    ConvLayer(Context& context, const Properties& props) : Layer(context, props)
+    {
+        activation_ = activationFromName(props.get<std::string>("activation", "logistic"));
+        batchNorm_ = props.get<bool>("batch_normalize", false);
+        filters_ = props.get<int>("filters", channels());
+        // shape of the conv RESULT; the delegated convolution owns kernel / stride / pad
+        const int oh = props.get<int>("out_height", height());
+        const int ow = props.get<int>("out_width", width());
+        setOutput(filters_, oh, ow);
+
+        const auto f = static_cast<std::size_t>(filters_);
+        biases_ = V(f, 0.0f);
+        if (batchNorm_) {
+            scales_ = V(f, 1.0f);
+            rollingMean_ = V(f, 0.0f);
+            rollingVar_ = V(f, 0.0f);
+            folded_ = DeviceVector<float>(pxh_bn_folded_bytes(filters_) / sizeof(float));
+        }
+        if (training()) {
+            biasUpdates_ = V(f, 0.0f);
+            biasM_ = V(f, 0.0f);
+            biasV_ = V(f, 0.0f);
+            if (batchNorm_) {
+                mean_ = V(f, 0.0f);
+                var_ = V(f, 0.0f);
+                scaleUpdates_ = V(f, 0.0f);
+                scaleM_ = V(f, 0.0f);
+                scaleV_ = V(f, 0.0f);
+            }
+        }
+    }
+
+    void setConvolution(Convolve fwd, ConvolveBackward bwd)
+    {
+        convolve_ = std::move(fwd);
+        convolveBackward_ = std::move(bwd);
+        result_ = V(output_.size());
+    }
+
+    // Parameter loading (reference: ConvLayer<D>::copyBiases etc., include/ConvLayer.h:48-54).
+    void copyBiases(const std::vector<float>& b) { load(biases_, b); foldedValid_ = false; }
+    void copyScales(const std::vector<float>& s) { load(scales_, s); foldedValid_ = false; }
+    void copyRollingMean(const std::vector<float>& m) { load(rollingMean_, m); foldedValid_ = false; }
+    void copyRollingVariance(const std::vector<float>& v) { load(rollingVar_, v); foldedValid_ = false; }
+
+    void forward(const V& input) override
+    {
+        Layer::forward(input);
+        const float* x = input.data();
+        if (convolve_) {
+            convolve_(input, result_);
+            x = result_.data();
+        } else {
+            PX_CHECK(input.size() == output_.size(), "ConvLayer: input is not a conv result of the output shape");
+        }
+        x_ = x;
+        const int spatial = outHeight() * outWidth();
+        if (!batchNorm_) {
+            PX_HIP_CHECK(pxh_bias_act_forward(x, output_.data(), nullptr, biases_.data(), batch(), filters_, spatial,
+                                              activation_, stream()));
+        } else if (training()) {
+            PX_HIP_CHECK(pxh_bn_train_act_forward(x, output_.data(), nullptr, nullptr, nullptr, mean_.data(),
+                                                  var_.data(), rollingMean_.data(), rollingVar_.data(),
+                                                  scales_.data(), biases_.data(), batch(), filters_, spatial,
+                                                  activation_, nullptr, 0, stream()));
+            foldedValid_ = false;       // the rolling statistics moved
+        } else {
+            if (!foldedValid_) {
+                PX_HIP_CHECK(pxh_bn_fold(rollingMean_.data(), rollingVar_.data(), scales_.data(), biases_.data(),
+                                         filters_, folded_.data(), stream()));
+                foldedValid_ = true;
+            }
+            PX_HIP_CHECK(pxh_bn_folded_act_forward(x, output_.data(), nullptr, folded_.data(), batch(), filters_,
+                                                   spatial, activation_, stream()));
+        }
+    }
+
+    // Needs the conv result of the matching forward to be unchanged (it is re-read instead of
+    // keeping saved copies of it, of x_hat and of the pre-activation).
+    void backward(const V& input, V* grad) override
+    {
+        Layer::backward(input, grad);
+        PX_CHECK(training() && x_ != nullptr, "ConvLayer: backward without a training forward");
+        const int spatial = outHeight() * outWidth();
+        if (batchNorm_) {
+            PX_HIP_CHECK(pxh_bn_act_backward(delta_.data(), x_, nullptr, mean_.data(), var_.data(), scales_.data(),
+                                             biases_.data(), scaleUpdates_.data(), biasUpdates_.data(), nullptr,
+                                             nullptr, batch(), filters_, spatial, activation_, nullptr, 0,
+                                             stream()));
+        } else {
+            // pre-activation = x + bias is not kept either; the linear head convs need none
+            preActivation(spatial);
+            PX_HIP_CHECK(pxh_bias_act_backward(delta_.data(), pre_.empty() ? nullptr : pre_.data(),
+                                               biasUpdates_.data(), batch(), filters_, spatial, activation_,
+                                               nullptr, 0, stream()));
+        }
+        if (convolveBackward_) {
+            convolveBackward_(input, delta_, grad);
+        } else if (grad) {
+            PX_HIP_CHECK(pxh_axpy(delta_.size(), 1.0f, delta_.data(), grad->data(), stream()));
+        }
+    }
+
+    // Adam on the biases and scales (the delegated convolution updates its own weights with
+    // the same Adam object: reference include/cuda/ConvLayer.h:388-413).
+    void update() override
+    {
+        const Adam adam(context());
+        adam.update(biases_, biasUpdates_, biasM_, biasV_, false);
+        if (batchNorm_) adam.update(scales_, scaleUpdates_, scaleM_, scaleV_, false);
+        foldedValid_ = false;
+    }
+
+    const V& biases() const noexcept { return biases_; }
+    const V& scales() const noexcept { return scales_; }
+    const V& rollingMean() const noexcept { return rollingMean_; }
+    const V& rollingVariance() const noexcept { return rollingVar_; }
+    const V& mean() const noexcept { return mean_; }
+    const V& variance() const noexcept { return var_; }
+    const V& biasUpdates() const noexcept { return biasUpdates_; }
+    const V& scaleUpdates() const noexcept { return scaleUpdates_; }
+
+private:
+    void load(V& dst, const std::vector<float>& src)
+    {
+        PX_CHECK(dst.size() == src.size(), "ConvLayer: parameter vector of the wrong size");
+        dst.copyHost(src);
+    }
+
+    // x + bias for a non-linear layer without batch norm (the gradient needs it)
+    void preActivation(int spatial)
+    {
+        if (activation_ == PXH_LINEAR) return;
+        if (pre_.empty()) pre_ = V(output_.size());
+        PX_HIP_CHECK(pxh_bias_act_forward(x_, pre_.data(), nullptr, biases_.data(), batch(), filters_, spatial,
+                                          PXH_LINEAR, stream()));
+    }
+
+    int activation_ = PXH_LOGISTIC, filters_ = 1;
+    bool batchNorm_ = false, foldedValid_ = false;
+    const float* x_ = nullptr;      // conv result of the last forward (borrowed)
+    V biases_, scales_, rollingMean_, rollingVar_, mean_, var_, folded_;
+    V biasUpdates_, scaleUpdates_, biasM_, biasV_, scaleM_, scaleV_;
+    V result_, pre_;
+    Convolve convolve_;
+    ConvolveBackward convolveBackward_;
+};
+
+// ---------------------------------------------------------------- max-pool
+// reference: include/MaxPoolLayer.h:50-158, include/cuda/MaxPoolLayer.h
+class MaxPoolLayer : public Layer
+{
+public:
+    MaxPoolLayer(Context& context, const Properties& props) : Layer(context, props)
+    {
+        kernel_ = props.get<int>("kernel", 1);
+        stride_ = props.get<int>("stride", 1);
+        padding_ = props.get<int>("padding", std::max(0, kernel_ - 1));
+        PX_CHECK(kernel_ > 0, "maxpool kernel must be positive");
+        PX_CHECK(stride_ > 0, "maxpool stride must be positive");
+        PX_CHECK(padding_ >= 0, "maxpool padding cannot be negative");
+        const int oh = (height() + padding_ - kernel_) / stride_ + 1;
+        const int ow = (width() + padding_ - kernel_) / stride_ + 1;
+        PX_CHECK(oh > 0 && ow > 0, "maxpool output dimensions must be positive");
+        setOutput(channels(), oh, ow);
+        if (training()) indexes_ = IntVector(output_.size());
+    }
+
+    void forward(const V& input) override
+    {
+        Layer::forward(input);
+        checkInput(input, "MaxPoolLayer");
+        if (indexes_.empty()) indexes_ = IntVector(output_.size());
+        PX_HIP_CHECK(pxh_maxpool_forward(input.data(), output_.data(), indexes_.data(), batch(), channels(),
+                                         height(), width(), outHeight(), outWidth(), kernel_, stride_, padding_,
+                                         stream()));
+    }
+
+    void backward(const V& input, V* grad) override
+    {
+        Layer::backward(input, grad);
+        if (grad == nullptr) return;
+        PX_HIP_CHECK(pxh_maxpool_backward(delta_.data(), indexes_.data(), grad->data(), batch(), channels(),
+                                          height(), width(), outHeight(), outWidth(), kernel_, stride_, padding_,
+                                          stream()));
+    }
+
+    const IntVector& indexes() const noexcept { return indexes_; }
+
+private:
+    int kernel_ = 1, stride_ = 1, padding_ = 0;
+    IntVector indexes_;
+};
+
+// ---------------------------------------------------------------- upsample
+// reference: include/UpsampleLayer.h:48-121, include/cuda/UpsampleLayer.h
+class UpsampleLayer : public Layer
+{
+public:
+    UpsampleLayer(Context& context, const Properties& props) : Layer(context, props)
+    {
+        stride_ = props.get<int>("stride", 2);
+        scale_ = props.get<float>("scale", 1.0f);
+        PX_CHECK(stride_ > 0, "upsample stride must be positive");
+        setOutput(channels(), height() * stride_, width() * stride_);
+    }
+
+    void forward(const V& input) override
+    {
+        Layer::forward(input);
+        checkInput(input, "UpsampleLayer");
+        PX_HIP_CHECK(pxh_upsample(input.data(), width(), height(), channels(), batch(), stride_, 1, scale_, nullptr,
+                                  output_.data(), stream()));
+    }
+
+    void backward(const V& input, V* grad) override
+    {
+        Layer::backward(input, grad);
+        if (grad == nullptr) return;
+        PX_HIP_CHECK(pxh_upsample(nullptr, width(), height(), channels(), batch(), stride_, 0, scale_, grad->data(),
+                                  delta_.data(), stream()));
+    }
+
+private:
+    int stride_ = 2;
+    float scale_ = 1.0f;
+};
+
+// ---------------------------------------------------------------- shortcut
+// reference: include/ShortcutLayer.h:45-141, include/cuda/ShortcutLayer.h:23-55
+class ShortcutLayer : public Layer
+{
+public:
+    ShortcutLayer(Context& context, const Properties& props, Layer::Ptr from) : Layer(context, props),
+                                                                                 from_(std::move(from))
+    {
+        PX_CHECK(from_ != nullptr, "shortcut needs its \"from\" layer");
+        activation_ = activationFromName(props.get<std::string>("activation", "linear"));
+        alpha_ = props.get<float>("alpha", 1.0f);
+        beta_ = props.get<float>("beta", 1.0f);
+        PX_CHECK(from_->batch() == batch(), "shortcut: batch sizes differ");
+        setOutput(channels(), height(), width());
+        sameShape_ = from_->outChannels() == outChannels() && from_->outHeight() == outHeight() &&
+                     from_->outWidth() == outWidth();
+        if (training() && (activation_ != PXH_LINEAR || !sameShape_)) preActivation_ = V(output_.size());
+    }
+
+    void forward(const V& input) override
+    {
+        Layer::forward(input);
+        checkInput(input, "ShortcutLayer");
+        float* pre = preActivation_.empty() ? nullptr : preActivation_.data();
+        if (sameShape_) {
+            PX_HIP_CHECK(pxh_shortcut_forward(input.data(), from_->output().data(), output_.data(), pre,
+                                              output_.size(), alpha_, beta_, activation_, stream()));
+            return;
+        }
+        // differing shapes: the index-mapped blend of the reference, then the activation
+        output_.copy(input, stream());
+        PX_HIP_CHECK(pxh_shortcut(batch(), outWidth(), outHeight(), outChannels(), from_->output().data(),
+                                  from_->outWidth(), from_->outHeight(), from_->outChannels(), alpha_, beta_,
+                                  output_.data(), stream()));
+        if (pre) preActivation_.copy(output_, stream());
+        PX_HIP_CHECK(pxh_activate(activation_, output_.data(), output_.size(), stream()));
+    }
+
+    void backward(const V& input, V* grad) override
+    {
+        Layer::backward(input, grad);
+        const float* pre = preActivation_.empty() ? nullptr : preActivation_.data();
+        if (sameShape_) {
+            PX_HIP_CHECK(pxh_shortcut_backward(delta_.data(), pre, from_->delta().data(),
+                                               grad ? grad->data() : nullptr, delta_.size(), alpha_, beta_,
+                                               activation_, stream()));
+            return;
+        }
+        if (activation_ != PXH_LINEAR)
+            PX_HIP_CHECK(pxh_gradient(activation_, pre, delta_.size(), delta_.data(), stream()));
+        PX_HIP_CHECK(pxh_shortcut(batch(), from_->outWidth(), from_->outHeight(), from_->outChannels(),
+                                  delta_.data(), outWidth(), outHeight(), outChannels(), 1.0f, beta_,
+                                  from_->delta().data(), stream()));
+        if (grad) PX_HIP_CHECK(pxh_axpy(delta_.size(), alpha_, delta_.data(), grad->data(), stream()));
+    }
+
+private:
+    Layer::Ptr from_;
+    int activation_ = PXH_LINEAR;
+    float alpha_ = 1.0f, beta_ = 1.0f;
+    bool sameShape_ = true;
+    V preActivation_;
+};
+
+// ---------------------------------------------------------------- route
+// reference: include/RouteLayer.h:39-137, include/cuda/RouteLayer.h:23-71
+class RouteLayer : public Layer
+{
+public:
+    RouteLayer(Context& context, const Properties& props, std::vector<Layer::Ptr> layers)
+            : Layer(context, props), layers_(std::move(layers))
+    {
+        PX_CHECK(!layers_.empty(), "route needs at least one source layer");
+        int outChannels = 0;
+        const int oh = layers_[0]->outHeight(), ow = layers_[0]->outWidth();
+        for (const auto& layer: layers_) {
+            PX_CHECK(layer->outHeight() == oh && layer->outWidth() == ow, "route: source layers differ in size");
+            PX_CHECK(layer->batch() == batch(), "route: batch sizes differ");
+            outChannels += layer->outChannels();
+        }
+        setOutput(outChannels, oh, ow);
+    }
+
+    void forward(const V& input) override
+    {
+        Layer::forward(input);
+        int offset = 0;
+        for (const auto& layer: layers_) {
+            PX_HIP_CHECK(pxh_route_forward(layer->output().data(), output_.data(), batch(), layer->outputs(),
+                                           outputs(), offset, stream()));
+            offset += layer->outputs();
+        }
+    }
+
+    void backward(const V& input, V* grad) override
+    {
+        Layer::backward(input, grad);
+        int offset = 0;
+        for (const auto& layer: layers_) {
+            PX_HIP_CHECK(pxh_route_backward(delta_.data(), layer->delta().data(), batch(), layer->outputs(),
+                                            outputs(), offset, stream()));
+            offset += layer->outputs();
+        }
+    }
+
+private:
+    std::vector<Layer::Ptr> layers_;
+};
+
+// ---------------------------------------------------------------- YOLO head
+// reference: include/YoloLayer.h:115-239, 390-547, include/cuda/YoloLayer.h:70-166.
+// The reference assigns the positive slots on the host and uploads them on every training
+// forward; here the assignment happens inside the same device pass as the decode.
+class YoloLayer : public Layer
+{
+public:
+    static constexpr int kStats = 12;
+
+    YoloLayer(Context& context, const Properties& props) : Layer(context, props)
+    {
+        anchors_ = props.get<std::vector<int>>("anchors");
+        mask_ = props.get<std::vector<int>>("mask");
+        numAnchors_ = props.get<int>("num", 1);
+        ignoreThresh_ = props.get<float>("ignore_thresh", 0.5f);
+        truthThresh_ = props.get<float>("truth_thresh", 1.0f);
+        coordScale_ = props.get<float>("coord_scale", 1.0f);
+        objectScale_ = props.get<float>("object_scale", 1.0f);
+        noObjectScale_ = props.get<float>("noobject_scale", 1.0f);
+        classScale_ = props.get<float>("class_scale", 1.0f);
+        PX_CHECK(static_cast<int>(anchors_.size()) == 2 * numAnchors_, "yolo: anchors must hold 2 * num values");
+        PX_CHECK(!mask_.empty(), "yolo: empty mask");
+        for (int m: mask_) PX_CHECK(m >= 0 && m < numAnchors_, "yolo: mask entry outside the anchors");
+        const int expect = static_cast<int>(mask_.size()) * (context.classes + 5);
+        PX_CHECK(channels() == expect, "yolo: channels must equal masks * (classes + 5)");
+        setOutput(channels(), height(), width());
+        if (training()) {
+            stats_ = V(kStats, 0.0f);
+            costDevice_ = V(1, 0.0f);
+        }
+    }
+
+    bool hasCost() const noexcept override { return true; }
+
+    void forward(const V& input) override
+    {
+        Layer::forward(input);
+        checkInput(input, "YoloLayer");
+        const auto& c = context();
+        const int masks = static_cast<int>(mask_.size());
+        if (inferring()) {
+            PX_HIP_CHECK(pxh_yolo_activate(input.data(), output_.data(), batch(), masks, c.classes,
+                                           width() * height(), stream()));
+            return;
+        }
+        PX_CHECK(static_cast<int>(c.truthCounts().size()) == batch(), "yolo: ground truth of another batch size");
+        PX_HIP_CHECK(pxh_yolo_forward_train(input.data(), output_.data(), delta_.data(), c.truths().data(),
+                                            c.truthCounts().data(), c.maxTruth(), mask_.data(), anchors_.data(),
+                                            stats_.data(), costDevice_.data(), batch(), masks, numAnchors_,
+                                            c.classes, width(), height(), c.width, c.height, ignoreThresh_,
+                                            truthThresh_, coordScale_, objectScale_, noObjectScale_, classScale_,
+                                            nullptr, 0, stream()));
+        costReady_ = false;
+    }
+
+    void backward(const V& input, V* grad) override
+    {
+        Layer::backward(input, grad);
+        if (grad == nullptr) return;
+        PX_HIP_CHECK(pxh_axpy(delta_.size(), 1.0f, delta_.data(), grad->data(), stream()));
+    }
+
+    // Blocking: cost = sum(delta^2) / max(1, batch) (reference: include/cuda/YoloLayer.h:132).
+    float fetchCost()
+    {
+        if (!costReady_ && !costDevice_.empty()) {
+            PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(stream()));
+            cost_ = costDevice_.asVector()[0] / static_cast<float>(std::max(1, batch()));
+            costReady_ = true;
+        }
+        return cost_;
+    }
+
+    // Blocking: the 12 counters of the last training forward.
+    std::vector<float> fetchStats() const
+    {
+        PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(stream()));
+        return stats_.asVector();
+    }
+
+private:
+    std::vector<int> anchors_, mask_;
+    int numAnchors_ = 1;
+    float ignoreThresh_, truthThresh_, coordScale_, objectScale_, noObjectScale_, classScale_;
+    V stats_, costDevice_;
+    bool costReady_ = false;
+};
+
+}   // px::hip

@@ -1,0 +1,448 @@
+// Drives the C++ layer interface (pixienn_amd/host) on the GPU and checks every layer against the
+// CPU checker on the inputs the GPU layer actually saw.  Test code: it links the checker, the
+// product headers do not.
+//
+//   host_check          all checks (needs a GPU)
+//   host_check --cpu    only the checks that touch no device (argument and property errors)
+//
+// Exit status 0 when every check passes.
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <string>
+#include <vector>
+
+#include "pixienn/Layers.h"
+#include "px_oracle.h"
+
+using namespace px::hip;
+using Host = std::vector<float>;
+
+namespace {
+
+int failures = 0;
+int checks = 0;
+
+void report(const std::string& what, bool ok, const std::string& detail = "")
+{
+    ++checks;
+    if (!ok) ++failures;
+    std::printf("%-58s %s %s\n", what.c_str(), ok ? "ok" : "FAILED", detail.c_str());
+    std::fflush(stdout);
+}
+
+// counter-based generator: the same values on every host
+struct Rng {
+    uint64_t state;
+    explicit Rng(uint64_t seed) : state(seed * 0x9E3779B97F4A7C15ull + 0x1234567ull) {}
+    uint32_t next()
+    {
+        state = state * 6364136223846793005ull + 1442695040888963407ull;
+        return static_cast<uint32_t>(state >> 33);
+    }
+    float uniform() { return (next() & 0xFFFFFF) / 16777216.0f; }
+    float normal()      // sum of 12 uniforms - 6
+    {
+        float s = 0;
+        for (int i = 0; i < 12; ++i) s += uniform();
+        return s - 6.0f;
+    }
+};
+
+Host normals(uint64_t seed, size_t n, float scale = 1.0f, float shift = 0.0f)
+{
+    Rng r(seed);
+    Host v(n);
+    for (auto& x: v) x = shift + scale * r.normal();
+    return v;
+}
+
+Host uniforms(uint64_t seed, size_t n, float lo, float hi)
+{
+    Rng r(seed);
+    Host v(n);
+    for (auto& x: v) x = lo + (hi - lo) * r.uniform();
+    return v;
+}
+
+void expectExact(const std::string& what, const Host& got, const Host& want)
+{
+    bool ok = got.size() == want.size();
+    size_t bad = 0;
+    for (size_t i = 0; ok && i < got.size(); ++i)
+        if (std::memcmp(&got[i], &want[i], 4) != 0 && !(std::isnan(got[i]) && std::isnan(want[i]))) ++bad;
+    report(what, ok && bad == 0, bad ? std::to_string(bad) + " elements differ" : "");
+}
+
+void expectExact(const std::string& what, const std::vector<int>& got, const std::vector<int>& want)
+{
+    report(what, got == want);
+}
+
+// |got - want| <= rtol * max(|want|, floor)
+void expectClose(const std::string& what, const Host& got, const Host& want, double rtol, double floor)
+{
+    bool ok = got.size() == want.size();
+    double worst = 0;
+    for (size_t i = 0; ok && i < got.size(); ++i) {
+        const double err = std::fabs(double(got[i]) - double(want[i]));
+        const double bound = rtol * std::max(std::fabs(double(want[i])), floor);
+        worst = std::max(worst, err / std::max(std::fabs(double(want[i])), floor));
+        if (!(err <= bound)) ok = false;
+    }
+    char buf[64];
+    std::snprintf(buf, sizeof buf, "max rel %.2e", worst);
+    report(what, ok, buf);
+}
+
+template<typename F>
+void expectThrows(const std::string& what, F&& f, const std::string& needle)
+{
+    try {
+        f();
+        report(what, false, "no exception");
+    } catch (const px::Error& e) {
+        const bool ok = std::string(e.what()).find(needle) != std::string::npos;
+        report(what, ok, ok ? "" : e.what());
+    }
+}
+
+// ---------------------------------------------------------------- checks without a device
+void hostOnlyChecks()
+{
+    Context ctx;
+    expectThrows("maxpool rejects kernel 0", [&] {
+        MaxPoolLayer l(ctx, { { "batch", 1 }, { "channels", 1 }, { "height", 4 }, { "width", 4 }, { "kernel", 0 } });
+    }, "kernel must be positive");
+    expectThrows("maxpool rejects negative padding", [&] {
+        MaxPoolLayer l(ctx, { { "batch", 1 }, { "channels", 1 }, { "height", 4 }, { "width", 4 }, { "kernel", 2 },
+                              { "stride", 2 }, { "padding", -1 } });
+    }, "padding cannot be negative");
+    expectThrows("yolo needs its anchors", [&] {
+        YoloLayer l(ctx, { { "batch", 1 }, { "channels", 8 }, { "height", 2 }, { "width", 2 } });
+    }, "no property named \"anchors\"");
+    expectThrows("unknown activation name", [&] { activationFromName("gelu"); }, "unknown activation");
+    expectThrows("C-ABI status becomes px::Error", [&] {
+        PX_HIP_CHECK(pxh_activate(99, reinterpret_cast<float*>(256), 4, nullptr));
+    }, "unknown activation");
+    Properties p{ { "stride", 3 }, { "scale", 2 } };
+    report("property int -> float conversion", p.get<float>("scale") == 2.0f && p.get<int>("stride", 1) == 3 &&
+                                                p.get<int>("absent", 7) == 7);
+}
+
+// ---------------------------------------------------------------- the mini network
+constexpr int N = 2, C = 8, S = 16, CLASSES = 3;
+
+struct Net {
+    Context ctx;
+    std::shared_ptr<ConvLayer> conv0, conv2, conv6;
+    std::shared_ptr<MaxPoolLayer> pool1;
+    std::shared_ptr<ShortcutLayer> short3;
+    std::shared_ptr<UpsampleLayer> up4;
+    std::shared_ptr<RouteLayer> route5;
+    std::shared_ptr<YoloLayer> yolo7;
+    std::vector<int> mask{ 0, 2 }, anchors{ 10, 14, 23, 27, 37, 58 };
+    Host scale0, bias0, scale2, bias2, bias6;
+
+    explicit Net(bool training)
+    {
+        ctx.training = training;
+        ctx.width = ctx.height = 128;
+        ctx.classes = CLASSES;
+        ctx.updateBatch = N;
+        ctx.timeStep = 3;
+        conv0 = std::make_shared<ConvLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S },
+                                                             { "width", S }, { "filters", C },
+                                                             { "batch_normalize", true },
+                                                             { "activation", std::string("leaky") } });
+        pool1 = std::make_shared<MaxPoolLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S },
+                                                                { "width", S }, { "kernel", 2 }, { "stride", 2 } });
+        conv2 = std::make_shared<ConvLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S / 2 },
+                                                             { "width", S / 2 }, { "filters", C },
+                                                             { "batch_normalize", true },
+                                                             { "activation", std::string("mish") } });
+        short3 = std::make_shared<ShortcutLayer>(ctx, Properties{ { "batch", N }, { "channels", C },
+                                                                  { "height", S / 2 }, { "width", S / 2 },
+                                                                  { "alpha", 1.0f }, { "beta", 0.5f } }, pool1);
+        up4 = std::make_shared<UpsampleLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S / 2 },
+                                                               { "width", S / 2 }, { "stride", 2 } });
+        route5 = std::make_shared<RouteLayer>(ctx, Properties{ { "batch", N }, { "channels", 2 * C },
+                                                               { "height", S }, { "width", S } },
+                                              std::vector<Layer::Ptr>{ up4, conv0 });
+        conv6 = std::make_shared<ConvLayer>(ctx, Properties{ { "batch", N }, { "channels", 2 * C }, { "height", S },
+                                                             { "width", S }, { "filters", 2 * C },
+                                                             { "activation", std::string("linear") } });
+        yolo7 = std::make_shared<YoloLayer>(ctx, Properties{ { "batch", N }, { "channels", 2 * C }, { "height", S },
+                                                             { "width", S }, { "num", 3 }, { "mask", mask },
+                                                             { "anchors", anchors }, { "ignore_thresh", 0.5f },
+                                                             { "object_scale", 2.0f }, { "noobject_scale", 0.5f } });
+        scale0 = uniforms(11, C, 0.5f, 1.5f); bias0 = normals(12, C, 0.1f);
+        scale2 = uniforms(13, C, 0.5f, 1.5f); bias2 = normals(14, C, 0.1f);
+        bias6 = normals(15, 2 * C, 0.1f);
+        conv0->copyScales(scale0); conv0->copyBiases(bias0);
+        conv0->copyRollingMean(normals(16, C, 0.1f)); conv0->copyRollingVariance(uniforms(17, C, 0.5f, 1.5f));
+        conv2->copyScales(scale2); conv2->copyBiases(bias2);
+        conv2->copyRollingMean(normals(18, C, 0.1f)); conv2->copyRollingVariance(uniforms(19, C, 0.5f, 1.5f));
+        conv6->copyBiases(bias6);
+    }
+};
+
+void convForwardCheck(const std::string& name, ConvLayer& layer, const Host& input, bool bn, bool training, int act,
+                      int channels, int size, Host* meanOut = nullptr, Host* varOut = nullptr)
+{
+    Host want = input;
+    Host mean(channels, 0.0f), var(channels, 0.0f);
+    Host rmean = layer.rollingMean().asVector(), rvar = layer.rollingVariance().asVector();
+    // the layer has already run: undo nothing, the inference path does not move the rolling values and
+    // the training check compares mean / var, which do not depend on them
+    Host scales = bn ? layer.scales().asVector() : Host(channels, 1.0f);
+    Host biases = layer.biases().asVector();
+    if (!bn) { rmean.assign(channels, 0.0f); rvar.assign(channels, 1.0f); }
+    Host x(training && bn ? input.size() : 0), xnorm(training && bn ? input.size() : 0);
+    pxo_conv_epilogue_forward(bn, training, act, N, channels, size, size, want.data(), nullptr, mean.data(),
+                              var.data(), rmean.data(), rvar.data(), scales.data(), biases.data(),
+                              x.empty() ? nullptr : x.data(), xnorm.empty() ? nullptr : xnorm.data(), 0);
+    expectClose(name + " forward", layer.output().asVector(), want, 1e-5, training ? 4.0 : 1.0);
+    if (training && bn) {
+        expectClose(name + " batch mean", layer.mean().asVector(), mean, 1e-5, 0.05);
+        expectClose(name + " batch variance", layer.variance().asVector(), var, 1e-5, 1.0);
+    }
+    if (meanOut) *meanOut = mean;
+    if (varOut) *varOut = var;
+}
+
+void inferenceChecks()
+{
+    Net net(false);
+    FloatVector input(normals(100, size_t(N) * C * S * S));
+    net.conv0->forward(input);
+    convForwardCheck("conv0 (bn, leaky, inference)", *net.conv0, input.asVector(), true, false, PXO_LEAKY, C, S);
+    net.conv0->forward(input);      // second call reuses the folded constants
+    convForwardCheck("conv0 again (folded constants reused)", *net.conv0, input.asVector(), true, false, PXO_LEAKY,
+                     C, S);
+    net.pool1->forward(net.conv0->output());
+    {
+        const Host in = net.conv0->output().asVector();
+        Host out(net.pool1->output().size());
+        std::vector<int> idx(out.size());
+        pxo_maxpool_forward(in.data(), out.data(), idx.data(), N, C, S, S, S / 2, S / 2, 2, 2, 1);
+        expectExact("pool1 forward values", net.pool1->output().asVector(), out);
+        expectExact("pool1 forward indexes", net.pool1->indexes().asVector(), idx);
+    }
+    net.conv2->forward(net.pool1->output());
+    convForwardCheck("conv2 (bn, mish, inference)", *net.conv2, net.pool1->output().asVector(), true, false,
+                     PXO_MISH, C, S / 2);
+    net.short3->forward(net.conv2->output());
+    {
+        const Host a = net.conv2->output().asVector(), b = net.pool1->output().asVector();
+        Host out(a.size()), pre(a.size());
+        pxo_shortcut_forward(PXO_LINEAR, N, S / 2, S / 2, C, a.data(), b.data(), 1.0f, 0.5f, out.data(), pre.data());
+        expectExact("short3 forward", net.short3->output().asVector(), out);
+    }
+    net.up4->forward(net.short3->output());
+    {
+        const Host in = net.short3->output().asVector();
+        Host out(net.up4->output().size(), 0.0f);
+        pxo_upsample(in.data(), S / 2, S / 2, C, N, 2, 1, 1.0f, nullptr, out.data());
+        expectExact("up4 forward", net.up4->output().asVector(), out);
+    }
+    net.route5->forward(net.up4->output());
+    {
+        const Host a = net.up4->output().asVector(), b = net.conv0->output().asVector();
+        Host out(net.route5->output().size(), -1.0f);
+        pxo_route_forward(a.data(), out.data(), N, C * S * S, 2 * C * S * S, 0);
+        pxo_route_forward(b.data(), out.data(), N, C * S * S, 2 * C * S * S, C * S * S);
+        expectExact("route5 forward", net.route5->output().asVector(), out);
+    }
+    net.conv6->forward(net.route5->output());
+    convForwardCheck("conv6 (bias, linear)", *net.conv6, net.route5->output().asVector(), false, false, PXO_LINEAR,
+                     2 * C, S);
+    net.yolo7->forward(net.conv6->output());
+    {
+        pxo_yolo_cfg cfg{ N, S, S, CLASSES, 2, 3, net.mask.data(), net.anchors.data(), 128, 128, 0.5f, 1.0f, 1.0f,
+                          2.0f, 0.5f, 1.0f };
+        const Host in = net.conv6->output().asVector();
+        Host out(in.size());
+        pxo_yolo_decode(&cfg, in.data(), out.data());
+        expectClose("yolo7 decode (inference)", net.yolo7->output().asVector(), out, 1e-5, 1e-3);
+    }
+}
+
+std::vector<GroundTruthVec> makeTruth()
+{
+    Rng r(77);
+    std::vector<GroundTruthVec> truth(N);
+    for (int b = 0; b < N; ++b) {
+        const int count = 3 + b * 2;
+        for (int t = 0; t < count; ++t) {
+            GroundTruth g;
+            g.x = r.uniform(); g.y = r.uniform();
+            g.w = 0.05f + 0.5f * r.uniform(); g.h = 0.05f + 0.5f * r.uniform();
+            g.classId = static_cast<int>(r.next() % CLASSES);
+            truth[b].push_back(g);
+        }
+    }
+    return truth;
+}
+
+void trainingChecks()
+{
+    Net net(true);
+    const auto truth = makeTruth();
+    net.ctx.setGroundTruth(truth);
+    FloatVector input(normals(200, size_t(N) * C * S * S));
+    const Host rmeanBefore = net.conv0->rollingMean().asVector();
+
+    // ---- forward
+    net.conv0->forward(input);
+    Host mean0, var0;
+    convForwardCheck("conv0 (bn, leaky, training)", *net.conv0, input.asVector(), true, true, PXO_LEAKY, C, S, &mean0,
+                     &var0);
+    {
+        Host want(C);
+        for (int c = 0; c < C; ++c) want[c] = 0.99f * rmeanBefore[c] + 0.01f * mean0[c];
+        expectClose("conv0 rolling mean moved", net.conv0->rollingMean().asVector(), want, 1e-5, 0.05);
+    }
+    net.pool1->forward(net.conv0->output());
+    net.conv2->forward(net.pool1->output());
+    Host mean2, var2;
+    convForwardCheck("conv2 (bn, mish, training)", *net.conv2, net.pool1->output().asVector(), true, true, PXO_MISH,
+                     C, S / 2, &mean2, &var2);
+    net.short3->forward(net.conv2->output());
+    net.up4->forward(net.short3->output());
+    net.route5->forward(net.up4->output());
+    net.conv6->forward(net.route5->output());
+    net.yolo7->forward(net.conv6->output());
+
+    // ---- YOLO head against the checker
+    const int maxTruth = net.ctx.maxTruth();
+    Host yoloDelta;
+    {
+        pxo_yolo_cfg cfg{ N, S, S, CLASSES, 2, 3, net.mask.data(), net.anchors.data(), 128, 128, 0.5f, 1.0f, 1.0f,
+                          2.0f, 0.5f, 1.0f };
+        const Host in = net.conv6->output().asVector();
+        const Host truths = net.ctx.truths().asVector();
+        const std::vector<int> counts = net.ctx.truthCounts().asVector();
+        Host out(in.size()), delta(in.size(), 0.0f), stats(12, 0.0f);
+        float cost = 0;
+        pxo_yolo_forward(&cfg, in.data(), truths.data(), counts.data(), maxTruth, out.data(), delta.data(), &cost,
+                         stats.data());
+        expectClose("yolo7 output (training)", net.yolo7->output().asVector(), out, 1e-5, 1e-3);
+        yoloDelta = net.yolo7->delta().asVector();
+        expectClose("yolo7 delta", yoloDelta, delta, 1e-5, 2.0);
+        expectClose("yolo7 cost", Host{ net.yolo7->fetchCost() }, Host{ cost }, 1e-5, 1e-3);
+        const Host gs = net.yolo7->fetchStats();
+        expectClose("yolo7 positives counted", Host{ gs[6] }, Host{ stats[6] }, 0.0, 1.0);
+    }
+
+    // ---- backward, last layer first; every layer accumulates into its predecessor's delta
+    net.yolo7->backward(net.conv6->output(), &net.conv6->delta());
+    expectExact("yolo7 backward: grad += delta", net.conv6->delta().asVector(), yoloDelta);
+
+    {   // conv6: bias backward, then (identity convolution) grad += delta
+        Host d = net.conv6->delta().asVector();
+        Host biasUpd(2 * C, 0.0f);
+        const Host pre = net.conv6->output().asVector();      // linear: the output is the pre-activation
+        pxo_conv_epilogue_backward(0, PXO_LINEAR, N, 2 * C, S, S, d.data(), pre.data(), nullptr, nullptr, nullptr,
+                                   nullptr, nullptr, nullptr, biasUpd.data(), nullptr, nullptr, 0);
+        net.conv6->backward(net.route5->output(), &net.route5->delta());
+        expectClose("conv6 bias updates", net.conv6->biasUpdates().asVector(), biasUpd, 1e-5, 1.0);
+        expectExact("conv6 backward into route5 delta", net.route5->delta().asVector(), d);
+    }
+    {   // route5 -> up4.delta and conv0.delta
+        const Host rd = net.route5->delta().asVector();
+        Host a(net.up4->delta().size(), 0.0f), b(net.conv0->delta().size(), 0.0f);
+        pxo_route_backward(rd.data(), a.data(), N, C * S * S, 2 * C * S * S, 0);
+        pxo_route_backward(rd.data(), b.data(), N, C * S * S, 2 * C * S * S, C * S * S);
+        net.route5->backward(net.up4->output(), &net.up4->delta());
+        expectExact("route5 backward into up4 delta", net.up4->delta().asVector(), a);
+        expectExact("route5 backward into conv0 delta", net.conv0->delta().asVector(), b);
+    }
+    {   // up4 -> short3.delta
+        const Host d = net.up4->delta().asVector();
+        Host acc(net.short3->delta().size(), 0.0f), dcopy = d;
+        pxo_upsample(nullptr, S / 2, S / 2, C, N, 2, 0, 1.0f, acc.data(), dcopy.data());
+        net.up4->backward(net.short3->output(), &net.short3->delta());
+        expectExact("up4 backward into short3 delta", net.short3->delta().asVector(), acc);
+    }
+    {   // short3 -> pool1.delta (from) and conv2.delta (grad)
+        Host d = net.short3->delta().asVector();
+        Host from(net.pool1->delta().size(), 0.0f), grad(net.conv2->delta().size(), 0.0f);
+        const Host pre = net.short3->output().asVector();     // linear: the output is the pre-activation
+        pxo_shortcut_backward(PXO_LINEAR, N, S / 2, S / 2, C, d.data(), pre.data(), from.data(), grad.data(), 1.0f,
+                              0.5f);
+        net.short3->backward(net.conv2->output(), &net.conv2->delta());
+        expectExact("short3 backward into pool1 delta", net.pool1->delta().asVector(), from);
+        expectExact("short3 backward into conv2 delta", net.conv2->delta().asVector(), grad);
+    }
+    {   // conv2: activation gradient + batch norm backward, accumulated into pool1.delta
+        Host d = net.conv2->delta().asVector();
+        const Host x = net.pool1->output().asVector();
+        const Host mean = net.conv2->mean().asVector(), var = net.conv2->variance().asVector();
+        // the checker wants x_hat and the pre-activation of the forward
+        Host xn = x, pre(x.size());
+        pxo_normalize(xn.data(), mean.data(), var.data(), N, C, (S / 2) * (S / 2));
+        for (size_t i = 0; i < x.size(); ++i) {
+            const int c = static_cast<int>(i / ((S / 2) * (S / 2))) % C;
+            const float scaled = xn[i] * net.scale2[c];
+            pre[i] = scaled + net.bias2[c];
+        }
+        Host md(C), vd(C), su(C, 0.0f), bu(C, 0.0f);
+        pxo_conv_epilogue_backward(1, PXO_MISH, N, C, S / 2, S / 2, d.data(), pre.data(), mean.data(), var.data(),
+                                   md.data(), vd.data(), net.scale2.data(), su.data(), bu.data(), x.data(), xn.data(),
+                                   0);
+        Host want = net.pool1->delta().asVector();
+        for (size_t i = 0; i < want.size(); ++i) want[i] += d[i];
+        net.conv2->backward(net.pool1->output(), &net.pool1->delta());
+        expectClose("conv2 scale updates", net.conv2->scaleUpdates().asVector(), su, 1e-5, 1.0);
+        expectClose("conv2 bias updates", net.conv2->biasUpdates().asVector(), bu, 1e-5, 1.0);
+        expectClose("conv2 backward into pool1 delta", net.pool1->delta().asVector(), want, 1e-5, 1.0);
+    }
+    {   // pool1 -> conv0.delta
+        const Host d = net.pool1->delta().asVector();
+        const std::vector<int> idx = net.pool1->indexes().asVector();
+        Host grad = net.conv0->delta().asVector();
+        pxo_maxpool_backward(d.data(), idx.data(), grad.data(), d.size());
+        net.pool1->backward(net.conv0->output(), &net.conv0->delta());
+        expectExact("pool1 backward into conv0 delta", net.conv0->delta().asVector(), grad);
+    }
+    net.conv0->backward(input, nullptr);
+
+    // ---- update: Adam on conv2's scales
+    {
+        Host w = net.conv2->scales().asVector(), d = net.conv2->scaleUpdates().asVector();
+        Host m(C, 0.0f), v(C, 0.0f);
+        pxo_adam_update(C, w.data(), d.data(), m.data(), v.data(), net.ctx.updateBatch, net.ctx.timeStep,
+                        net.ctx.learningRate, net.ctx.adamBeta1, net.ctx.adamBeta2, net.ctx.adamEpsilon,
+                        net.ctx.decay, 0);
+        net.conv2->update();
+        expectClose("conv2 Adam update of the scales", net.conv2->scales().asVector(), w, 1e-6, 1e-3);
+        expectExact("conv2 scale updates consumed", net.conv2->scaleUpdates().asVector(), Host(C, 0.0f));
+    }
+}
+
+}   // namespace
+
+int main(int argc, char** argv)
+{
+    const bool cpuOnly = argc > 1 && std::strcmp(argv[1], "--cpu") == 0;
+    try {
+        hostOnlyChecks();
+        if (!cpuOnly) {
+            int devices = 0;
+            if (hipGetDeviceCount(&devices) != hipSuccess || devices == 0) {
+                std::printf("no GPU visible\n");
+                return 2;
+            }
+            inferenceChecks();
+            trainingChecks();
+        }
+    } catch (const std::exception& e) {
+        std::printf("unexpected exception: %s\n", e.what());
+        return 3;
+    }
+    std::printf("%d checks, %d failed\n", checks, failures);
+    return failures ? 1 : 0;
+}
