@@ -42,7 +42,9 @@ def gpu_head(ops, x, truths, counts, W, H, K, mask, anchors, net, ignore_thresh=
     return host(gout), host(gdelta), float(host(cost)[0]), host(stats)
 
 
-def compare_head(got, want, what):
+def compare_head(got, want, what, sum_rtol=2e-5):
+    """sum_rtol bounds the statistics that are running fp32 sums over every slot in the CPU layer
+    (at a million slots its sequential accumulation is itself only good to ~1e-4)."""
     out, delta, cost, stats = got
     out_w, delta_w, cost_w, stats_w = want
     assert_close(out, out_w, 1e-5, 1e-6, what + " output")
@@ -54,7 +56,7 @@ def compare_head(got, want, what):
     assert stats[6] == stats_w[6] and stats[7] == stats_w[7], (what, stats, stats_w)
     assert stats[1] == stats_w[1] and stats[2] == stats_w[2], (what, stats, stats_w)
     for k in (0, 3, 4, 5, 8, 9, 10, 11):
-        assert abs(stats[k] - stats_w[k]) <= 2e-5 * max(abs(stats_w[k]), 1.0), (what, k, stats[k], stats_w[k])
+        assert abs(stats[k] - stats_w[k]) <= sum_rtol * max(abs(stats_w[k]), 1.0), (what, k, stats[k], stats_w[k])
 
 
 def test_yolo_decode_matches_oracle(ops, oracle, kats):
