@@ -2,15 +2,15 @@
 // statistics).
 //
 // Layout [batch][mask][5 + classes][area].  The training pass is two launches:
-//   pass 1  two kinds of workgroup share one grid.  HEAD workgroups give one lane to every slot
-//           (image, anchor, cell): the 5 box/objectness rows, the best-truth search, the decision
-//           what the slot is supervised with (one int per slot), box/objectness deltas, every
-//           statistic and the whole cost (the class rows of the few supervised slots are visited
-//           for it).  They are instruction bound.  CLASS workgroups stream the class rows, 94 %
-//           of the tensor: logit -> probability -> `out`.  They are bandwidth bound, and the two
-//           kinds are interleaved in the grid so that they overlap on every compute unit.
-//   pass 2  the dense class delta from the slots' decisions, a write-only stream; its first
-//           workgroups also add up the per-workgroup sums of pass 1 in a fixed order.
+//   head   one lane per slot (image, anchor, cell): the 5 box/objectness rows, the best-truth
+//          search against the image's truths staged in LDS, the decision what the slot is
+//          supervised with (one int per slot), box/objectness deltas, every statistic and the
+//          whole cost (the class rows of the few supervised slots are visited for it).  Latency
+//          bound: a few dependent memory round trips and ~20 IoU tests per lane, so the kernel is
+//          written for instruction-level parallelism rather than for occupancy.
+//   class  streams the class rows, 94 % of the tensor: logit -> probability -> `out`, and the
+//          dense class delta from the slots' decisions, 12 bytes per element.  Its first
+//          workgroups also add up the per-workgroup sums of the head kernel in a fixed order.
 // Box arithmetic follows the CPU layer (include/YoloLayer.h, src/DarkBox.cpp of the reference).
 #include "stream.h"
 
@@ -60,36 +60,39 @@ __device__ __forceinline__ float box_iou(const Box& a, const Box& b)
     return inter / uni;
 }
 
-// IoU of a prediction rectangle (pl, pt, pw, ph; not empty) with an unpacked truth: the same
-// operations as box_iou, ordered so that a pair that is disjoint along x or along y leaves after
-// a handful of instructions.  With lo/hi the rectangles ordered by left edge, the overlap width is
-// min(lo.w - (hi.left - lo.left), hi.w) <= lo.w - (hi.left - lo.left): when that bound is not
-// positive the intersection is empty whatever the rest says.
-__device__ __forceinline__ float rect_iou(float pl, float pt, float pw, float ph, float tl, float tt, float tw,
-                                          float th)
+// Overlap area of a prediction rectangle (pl, pt, pw, ph; not empty) with an unpacked truth: the
+// operations of box_intersection without its branches, so that several pairs can be in flight
+// in one lane.  With lo/hi the rectangles ordered by left edge, the overlap width is
+// min(lo.w - (hi.left - lo.left), hi.w); an empty truth carries left = +inf and drops out here.
+__device__ __forceinline__ float rect_overlap(float pl, float pt, float pw, float ph, float tl, float tt, float tw,
+                                              float th)
 {
     const bool p_left = pl < tl;
     const float xlo = p_left ? pl : tl, xlo_w = p_left ? pw : tw;
     const float xhi = p_left ? tl : pl, xhi_w = p_left ? tw : pw;
     const float bx = xlo_w - (xhi - xlo);
-    if (!(bx > 0.0f)) return 0.0f;
     const bool p_top = pt < tt;
     const float ylo = p_top ? pt : tt, ylo_h = p_top ? ph : th;
     const float yhi = p_top ? tt : pt, yhi_h = p_top ? th : ph;
     const float by = ylo_h - (yhi - ylo);
-    if (!(by > 0.0f)) return 0.0f;
-    if ((xlo < 0.0f && xlo + xlo_w < xhi) || (ylo < 0.0f && ylo + ylo_h < yhi)) return 0.0f;
+    // bitwise on purpose: no short-circuit branches, the lanes of a wave rarely agree
+    const bool meet = (bx > 0.0f) & (by > 0.0f) & !((xlo < 0.0f) & (xlo + xlo_w < xhi)) &
+                      !((ylo < 0.0f) & (ylo + ylo_h < yhi));
     const float iw = fminf(bx, xhi_w);
     const float ih = fminf(by, yhi_h);
-    const float inter = iw * ih;
-    if (inter == 0.0f) return 0.0f;
+    return meet ? iw * ih : 0.0f;
+}
+
+// inter / union as box_iou forms it; 0 when either is 0.  No branches.
+__device__ __forceinline__ float overlap_ratio(float inter, float pw, float ph, float tw, float th)
+{
     const float ap = pw * ph;
     const float at = tw * th;
     float uni = ap + at;
     uni = uni - inter;
-    uni = uni > 0.0f ? uni : 0.0f;
-    if (uni == 0.0f) return 0.0f;
-    return inter / uni;
+    const bool some = (uni > 0.0f) & (inter > 0.0f);
+    const float q = inter / (some ? uni : 1.0f);
+    return some ? q : 0.0f;
 }
 
 // Logistic for the class rows: exp2 and reciprocal in hardware, two multiplies and an add.  The
@@ -134,6 +137,7 @@ struct YoloParams {
     float ignore_thresh, truth_thresh, coord_scale, object_scale, noobject_scale, class_scale;
     int masks[kMaxMasks];
     float anchors[2 * kMaxAnchors];   // integer pixel sizes held as float
+    float anchors_rel[2 * kMaxAnchors];   // anchors[2a] / net_width, anchors[2a+1] / net_height (fp32 division)
     FastDiv by_tiles;    // workgroups per (image, anchor) in the head sweep
     FastDiv by_masks;
     FastDiv by_width;
@@ -204,22 +208,27 @@ __device__ __forceinline__ TruthSlot make_truth_slot(const float* __restrict__ g
     s.cls = static_cast<int>(g[4]);
     s.target = -1;
     if constexpr (FUSED) {
-        const Box shifted{ 0.0f, 0.0f, box.w, box.h };
+        // Both boxes are centred on the origin, where DarkBox's rectangle intersection reduces to
+        // min(w) * min(h) exactly: ordered by left edge the wider box comes first, its overlap bound
+        // W - (W/2 - n/2) is never below the narrower width n, and the negative-left test
+        // (-W/2 + W < -n/2) is false.  The IoU is then formed as box_iou forms it.
         float ba = -FLT_MAX;
         int bi = 0;
-        // four anchors at a time: the four IoU chains are independent and overlap in the pipeline
-        for (int a0 = 0; a0 < p.anchor_count; a0 += 4) {
-            float iou[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int a = min(a0 + u, p.anchor_count - 1);
-                const Box cand{ 0.0f, 0.0f, p.anchors[2 * a] / static_cast<float>(p.net_width),
-                                p.anchors[2 * a + 1] / static_cast<float>(p.net_height) };
-                iou[u] = box_iou(cand, shifted);
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-                if (a0 + u < p.anchor_count && iou[u] > ba) { ba = iou[u]; bi = a0 + u; }
+        const bool truth_empty = empty;
+        const float ab = box.w * box.h;
+        for (int a = 0; a < p.anchor_count; ++a) {
+            const float cw = p.anchors_rel[2 * a], ch = p.anchors_rel[2 * a + 1];
+            const bool none = truth_empty | (cw <= 0.0f) | (ch <= 0.0f);
+            const float inter = none ? 0.0f : fminf(cw, box.w) * fminf(ch, box.h);
+            const float aa = cw * ch;
+            float uni = aa + ab;
+            uni = uni - inter;
+            const bool some = (uni > 0.0f) & (inter > 0.0f);
+            const float q = inter / (some ? uni : 1.0f);
+            const float iou = some ? q : 0.0f;
+            const bool better = iou > ba;
+            ba = better ? iou : ba;
+            bi = better ? a : bi;
         }
         int ms = -1;
         for (int m = 0; m < p.mask_count; ++m)
@@ -260,15 +269,25 @@ struct HeadArgs {
     double* partial;
 };
 
+// Sum of 64 lanes, pairwise (butterfly): at most 6 roundings on any path.
+__device__ __forceinline__ float wave_sum_pairwise(float v)
+{
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+constexpr int kWaves = kBlock / kWave;
+constexpr int kTruthUnroll = 4;
+
+// Returns, in threads 0..kSums-1, the tile's sum of statistic threadIdx.x.
 template<bool FUSED>
-__device__ __forceinline__ void head_workgroup(uint32_t head_block, const HeadArgs& a, const YoloParams& p,
-                                               const YoloTables& tb, TruthSlot* tile, double* slots)
+__device__ __forceinline__ double head_tile(const uint32_t head_block, const HeadArgs& a, const YoloParams& p,
+                                          const YoloTables& tb, TruthSlot* tile, double (*wave_sums)[kWaves])
 {
     const float* __restrict__ in = a.in;
     float* __restrict__ out = a.out;
     float* __restrict__ delta = a.delta;
-    int* __restrict__ decision = a.decision;
-    double* __restrict__ partial = a.partial;
     uint32_t bn, tile_id, b, n;
     p.by_tiles.divmod(head_block, bn, tile_id);
     p.by_masks.divmod(bn, b, n);
@@ -277,6 +296,10 @@ __device__ __forceinline__ void head_workgroup(uint32_t head_block, const HeadAr
     const int area = p.area;
     const int entries = p.classes + 5;
     const size_t base = (static_cast<size_t>(bn) * entries) * area + (live ? cell : 0);
+
+    // issued first, used last: the truth count and this lane's truth do not depend on each other
+    const int count = a.truth_counts[b];
+    const float* image_truths = a.truths + static_cast<size_t>(b) * p.max_truth * 5;
 
     int mask_anchor;
     float aw, ah;
@@ -314,59 +337,82 @@ __device__ __forceinline__ void head_workgroup(uint32_t head_block, const HeadAr
     }
     const Box pred = decode_box(sx, sy, rw, rh, i, j, aw, ah, p);
     const bool pred_empty = pred.w <= 0.0f || pred.h <= 0.0f;
-    const float pl = pred.x - pred.w / 2.0f, pt = pred.y - pred.h / 2.0f;
+    // an empty prediction overlaps nothing: park it where every overlap test fails
+    const float pl = pred_empty ? INFINITY : pred.x - pred.w / 2.0f, pt = pred.y - pred.h / 2.0f;
 
     // Sweep the image's truths through LDS: best IoU (strict >, first wins) and, in the fused
     // form, the truths that claim this slot as their positive (the last one writes the delta).
     // IoU is never negative, so "first wins from the lowest float" is: start at truth 0 with 0.
-    const int count = a.truth_counts[b];
-    const float* image_truths = a.truths + static_cast<size_t>(b) * p.max_truth * 5;
     float best = 0.0f;
     int best_k = count > 0 ? 0 : -1;
-    int pos_k = -1;
+    int pos_cls = -1, pos_anchor = mask_anchor;
+    Box pos_box{ 0, 0, 0, 0 };
     float st_iou = 0, st_r50 = 0, st_r75 = 0, st_cat = 0, st_obj = 0, st_count = 0;
-    const int my_slot = n * area + cell;
+    const int my_slot = live ? static_cast<int>(n) * area + cell : -2;
 
     for (int t0 = 0; t0 < count; t0 += kTruthTile) {
         const int t = t0 + threadIdx.x;
-        __syncthreads();
+        __syncthreads();       // the previous tile (or the previous head tile of this workgroup) is done with
         if (t < count) tile[threadIdx.x] = make_truth_slot<FUSED>(image_truths + 5 * static_cast<size_t>(t), p);
         __syncthreads();
         const int tn = min(kTruthTile, count - t0);
-        if (live) {
-            for (int k = 0; k < tn; ++k) {
+        // kTruthUnroll truths per step: their overlap tests are independent and interleave; the
+        // ordered part (best so far, claims) follows in truth order.  Steps past the last truth
+        // re-read it with an empty overlap and no target.
+        for (int k0 = 0; k0 < tn; k0 += kTruthUnroll) {
+            float inter[kTruthUnroll], tw[kTruthUnroll], th[kTruthUnroll], iou[kTruthUnroll];
+            int target[kTruthUnroll];
+            bool touch = false, claimed = false;
+#pragma unroll
+            for (int u = 0; u < kTruthUnroll; ++u) {
+                const bool real = k0 + u < tn;
+                const int k = real ? k0 + u : tn - 1;
                 const float4 r = *reinterpret_cast<const float4*>(&tile[k].left);
-                const float iou = pred_empty ? 0.0f : rect_iou(pl, pt, pred.w, pred.h, r.x, r.y, r.z, r.w);
-                if (iou > best) {
-                    best = iou;
-                    best_k = t0 + k;
+                target[u] = real ? tile[k].target : -1;
+                tw[u] = r.z; th[u] = r.w;
+                const float ov = rect_overlap(pl, pt, pred.w, pred.h, r.x, r.y, r.z, r.w);
+                inter[u] = real ? ov : 0.0f;
+                touch = touch | (inter[u] > 0.0f);
+                claimed = claimed | (target[u] == my_slot);
+            }
+            // most steps touch nothing in the whole wave: no divisions then
+            if (__ballot(touch)) {
+#pragma unroll
+                for (int u = 0; u < kTruthUnroll; ++u) iou[u] = overlap_ratio(inter[u], pred.w, pred.h, tw[u], th[u]);
+#pragma unroll
+                for (int u = 0; u < kTruthUnroll; ++u) {
+                    const bool better = iou[u] > best;
+                    best = better ? iou[u] : best;
+                    best_k = better ? t0 + k0 + u : best_k;
                 }
-                if constexpr (FUSED) {
-                    if (tile[k].target == my_slot) {
-                        // every claiming truth is counted (include/YoloLayer.h:480-507); the claimed
-                        // slot's anchor is this mask's, so `iou` is the IoU the CPU layer records
-                        pos_k = t0 + k;
-                        st_cat += fminf(1.0f, class_prob<FUSED>(in, base, tile[k].cls, area));
-                        st_iou += iou;
-                        if (iou > .5f) st_r50 += 1.0f;
-                        if (iou > .75f) st_r75 += 1.0f;
-                        st_obj += so;
-                        st_count += 1.0f;
+            } else {
+#pragma unroll
+                for (int u = 0; u < kTruthUnroll; ++u) iou[u] = 0.0f;
+            }
+            if constexpr (FUSED) {
+                if (__ballot(claimed)) {
+#pragma unroll
+                    for (int u = 0; u < kTruthUnroll; ++u) {
+                        if (target[u] == my_slot) {
+                            // every claiming truth is counted (include/YoloLayer.h:480-507); the claimed
+                            // slot's anchor is this mask's, so iou[u] is the IoU the CPU layer records
+                            const TruthSlot& ts = tile[k0 + u];
+                            pos_cls = ts.cls;
+                            pos_box = Box{ ts.x, ts.y, ts.w, ts.h };
+                            st_cat += fminf(1.0f, class_prob<FUSED>(in, base, ts.cls, area));
+                            st_iou += iou[u];
+                            if (iou[u] > .5f) st_r50 += 1.0f;
+                            if (iou[u] > .75f) st_r75 += 1.0f;
+                            st_obj += so;
+                            st_count += 1.0f;
+                        }
                     }
                 }
             }
         }
     }
 
-    int pos_cls = -1, pos_anchor = mask_anchor;
-    Box pos_box{ 0, 0, 0, 0 };
-    if constexpr (FUSED) {
-        if (pos_k >= 0) {
-            const float* g = image_truths + 5 * static_cast<size_t>(pos_k);
-            pos_cls = static_cast<int>(g[4]);
-            pos_box = Box{ g[0], g[1], g[2], g[3] };
-        }
-    } else {
+    if constexpr (!FUSED) {
         if (live) {
             const size_t slot = static_cast<size_t>(bn) * area + cell;
             const int acls = tb.assigned_classes[slot];
@@ -391,7 +437,7 @@ __device__ __forceinline__ void head_workgroup(uint32_t head_block, const HeadAr
     float d_obj = 0.0f;
     int cls = -1;            // class the dense class delta is written for, -1: zeros
     BoxDelta bd{ { 0, 0, 0, 0 } };
-    float c_box = 0, c_obj = 0, c_noobj = 0, c_cls = 0;
+    float c_box = 0, c_obj = 0, c_noobj = 0;
     if (live) {
         const bool have_best = best_k >= 0;
         if (!have_best || best < p.ignore_thresh) d_obj = p.noobject_scale * (0.0f - so);
@@ -420,46 +466,68 @@ __device__ __forceinline__ void head_workgroup(uint32_t head_block, const HeadAr
         }
         delta[base + 4 * static_cast<size_t>(area)] = d_obj;
         if (d_obj >= 0.0f) c_obj = d_obj * d_obj; else c_noobj = d_obj * d_obj;
-        decision[static_cast<size_t>(bn) * area + cell] = cls;
-        // class deltas are zero except for the supervised slots: their cost is taken here, with
-        // the probabilities the class sweep will write
-        if (cls >= 0) {
-            // 16 independent loads per round trip (rows past the last class re-read it and are
-            // masked out); the sum keeps the class order
-            constexpr int kRows = 16;
-            const float* src = in + base + 5 * static_cast<size_t>(area);
-            for (int c0 = 0; c0 < p.classes; c0 += kRows) {
-                float v[kRows];
-#pragma unroll
-                for (int u = 0; u < kRows; ++u) v[u] = src[min(c0 + u, p.classes - 1) * static_cast<size_t>(area)];
-#pragma unroll
-                for (int u = 0; u < kRows; ++u) {
-                    const float prob = FUSED ? sigmoid_fast(v[u]) : v[u];
-                    const float t = (c0 + u == cls) ? 1.0f : 0.0f;
-                    const float d = p.class_scale * (t - prob);
-                    c_cls += (c0 + u < p.classes) ? d * d : 0.0f;
-                }
-            }
-        }
+        a.decision[static_cast<size_t>(bn) * area + cell] = cls;
     }
 
-    // Only the objectness sum and the no-object cost exist for every slot; the rest is non-zero
-    // only where a slot is supervised, which most workgroups never see.
-    const bool any_pos = __syncthreads_or(cls >= 0 || st_count != 0.0f);
-    const float sums[12] = { st_iou, st_r50, st_r75, st_cat, st_obj, live ? so : 0.0f, st_count, st_count,
-                             c_box, c_obj, c_noobj, c_cls };
-    double* dst = partial + head_block;     // [12][blocks]
-    const size_t stride = p.blocks;
+    // Workgroup sums.  The objectness sum and the no-object cost exist for every slot: pairwise
+    // over the wave.  Everything else is non-zero only at supervised slots, which most waves never
+    // see: their lanes are visited one by one, in lane order.  The class deltas are zero except at
+    // those slots too; the wave takes their cost together, one class row per lane, from the
+    // probabilities the class stream writes (the same function of the same logits).
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const float dense_obj = wave_sum_pairwise(live ? so : 0.0f);
+    const float dense_noobj = wave_sum_pairwise(c_noobj);
+    const float sparse[9] = { st_iou, st_r50, st_r75, st_cat, st_obj, st_count, st_count, c_box, c_obj };
+    constexpr int slot_of[9] = { 0, 1, 2, 3, 4, 6, 7, 8, 9 };
+    double acc[9] = { 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+    double class_cost = 0.0;
+    unsigned long long todo = __ballot(cls >= 0 || st_count != 0.0f);
+    while (todo) {
+        const int src_lane = __builtin_ctzll(todo);
+        todo &= todo - 1;
 #pragma unroll
-    for (int k = 0; k < 12; ++k) {
-        const bool dense = (k == 5 || k == 10);
-        if (dense || any_pos) {
-            const double total = block_sum(static_cast<double>(sums[k]), slots);
-            if (threadIdx.x == 0) dst[k * stride] = total;
-        } else if (threadIdx.x == 0) {
-            dst[k * stride] = 0.0;
+        for (int k = 0; k < 9; ++k)
+            acc[k] += static_cast<double>(__shfl(sparse[k], src_lane, kWave));
+        const int s_cls = __shfl(cls, src_lane, kWave);
+        if (s_cls >= 0) {
+            const int s_cell = __shfl(cell, src_lane, kWave);
+            const float* rows = in + (static_cast<size_t>(bn) * entries + 5) * area + s_cell;
+            float sq = 0.0f;
+            for (int c = lane; c < p.classes; c += kWave) {
+                const float v = rows[static_cast<size_t>(c) * area];
+                const float prob = FUSED ? sigmoid_fast(v) : v;
+                const float t = (c == s_cls) ? 1.0f : 0.0f;
+                const float d = p.class_scale * (t - prob);
+                sq += d * d;
+            }
+            class_cost += static_cast<double>(wave_sum_pairwise(sq));
         }
     }
+    if (lane == 0) {
+#pragma unroll
+        for (int k = 0; k < 9; ++k) wave_sums[slot_of[k]][wave] = acc[k];
+        wave_sums[5][wave] = static_cast<double>(dense_obj);
+        wave_sums[10][wave] = static_cast<double>(dense_noobj);
+        wave_sums[11][wave] = class_cost;
+    }
+    __syncthreads();
+    double total = 0.0;
+    if (threadIdx.x < kSums) {
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) total += wave_sums[threadIdx.x][w];
+    }
+    return total;
+}
+
+// One workgroup per head tile (the decoded-input form of the reference's signature).
+template<bool FUSED>
+__global__ __launch_bounds__(kBlock) void yolo_head_kernel(HeadArgs a, YoloParams p, YoloTables tb)
+{
+    __shared__ TruthSlot tile[kTruthTile];
+    __shared__ double wave_sums[kSums][kWaves];
+    const double total = head_tile<FUSED>(blockIdx.x, a, p, tb, tile, wave_sums);
+    if (threadIdx.x < kSums) a.partial[static_cast<size_t>(threadIdx.x) * gridDim.x + blockIdx.x] = total;   // [12][n]
 }
 
 // The class rows as a flat index space over [batch*mask][classes][area] (the 5 head rows of every
@@ -481,45 +549,10 @@ struct ClassSpace {
     }
 };
 
-// ---- pass 1: HEAD workgroups and CLASS (decode) workgroups in one grid ------------------------
-struct Pass1Args {
-    HeadArgs head;
-    ClassSpace space;
-    uint32_t head_blocks, class_blocks;   // HEAD workgroups come first in the grid
-};
-
-// V = 4 needs area % 4 == 0 (a vector then never leaves its row) and 16-byte aligned tensors.
-template<bool FUSED, int V, bool NT>
-__global__ __launch_bounds__(kBlock) void yolo_pass1_kernel(Pass1Args a, YoloParams p, YoloTables tb)
-{
-    __shared__ TruthSlot tile[kTruthTile];
-    __shared__ double slots[kBlock / kWave];
-    const uint32_t b = blockIdx.x;
-    // The long-lived HEAD workgroups are dispatched first, so that the short CLASS workgroups fill the
-    // machine as they retire; spreading them through the grid leaves them holding wave slots that
-    // the streaming workgroups need.
-    if (b < a.head_blocks) {
-        head_workgroup<FUSED>(b, a.head, p, tb, tile, slots);
-        return;
-    }
-    if constexpr (FUSED) {
-        const uint32_t cb = b - a.head_blocks;
-        const uint32_t e = (cb * kBlock + threadIdx.x) * V;
-        if (e >= a.space.elems) return;
-        uint32_t bn, c, cell;
-        a.space.locate(e, bn, c, cell);
-        const size_t at = a.space.offset(bn, c, cell);
-        const Pack<V> x = ld<V, NT>(a.head.in, at);
-        Pack<V> prob;
-#pragma unroll
-        for (int k = 0; k < V; ++k) prob.v[k] = sigmoid_fast(x.v[k]);
-        st<V, NT>(a.head.out, at, prob);
-    }
-}
-
-// ---- pass 2: dense class delta from the decisions; the first workgroups add up the sums -------
-struct Pass2Args {
-    const float* prob;     // decoded head (pass 1's `out`, or the caller's decoded input)
+// ---- class sweep: decode + dense class delta; the first workgroups add up the head sums --------
+struct ClassArgs {
+    const float* in;       // FUSED: raw logits; otherwise the decoded head
+    float* out;            // FUSED only
     float* delta;
     const int* decision;
     const double* partial;
@@ -531,14 +564,21 @@ struct Pass2Args {
     int accumulate;
 };
 
-// statistic k (k < 12) or the cost (k == 12, slots 8..11) over all HEAD workgroups, fixed order
-__device__ __forceinline__ void finish_statistic(int k, const Pass2Args& a, double* slots)
+// statistic k (k < 12) or the cost (k == 12, slots 8..11) over all head workgroups, fixed order
+__device__ __forceinline__ void finish_statistic(int k, const ClassArgs& a, double* slots)
 {
     const int first = k < 12 ? k : 8, last = k < 12 ? k : 11;
     double s = 0.0;
     for (int kk = first; kk <= last; ++kk) {
         const double* src = a.partial + static_cast<size_t>(kk) * a.head_blocks;
-        for (uint32_t j = threadIdx.x; j < a.head_blocks; j += kBlock) s += src[j];
+        // four loads in flight per lane; the order of the additions does not depend on it
+        for (uint32_t j = threadIdx.x; j < a.head_blocks; j += 4 * kBlock) {
+            double v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = j + u * kBlock < a.head_blocks ? src[j + u * kBlock] : 0.0;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) s += v[u];
+        }
     }
     const double total = block_sum(s, slots);
     if (threadIdx.x == 0) {
@@ -551,8 +591,9 @@ __device__ __forceinline__ void finish_statistic(int k, const Pass2Args& a, doub
     }
 }
 
-template<int V, bool NT>
-__global__ __launch_bounds__(kBlock) void yolo_pass2_kernel(Pass2Args a)
+// V = 4 needs area % 4 == 0 (a vector then never leaves its row) and 16-byte aligned tensors.
+template<bool FUSED, int V, bool NT>
+__global__ __launch_bounds__(kBlock) void yolo_class_kernel(ClassArgs a)
 {
     __shared__ double slots[kBlock / kWave];
     if (blockIdx.x < 13) finish_statistic(blockIdx.x, a, slots);
@@ -562,16 +603,101 @@ __global__ __launch_bounds__(kBlock) void yolo_pass2_kernel(Pass2Args a)
     a.space.locate(e, bn, c, cell);
     const size_t at = a.space.offset(bn, c, cell);
     const IPack<V> cls = ldi<V, false>(a.decision, static_cast<size_t>(bn) * a.space.area + cell);
-    Pack<V> d;
+    Pack<V> prob, d;
+    if constexpr (FUSED) {
+        const Pack<V> x = ld<V, NT>(a.in, at);
+#pragma unroll
+        for (int k = 0; k < V; ++k) prob.v[k] = sigmoid_fast(x.v[k]);
+        st<V, NT>(a.out, at, prob);
+    }
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         d.v[k] = 0.0f;
         if (cls.v[k] >= 0) {      // rare: a supervised slot
             const float t = (static_cast<int>(c) == cls.v[k]) ? 1.0f : 0.0f;
-            d.v[k] = a.class_scale * (t - a.prob[at + k]);
+            float pr;
+            if constexpr (FUSED) pr = prob.v[k]; else pr = a.in[at + k];
+            d.v[k] = a.class_scale * (t - pr);
         }
     }
     st<V, NT>(a.delta, at, d);
+}
+
+// ---- fused pass: persistent head workgroups + class decode stream in one grid ------------------
+// The head tiles are instruction bound and the class stream is bandwidth bound, so they run side
+// by side: the first `head_workers` workgroups of the grid (dispatched first, about two per
+// compute unit) walk the head tiles with a stride, every other workgroup decodes one vector per
+// lane of the class rows and writes a zero class delta.  The few supervised slots get their class
+// delta from yolo_patch_kernel afterwards, so nothing in this grid waits for anything else in it.
+struct FusedArgs {
+    HeadArgs head;
+    ClassSpace space;
+    uint32_t head_workers;
+};
+
+// Eight waves per SIMD (at most 64 vector registers): the class stream needs the occupancy.
+template<int V, bool NT>
+__global__ __launch_bounds__(kBlock, 8) void yolo_fused_kernel(FusedArgs a, YoloParams p, YoloTables tb)
+{
+    __shared__ TruthSlot tile[kTruthTile];
+    __shared__ double wave_sums[kSums][kWaves];
+    if (blockIdx.x < a.head_workers) {
+        // one sum per worker and statistic, over its tiles in walking order
+        double total = 0.0;
+        for (uint32_t t = blockIdx.x; t < p.blocks; t += a.head_workers) {
+            total += head_tile<true>(t, a.head, p, tb, tile, wave_sums);
+            __syncthreads();      // wave_sums is read by the first lanes until here
+        }
+        if (threadIdx.x < kSums)
+            a.head.partial[static_cast<size_t>(threadIdx.x) * a.head_workers + blockIdx.x] = total;
+        return;
+    }
+    const uint32_t e = ((blockIdx.x - a.head_workers) * kBlock + threadIdx.x) * V;
+    if (e >= a.space.elems) return;
+    uint32_t bn, c, cell;
+    a.space.locate(e, bn, c, cell);
+    const size_t at = a.space.offset(bn, c, cell);
+    const Pack<V> x = ld<V, NT>(a.head.in, at);
+    Pack<V> prob, zero;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        prob.v[k] = sigmoid_fast(x.v[k]);
+        zero.v[k] = 0.0f;
+    }
+    st<V, NT>(a.head.out, at, prob);
+    st<V, NT>(a.head.delta, at, zero);
+}
+
+// One lane per slot finds the supervised ones; a wave then writes the class delta of each of its
+// supervised slots together (one class row per lane) from the probabilities the fused pass wrote.
+// The first workgroups also add up the head sums.
+struct PatchArgs {
+    ClassArgs cls;        // in = the decoded head; out unused
+    uint32_t slots;       // batch * masks * area
+    int classes;
+};
+
+__global__ __launch_bounds__(kBlock) void yolo_patch_kernel(PatchArgs a)
+{
+    __shared__ double slots[kBlock / kWave];
+    const uint32_t slot = blockIdx.x * kBlock + threadIdx.x;
+    const int cls = slot < a.slots ? a.cls.decision[slot] : -1;
+    const int lane = threadIdx.x & (kWave - 1);
+    unsigned long long todo = __ballot(cls >= 0);
+    while (todo) {
+        const int src = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const uint32_t s_slot = __shfl(slot, src, kWave);
+        const int s_cls = __shfl(cls, src, kWave);
+        uint32_t bn, cell;
+        a.cls.space.by_area.divmod(s_slot, bn, cell);
+        for (int c = lane; c < a.classes; c += kWave) {
+            const size_t at = a.cls.space.offset(bn, c, cell);
+            const float t = (c == s_cls) ? 1.0f : 0.0f;
+            a.cls.delta[at] = a.cls.class_scale * (t - a.cls.in[at]);
+        }
+    }
+    if (blockIdx.x < 13) finish_statistic(blockIdx.x, a.cls, slots);
 }
 
 int fill_params(const char* who, YoloParams& p, int batch, int mask_count, int anchor_count, int classes, int width,
@@ -629,6 +755,18 @@ YoloWorkspace carve(void* ws, const YoloParams& p)
     return w;
 }
 
+// Persistent head workgroups of the fused pass.  A head tile takes about kTileMicros however
+// many run side by side, so enough of them are started to be through in the time the class rows
+// take to stream, and no more: every one holds wave slots the stream could use.
+uint32_t head_workers(uint32_t tiles, double stream_us)
+{
+    constexpr double kTileMicros = 22.0;
+    double rounds = stream_us * 0.85 / kTileMicros;
+    if (rounds < 1.0) rounds = 1.0;
+    uint32_t want = static_cast<uint32_t>(static_cast<double>(tiles) / rounds) + 1;
+    return want < tiles ? want : tiles;
+}
+
 template<bool FUSED>
 int run_training_pass(const char* who, const float* in, float* out, float* delta, const float* truths,
                       const int* truth_counts, const YoloParams& p, const YoloTables& tb, float* stats, float* cost,
@@ -642,36 +780,46 @@ int run_training_pass(const char* who, const float* in, float* out, float* delta
     const uint32_t per_block = kBlock * (vec ? 4 : 1);
     const uint32_t class_blocks = (space.elems + per_block - 1) / per_block;
 
-    Pass1Args a1{};
-    a1.head = HeadArgs{ in, out, delta, truths, truth_counts, w.decision, w.partial };
-    a1.space = space;
-    a1.head_blocks = p.blocks;
-    a1.class_blocks = FUSED ? class_blocks : 0;
-    const uint32_t total1 = a1.head_blocks + a1.class_blocks;
-    const bool nt1 = static_cast<size_t>(space.elems) * 8 >= kStreamingBytes;
-    if (vec && nt1) hipLaunchKernelGGL((yolo_pass1_kernel<FUSED, 4, true>), dim3(total1), dim3(kBlock), 0, s, a1, p, tb);
-    else if (vec) hipLaunchKernelGGL((yolo_pass1_kernel<FUSED, 4, false>), dim3(total1), dim3(kBlock), 0, s, a1, p, tb);
-    else hipLaunchKernelGGL((yolo_pass1_kernel<FUSED, 1, false>), dim3(total1), dim3(kBlock), 0, s, a1, p, tb);
-    int rc = check_launch(who);
-    if (rc) return rc;
+    ClassArgs ca{};
+    ca.in = FUSED ? out : in;      // the decoded head
+    ca.out = nullptr;
+    ca.delta = delta;
+    ca.decision = w.decision;
+    ca.partial = w.partial;
+    ca.stats = stats;
+    ca.cost = cost;
+    ca.space = space;
+    ca.head_blocks = p.blocks;
+    ca.class_scale = p.class_scale;
+    ca.accumulate = accumulate;
+    const HeadArgs ha{ in, out, delta, truths, truth_counts, w.decision, w.partial };
 
-    Pass2Args a2{};
-    a2.prob = FUSED ? out : in;
-    a2.delta = delta;
-    a2.decision = w.decision;
-    a2.partial = w.partial;
-    a2.stats = stats;
-    a2.cost = cost;
-    a2.space = space;
-    a2.head_blocks = p.blocks;
-    a2.class_scale = p.class_scale;
-    a2.accumulate = accumulate;
-    const uint32_t total2 = class_blocks < 13 ? 13 : class_blocks;
-    const bool nt2 = static_cast<size_t>(space.elems) * 4 >= kStreamingBytes;
-    if (vec && nt2) hipLaunchKernelGGL((yolo_pass2_kernel<4, true>), dim3(total2), dim3(kBlock), 0, s, a2);
-    else if (vec) hipLaunchKernelGGL((yolo_pass2_kernel<4, false>), dim3(total2), dim3(kBlock), 0, s, a2);
-    else hipLaunchKernelGGL((yolo_pass2_kernel<1, false>), dim3(total2), dim3(kBlock), 0, s, a2);
-    return check_launch(who);
+    if constexpr (FUSED) {
+        const double stream_us = static_cast<double>(space.elems) * 12.0 / 6.0e6;   // class stream at 6 TB/s
+        FusedArgs fa{ ha, space, head_workers(p.blocks, stream_us) };
+        ca.head_blocks = fa.head_workers;      // one partial sum per worker
+        const uint32_t grid = fa.head_workers + class_blocks;
+        const bool nt = static_cast<size_t>(space.elems) * 12 >= kStreamingBytes;
+        if (vec && nt) hipLaunchKernelGGL((yolo_fused_kernel<4, true>), dim3(grid), dim3(kBlock), 0, s, fa, p, tb);
+        else if (vec) hipLaunchKernelGGL((yolo_fused_kernel<4, false>), dim3(grid), dim3(kBlock), 0, s, fa, p, tb);
+        else hipLaunchKernelGGL((yolo_fused_kernel<1, false>), dim3(grid), dim3(kBlock), 0, s, fa, p, tb);
+        int rc = check_launch(who);
+        if (rc) return rc;
+        PatchArgs pa{ ca, static_cast<uint32_t>(p.batch) * p.mask_count * p.area, p.classes };
+        const uint32_t pgrid = grid_for(pa.slots, kBlock);
+        hipLaunchKernelGGL(yolo_patch_kernel, dim3(pgrid < 13 ? 13 : pgrid), dim3(kBlock), 0, s, pa);
+        return check_launch(who);
+    } else {
+        hipLaunchKernelGGL((yolo_head_kernel<false>), dim3(p.blocks), dim3(kBlock), 0, s, ha, p, tb);
+        int rc = check_launch(who);
+        if (rc) return rc;
+        const uint32_t grid = class_blocks < 13 ? 13 : class_blocks;
+        const bool nt = static_cast<size_t>(space.elems) * 4 >= kStreamingBytes;
+        if (vec && nt) hipLaunchKernelGGL((yolo_class_kernel<false, 4, true>), dim3(grid), dim3(kBlock), 0, s, ca);
+        else if (vec) hipLaunchKernelGGL((yolo_class_kernel<false, 4, false>), dim3(grid), dim3(kBlock), 0, s, ca);
+        else hipLaunchKernelGGL((yolo_class_kernel<false, 1, false>), dim3(grid), dim3(kBlock), 0, s, ca);
+        return check_launch(who);
+    }
 }
 
 }  // namespace
@@ -725,7 +873,10 @@ int pxh_yolo_forward_train(const float* input, float* output, float* delta, cons
             return fail_invalid("pxh_yolo_forward_train: mask %d names anchor %d of %d", m, host_masks[m], anchor_count);
         p.masks[m] = host_masks[m];
     }
-    for (int a = 0; a < 2 * anchor_count; ++a) p.anchors[a] = static_cast<float>(host_anchors[a]);
+    for (int a = 0; a < 2 * anchor_count; ++a) {
+        p.anchors[a] = static_cast<float>(host_anchors[a]);
+        p.anchors_rel[a] = p.anchors[a] / static_cast<float>(a % 2 ? net_height : net_width);
+    }
     void* ws;
     rc = resolve_workspace(workspace, workspace_bytes,
                            yolo_workspace_bytes(batch, mask_count, width, height), &ws);
