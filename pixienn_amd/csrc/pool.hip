@@ -45,7 +45,7 @@ __global__ __launch_bounds__(kBlock) void maxpool_fwd_generic_kernel(const float
 
 // 2x2 / stride 2 windows that all lie inside the input: VX outputs per lane from two
 // (2*VX)-wide row loads, stored as VX-wide value and index vectors.
-template<int VX>
+template<int VX, bool NT>
 __global__ __launch_bounds__(kBlock) void maxpool_fwd_2x2_kernel(const float* in, float* out, int* indexes,
                                                                  uint32_t units, int iw, int ow, FastDiv by_owv,
                                                                  FastDiv by_oh)
@@ -58,8 +58,8 @@ __global__ __launch_bounds__(kBlock) void maxpool_fwd_2x2_kernel(const float* in
     const uint32_t ih = by_oh.d * 2;
     const uint32_t ox = oxv * VX;
     const uint32_t in0 = (plane * ih + 2 * oy) * iw + 2 * ox;   // < 2^31 checked by the host
-    const Pack<2 * VX> r0 = ld<2 * VX>(in, in0);
-    const Pack<2 * VX> r1 = ld<2 * VX>(in, in0 + iw);
+    const Pack<2 * VX> r0 = ld<2 * VX, NT>(in, in0);
+    const Pack<2 * VX> r1 = ld<2 * VX, NT>(in, in0 + iw);
     Pack<VX> v;
     IPack<VX> ix;
 #pragma unroll
@@ -73,8 +73,57 @@ __global__ __launch_bounds__(kBlock) void maxpool_fwd_2x2_kernel(const float* in
         ix.v[k] = at;
     }
     const uint32_t o = (plane * by_oh.d + oy) * ow + ox;
-    st<VX>(out, o, v);
-    sti<VX>(indexes, o, ix);
+    st<VX, NT>(out, o, v);
+    sti<VX, NT>(indexes, o, ix);
+}
+
+// The same for an even output width (input rows of a multiple of 4 floats) and a multiple of 4
+// outputs in all, with one 128-bit access per lane and stream: a lane takes 2 consecutive
+// outputs of the flat output tensor (they share a row), i.e. 4 floats of each of two input rows;
+// the lanes of a pair then swap halves so that the even lane stores the pair's 4 values and the
+// odd lane its 4 indexes.  Every address is 16-byte aligned: rows start at multiples of 4 floats.
+template<bool NT>
+__global__ __launch_bounds__(kBlock) void maxpool_fwd_2x2_pair_kernel(const float* in, float* out, int* indexes,
+                                                                      uint32_t lanes, int iw, int ow, FastDiv by_owh,
+                                                                      FastDiv by_oh)
+{
+    // the grid is a whole number of waves and `lanes` is even: a pair is never split by the guard
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    const bool live = t < lanes;
+    const uint32_t u = live ? t : 0;
+    const uint32_t half = u & 1;
+    uint32_t rows, oxh, plane, oy;
+    by_owh.divmod(u, rows, oxh);
+    by_oh.divmod(rows, plane, oy);
+    const uint32_t ih = by_oh.d * 2;
+    const uint32_t ox = oxh * 2;
+    const uint32_t in0 = (plane * ih + 2 * oy) * iw + 2 * ox;   // < 2^31 checked by the host
+    const Pack<4> r0 = ld<4, NT>(in, in0);
+    const Pack<4> r1 = ld<4, NT>(in, in0 + iw);
+    float v[2];
+    int ix[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        float best = r0.v[2 * k];
+        int at = in0 + 2 * k;
+        if (r0.v[2 * k + 1] > best) { best = r0.v[2 * k + 1]; at = in0 + 2 * k + 1; }
+        if (r1.v[2 * k] > best) { best = r1.v[2 * k]; at = in0 + iw + 2 * k; }
+        if (r1.v[2 * k + 1] > best) { best = r1.v[2 * k + 1]; at = in0 + iw + 2 * k + 1; }
+        v[k] = best;
+        ix[k] = at;
+    }
+    // even lane: gives its indexes, takes the partner's values; odd lane the other way round
+    const float pv0 = __shfl_xor(v[0], 1, kWave), pv1 = __shfl_xor(v[1], 1, kWave);
+    const int pi0 = __shfl_xor(ix[0], 1, kWave), pi1 = __shfl_xor(ix[1], 1, kWave);
+    if (!live) return;
+    const uint32_t o = (u >> 1) * 4;       // the pair's 4 flat outputs
+    if (half == 0) {
+        const Pack<4> w{ { v[0], v[1], pv0, pv1 } };
+        st<4, NT>(out, o, w);
+    } else {
+        const IPack<4> w{ { pi0, pi1, ix[0], ix[1] } };
+        sti<4, NT>(indexes, o, w);
+    }
 }
 
 // Backward, any geometry: one input cell per lane gathers, in ascending output order, the
@@ -112,7 +161,7 @@ __global__ __launch_bounds__(kBlock) void maxpool_bwd_generic_kernel(const float
 
 // Backward for the 2x2 / stride 2 in-bounds case: one window per output, VX windows per lane,
 // the two grad rows are updated as full vectors so the read-modify-write stays coalesced.
-template<int VX>
+template<int VX, bool NT>
 __global__ __launch_bounds__(kBlock) void maxpool_bwd_2x2_kernel(const float* delta, const int* indexes, float* grad,
                                                                  uint32_t units, int iw, int ow, FastDiv by_owv,
                                                                  FastDiv by_oh)
@@ -126,10 +175,10 @@ __global__ __launch_bounds__(kBlock) void maxpool_bwd_2x2_kernel(const float* de
     const uint32_t ox = oxv * VX;
     const uint32_t in0 = (plane * ih + 2 * oy) * iw + 2 * ox;
     const uint32_t o = (plane * by_oh.d + oy) * ow + ox;
-    const Pack<VX> d = ld<VX>(delta, o);
-    const IPack<VX> ix = ldi<VX>(indexes, o);
-    Pack<2 * VX> g0 = ld<2 * VX>(grad, in0);
-    Pack<2 * VX> g1 = ld<2 * VX>(grad, in0 + iw);
+    const Pack<VX> d = ld<VX, NT>(delta, o);
+    const IPack<VX> ix = ldi<VX, NT>(indexes, o);
+    Pack<2 * VX> g0 = ld<2 * VX, NT>(grad, in0);
+    Pack<2 * VX> g1 = ld<2 * VX, NT>(grad, in0 + iw);
 #pragma unroll
     for (int k = 0; k < VX; ++k) {
         const int at = ix.v[k];
@@ -139,8 +188,57 @@ __global__ __launch_bounds__(kBlock) void maxpool_bwd_2x2_kernel(const float* de
         else if (at == base + iw) g1.v[2 * k] += d.v[k];
         else if (at == base + iw + 1) g1.v[2 * k + 1] += d.v[k];
     }
-    st<2 * VX>(grad, in0, g0);
-    st<2 * VX>(grad, in0 + iw, g1);
+    st<2 * VX, NT>(grad, in0, g0);
+    st<2 * VX, NT>(grad, in0 + iw, g1);
+}
+
+// The pair form of the backward pass: the even lane reads the pair's 4 deltas, the odd lane its
+// 4 indexes, they swap halves, and every lane updates 4 floats of each of the two grad rows.
+template<bool NT>
+__global__ __launch_bounds__(kBlock) void maxpool_bwd_2x2_pair_kernel(const float* delta, const int* indexes,
+                                                                      float* grad, uint32_t lanes, int iw, int ow,
+                                                                      FastDiv by_owh, FastDiv by_oh)
+{
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    const bool live = t < lanes;
+    const uint32_t u = live ? t : 0;
+    const uint32_t half = u & 1;
+    uint32_t rows, oxh, plane, oy;
+    by_owh.divmod(u, rows, oxh);
+    by_oh.divmod(rows, plane, oy);
+    const uint32_t ih = by_oh.d * 2;
+    const uint32_t ox = oxh * 2;
+    const uint32_t in0 = (plane * ih + 2 * oy) * iw + 2 * ox;
+    const uint32_t o = (u >> 1) * 4;
+    // one 128-bit load per lane: deltas (even) or indexes (odd), as raw bits
+    const Pack<4> mine = half == 0 ? ld<4, NT>(delta, o) : ld<4, NT>(reinterpret_cast<const float*>(indexes), o);
+    Pack<4> theirs;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) theirs.v[k] = __shfl_xor(mine.v[k], 1, kWave);
+    // this lane's two windows are outputs 2*half, 2*half + 1 of the pair
+    float d[2];
+    int ix[2];
+    if (half == 0) {
+        d[0] = mine.v[0]; d[1] = mine.v[1];
+        ix[0] = __float_as_int(theirs.v[0]); ix[1] = __float_as_int(theirs.v[1]);
+    } else {
+        d[0] = theirs.v[2]; d[1] = theirs.v[3];
+        ix[0] = __float_as_int(mine.v[2]); ix[1] = __float_as_int(mine.v[3]);
+    }
+    if (!live) return;
+    Pack<4> g0 = ld<4, NT>(grad, in0);
+    Pack<4> g1 = ld<4, NT>(grad, in0 + iw);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int at = ix[k];
+        const int base = static_cast<int>(in0) + 2 * k;
+        if (at == base) g0.v[2 * k] += d[k];
+        else if (at == base + 1) g0.v[2 * k + 1] += d[k];
+        else if (at == base + iw) g1.v[2 * k] += d[k];
+        else if (at == base + iw + 1) g1.v[2 * k + 1] += d[k];
+    }
+    st<4, NT>(grad, in0, g0);
+    st<4, NT>(grad, in0 + iw, g1);
 }
 
 __global__ __launch_bounds__(kBlock) void maxpool_bwd_scatter_kernel(const float* delta, const int* indexes,
@@ -269,17 +367,29 @@ int pxh_maxpool_forward(const float* in, float* out, int* indexes, int batch, in
     const uint32_t total = planes * oh * ow;
     if (is_2x2_inbounds(ih, iw, oh, ow, kernel, stride, padding) && aligned16(in) && aligned16(out) &&
         aligned16(indexes)) {
-        if (iw % 8 == 0) {
-            const uint32_t units = total / 4;
-            hipLaunchKernelGGL((maxpool_fwd_2x2_kernel<4>), dim3(grid_for(units, kBlock)), dim3(kBlock), 0, s, in, out,
-                               indexes, units, iw, ow, FastDiv(ow / 4), FastDiv(oh));
+        // 4 bytes in, 8 bytes out per input element / 4
+        const bool nt = static_cast<size_t>(total) * 24 >= kStreamingBytes;
+        // the pair form needs an even output width and whole output quads; it pays for wide rows
+        if (iw % 8 == 0 && total % 4 == 0) {
+            const uint32_t lanes = total / 2;
+            const dim3 grid(grid_for(lanes, kBlock));
+            if (nt) hipLaunchKernelGGL((maxpool_fwd_2x2_pair_kernel<true>), grid, dim3(kBlock), 0, s, in, out, indexes,
+                                       lanes, iw, ow, FastDiv(ow / 2), FastDiv(oh));
+            else hipLaunchKernelGGL((maxpool_fwd_2x2_pair_kernel<false>), grid, dim3(kBlock), 0, s, in, out, indexes,
+                                    lanes, iw, ow, FastDiv(ow / 2), FastDiv(oh));
         } else if (iw % 4 == 0) {
             const uint32_t units = total / 2;
-            hipLaunchKernelGGL((maxpool_fwd_2x2_kernel<2>), dim3(grid_for(units, kBlock)), dim3(kBlock), 0, s, in, out,
-                               indexes, units, iw, ow, FastDiv(ow / 2), FastDiv(oh));
+            const dim3 grid(grid_for(units, kBlock));
+            if (nt) hipLaunchKernelGGL((maxpool_fwd_2x2_kernel<2, true>), grid, dim3(kBlock), 0, s, in, out, indexes,
+                                       units, iw, ow, FastDiv(ow / 2), FastDiv(oh));
+            else hipLaunchKernelGGL((maxpool_fwd_2x2_kernel<2, false>), grid, dim3(kBlock), 0, s, in, out, indexes,
+                                    units, iw, ow, FastDiv(ow / 2), FastDiv(oh));
         } else {
-            hipLaunchKernelGGL((maxpool_fwd_2x2_kernel<1>), dim3(grid_for(total, kBlock)), dim3(kBlock), 0, s, in, out,
-                               indexes, total, iw, ow, FastDiv(ow), FastDiv(oh));
+            const dim3 grid(grid_for(total, kBlock));
+            if (nt) hipLaunchKernelGGL((maxpool_fwd_2x2_kernel<1, true>), grid, dim3(kBlock), 0, s, in, out, indexes,
+                                       total, iw, ow, FastDiv(ow), FastDiv(oh));
+            else hipLaunchKernelGGL((maxpool_fwd_2x2_kernel<1, false>), grid, dim3(kBlock), 0, s, in, out, indexes,
+                                    total, iw, ow, FastDiv(ow), FastDiv(oh));
         }
         return check_launch("pxh_maxpool_forward");
     }
@@ -300,17 +410,28 @@ int pxh_maxpool_backward(const float* delta, const int* indexes, float* grad, in
     const uint32_t out_total = planes * oh * ow;
     if (is_2x2_inbounds(ih, iw, oh, ow, kernel, stride, padding) && aligned16(delta) && aligned16(indexes) &&
         aligned16(grad)) {
-        if (iw % 8 == 0) {
-            const uint32_t units = out_total / 4;
-            hipLaunchKernelGGL((maxpool_bwd_2x2_kernel<4>), dim3(grid_for(units, kBlock)), dim3(kBlock), 0, s, delta,
-                               indexes, grad, units, iw, ow, FastDiv(ow / 4), FastDiv(oh));
+        // 8 bytes per output, 8 bytes per grad cell
+        const bool nt = static_cast<size_t>(out_total) * 40 >= kStreamingBytes;
+        if (iw % 8 == 0 && out_total % 4 == 0) {
+            const uint32_t lanes = out_total / 2;
+            const dim3 grid(grid_for(lanes, kBlock));
+            if (nt) hipLaunchKernelGGL((maxpool_bwd_2x2_pair_kernel<true>), grid, dim3(kBlock), 0, s, delta, indexes,
+                                       grad, lanes, iw, ow, FastDiv(ow / 2), FastDiv(oh));
+            else hipLaunchKernelGGL((maxpool_bwd_2x2_pair_kernel<false>), grid, dim3(kBlock), 0, s, delta, indexes,
+                                    grad, lanes, iw, ow, FastDiv(ow / 2), FastDiv(oh));
         } else if (iw % 4 == 0) {
             const uint32_t units = out_total / 2;
-            hipLaunchKernelGGL((maxpool_bwd_2x2_kernel<2>), dim3(grid_for(units, kBlock)), dim3(kBlock), 0, s, delta,
-                               indexes, grad, units, iw, ow, FastDiv(ow / 2), FastDiv(oh));
+            const dim3 grid(grid_for(units, kBlock));
+            if (nt) hipLaunchKernelGGL((maxpool_bwd_2x2_kernel<2, true>), grid, dim3(kBlock), 0, s, delta, indexes,
+                                       grad, units, iw, ow, FastDiv(ow / 2), FastDiv(oh));
+            else hipLaunchKernelGGL((maxpool_bwd_2x2_kernel<2, false>), grid, dim3(kBlock), 0, s, delta, indexes, grad,
+                                    units, iw, ow, FastDiv(ow / 2), FastDiv(oh));
         } else {
-            hipLaunchKernelGGL((maxpool_bwd_2x2_kernel<1>), dim3(grid_for(out_total, kBlock)), dim3(kBlock), 0, s,
-                               delta, indexes, grad, out_total, iw, ow, FastDiv(ow), FastDiv(oh));
+            const dim3 grid(grid_for(out_total, kBlock));
+            if (nt) hipLaunchKernelGGL((maxpool_bwd_2x2_kernel<1, true>), grid, dim3(kBlock), 0, s, delta, indexes,
+                                       grad, out_total, iw, ow, FastDiv(ow), FastDiv(oh));
+            else hipLaunchKernelGGL((maxpool_bwd_2x2_kernel<1, false>), grid, dim3(kBlock), 0, s, delta, indexes, grad,
+                                    out_total, iw, ow, FastDiv(ow), FastDiv(oh));
         }
         return check_launch("pxh_maxpool_backward");
     }

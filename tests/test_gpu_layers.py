@@ -54,7 +54,7 @@ def test_maxpool_reference_kat(ops, kats):
 
 
 @pytest.mark.parametrize("shape", [(2, 3, 304, 304), (2, 4, 76, 76), (2, 5, 38, 38), (3, 4, 26, 26),
-                                   (1, 2, 416, 416), (2, 3, 6, 10), (2, 2, 20, 12)])
+                                   (1, 2, 416, 416), (2, 3, 6, 10), (2, 2, 20, 12), (1, 1, 6, 4), (1, 3, 2, 12)])
 def test_maxpool_2x2_stride2(ops, oracle, shape):
     x = wl.normal(1000 + shape[2], shape)
     run_maxpool(ops, oracle, x, 2, 2, 1, 1100)
