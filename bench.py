@@ -54,22 +54,45 @@ def parse_args():
 
 
 class Timer:
-    """Mean duration of a launch sequence from HIP events on the current stream."""
+    """Mean duration of a launch sequence from HIP events on the stream it runs on.
+
+    The repetitions are recorded into one HIP graph and the graph is replayed between the two
+    events: a launch through Python and ctypes costs several microseconds of host time, more than
+    the small kernels of this path run, and the graph takes that out of the measurement.  If the
+    capture fails the repetitions are launched eagerly."""
 
     def __init__(self, torch):
         self.torch = torch
+        self.use_graphs = True
 
     def time(self, fn, reps, warm=2, rotate=1):
         """fn(i) launches one repetition using buffer set i % rotate.  Returns ms per repetition."""
         t = self.torch
-        for i in range(warm):
+        for i in range(max(warm, rotate)):
             fn(i % rotate)
         t.cuda.synchronize()
+        graph = None
+        if self.use_graphs:
+            try:
+                graph = t.cuda.CUDAGraph()
+                with t.cuda.graph(graph):
+                    for i in range(reps):
+                        fn(i % rotate)
+                graph.replay()
+                t.cuda.synchronize()
+            except Exception as e:      # noqa: BLE001 - any capture problem means: measure eagerly
+                log("graph capture failed (%s): timing eagerly" % e)
+                graph = None
+                self.use_graphs = False
+                t.cuda.synchronize()
         start = t.cuda.Event(enable_timing=True)
         stop = t.cuda.Event(enable_timing=True)
         start.record()
-        for i in range(reps):
-            fn(i % rotate)
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(reps):
+                fn(i % rotate)
         stop.record()
         t.cuda.synchronize()
         return start.elapsed_time(stop) / reps

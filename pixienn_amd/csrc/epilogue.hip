@@ -294,8 +294,46 @@ __global__ __launch_bounds__(kBlock) void bn_stats_partial_kernel(const float* x
     if (threadIdx.x == 0) partial[blockIdx.x] = make_double2(t1, t2);
 }
 
-// One wavefront per channel adds the channel's partials, finishes mean / variance, updates the
-// rolling statistics and (when asked) folds the constants the apply pass needs.
+// Mean / variance from the shifted sums S1 = sum(x - K), S2 = sum((x - K)^2) over `count` values,
+// and the rolling statistics moved towards them.
+struct ChannelStats { float mean, var, rolling_mean, rolling_var; };
+
+__device__ __forceinline__ ChannelStats channel_stats(double s1, double s2, float shift_value, double count,
+                                                      float rolling_mean, float rolling_var)
+{
+    const double shift = static_cast<double>(shift_value);
+    const double m = s1 / count;
+    double v = (s2 - s1 * m) / count;
+    if (v < 0.0) v = 0.0;
+    ChannelStats st;
+    st.mean = static_cast<float>(shift + m);
+    st.var = static_cast<float>(v);
+    // sscal then saxpy: two fp32 roundings each (src/BatchNorm.cpp:53-56)
+    float r = 0.99f * rolling_mean;
+    st.rolling_mean = r + .01f * st.mean;
+    r = 0.99f * rolling_var;
+    st.rolling_var = r + .01f * st.var;
+    return st;
+}
+
+// The same for channel c of the tensors: writes the statistics and folds the constants the apply
+// pass needs.
+__device__ __forceinline__ FoldCoef finish_stats(double s1, double s2, float shift_value, double count, int c,
+                                                 float* mean, float* var, float* rolling_mean, float* rolling_var,
+                                                 const float* scale, const float* bias)
+{
+    const ChannelStats st = channel_stats(s1, s2, shift_value, count, rolling_mean ? rolling_mean[c] : 0.0f,
+                                          rolling_var ? rolling_var[c] : 0.0f);
+    mean[c] = st.mean;
+    var[c] = st.var;
+    if (rolling_mean) {
+        rolling_mean[c] = st.rolling_mean;
+        rolling_var[c] = st.rolling_var;
+    }
+    return make_coef(st.mean, st.var, scale ? scale[c] : 1.0f, bias ? bias[c] : 0.0f);
+}
+
+// One wavefront per channel adds the channel's partials and finishes the statistics.
 __global__ __launch_bounds__(kBlock) void bn_stats_finish_kernel(const float* x, const double2* partial, int channels,
                                                                  int spatial, int blocks, double count, float* mean,
                                                                  float* var, float* rolling_mean, float* rolling_var,
@@ -314,22 +352,9 @@ __global__ __launch_bounds__(kBlock) void bn_stats_finish_kernel(const float* x,
     s1 = wave_sum(s1);
     s2 = wave_sum(s2);
     if (lane == 0) {
-        const double shift = static_cast<double>(x[static_cast<size_t>(c) * spatial]);
-        const double m = s1 / count;
-        double v = (s2 - s1 * m) / count;
-        if (v < 0.0) v = 0.0;
-        const float fm = static_cast<float>(shift + m);
-        const float fv = static_cast<float>(v);
-        mean[c] = fm;
-        var[c] = fv;
-        if (rolling_mean) {
-            // sscal then saxpy: two fp32 roundings each (src/BatchNorm.cpp:53-56)
-            float r = 0.99f * rolling_mean[c];
-            rolling_mean[c] = r + .01f * fm;
-            r = 0.99f * rolling_var[c];
-            rolling_var[c] = r + .01f * fv;
-        }
-        if (table) table[c] = make_coef(fm, fv, scale[c], bias[c]);
+        const FoldCoef k = finish_stats(s1, s2, x[static_cast<size_t>(c) * spatial], count, c, mean, var, rolling_mean,
+                                        rolling_var, scale, bias);
+        if (table) table[c] = k;
     }
 }
 
@@ -406,6 +431,39 @@ struct __attribute__((aligned(16))) DxCoef {
     double pad;
 };
 
+// Channel c from A = sum d' and B = sum d' * (x - mean): accumulates the parameter updates and
+// returns the constants of the dx pass.
+template<bool BN>
+__device__ __forceinline__ DxCoef finish_backward(double sa, double sb, int c, int count, const float* mean,
+                                                  const float* var, const float* scale, const float* bias,
+                                                  float* scale_updates, float* bias_updates, float* mean_delta,
+                                                  float* var_delta)
+{
+    DxCoef k{};
+    bias_updates[c] += static_cast<float>(sa);
+    if constexpr (BN) {
+        const float v = var[c];
+        const float s = scale[c];
+        // sum d' * x_hat with x_hat = (x - mean) / (sqrt(var) + eps)
+        const double denom = sqrt(static_cast<double>(v)) + static_cast<double>(kEps);
+        scale_updates[c] += static_cast<float>(sb / denom);
+        // sums of d'' = d' * scale
+        const float sum_dd = static_cast<float>(sa * static_cast<double>(s));
+        const float sum_ddx = static_cast<float>(sb * static_cast<double>(s));
+        const float ve = v + kEps;
+        const float md = static_cast<float>(static_cast<double>(sum_dd) * (-1. / static_cast<double>(sqrtf(ve))));
+        const float vd = sum_ddx * (-.5f * powf(ve, -3.0f / 2.0f));
+        if (mean_delta) mean_delta[c] = md;
+        if (var_delta) var_delta[c] = vd;
+        k.f = make_coef(mean[c], v, s, bias[c]);
+        k.rroot = 1.0 / sqrt(static_cast<double>(ve));
+        k.c2 = static_cast<double>(vd) * 2. / static_cast<double>(count);
+        k.md_term = static_cast<double>(md / static_cast<float>(count));
+        k.pad = 0.0;
+    }
+    return k;
+}
+
 template<bool BN>
 __global__ __launch_bounds__(kBlock) void bwd_finish_kernel(const double2* partial, int channels, int blocks, int count,
                                                             const float* mean, const float* var, const float* scale,
@@ -425,29 +483,9 @@ __global__ __launch_bounds__(kBlock) void bwd_finish_kernel(const double2* parti
     sa = wave_sum(sa);
     sb = wave_sum(sb);
     if (lane == 0) {
-        bias_updates[c] += static_cast<float>(sa);
-        if constexpr (BN) {
-            const float v = var[c];
-            const float s = scale[c];
-            // sum d' * x_hat with x_hat = (x - mean) / (sqrt(var) + eps)
-            const double denom = sqrt(static_cast<double>(v)) + static_cast<double>(kEps);
-            scale_updates[c] += static_cast<float>(sb / denom);
-            // sums of d'' = d' * scale
-            const float sum_dd = static_cast<float>(sa * static_cast<double>(s));
-            const float sum_ddx = static_cast<float>(sb * static_cast<double>(s));
-            const float ve = v + kEps;
-            const float md = static_cast<float>(static_cast<double>(sum_dd) * (-1. / static_cast<double>(sqrtf(ve))));
-            const float vd = sum_ddx * (-.5f * powf(ve, -3.0f / 2.0f));
-            if (mean_delta) mean_delta[c] = md;
-            if (var_delta) var_delta[c] = vd;
-            DxCoef k;
-            k.f = make_coef(mean[c], v, s, bias[c]);
-            k.rroot = 1.0 / sqrt(static_cast<double>(ve));
-            k.c2 = static_cast<double>(vd) * 2. / static_cast<double>(count);
-            k.md_term = static_cast<double>(md / static_cast<float>(count));
-            k.pad = 0.0;
-            coef[c] = k;
-        }
+        const DxCoef k = finish_backward<BN>(sa, sb, c, count, mean, var, scale, bias, scale_updates, bias_updates,
+                                             mean_delta, var_delta);
+        if constexpr (BN) coef[c] = k;
     }
 }
 
@@ -536,6 +574,214 @@ __global__ __launch_bounds__(kBlock) void bn_dx_scalar_kernel(DxArgs a)
     const bool recompute = a.pre == nullptr;
     const float pre = (ACT != PXH_LINEAR && !recompute) ? a.pre[e] : 0.0f;
     a.delta[e] = dx_value<ACT>(a.delta[e], a.x[e], pre, recompute, a.coef[c]);
+}
+
+// ---------------------------------------------------------------- channel-resident training passes
+// For a tensor whose per-channel slice (batch * spatial floats) fits the registers of one
+// workgroup, the three launches above (partial sums, finish, apply) collapse into one: workgroup c
+// holds channel c, reduces it, finishes the statistics and applies them.  The tensor is read from
+// memory once, and a small layer costs one launch instead of three.
+constexpr int kResidentThreads = 1024;
+constexpr int kResidentWaves = kResidentThreads / kWave;
+
+// Sum of two doubles over the workgroup; every thread returns both totals.
+__device__ __forceinline__ void resident_sum2(double& a, double& b, double (*slots)[kResidentWaves])
+{
+    a = wave_sum(a);
+    b = wave_sum(b);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) {
+        slots[0][wave] = a;
+        slots[1][wave] = b;
+    }
+    __syncthreads();
+    double ta = 0.0, tb = 0.0;
+#pragma unroll
+    for (int w = 0; w < kResidentWaves; ++w) {
+        ta += slots[0][w];
+        tb += slots[1][w];
+    }
+    a = ta;
+    b = tb;
+}
+
+struct ResidentGeom {
+    int channels, spatial;
+    uint32_t per_channel;     // batch * spatial
+    FastDiv by_spatial;
+    // offset of element e of channel c's slice (e counts through the images)
+    __device__ __forceinline__ size_t at(uint32_t c, uint32_t e) const
+    {
+        uint32_t n, r;
+        by_spatial.divmod(e, n, r);
+        return (static_cast<size_t>(n) * channels + c) * spatial + r;
+    }
+};
+
+struct ResidentFwdArgs {
+    const float* x;
+    float* y;
+    float* pre;        // nullable
+    float* x_saved;    // nullable
+    float* x_norm;     // nullable
+    float* mean;
+    float* var;
+    float* rolling_mean;
+    float* rolling_var;
+    const float* scale;
+    const float* bias;
+    ResidentGeom g;
+};
+
+// V = 4 needs spatial % 4 == 0 and 16-byte aligned tensors.  R vectors per thread at most.
+template<int ACT, int V, int R>
+__global__ __launch_bounds__(kResidentThreads) void bn_resident_fwd_kernel(ResidentFwdArgs a)
+{
+    __shared__ double slots[2][kResidentWaves];
+    __shared__ FoldCoef shared_coef;
+    const uint32_t c = blockIdx.x;
+    const float shift = a.x[static_cast<size_t>(c) * a.g.spatial];
+    // issued now, needed after the reduction
+    const float rm_in = a.rolling_mean[c], rv_in = a.rolling_var[c], scale_in = a.scale[c], bias_in = a.bias[c];
+    Pack<V> v[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+        if (e < a.g.per_channel) v[r] = ld<V, false>(a.x, a.g.at(c, e));
+    }
+    float a1 = 0.0f, a2 = 0.0f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if ((r * kResidentThreads + threadIdx.x) * V < a.g.per_channel) {
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                const float d = v[r].v[k] - shift;
+                a1 += d;
+                a2 += d * d;
+            }
+        }
+    }
+    double s1 = static_cast<double>(a1), s2 = static_cast<double>(a2);
+    resident_sum2(s1, s2, slots);
+    if (threadIdx.x == 0) {
+        const ChannelStats st = channel_stats(s1, s2, shift, static_cast<double>(a.g.per_channel), rm_in, rv_in);
+        a.mean[c] = st.mean;
+        a.var[c] = st.var;
+        a.rolling_mean[c] = st.rolling_mean;
+        a.rolling_var[c] = st.rolling_var;
+        shared_coef = make_coef(st.mean, st.var, scale_in, bias_in);
+    }
+    __syncthreads();
+    const FoldCoef k = shared_coef;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+        if (e < a.g.per_channel) {
+            const size_t where = a.g.at(c, e);
+            Pack<V> xn, pre, out;
+#pragma unroll
+            for (int q = 0; q < V; ++q) {
+                xn.v[q] = normalize(v[r].v[q], k);
+                pre.v[q] = affine(xn.v[q], k);
+                out.v[q] = act_apply<ACT>(pre.v[q]);
+            }
+            if (a.x_saved) st<V, false>(a.x_saved, where, v[r]);
+            if (a.x_norm) st<V, false>(a.x_norm, where, xn);
+            if (a.pre) st<V, false>(a.pre, where, pre);
+            st<V, false>(a.y, where, out);
+        }
+    }
+}
+
+struct ResidentBwdArgs {
+    BackwardArgs b;
+    float* scale_updates;
+    float* bias_updates;
+    float* mean_delta;   // nullable
+    float* var_delta;    // nullable
+    ResidentGeom g;
+};
+
+// The workgroup keeps d' = delta * act'(pre) in registers; x is read again for the dx phase
+// (it is still in the cache: one channel's slice is a few hundred KB).
+template<int ACT, int V, int R>
+__global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(ResidentBwdArgs a)
+{
+    __shared__ double slots[2][kResidentWaves];
+    __shared__ DxCoef shared_coef;
+    const uint32_t c = blockIdx.x;
+    const FoldCoef k = make_coef(a.b.mean[c], a.b.var[c], a.b.scale[c], a.b.bias[c]);
+    const bool recompute = a.b.pre == nullptr;
+    Pack<V> d[R];
+    float fa = 0.0f, fb = 0.0f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+        if (e < a.g.per_channel) {
+            const size_t where = a.g.at(c, e);
+            d[r] = ld<V, false>(a.b.delta, where);
+            const Pack<V> xv = ld<V, false>(a.b.x, where);
+            Pack<V> pv;
+            if constexpr (ACT != PXH_LINEAR) {
+                if (!recompute) pv = ld<V, false>(a.b.pre, where);
+            }
+#pragma unroll
+            for (int q = 0; q < V; ++q) {
+                float dv = d[r].v[q];
+                if constexpr (ACT != PXH_LINEAR) {
+                    float pre;
+                    if (recompute) pre = affine(normalize(xv.v[q], k), k);
+                    else pre = pv.v[q];
+                    dv = dv * act_grad<ACT>(pre);
+                    d[r].v[q] = dv;
+                }
+                fa += dv;
+                fb += dv * (xv.v[q] - k.mean);
+            }
+        }
+    }
+    double sa = static_cast<double>(fa), sb = static_cast<double>(fb);
+    resident_sum2(sa, sb, slots);
+    if (threadIdx.x == 0)
+        shared_coef = finish_backward<true>(sa, sb, c, static_cast<int>(a.g.per_channel), a.b.mean, a.b.var, a.b.scale,
+                                            a.b.bias, a.scale_updates, a.bias_updates, a.mean_delta, a.var_delta);
+    __syncthreads();
+    const DxCoef kd = shared_coef;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+        if (e < a.g.per_channel) {
+            const size_t where = a.g.at(c, e);
+            const Pack<V> xv = ld<V, false>(a.b.x, where);
+            Pack<V> out;
+#pragma unroll
+            for (int q = 0; q < V; ++q) out.v[q] = dx_value<PXH_LINEAR>(d[r].v[q], xv.v[q], 0.0f, false, kd);
+            st<V, false>(a.b.delta, where, out);
+        }
+    }
+}
+
+// Vectors per thread the resident kernels are built for, and whether a shape takes that path:
+// the channel slice must fit, and there must be enough channels to occupy the machine.  (Measured
+// with 24 vectors per thread: the registers spill and 128 workgroups of 16x128x76^2 are slower than
+// the three launches.)
+constexpr int kResidentVectors = 8;
+
+int resident_vectors(int batch, int channels, int spatial, bool vec)
+{
+    if (channels < 96) return 0;
+    const size_t per_channel = static_cast<size_t>(batch) * spatial;
+    const size_t vectors = (per_channel + (vec ? 3 : 0)) / (vec ? 4 : 1);
+    const size_t per_thread = (vectors + kResidentThreads - 1) / kResidentThreads;
+    return per_thread <= kResidentVectors ? kResidentVectors : 0;
+}
+
+ResidentGeom resident_geom(int batch, int channels, int spatial)
+{
+    return ResidentGeom{ channels, spatial, static_cast<uint32_t>(batch) * static_cast<uint32_t>(spatial),
+                         FastDiv(static_cast<uint32_t>(spatial)) };
 }
 
 // workspace: [partial sums][per-channel constants]
@@ -687,10 +933,26 @@ int pxh_bn_train_act_forward(const float* x, float* y, float* pre_activation, fl
     EpilogueArgs a{};
     int rc = check_shape("pxh_bn_train_act_forward", batch, channels, spatial, &a.total);
     if (rc) return rc;
+    hipStream_t s = as_stream(stream);
+    {
+        const bool vec = spatial % 4 == 0 && aligned16(x) && aligned16(y) && aligned16(pre_activation) &&
+                         aligned16(x_saved) && aligned16(x_norm);
+        const int per_thread = resident_vectors(batch, channels, spatial, vec);
+        if (per_thread) {
+            const ResidentFwdArgs r{ x, y, pre_activation, x_saved, x_norm, mean, var, rolling_mean, rolling_var,
+                                     scale, bias, resident_geom(batch, channels, spatial) };
+            const dim3 grid(channels), block(kResidentThreads);
+            const bool known = dispatch_activation(activation, [&]<int ACT>() {
+                if (vec) hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 4, kResidentVectors>), grid, block, 0, s, r);
+                else hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 1, kResidentVectors>), grid, block, 0, s, r);
+            });
+            if (!known) return fail_invalid("pxh_bn_train_act_forward: unknown activation %d", activation);
+            return check_launch("pxh_bn_train_act_forward");
+        }
+    }
     void* ws;
     rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws);
     if (rc) return rc;
-    hipStream_t s = as_stream(stream);
     FoldCoef* table = static_cast<FoldCoef*>(coef_region(ws, batch, channels, spatial));
     rc = launch_stats(x, mean, var, rolling_mean, rolling_var, scale, bias, table, batch, channels, spatial, a.total,
                       ws, s);
@@ -711,10 +973,25 @@ int pxh_bn_act_backward(float* delta, const float* x, const float* pre_activatio
     uint32_t total;
     int rc = check_shape("pxh_bn_act_backward", batch, channels, spatial, &total);
     if (rc) return rc;
+    hipStream_t s = as_stream(stream);
+    {
+        const bool rvec = spatial % 4 == 0 && aligned16(delta) && aligned16(x) && aligned16(pre_activation);
+        const int per_thread = resident_vectors(batch, channels, spatial, rvec);
+        if (per_thread) {
+            const ResidentBwdArgs r{ BackwardArgs{ delta, x, pre_activation, mean, var, scale, bias }, scale_updates,
+                                     bias_updates, mean_delta, var_delta, resident_geom(batch, channels, spatial) };
+            const dim3 grid(channels), block(kResidentThreads);
+            const bool known = dispatch_activation(activation, [&]<int ACT>() {
+                if (rvec) hipLaunchKernelGGL((bn_resident_bwd_kernel<ACT, 4, kResidentVectors>), grid, block, 0, s, r);
+                else hipLaunchKernelGGL((bn_resident_bwd_kernel<ACT, 1, kResidentVectors>), grid, block, 0, s, r);
+            });
+            if (!known) return fail_invalid("pxh_bn_act_backward: unknown activation %d", activation);
+            return check_launch("pxh_bn_act_backward");
+        }
+    }
     void* ws;
     rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws);
     if (rc) return rc;
-    hipStream_t s = as_stream(stream);
     const ReduceGeom g = make_geom(batch, channels, spatial);
     double2* partial = static_cast<double2*>(ws);
     DxCoef* coef = static_cast<DxCoef*>(coef_region(ws, batch, channels, spatial));
