@@ -284,6 +284,22 @@ def measure_extras(torch, ops, wl, timer):
     ms_adam = max(ms_both - ms_copy, 1e-6)
     add("adam_update", "%d params" % P, 32 * P, ms_adam, "32B/param, L2 folded into the update")
 
+    # ---- SGD with momentum over the same buffer (the optimiser of the shipped presets)
+    ms_sgd = timer.time(lambda i: ops.sgd_update(w, d, 16, 1e-3, 0.9, 5e-4, True), 10)
+    add("sgd_update", "%d params" % P, 16 * P, ms_sgd, "16B/param; not in ms/batch (Adam is)")
+    del w, g, m, v, d
+    # ---- gradient rescale + clamp of a delta tensor: 4B/elem for the norm, 8B/elem to rewrite
+    for c, s_ in [(256, 76), (64, 304)]:
+        e = N * c * s_ * s_
+        rot = rotation_for(12 * e)
+        xs = [randn(N, c, s_, s_) for _ in range(rot)]
+        # a threshold far below the norm: every call rescales and clamps
+        ms = timer.time(lambda i: ops.rescale_clip(xs[i], 1e-3, 1e-6), 10, rotate=rot)
+        add("rescale_clip", "%dx%dx%d^2" % (N, c, s_), 12 * e, ms, "norm 4B + rewrite 8B per elem")
+        ms = timer.time(lambda i: ops.rescale_clip(xs[i], 1e30, 0.0), 10, rotate=rot)
+        add("rescale_clip(no-op)", "%dx%dx%d^2" % (N, c, s_), 4 * e, ms, "below the threshold: norm only, 4B/elem")
+        del xs
+
     # ---- non-conv ms per batch, YOLOv3 @608, batch 16, one training step:
     # 72 BN'd conv epilogues fwd+bwd, 3 bias epilogues, 23 shortcuts fwd+bwd, 2 upsamples and 2 route
     # concats fwd+bwd, the four max-pools of the data-movement configuration fwd+bwd, 3 heads (fused

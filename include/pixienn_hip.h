@@ -250,6 +250,29 @@ int pxh_yolo_forward_train(const float* input, float* output, float* delta, cons
                            float class_scale, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------
+ * SGD with momentum.  The three BLAS calls of ConvLayer::update for one parameter tensor
+ * (include/ConvLayer.h:309-321, include/cuda/ConvLayer.h:388-413) in one pass:
+ *   if apply_decay d += (-decay*batch)*w;  w += (lr/batch)*d;  d *= momentum.
+ * The reference applies the decay to the weights only, not to biases and scales.
+ * ---------------------------------------------------------------------- */
+int pxh_sgd_update(size_t n, float* w, float* d, int batch, float lr, float momentum, float decay,
+                   int apply_decay, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Gradient rescale and clip, the two helpers Layer::backward runs on delta before a layer's own
+ * backward (include/Layer.h:385-397, 479-499; include/cuda/Layer.h:24-39: cublasSnrm2 +
+ * cublasSscal, then constrainGpu) without the host round trip of the norm:
+ *   norm = |x|_2;  if (threshold > 0 && norm > 0 && norm > threshold) x *= threshold/norm;
+ *   if (clip > 0) x = clamp(x, -clip, clip).
+ * norm_out (nullable, device) receives the norm before rescaling.  When nothing has to change,
+ * the tensor is read once and not written.  workspace: pxh_rescale_workspace_bytes() bytes or
+ * NULL for the library's per-device buffer.
+ * ---------------------------------------------------------------------- */
+size_t pxh_rescale_workspace_bytes(void);
+int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* norm_out,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
  * Adam.  include/Adam.cuh:21, include/cuda/Adam.h:49-90.
  * ---------------------------------------------------------------------- */
 

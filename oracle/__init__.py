@@ -295,3 +295,15 @@ def yolo_build_targets(cfg, truths, count, classes, anchors, boxes):
 def adam_update(w, d, m, v, batch, t, lr, beta1, beta2, eps, decay, apply_decay):
     lib().pxo_adam_update(_c_size(w.size), _f(w), _f(d), _f(m), _f(v), int(batch), int(t), _c_float(lr),
                           _c_float(beta1), _c_float(beta2), _c_float(eps), _c_float(decay), int(apply_decay))
+
+
+# ---------------- SGD / gradient rescale ----------------
+def sgd_update(w, d, batch, lr, momentum, decay, apply_decay):
+    lib().pxo_sgd_update(_c_size(w.size), _f(w), _f(d), int(batch), _c_float(lr), _c_float(momentum),
+                         _c_float(decay), int(apply_decay))
+
+
+def rescale_clip(x, threshold, clip):
+    fn = lib().pxo_rescale_clip
+    fn.restype = _c_float
+    return float(fn(_f(x), _c_size(x.size), _c_float(threshold), _c_float(clip)))

@@ -962,3 +962,34 @@ void pxo_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch
         d[i] = 0.0f;
     }
 }
+
+/* ------------------------------------------------------------------ */
+/* SGD with momentum -- include/ConvLayer.h:309-311                    */
+/* ------------------------------------------------------------------ */
+
+/* three BLAS passes: saxpy(-decay*batch, w, d); saxpy(lr/batch, d, w); sscal(momentum, d) */
+void pxo_sgd_update(size_t n, float* w, float* d, int batch, float lr, float momentum, float decay,
+                    int apply_decay)
+{
+    const float a0 = -decay * (float) batch;
+    const float a1 = lr / (float) batch;
+    if (apply_decay) pxo_axpy(n, a0, w, d);
+    pxo_axpy(n, a1, d, w);
+    for (size_t i = 0; i < n; ++i) d[i] = momentum * d[i];
+}
+
+/* ------------------------------------------------------------------ */
+/* gradient rescale + clip -- include/Layer.h:385-397, 479-499         */
+/* ------------------------------------------------------------------ */
+
+/* scaleTensor (when threshold > 0) then constrain (when clip > 0); returns the norm before */
+float pxo_rescale_clip(float* x, size_t n, float threshold, float clip)
+{
+    const float norm = pxo_mag_array(x, n);
+    if (threshold > 0.0f && norm > 0.0f && norm > threshold) {
+        const float scale = threshold / norm;
+        for (size_t i = 0; i < n; ++i) x[i] = scale * x[i];
+    }
+    if (clip > 0.0f) pxo_constrain((int) n, clip, x);
+    return norm;
+}

@@ -139,6 +139,15 @@ void pxo_route_backward(const float* route_delta, float* layer_delta, int batch,
 void pxo_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch, int t, float lr,
                      float beta1, float beta2, float eps, float decay, int apply_decay);
 
+/* ---- SGD with momentum: include/ConvLayer.h:309-311.  Parity unpinned by reference tests (no
+ * numeric test of update() exists); pinned by the closed form of one step and an fp64 recurrence. */
+void pxo_sgd_update(size_t n, float* w, float* d, int batch, float lr, float momentum, float decay,
+                    int apply_decay);
+
+/* ---- gradient rescale + clip: include/Layer.h:385-397, 479-499.  cblas_snrm2's internal summation
+ * is implementation defined; the norm is carried in double here (pxo_mag_array). */
+float pxo_rescale_clip(float* x, size_t n, float threshold, float clip);
+
 #ifdef __cplusplus
 }
 #endif

@@ -49,6 +49,8 @@ SIGNATURES = {
     "pxh_yolo_activate": [P, P, I, I, I, I, P],
     "pxh_yolo_loss": [P, P, P, P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, F, F, F, F, F, P, Z, P],
     "pxh_yolo_forward_train": [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, F, F, F, F, P, Z, P],
+    "pxh_sgd_update": [Z, P, P, I, F, F, F, I, P],
+    "pxh_rescale_clip": [P, Z, F, F, P, P, Z, P],
     "pxh_adam": [I, P, P, P, F, F, F, F, I, P],
     "pxh_adam_update": [Z, P, P, P, P, I, I, F, F, F, F, F, I, P],
 }
@@ -57,6 +59,7 @@ _OTHER_RETURNS = {
     "pxh_abi_version": (I, []),
     "pxh_bn_workspace_bytes": (Z, [I, I, I]),
     "pxh_bn_folded_bytes": (Z, [I]),
+    "pxh_rescale_workspace_bytes": (Z, []),
     "pxh_yolo_workspace_bytes": (Z, [I, I, I, I, I, I]),
     "pxh_debug_fastdiv": (ctypes.c_uint, [ctypes.c_uint, ctypes.c_uint]),
 }

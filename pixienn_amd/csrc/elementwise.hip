@@ -251,6 +251,126 @@ __global__ __launch_bounds__(kBlock) void shortcut_mapped_kernel(uint32_t size, 
     out[oi] = po + pa;
 }
 
+// ---------------------------------------------------------------- SGD with momentum
+// The three BLAS calls of ConvLayer::update (include/ConvLayer.h:309-311, cuda 391-400) in one
+// pass, one fp32 rounding per product and sum as there:
+//   d += (-decay*batch) * w   (weights only);  w += (lr/batch) * d;  d *= momentum
+struct SgdUpdateOp {
+    float* w;
+    float* d;
+    float neg_decay_batch, rate, momentum;
+    int apply_decay;
+    template<int V> struct Regs { Pack<V> w, d; };
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
+    {
+        r.w = ld<V, NT>(w, e);
+        r.d = ld<V, NT>(d, e);
+    }
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> ow, od;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            float g = r.d.v[k];
+            if (apply_decay) {
+                const float l2 = neg_decay_batch * r.w.v[k];
+                g = g + l2;
+            }
+            const float step = rate * g;
+            ow.v[k] = r.w.v[k] + step;
+            od.v[k] = momentum * g;
+        }
+        st<V, NT>(w, e, ow);
+        st<V, NT>(d, e, od);
+    }
+};
+
+// ---------------------------------------------------------------- gradient rescale + clip
+// Layer::backward's two helpers (include/Layer.h:385-397, 479-499; cuda/Layer.h:24-39):
+//   norm = |x|_2;  if (norm > 0 && norm > threshold) x *= threshold / norm;  then clamp to +-clip.
+// Pass 1: a fixed number of workgroups walk the tensor and leave one partial sum of squares each;
+// pass 2: every workgroup adds up those partials (the same order everywhere), derives the factor
+// and rewrites its part of the tensor; when nothing is to be done it leaves without touching it.
+constexpr int kNormBlocks = 2048;     // 8 per compute unit: full occupancy
+constexpr int kNormLoads = 4;      // 128-bit loads in flight per lane
+
+template<int V, bool NT>
+__global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, size_t n_vec, double* partial)
+{
+    __shared__ double slots[kBlock / kWave];
+    const size_t per_step = static_cast<size_t>(kBlock) * V * kNormLoads;
+    double s = 0.0;
+    for (size_t base = static_cast<size_t>(blockIdx.x) * per_step; base < n_vec;
+         base += static_cast<size_t>(gridDim.x) * per_step) {
+        Pack<V> v[kNormLoads];
+#pragma unroll
+        for (int u = 0; u < kNormLoads; ++u) {
+            const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
+            if (e < n_vec) v[u] = ld<V, NT>(x, e);
+        }
+        float a = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kNormLoads; ++u) {
+            const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
+            if (e < n_vec) {
+#pragma unroll
+                for (int k = 0; k < V; ++k) a += v[u].v[k] * v[u].v[k];
+            }
+        }
+        s += static_cast<double>(a);
+    }
+    const double total = block_sum(s, slots);
+    if (threadIdx.x == 0) partial[blockIdx.x] = total;
+}
+
+// One workgroup: the norm from the partial sums, and the factor the rewrite applies.
+__global__ __launch_bounds__(kBlock) void rescale_factor_kernel(const double* partial, int partials, float threshold,
+                                                                float* factor_out, float* norm_out)
+{
+    __shared__ double slots[kBlock / kWave];
+    double s = 0.0;
+    for (int j = threadIdx.x; j < partials; j += kBlock) s += partial[j];
+    const double total = block_sum(s, slots);
+    if (threadIdx.x == 0) {
+        const float norm = static_cast<float>(sqrt(total));
+        if (norm_out) *norm_out = norm;
+        float factor = 1.0f;
+        if (threshold > 0.0f && norm > 0.0f && norm > threshold) factor = threshold / norm;
+        *factor_out = factor;
+    }
+}
+
+// x = clamp(factor * x); leaves without touching the tensor when there is nothing to do.
+// factor_in == nullptr: no rescaling was asked for.
+template<int V, bool NT>
+__global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n_vec, const float* factor_in,
+                                                              float clip)
+{
+    const float factor = factor_in ? *factor_in : 1.0f;
+    if (factor == 1.0f && !(clip > 0.0f)) return;
+    // kNormLoads vectors per lane: a quarter of the workgroups to dispatch when there is nothing to do
+    const size_t base = static_cast<size_t>(blockIdx.x) * kBlock * V * kNormLoads;
+    Pack<V> v[kNormLoads];
+#pragma unroll
+    for (int u = 0; u < kNormLoads; ++u) {
+        const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
+        if (e < n_vec) v[u] = ld<V, NT>(x, e);
+    }
+#pragma unroll
+    for (int u = 0; u < kNormLoads; ++u) {
+        const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
+        if (e < n_vec) {
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                float t = factor == 1.0f ? v[u].v[k] : factor * v[u].v[k];
+                if (clip > 0.0f) t = fminf(clip, fmaxf(-clip, t));
+                v[u].v[k] = t;
+            }
+            st<V, NT>(x, e, v[u]);
+        }
+    }
+}
+
 // ---------------------------------------------------------------- Adam
 // One fp32 rounding per BLAS call of the reference sequence (include/cuda/Adam.h:49-90).
 struct AdamUpdateOp {
@@ -482,6 +602,61 @@ int pxh_shortcut_backward(float* delta, const float* pre_activation, float* from
     });
     if (!known) return fail_invalid("pxh_shortcut_backward: unknown activation %d", activation);
     return rc;
+}
+
+int pxh_sgd_update(size_t n, float* w, float* d, int batch, float lr, float momentum, float decay, int apply_decay,
+                   void* stream)
+{
+    if (batch <= 0) return fail_invalid("pxh_sgd_update: batch must be positive");
+    if ((!w || !d) && n) return fail_invalid("pxh_sgd_update: null pointer");
+    const SgdUpdateOp op{ w, d, -decay * static_cast<float>(batch), lr / static_cast<float>(batch), momentum,
+                          apply_decay };
+    return launch_stream("pxh_sgd_update", n, aligned16(w) && aligned16(d), 16, op, as_stream(stream));
+}
+
+size_t pxh_rescale_workspace_bytes(void)
+{
+    return kNormBlocks * sizeof(double) + 256;      // partial sums, then the factor
+}
+
+int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* norm_out, void* workspace,
+                     size_t workspace_bytes, void* stream)
+{
+    if (!x && n) return fail_invalid("pxh_rescale_clip: null pointer");
+    if (n == 0) return PXH_OK;
+    const bool rescale = threshold > 0.0f || norm_out != nullptr;
+    if (!rescale && !(clip > 0.0f)) return PXH_OK;
+    void* ws = nullptr;
+    int rc = resolve_workspace(workspace, workspace_bytes, pxh_rescale_workspace_bytes(), &ws);
+    if (rc) return rc;
+    double* partial = static_cast<double*>(ws);
+    float* factor = reinterpret_cast<float*>(partial + kNormBlocks);
+    hipStream_t s = as_stream(stream);
+    const bool vec = aligned16(x) && n % 4 == 0;
+    const int v = vec ? 4 : 1;
+    // a tensor past the last-level cache gains nothing from being kept for the next pass
+    const bool nt = vec && n * 4 >= kStreamingBytes;
+    if (rescale) {
+        const size_t per_step = static_cast<size_t>(kBlock) * v * kNormLoads;
+        const size_t want = (n + per_step - 1) / per_step;
+        const int blocks = static_cast<int>(want < static_cast<size_t>(kNormBlocks) ? want : kNormBlocks);
+        if (nt) hipLaunchKernelGGL((sumsq_partial_kernel<4, true>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
+        else if (vec) hipLaunchKernelGGL((sumsq_partial_kernel<4, false>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
+        else hipLaunchKernelGGL((sumsq_partial_kernel<1, false>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
+        rc = check_launch("pxh_rescale_clip");
+        if (rc) return rc;
+        hipLaunchKernelGGL(rescale_factor_kernel, dim3(1), dim3(kBlock), 0, s, partial, blocks, threshold, factor,
+                           norm_out);
+        rc = check_launch("pxh_rescale_clip");
+        if (rc) return rc;
+        if (!(threshold > 0.0f) && !(clip > 0.0f)) return PXH_OK;      // only the norm was asked for
+    }
+    const float* factor_in = threshold > 0.0f ? factor : nullptr;
+    const dim3 grid(grid_for(n, static_cast<size_t>(kBlock) * v * kNormLoads));
+    if (nt) hipLaunchKernelGGL((rescale_clip_kernel<4, true>), grid, dim3(kBlock), 0, s, x, n, factor_in, clip);
+    else if (vec) hipLaunchKernelGGL((rescale_clip_kernel<4, false>), grid, dim3(kBlock), 0, s, x, n, factor_in, clip);
+    else hipLaunchKernelGGL((rescale_clip_kernel<1, false>), grid, dim3(kBlock), 0, s, x, n, factor_in, clip);
+    return check_launch("pxh_rescale_clip");
 }
 
 int pxh_adam(int n, float* x, const float* m, const float* v, float beta1, float beta2, float rate, float eps, int t,

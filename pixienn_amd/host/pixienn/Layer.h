@@ -92,8 +92,10 @@ public:
     int width = 0, height = 0;      // network input size
     int classes = 0;
 
-    // optimiser (reference: Model<D>::adam*, learningRate, decay, include/Model.h)
-    float learningRate = 1e-3f, decay = 5e-4f;
+    // optimiser (reference: Model<D>::adam*, learningRate, momentum, decay, include/Model.h);
+    // the shipped presets train with SGD + momentum (adam.enabled: False)
+    bool adamEnabled = false;
+    float learningRate = 1e-3f, momentum = 0.9f, decay = 5e-4f;
     float adamBeta1 = 0.9f, adamBeta2 = 0.999f, adamEpsilon = 1e-8f;
     int timeStep = 1;               // Adam's t
     int updateBatch = 1;            // images a parameter update averages over (batch * subdivisions)
@@ -161,10 +163,14 @@ public:
 
     // delta_ holds dL/d(output) on entry; a layer turns it into dL/d(input) and ACCUMULATES that
     // into *grad (nullptr for the first layer).
+    // First the reference's two helpers on delta_ (include/Layer.h:385-397): rescale to a norm
+    // threshold, then clamp; one fused call here.
     virtual void backward(const V& /*input*/, V* /*grad*/)
     {
-        if (gradientClipping_) PX_HIP_CHECK(pxh_constrain(static_cast<int>(delta_.size()), gradientClipValue_,
-                                                          delta_.data(), stream()));
+        if (gradientRescaling_ || gradientClipping_)
+            PX_HIP_CHECK(pxh_rescale_clip(delta_.data(), delta_.size(), gradientRescaling_ ? gradientThreshold_ : 0.0f,
+                                          gradientClipping_ ? gradientClipValue_ : 0.0f, nullptr, nullptr, 0,
+                                          stream()));
     }
 
     virtual void update() {}
@@ -187,6 +193,7 @@ public:
     V& delta() noexcept { return delta_; }
 
     void setGradientClipping(bool on, float value) { gradientClipping_ = on; gradientClipValue_ = value; }
+    void setGradientRescaling(bool on, float threshold) { gradientRescaling_ = on; gradientThreshold_ = threshold; }
 
 protected:
     // Sets the output shape and allocates output_ (and delta_, which inference never touches,
@@ -224,8 +231,8 @@ private:
     Properties props_;
     int batch_, channels_, height_, width_, index_, inputs_;
     int outChannels_ = 0, outHeight_ = 0, outWidth_ = 0, outputs_ = 0;
-    bool gradientClipping_ = false;
-    float gradientClipValue_ = 1.0f;
+    bool gradientClipping_ = false, gradientRescaling_ = false;
+    float gradientClipValue_ = 1.0f, gradientThreshold_ = 0.0f;
 };
 
 }   // px::hip

@@ -137,13 +137,23 @@ public:
         }
     }
 
-    // Adam on the biases and scales (the delegated convolution updates its own weights with
-    // the same Adam object: reference include/cuda/ConvLayer.h:388-413).
+    // Adam or SGD with momentum on the biases and scales, neither with weight decay (the
+    // delegated convolution updates its own weights the same way, with decay: reference
+    // include/cuda/ConvLayer.h:362-413).
     void update() override
     {
-        const Adam adam(context());
-        adam.update(biases_, biasUpdates_, biasM_, biasV_, false);
-        if (batchNorm_) adam.update(scales_, scaleUpdates_, scaleM_, scaleV_, false);
+        const auto& c = context();
+        if (c.adamEnabled) {
+            const Adam adam(c);
+            adam.update(biases_, biasUpdates_, biasM_, biasV_, false);
+            if (batchNorm_) adam.update(scales_, scaleUpdates_, scaleM_, scaleV_, false);
+        } else {
+            PX_HIP_CHECK(pxh_sgd_update(biases_.size(), biases_.data(), biasUpdates_.data(), c.updateBatch,
+                                        c.learningRate, c.momentum, c.decay, 0, stream()));
+            if (batchNorm_)
+                PX_HIP_CHECK(pxh_sgd_update(scales_.size(), scales_.data(), scaleUpdates_.data(), c.updateBatch,
+                                            c.learningRate, c.momentum, c.decay, 0, stream()));
+        }
         foldedValid_ = false;
     }
 

@@ -290,3 +290,16 @@ def adam_update(w, d, m, v, batch, t, lr, beta1=0.9, beta2=0.999, eps=1e-8, deca
     _chk_all(w, d, m, v)
     call("pxh_adam_update", w.numel(), ptr(w), ptr(d), ptr(m), ptr(v), int(batch), int(t), float(lr), float(beta1),
          float(beta2), float(eps), float(decay), int(bool(apply_decay)), _stream())
+
+
+def sgd_update(w, d, batch, lr, momentum, decay=0.0, apply_decay=False):
+    """include/ConvLayer.h:309-311 of the reference for one parameter tensor."""
+    _chk_all(w, d)
+    call("pxh_sgd_update", w.numel(), ptr(w), ptr(d), int(batch), float(lr), float(momentum), float(decay),
+         int(bool(apply_decay)), _stream())
+
+
+def rescale_clip(x, threshold=0.0, clip=0.0, norm_out=None):
+    """Gradient rescale to a norm threshold, then clamp (include/Layer.h:385-397 of the reference)."""
+    _chk_all(x, norm_out)
+    call("pxh_rescale_clip", ptr(x), x.numel(), float(threshold), float(clip), ptr(norm_out), None, 0, _stream())

@@ -337,8 +337,19 @@ void trainingChecks()
         expectClose("yolo7 positives counted", Host{ gs[6] }, Host{ stats[6] }, 0.0, 1.0);
     }
 
-    // ---- backward, last layer first; every layer accumulates into its predecessor's delta
-    net.yolo7->backward(net.conv6->output(), &net.conv6->delta());
+    // ---- backward, last layer first; every layer accumulates into its predecessor's delta.
+    // The head rescales its delta to a norm threshold and clamps it first.
+    {
+        Host want = yoloDelta;
+        const float norm = pxo_rescale_clip(want.data(), want.size(), 0.0f, 0.0f);
+        want = yoloDelta;
+        pxo_rescale_clip(want.data(), want.size(), 0.5f * norm, 0.05f);
+        net.yolo7->setGradientRescaling(true, 0.5f * norm);
+        net.yolo7->setGradientClipping(true, 0.05f);
+        net.yolo7->backward(net.conv6->output(), &net.conv6->delta());
+        yoloDelta = net.yolo7->delta().asVector();
+        expectClose("yolo7 delta rescaled and clamped", yoloDelta, want, 1e-6, 1e-6);
+    }
     expectExact("yolo7 backward: grad += delta", net.conv6->delta().asVector(), yoloDelta);
 
     {   // conv6: bias backward, then (identity convolution) grad += delta
@@ -410,7 +421,17 @@ void trainingChecks()
     }
     net.conv0->backward(input, nullptr);
 
-    // ---- update: Adam on conv2's scales
+    // ---- update: SGD with momentum on conv0's biases, then Adam on conv2's scales
+    {
+        Host w = net.conv0->biases().asVector(), d = net.conv0->biasUpdates().asVector();
+        pxo_sgd_update(C, w.data(), d.data(), net.ctx.updateBatch, net.ctx.learningRate, net.ctx.momentum,
+                       net.ctx.decay, 0);
+        net.ctx.adamEnabled = false;
+        net.conv0->update();
+        expectClose("conv0 SGD update of the biases", net.conv0->biases().asVector(), w, 1e-6, 1e-3);
+        expectClose("conv0 bias updates keep the momentum term", net.conv0->biasUpdates().asVector(), d, 1e-6, 1e-3);
+    }
+    net.ctx.adamEnabled = true;
     {
         Host w = net.conv2->scales().asVector(), d = net.conv2->scaleUpdates().asVector();
         Host m(C, 0.0f), v(C, 0.0f);

@@ -282,3 +282,49 @@ def test_adam_step_reference_signature(ops):
     c1 = float(F(1) - np.power(F(0.9), F(7))); c2 = float(F(1) - np.power(F(0.999), F(7)))
     want = x0 + 1e-3 * (m.astype(np.float64) / c1) / (np.sqrt(v.astype(np.float64) / c2) + 1e-8)
     assert_close(host(gx), want, 2e-6, 1e-3, "adamGpu")
+
+
+# ---------------------------------------------------------------- SGD, gradient rescale + clip
+@pytest.mark.parametrize("n", [1, 7, 1024, 4099, 1 << 20])
+def test_sgd_update_matches_oracle(ops, oracle, n):
+    w0 = wl.normal(3300 + n % 97, n, std=0.02); d0 = wl.normal(3301 + n % 97, n, std=0.5)
+    for apply_decay in (True, False):
+        w = w0.copy(); d = d0.copy()
+        gw = gpu(w0); gd = gpu(d0)
+        for step in range(3):
+            oracle.sgd_update(w, d, 16, 1e-3, 0.9, 5e-4, apply_decay)
+            ops.sgd_update(gw, gd, 16, 1e-3, 0.9, 5e-4, apply_decay)
+            # the next step accumulates a fresh gradient on top of the momentum term
+            g = wl.normal(3310 + step, n, std=0.5)
+            d += g
+            gd += gpu(g)
+        assert_close(host(gw), w, 1e-6, 1e-3, "sgd weights n=%d decay=%s" % (n, apply_decay))
+        assert_close(host(gd), d, 1e-6, 1e-3, "sgd updates n=%d decay=%s" % (n, apply_decay))
+
+
+@pytest.mark.parametrize("n", [5, 1024, 4 * 1024 * 1024 + 4, 1234567])
+@pytest.mark.parametrize("mode", ["rescale", "clip", "both", "below", "none"])
+def test_rescale_clip_matches_oracle(ops, oracle, n, mode):
+    import torch
+    x0 = wl.normal(3400 + n % 89, n)
+    norm_true = float(np.sqrt(np.square(x0.astype(np.float64)).sum()))
+    threshold = {"rescale": 0.5 * norm_true, "both": 0.25 * norm_true, "below": 2.0 * norm_true}.get(mode, 0.0)
+    clip = {"clip": 0.7, "both": 0.3 * 0.25}.get(mode, 0.0)
+    want = x0.copy()
+    norm_w = oracle.rescale_clip(want, threshold, clip)
+    gx = gpu(x0)
+    gnorm = torch.full((1,), -1.0, device="cuda")
+    ops.rescale_clip(gx, threshold, clip, norm_out=gnorm)
+    assert abs(float(host(gnorm)[0]) - norm_w) <= 1e-6 * norm_w
+    assert abs(norm_w - norm_true) <= 1e-6 * norm_true
+    if mode in ("below", "none"):
+        assert_bit_exact(host(gx), x0, "untouched when nothing is to be done")
+    else:
+        # the factor is threshold / norm with the norm good to 1e-7: 1e-6 of the value
+        assert_close(host(gx), want, 1e-6, 1e-6, "rescale/clip %s n=%d" % (mode, n))
+    if clip > 0:
+        assert np.abs(host(gx)).max() <= np.float32(clip)
+    # without norm_out the result is the same
+    gy = gpu(x0)
+    ops.rescale_clip(gy, threshold, clip)
+    assert_bit_exact(host(gy), host(gx), "with and without norm_out")

@@ -517,3 +517,61 @@ def test_adam_10_steps_vs_fp64_l2(oracle):
     assert np.max(np.abs(w - w64) / np.maximum(np.abs(w64), 1e-2)) < 1e-5
     # a decoupled-decay (AdamW) recurrence is measurably different: the restatement is not that
     assert np.max(np.abs(w - w64)) < 1e-6
+
+
+def test_sgd_closed_form_and_fp64_recurrence(oracle):
+    """The reference holds no numeric test of ConvLayer::update: one step against its closed form,
+    ten steps against the same recurrence carried in fp64."""
+    rng = np.random.default_rng(11)
+    n = 4096
+    w0 = rng.normal(0, 0.02, n).astype(F); g = rng.normal(0, 0.5, (10, n)).astype(F)
+    lr, mom, decay, batch = 1e-3, 0.9, 5e-4, 16
+    w = w0.copy(); d = g[0].copy()
+    oracle.sgd_update(w, d, batch, lr, mom, decay, True)
+    d_eff = g[0].astype(np.float64) - decay * batch * w0.astype(np.float64)
+    assert np.allclose(w, w0 + lr / batch * d_eff, rtol=1e-6, atol=1e-9)
+    assert np.allclose(d, mom * d_eff, rtol=1e-6, atol=1e-9)
+    # without decay the weights do not enter the update
+    w2 = w0.copy(); d2 = g[0].copy()
+    oracle.sgd_update(w2, d2, batch, lr, mom, decay, False)
+    assert np.allclose(w2, w0 + lr / batch * g[0].astype(np.float64), rtol=1e-6, atol=1e-9)
+    assert np.allclose(d2, mom * g[0].astype(np.float64), rtol=1e-6, atol=1e-9)
+    # ten steps
+    w = w0.copy(); d = np.zeros(n, F)
+    w64 = w0.astype(np.float64); d64 = np.zeros(n)
+    for t in range(10):
+        d += g[t]; d64 += g[t]
+        oracle.sgd_update(w, d, batch, lr, mom, decay, True)
+        d64 = d64 - decay * batch * w64
+        w64 = w64 + lr / batch * d64
+        d64 = mom * d64
+    assert np.allclose(w, w64, rtol=1e-5, atol=1e-8)
+    assert np.allclose(d, d64, rtol=1e-5, atol=2e-6)      # sums of O(1) terms rounded to fp32 ten times
+
+
+def test_rescale_clip_invariants(oracle):
+    rng = np.random.default_rng(12)
+    x0 = rng.normal(0, 1.0, 10000).astype(F)
+    norm = np.sqrt(np.square(x0.astype(np.float64)).sum())
+    # above the threshold: the result has the threshold as its norm and the direction of x
+    x = x0.copy()
+    got = oracle.rescale_clip(x, 0.5 * norm, 0.0)
+    assert abs(got - norm) <= 1e-6 * norm
+    assert abs(np.sqrt(np.square(x.astype(np.float64)).sum()) - 0.5 * norm) <= 1e-6 * norm
+    assert np.allclose(x, 0.5 * x0, rtol=1e-6)
+    # below the threshold, or no threshold: untouched
+    for thr in (2.0 * norm, 0.0):
+        x = x0.copy()
+        oracle.rescale_clip(x, thr, 0.0)
+        assert np.array_equal(x, x0)
+    # clip only: clamp
+    x = x0.copy()
+    oracle.rescale_clip(x, 0.0, 0.7)
+    assert np.array_equal(x, np.clip(x0, -0.7, 0.7))
+    # both: rescale first, then clamp (the order of Layer::backward)
+    x = x0.copy()
+    oracle.rescale_clip(x, 0.5 * norm, 0.3)
+    assert np.allclose(x, np.clip(0.5 * x0, -0.3, 0.3), rtol=1e-6)
+    # zero tensor: the norm test keeps it untouched
+    z = np.zeros(8, F)
+    assert oracle.rescale_clip(z, 1.0, 0.0) == 0.0 and not z.any()
