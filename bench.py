@@ -35,7 +35,7 @@ EPILOGUE_ACTS = ["leaky", "mish", "logistic"]
 # HBM bytes per launch of the leaky epilogue kernel relative to its algorithmic bytes, from two
 # rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of this script, each scaled by what the counter
 # reads for the 2 x 512 MiB plain copy below (profiles/epilogue_sweep_hbm_traffic.txt)
-EPILOGUE_TRAFFIC_RATIO = 0.9998
+EPILOGUE_TRAFFIC_RATIO = 0.9999
 
 
 def log(*a):
