@@ -1,0 +1,72 @@
+"""The entry points inside a HIP graph: a layer sequence is captured once and replayed several
+times on new data, with eager work and synchronisations in between; every replay must give
+exactly what the same calls give when launched eagerly."""
+import numpy as np
+import pytest
+
+from pixienn_amd import workloads as wl
+from util import F, gpu, host
+
+pytestmark = pytest.mark.gpu
+
+
+def test_layer_sequence_in_a_graph_matches_eager():
+    import torch
+    from pixienn_amd import ops
+    N, C, S, K = 4, 128, 38, 80
+    dev = "cuda"
+    scale, bias, rmean0, rvar0 = (gpu(a) for a in wl.bn_params(9000, C))
+    truths_np, counts_np = wl.yolo_truths(9001, N)
+    truths, counts = gpu(truths_np), gpu(counts_np)
+    mask = wl.YOLOV3_MASKS[38]
+
+    # static buffers of the captured sequence
+    x = torch.zeros((N, C, S, S), device=dev); d_in = torch.zeros_like(x)
+    head_in = torch.zeros((N, 3 * (K + 5), S, S), device=dev)
+    buf = dict(y=torch.empty_like(x), mean=torch.zeros(C, device=dev), var=torch.zeros(C, device=dev),
+               rmean=rmean0.clone(), rvar=rvar0.clone(), su=torch.zeros(C, device=dev), bu=torch.zeros(C, device=dev),
+               d=torch.empty_like(x), pool=torch.empty((N, C, S // 2, S // 2), device=dev),
+               idx=torch.empty((N, C, S // 2, S // 2), device=dev, dtype=torch.int32),
+               up=torch.empty_like(x), head_out=torch.empty_like(head_in), head_delta=torch.empty_like(head_in),
+               stats=torch.zeros(12, device=dev), cost=torch.zeros(1, device=dev), norm=torch.zeros(1, device=dev),
+               w=torch.zeros(C * 9, device=dev), wd=torch.zeros(C * 9, device=dev))
+
+    def sequence(b):
+        ops.bn_train_act_forward(x, b["y"], b["mean"], b["var"], b["rmean"], b["rvar"], scale, bias, "leaky")
+        ops.maxpool_forward(b["y"], b["pool"], b["idx"], 2, 2, 1)
+        ops.upsample_forward(b["pool"], b["up"], 2, 1.0)
+        b["d"].copy_(d_in)
+        ops.rescale_clip(b["d"], 50.0, 0.5, norm_out=b["norm"])
+        ops.bn_act_backward(b["d"], x, b["mean"], b["var"], scale, bias, b["su"], b["bu"], "leaky")
+        ops.yolo_forward_train(head_in, b["head_out"], b["head_delta"], truths, counts, truths.shape[1], mask,
+                               wl.YOLOV3_ANCHORS, b["stats"], b["cost"], N, K, S, S, 608, 608, 0.7, 1.0, 1.0, 2.0,
+                               0.1, 1.0)
+        b["wd"].add_(1.0)
+        ops.sgd_update(b["w"], b["wd"], 16, 1e-3, 0.9, 5e-4, True)
+
+    def load(step):
+        x.copy_(gpu(wl.normal(9100 + step, tuple(x.shape))))
+        d_in.copy_(gpu(wl.normal(9200 + step, tuple(x.shape))))
+        head_in.copy_(gpu(wl.normal(9300 + step, tuple(head_in.shape), std=2.0)))
+
+    load(0)
+    sequence({k: v.clone() for k, v in buf.items()})       # first call: the library allocates its workspace
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sequence(buf)
+    eager = {k: v.clone() for k, v in buf.items()}
+    for k in ("rmean", "rvar"):
+        eager[k].copy_({"rmean": rmean0, "rvar": rvar0}[k]); buf[k].copy_(eager[k])
+    for k in ("su", "bu", "w", "wd"):
+        eager[k].zero_(); buf[k].zero_()
+    for step in range(1, 4):
+        load(step)
+        graph.replay()
+        torch.cuda.synchronize()
+        sequence(eager)                                      # eager work between the replays
+        torch.cuda.synchronize()
+        for k in buf:
+            assert torch.equal(buf[k], eager[k]), "replay %d differs from eager in %s" % (step, k)
+    assert float(buf["stats"][6]) > 0 and float(buf["norm"][0]) > 50.0
