@@ -145,8 +145,9 @@ def run_epilogue_step(ops, shapes, events=None, torch=None, raw=False):
             events.append((act, a, b))
 
 
-def measure_extras(torch, ops, wl, timer):
+def measure_extras(torch, ops, wl, timer, capi):
     """The other kernels of the path at the baseline's shapes.  Returns (rows, ms_per_batch)."""
+    import numpy as np
     dev = torch.device("cuda:0")
     rows = []
 
@@ -238,6 +239,27 @@ def measure_extras(torch, ops, wl, timer):
             cost, NB, 80, s, s, 608, 608, 0.7, 1.0, 1.0, 2.0, 0.1, 1.0), 20, rotate=rot)
         add("yolo_decode+delta+cost", "%dx255x%d^2" % (NB, s), 12 * e, ms_t, "fused 12B/elem")
         head_ms[s] = (ms_d, ms_t)
+        if s == 76:
+            # detections of the decoded head at a confidence threshold of 0.5: the objectness row of every
+            # slot, the box and class rows of the slots that pass (about half of them on these logits)
+            cap = 1 << 22
+            rec = torch.empty((cap, 8), device=dev, dtype=torch.int32)
+            cnt = torch.zeros(1, device=dev, dtype=torch.int32)
+            m = np.ascontiguousarray(wl.YOLOV3_MASKS[s], dtype=np.int32)
+            a = np.ascontiguousarray(wl.YOLOV3_ANCHORS, dtype=np.int32)
+
+            def detect(i):
+                capi.call("pxh_yolo_detections", out[i].data_ptr(), NB, m.ctypes.data, len(m), a.ctypes.data,
+                          len(a) // 2, 80, s, s, 608, 608, 0, 0, 0.5, rec.data_ptr(), cap, cnt.data_ptr(),
+                          torch.cuda.current_stream().cuda_stream)
+
+            ms_det = timer.time(detect, 10, rotate=rot)
+            found = int(cnt.item())
+            passing = float((out[0].view(NB, 3, 85, s * s)[:, :, 4] >= 0.5).float().mean())
+            slots = NB * 3 * s * s
+            add("yolo_detections(thr .5)", "%dx255x%d^2" % (NB, s), 4 * slots * (1 + passing * 84) + 32 * min(found, cap),
+                ms_det, "%d records; %.0f%% of the slots pass" % (found, 100 * passing))
+            del rec
         del xin, out, dl
     # ---- BN training forward / backward (config 4): batch 16 @608, 13 shapes
     bn_ms = {}
@@ -436,7 +458,7 @@ def main():
 
     extras, ms_batch = (None, None)
     if not args.no_extras:
-        extras, ms_batch = measure_extras(torch, ops, wl, timer)
+        extras, ms_batch = measure_extras(torch, ops, wl, timer, capi)
         for r in extras:
             log("%-24s %-18s %9.1f MB %8.4f ms %8.1f GB/s  %4.1f%%  %s"
                 % (r["kernel"], r["shape"], r["MB"], r["ms"], r["GBps"], 100 * r["frac"], r["note"]))

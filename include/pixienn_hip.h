@@ -233,6 +233,27 @@ int pxh_yolo_loss(const float* output, float* delta, const float* truths, const 
                   float noobject_scale, float class_scale, void* workspace, size_t workspace_bytes,
                   void* stream);
 
+/* Detections of a decoded head without copying the head to the host: YoloLayer::addDetects
+ * (include/YoloLayer.h:601-698) as a thresholded compaction on the device.  A slot passes when its
+ * objectness is not below `threshold`; each of its classes with objectness * probability >=
+ * threshold gives one record.  image_width/height > 0 selects scaledYoloBox (integer pixel box of
+ * the letterboxed image, x/y = left/top), else yoloBox(...).rect() (relative left, top, w, h).
+ * *count (device int, cleared by the call) receives the number found, which may exceed `capacity`;
+ * only the first `capacity` places are written.  Records are in no particular order; `order` is the
+ * position in the reference's emission order (image, cell, mask, class), sort by it to restore it.
+ * No counterpart among the reference's device kernels: its CUDA path copies the head to the host. */
+typedef struct pxh_detection {
+    float x, y, w, h;
+    float prob;
+    int batch;
+    int class_index;
+    unsigned order;
+} pxh_detection;
+int pxh_yolo_detections(const float* predictions, int batch, const int* host_masks, int mask_count,
+                        const int* host_anchors, int anchor_count, int classes, int width, int height,
+                        int net_width, int net_height, int image_width, int image_height,
+                        float threshold, pxh_detection* out, int capacity, int* count, void* stream);
+
 size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int width, int height,
                                 int max_truth);
 

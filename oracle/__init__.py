@@ -307,3 +307,18 @@ def rescale_clip(x, threshold, clip):
     fn = lib().pxo_rescale_clip
     fn.restype = _c_float
     return float(fn(_f(x), _c_size(x.size), _c_float(threshold), _c_float(clip)))
+
+
+# ---------------- detections ----------------
+DETECTION_DTYPE = np.dtype([("x", "f4"), ("y", "f4"), ("w", "f4"), ("h", "f4"), ("prob", "f4"), ("batch", "i4"),
+                            ("class_index", "i4"), ("order", "u4")])
+
+
+def yolo_detections(cfg, predictions, threshold, capacity, image_width=0, image_height=0):
+    """Returns (records in the reference's emission order, total number found)."""
+    out = np.zeros(max(1, capacity), DETECTION_DTYPE)
+    fn = lib().pxo_yolo_detections
+    fn.restype = _c_int
+    found = fn(ctypes.byref(cfg), _f(predictions), _c_float(threshold), int(image_width), int(image_height),
+               out.ctypes.data_as(ctypes.c_void_p), int(capacity))
+    return out[:min(found, capacity)], int(found)

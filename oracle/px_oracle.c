@@ -993,3 +993,84 @@ float pxo_rescale_clip(float* x, size_t n, float threshold, float clip)
     if (clip > 0.0f) pxo_constrain((int) n, clip, x);
     return norm;
 }
+
+/* ------------------------------------------------------------------ */
+/* detections -- include/YoloLayer.h:601-698                           */
+/* ------------------------------------------------------------------ */
+
+/* YoloLayer.h:601-634: box in pixels of a w x h image that was letterboxed into the network input.
+ * The float expressions are converted to int by std::max<int> / std::min<int> (truncation). */
+static void yolo_scaled_box(const pxo_yolo_cfg* g, const float* p, int anchor, size_t index, int i, int j,
+                            int w, int h, float box[4])
+{
+    const size_t stride = (size_t) g->width * g->height;
+    const int netW = g->net_width, netH = g->net_height;
+    int newW, newH;
+    if (((float) netW / w) < ((float) netH / h)) {
+        newW = netW;
+        newH = (h * netW) / w;
+    } else {
+        newH = netH;
+        newW = (w * netH) / h;
+    }
+    float x = ((float) i + p[index]) / (float) g->width;
+    x = (x - (float) (netW - newW) / 2.0f / (float) netW) / ((float) newW / (float) netW);
+    float y = ((float) j + p[index + stride]) / (float) g->height;
+    y = (y - (float) (netH - newH) / 2.0f / (float) netH) / ((float) newH / (float) netH);
+    float width = expf(p[index + 2 * stride]) * (float) g->anchors[2 * anchor] / (float) netW;
+    width *= (float) netW / (float) newW;
+    float height = expf(p[index + 3 * stride]) * (float) g->anchors[2 * anchor + 1] / (float) netH;
+    height *= (float) netH / (float) newH;
+    int left = (int) ((x - width / 2) * (float) w);
+    if (left < 0) left = 0;
+    int right = (int) ((x + width / 2) * (float) w);
+    if (right > w - 1) right = w - 1;
+    int top = (int) ((y - height / 2) * (float) h);
+    if (top < 0) top = 0;
+    int bottom = (int) ((y + height / 2) * (float) h);
+    if (bottom > h - 1) bottom = h - 1;
+    box[0] = (float) left; box[1] = (float) top;
+    box[2] = (float) (right - left); box[3] = (float) (bottom - top);
+}
+
+int pxo_yolo_detections(const pxo_yolo_cfg* g, const float* predictions, float threshold,
+                        int image_width, int image_height, pxo_detection* out, int capacity)
+{
+    const int scaled = image_width > 0 && image_height > 0;
+    int area = g->width * g->height;
+    if (area < 1) area = 1;
+    int found = 0;
+    for (int b = 0; b < g->batch; ++b)
+        for (int i = 0; i < area; ++i) {
+            const int row = i / g->width, col = i % g->width;
+            for (int n = 0; n < g->num_masks; ++n) {
+                const float objectness = predictions[yolo_entry(g, b, n * area + i, 4)];
+                if (objectness < threshold) continue;
+                const size_t box_index = yolo_entry(g, b, n * area + i, 0);
+                float box[4];
+                if (scaled) {
+                    yolo_scaled_box(g, predictions, g->mask[n], box_index, col, row, image_width, image_height, box);
+                } else {
+                    /* yoloBox(...).rect(): left/top fall back to the centre for a non-positive size */
+                    float c[4];
+                    yolo_box(g, predictions, g->mask[n], box_index, col, row, c);
+                    box[0] = c[2] > 0.0f ? c[0] - c[2] / 2.0f : c[0];
+                    box[1] = c[3] > 0.0f ? c[1] - c[3] / 2.0f : c[1];
+                    box[2] = c[2]; box[3] = c[3];
+                }
+                for (int j = 0; j < g->classes; ++j) {
+                    const float prob = objectness * predictions[yolo_entry(g, b, n * area + i, 5 + j)];
+                    if (prob >= threshold) {
+                        if (found < capacity) {
+                            pxo_detection* d = out + found;
+                            d->x = box[0]; d->y = box[1]; d->w = box[2]; d->h = box[3];
+                            d->prob = prob; d->batch = b; d->class_index = j;
+                            d->order = (unsigned) ((((size_t) b * area + i) * g->num_masks + n) * g->classes + j);
+                        }
+                        ++found;
+                    }
+                }
+            }
+        }
+    return found;
+}

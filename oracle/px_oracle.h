@@ -139,6 +139,21 @@ void pxo_route_backward(const float* route_delta, float* layer_delta, int batch,
 void pxo_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch, int t, float lr,
                      float beta1, float beta2, float eps, float decay, int apply_decay);
 
+/* ---- detections of a decoded head: include/YoloLayer.h:601-698 (addDetects, yoloBox, scaledYoloBox).
+ * image_width/height > 0 selects the letterbox-corrected integer pixel boxes, else the relative
+ * DarkBox rectangle (left, top, w, h).  Records come in the reference's order: image, cell, mask,
+ * class.  Returns the number found; at most `capacity` are written.  Parity unpinned by reference
+ * tests (they need downloaded weights); pinned by hand-computed cases and brute force. */
+typedef struct pxo_detection {
+    float x, y, w, h;
+    float prob;
+    int batch;
+    int class_index;
+    unsigned order;      /* ((image*area + cell)*masks + mask)*classes + class */
+} pxo_detection;
+int pxo_yolo_detections(const pxo_yolo_cfg* cfg, const float* predictions, float threshold,
+                        int image_width, int image_height, pxo_detection* out, int capacity);
+
 /* ---- SGD with momentum: include/ConvLayer.h:309-311.  Parity unpinned by reference tests (no
  * numeric test of update() exists); pinned by the closed form of one step and an fp64 recurrence. */
 void pxo_sgd_update(size_t n, float* w, float* d, int batch, float lr, float momentum, float decay,

@@ -51,6 +51,7 @@ SIGNATURES = {
     "pxh_yolo_forward_train": [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, F, F, F, F, P, Z, P],
     "pxh_sgd_update": [Z, P, P, I, F, F, F, I, P],
     "pxh_rescale_clip": [P, Z, F, F, P, P, Z, P],
+    "pxh_yolo_detections": [P, I, P, I, P, I, I, I, I, I, I, I, I, F, P, I, P, P],
     "pxh_adam": [I, P, P, P, F, F, F, F, I, P],
     "pxh_adam_update": [Z, P, P, P, P, I, I, F, F, F, F, F, I, P],
 }

@@ -700,6 +700,137 @@ __global__ __launch_bounds__(kBlock) void yolo_patch_kernel(PatchArgs a)
     if (blockIdx.x < 13) finish_statistic(blockIdx.x, a.cls, slots);
 }
 
+// ---------------------------------------------------------------- detections
+// Thresholded compaction of a decoded head (include/YoloLayer.h:601-698): one lane per slot; a slot
+// whose objectness passes walks its class rows, and the lanes of a wave that found a detection in
+// the same class step reserve their output places with one atomic between them.  The records
+// carry their position in the reference's emission order, so sorting by it restores that order.
+struct DetectArgs {
+    const float* pred;
+    pxh_detection* out;
+    int* count;
+    int capacity;
+    float threshold;
+    int image_width, image_height;    // > 0: letterbox-corrected pixel boxes
+    uint32_t slots;                   // batch * masks * area
+    FastDiv by_area;
+};
+
+__global__ __launch_bounds__(kBlock) void yolo_detect_kernel(DetectArgs a, YoloParams p)
+{
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    const bool live = t < a.slots;
+    const uint32_t slot = live ? t : 0;
+    uint32_t bn, cell, b, n;
+    a.by_area.divmod(slot, bn, cell);
+    p.by_masks.divmod(bn, b, n);
+    const int area = p.area;
+    const size_t base = static_cast<size_t>(bn) * (p.classes + 5) * area + cell;
+    const float objectness = live ? a.pred[base + 4 * static_cast<size_t>(area)] : -INFINITY;
+    bool pass = live && !(objectness < a.threshold);
+    float bx = 0, by = 0, bw = 0, bh = 0;
+    if (pass) {
+        uint32_t row, col;
+        p.by_width.divmod(cell, row, col);
+        const int anchor = p.masks[n];
+        const float p0 = a.pred[base], p1 = a.pred[base + area], p2 = a.pred[base + 2 * static_cast<size_t>(area)],
+                    p3 = a.pred[base + 3 * static_cast<size_t>(area)];
+        if (a.image_width > 0 && a.image_height > 0) {
+            const int w = a.image_width, h = a.image_height;
+            const int netW = p.net_width, netH = p.net_height;
+            int newW, newH;
+            if ((static_cast<float>(netW) / w) < (static_cast<float>(netH) / h)) {
+                newW = netW;
+                newH = (h * netW) / w;
+            } else {
+                newH = netH;
+                newW = (w * netH) / h;
+            }
+            float x = (static_cast<float>(col) + p0) / static_cast<float>(p.width);
+            x = (x - static_cast<float>(netW - newW) / 2.0f / static_cast<float>(netW)) /
+                (static_cast<float>(newW) / static_cast<float>(netW));
+            float y = (static_cast<float>(row) + p1) / static_cast<float>(p.height);
+            y = (y - static_cast<float>(netH - newH) / 2.0f / static_cast<float>(netH)) /
+                (static_cast<float>(newH) / static_cast<float>(netH));
+            float width = expf(p2) * p.anchors[2 * anchor] / static_cast<float>(netW);
+            width *= static_cast<float>(netW) / static_cast<float>(newW);
+            float height = expf(p3) * p.anchors[2 * anchor + 1] / static_cast<float>(netH);
+            height *= static_cast<float>(netH) / static_cast<float>(newH);
+            const int left = max(0, static_cast<int>((x - width / 2) * static_cast<float>(w)));
+            const int right = min(w - 1, static_cast<int>((x + width / 2) * static_cast<float>(w)));
+            const int top = max(0, static_cast<int>((y - height / 2) * static_cast<float>(h)));
+            const int bottom = min(h - 1, static_cast<int>((y + height / 2) * static_cast<float>(h)));
+            bx = static_cast<float>(left); by = static_cast<float>(top);
+            bw = static_cast<float>(right - left); bh = static_cast<float>(bottom - top);
+        } else {
+            const float x = (static_cast<float>(col) + p0) / static_cast<float>(p.width);
+            const float y = (static_cast<float>(row) + p1) / static_cast<float>(p.height);
+            bw = expf(p2) * p.anchors[2 * anchor] / static_cast<float>(p.net_width);
+            bh = expf(p3) * p.anchors[2 * anchor + 1] / static_cast<float>(p.net_height);
+            // DarkBox::rect(): the corner falls back to the centre for a non-positive size
+            bx = bw > 0.0f ? x - bw / 2.0f : x;
+            by = bh > 0.0f ? y - bh / 2.0f : y;
+        }
+    }
+    if (!__ballot(pass)) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t order0 = ((b * static_cast<uint32_t>(area) + cell) * p.mask_count + n) * p.classes;
+    const float* rows = a.pred + base + 5 * static_cast<size_t>(area);
+    // 128 classes at a time: each lane notes its hits in a bit mask, the wave reserves the places
+    // of all of them with ONE atomic (a counter shared by the whole grid cannot take one per hit),
+    // then every lane writes its records one after the other.
+    constexpr int kWords = 4;
+    for (int j0 = 0; j0 < p.classes; j0 += 32 * kWords) {
+        uint32_t hits[kWords];
+        int mine = 0;
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) {
+            hits[w] = 0u;
+            const int first = j0 + 32 * w;
+            const int last = min(first + 32, p.classes);
+            if (pass) {
+                for (int j = first; j < last; ++j) {
+                    const float prob = objectness * rows[static_cast<size_t>(j) * area];
+                    if (prob >= a.threshold) {
+                        hits[w] |= 1u << (j - first);
+                        ++mine;
+                    }
+                }
+            }
+        }
+        int upto = mine;      // inclusive prefix sum over the lanes
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const int v = __shfl_up(upto, off, kWave);
+            if (lane >= off) upto += v;
+        }
+        const int total = __shfl(upto, kWave - 1, kWave);
+        if (total == 0) continue;
+        int first_place = 0;
+        if (lane == kWave - 1) first_place = atomicAdd(a.count, total);
+        first_place = __shfl(first_place, kWave - 1, kWave);
+        int at = first_place + upto - mine;
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) {
+            uint32_t bits = hits[w];
+            while (bits) {
+                const int j = j0 + 32 * w + __builtin_ctz(bits);
+                bits &= bits - 1;
+                if (at < a.capacity) {
+                    pxh_detection d;
+                    d.x = bx; d.y = by; d.w = bw; d.h = bh;
+                    d.prob = objectness * rows[static_cast<size_t>(j) * area];
+                    d.batch = static_cast<int>(b);
+                    d.class_index = j;
+                    d.order = order0 + j;
+                    a.out[at] = d;
+                }
+                ++at;
+            }
+        }
+    }
+}
+
 int fill_params(const char* who, YoloParams& p, int batch, int mask_count, int anchor_count, int classes, int width,
                 int height, int net_width, int net_height, int max_truth, float ignore_thresh, float truth_thresh,
                 float coord_scale, float object_scale, float noobject_scale, float class_scale)
@@ -842,6 +973,36 @@ int pxh_yolo_activate(const float* input, float* output, int batch, int masks, i
     // the 128-bit path steps a row boundary at most once per vector: needs area >= 4
     const bool vec = area >= 4 && aligned16(input) && aligned16(output);
     return launch_stream("pxh_yolo_activate", static_cast<size_t>(total), vec, 8, op, as_stream(stream));
+}
+
+int pxh_yolo_detections(const float* predictions, int batch, const int* host_masks, int mask_count,
+                        const int* host_anchors, int anchor_count, int classes, int width, int height,
+                        int net_width, int net_height, int image_width, int image_height, float threshold,
+                        pxh_detection* out, int capacity, int* count, void* stream)
+{
+    if (!predictions || !host_masks || !host_anchors || !count || (!out && capacity > 0))
+        return fail_invalid("pxh_yolo_detections: null pointer");
+    if (capacity < 0) return fail_invalid("pxh_yolo_detections: negative capacity");
+    YoloParams p{};
+    int rc = fill_params("pxh_yolo_detections", p, batch, mask_count, anchor_count, classes, width, height, net_width,
+                         net_height, 0, 0.0f, 0.0f, 1.0f, 1.0f, 1.0f, 1.0f);
+    if (rc) return rc;
+    for (int m = 0; m < mask_count; ++m) {
+        if (host_masks[m] < 0 || host_masks[m] >= anchor_count)
+            return fail_invalid("pxh_yolo_detections: mask %d names anchor %d of %d", m, host_masks[m], anchor_count);
+        p.masks[m] = host_masks[m];
+    }
+    for (int a = 0; a < 2 * anchor_count; ++a) p.anchors[a] = static_cast<float>(host_anchors[a]);
+    hipStream_t s = as_stream(stream);
+    rc = pxh_fill_i32(count, 1, 0, stream);
+    if (rc) return rc;
+    DetectArgs a{};
+    a.pred = predictions; a.out = out; a.count = count; a.capacity = capacity; a.threshold = threshold;
+    a.image_width = image_width; a.image_height = image_height;
+    a.slots = static_cast<uint32_t>(batch) * mask_count * p.area;
+    a.by_area = FastDiv(p.area);
+    hipLaunchKernelGGL(yolo_detect_kernel, dim3(grid_for(a.slots, kBlock)), dim3(kBlock), 0, s, a, p);
+    return check_launch("pxh_yolo_detections");
 }
 
 size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int width, int height, int max_truth)

@@ -4,6 +4,7 @@
 // fused C-ABI calls where the reference issues several library calls and copies.
 #pragma once
 
+#include <cstring>
 #include <functional>
 
 #include "Adam.h"
@@ -381,6 +382,18 @@ private:
     std::vector<Layer::Ptr> layers_;
 };
 
+// ---------------------------------------------------------------- detections
+// reference: Detection, include/Detection.h:23-40 (the box is left, top, width, height)
+struct Detection
+{
+    float x, y, w, h;
+    int batchId;
+    int classIndex;
+    float prob;
+};
+
+using Detections = std::vector<Detection>;
+
 // ---------------------------------------------------------------- YOLO head
 // reference: include/YoloLayer.h:115-239, 390-547, include/cuda/YoloLayer.h:70-166.
 // The reference assigns the positive slots on the host and uploads them on every training
@@ -443,6 +456,34 @@ public:
         PX_HIP_CHECK(pxh_axpy(delta_.size(), 1.0f, delta_.data(), grad->data(), stream()));
     }
 
+    // Appends the detections of the last forward, in the reference's order (image, cell, mask,
+    // class), relative boxes (reference: include/YoloLayer.h:713-720).  Blocking; only the
+    // detections cross to the host, not the head.
+    void addDetects(Detections& detections, float threshold) { addDetects(detections, 0, 0, threshold); }
+
+    // The same with boxes in pixels of a width x height image that was letterboxed into the
+    // network input (reference: include/YoloLayer.h:700-711).
+    void addDetects(Detections& detections, int width, int height, float threshold)
+    {
+        const auto& c = context();
+        if (detectCount_.empty()) detectCount_ = IntVector(1, 0);
+        if (detectCapacity_ == 0) growDetections(4096);
+        for (;;) {
+            PX_HIP_CHECK(pxh_yolo_detections(output_.data(), batch(), mask_.data(), static_cast<int>(mask_.size()),
+                                             anchors_.data(), numAnchors_, c.classes, this->width(), this->height(),
+                                             c.width, c.height, width, height, threshold,
+                                             reinterpret_cast<pxh_detection*>(detectRecords_.data()),
+                                             detectCapacity_, detectCount_.data(), stream()));
+            PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(stream()));
+            const int found = detectCount_.asVector()[0];
+            if (found <= detectCapacity_) {
+                appendSorted(detections, found);
+                return;
+            }
+            growDetections(found);
+        }
+    }
+
     // Blocking: cost = sum(delta^2) / max(1, batch) (reference: include/cuda/YoloLayer.h:132).
     float fetchCost()
     {
@@ -462,11 +503,30 @@ public:
     }
 
 private:
+    void growDetections(int capacity)
+    {
+        detectCapacity_ = capacity;
+        detectRecords_ = IntVector(static_cast<std::size_t>(capacity) * (sizeof(pxh_detection) / sizeof(int)));
+    }
+
+    void appendSorted(Detections& detections, int found)
+    {
+        static_assert(sizeof(pxh_detection) == 8 * sizeof(int), "record layout");
+        const std::vector<int> raw = detectRecords_.asVector();
+        std::vector<pxh_detection> records(static_cast<std::size_t>(found));
+        if (found) std::memcpy(records.data(), raw.data(), records.size() * sizeof(pxh_detection));
+        std::sort(records.begin(), records.end(),
+                  [](const pxh_detection& a, const pxh_detection& b) { return a.order < b.order; });
+        for (const auto& r: records) detections.push_back(Detection{ r.x, r.y, r.w, r.h, r.batch, r.class_index, r.prob });
+    }
+
     std::vector<int> anchors_, mask_;
     int numAnchors_ = 1;
     float ignoreThresh_, truthThresh_, coordScale_, objectScale_, noObjectScale_, classScale_;
     V stats_, costDevice_;
     bool costReady_ = false;
+    IntVector detectRecords_, detectCount_;
+    int detectCapacity_ = 0;
 };
 
 }   // px::hip

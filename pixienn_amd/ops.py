@@ -303,3 +303,25 @@ def rescale_clip(x, threshold=0.0, clip=0.0, norm_out=None):
     """Gradient rescale to a norm threshold, then clamp (include/Layer.h:385-397 of the reference)."""
     _chk_all(x, norm_out)
     call("pxh_rescale_clip", ptr(x), x.numel(), float(threshold), float(clip), ptr(norm_out), None, 0, _stream())
+
+
+DETECTION_DTYPE = np.dtype([("x", "f4"), ("y", "f4"), ("w", "f4"), ("h", "f4"), ("prob", "f4"), ("batch", "i4"),
+                            ("class_index", "i4"), ("order", "u4")])
+
+
+def yolo_detections(predictions, batch, masks, anchors, classes, width, height, net_width, net_height, threshold,
+                    capacity, image_width=0, image_height=0):
+    """Thresholded compaction of a decoded head.  Returns (records sorted into the reference's
+    emission order as a numpy structured array, total number found)."""
+    _chk_all(predictions)
+    m = np.ascontiguousarray(masks, dtype=np.int32)
+    a = np.ascontiguousarray(anchors, dtype=np.int32)
+    out = torch.zeros((max(1, capacity), 8), device=predictions.device, dtype=torch.int32)
+    count = torch.zeros(1, device=predictions.device, dtype=torch.int32)
+    call("pxh_yolo_detections", ptr(predictions), batch, m.ctypes.data, len(m), a.ctypes.data, len(a) // 2, classes,
+         width, height, net_width, net_height, int(image_width), int(image_height), float(threshold), ptr(out),
+         int(capacity), ptr(count), _stream())
+    torch.cuda.current_stream().synchronize()
+    found = int(count.item())
+    rec = out[:min(found, capacity)].cpu().numpy().view(DETECTION_DTYPE).reshape(-1)
+    return rec[np.argsort(rec["order"], kind="stable")], found

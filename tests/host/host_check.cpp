@@ -267,6 +267,29 @@ void inferenceChecks()
         Host out(in.size());
         pxo_yolo_decode(&cfg, in.data(), out.data());
         expectClose("yolo7 decode (inference)", net.yolo7->output().asVector(), out, 1e-5, 1e-3);
+
+        // detections of that head, from the decoded values the layer holds
+        const Host decoded = net.yolo7->output().asVector();
+        for (int scaled = 0; scaled < 2; ++scaled) {
+            const int iw = scaled ? 320 : 0, ih = scaled ? 200 : 0;
+            std::vector<pxo_detection> want(4096);
+            const int found = pxo_yolo_detections(&cfg, decoded.data(), 0.3f, iw, ih, want.data(), 4096);
+            Detections got;
+            if (scaled) net.yolo7->addDetects(got, iw, ih, 0.3f); else net.yolo7->addDetects(got, 0.3f);
+            bool same = found > 0 && found <= 4096 && static_cast<int>(got.size()) == found;
+            Host gb, wb;
+            for (int k = 0; same && k < found; ++k) {
+                same = got[k].batchId == want[k].batch && got[k].classIndex == want[k].class_index &&
+                       got[k].prob == want[k].prob;
+                gb.insert(gb.end(), { got[k].x, got[k].y, got[k].w, got[k].h });
+                wb.insert(wb.end(), { want[k].x, want[k].y, want[k].w, want[k].h });
+            }
+            report(std::string("yolo7 detections, order and scores") + (scaled ? " (pixel boxes)" : ""), same,
+                   std::to_string(found) + " found");
+            // integer pixel boxes may differ by one where a last-place difference in exp moves a truncation
+            expectClose(std::string("yolo7 detection boxes") + (scaled ? " (pixel boxes)" : ""), gb, wb,
+                        scaled ? 1.0 / 320.0 : 1e-5, scaled ? 320.0 : 4.0);
+        }
     }
 }
 

@@ -328,3 +328,52 @@ def test_rescale_clip_matches_oracle(ops, oracle, n, mode):
     gy = gpu(x0)
     ops.rescale_clip(gy, threshold, clip)
     assert_bit_exact(host(gy), host(gx), "with and without norm_out")
+
+
+# ---------------------------------------------------------------- detections (device-side compaction)
+@pytest.mark.parametrize("case", [(2, 3, 80, 19, 0.5), (4, 3, 80, 38, 0.4), (1, 2, 5, 7, 0.1), (3, 3, 20, 13, 0.9)])
+@pytest.mark.parametrize("image", [(0, 0), (640, 480), (333, 500)])
+def test_yolo_detections_match_oracle(ops, oracle, case, image):
+    import torch
+    N, A, K, W, thr = case
+    mask = list(range(A)); anchors = wl.YOLOV3_ANCHORS[:2 * A]
+    logits = wl.normal(3500 + W, (N, A * (K + 5), W, W), std=2.0)
+    cfg, keep = oracle.yolo_cfg(N, W, W, K, mask, anchors, 608, 608)
+    decoded = np.zeros_like(logits)
+    oracle.yolo_decode(cfg, logits, decoded)
+    cap = 1 << 20
+    want, found_w = oracle.yolo_detections(cfg, decoded, thr, cap, image_width=image[0], image_height=image[1])
+    got, found_g = ops.yolo_detections(gpu(decoded), N, mask, anchors, K, W, W, 608, 608, thr, cap,
+                                       image_width=image[0], image_height=image[1])
+    assert 0 < found_w <= cap, "the case must produce detections, and all must fit"
+    assert found_g == found_w and len(got) == len(want)
+    for k in ("order", "batch", "class_index"):
+        assert np.array_equal(got[k], want[k]), k
+    assert_bit_exact(got["prob"], want["prob"], "probabilities")
+    if image[0]:
+        # integer pixel boxes: a last-place difference in exp can move a truncation by one pixel
+        for k in ("x", "y", "w", "h"):
+            d = np.abs(got[k] - want[k])
+            assert d.max() <= 1.0 and (d > 0).mean() < 1e-3, (k, d.max(), (d > 0).mean())
+    else:
+        # left = x - w/2 cancels: bounded relative to its operands (the centre is O(1), the size any)
+        assert_close(got["w"], want["w"], 1e-5, 1e-6, "box w")
+        assert_close(got["h"], want["h"], 1e-5, 1e-6, "box h")
+        assert_close(got["x"], want["x"], 1e-5, np.maximum(1.0, want["w"]), "box x")
+        assert_close(got["y"], want["y"], 1e-5, np.maximum(1.0, want["h"]), "box y")
+
+
+def test_yolo_detections_capacity_and_empty(ops, oracle):
+    N, A, K, W = 2, 3, 8, 13
+    mask = [0, 1, 2]; anchors = wl.YOLOV3_ANCHORS[:6]
+    logits = wl.normal(3600, (N, A * (K + 5), W, W), std=2.0)
+    cfg, keep = oracle.yolo_cfg(N, W, W, K, mask, anchors, 416, 416)
+    decoded = np.zeros_like(logits)
+    oracle.yolo_decode(cfg, logits, decoded)
+    want, found_w = oracle.yolo_detections(cfg, decoded, 0.3, 1 << 16)
+    got, found_g = ops.yolo_detections(gpu(decoded), N, mask, anchors, K, W, W, 416, 416, 0.3, 10)
+    assert found_g == found_w > 10 and len(got) == 10
+    # the ten that fit are ten of the true ones
+    assert set(got["order"]) <= set(want["order"])
+    got, found_g = ops.yolo_detections(gpu(decoded), N, mask, anchors, K, W, W, 416, 416, 1.5, 10)
+    assert found_g == 0 and len(got) == 0

@@ -575,3 +575,36 @@ def test_rescale_clip_invariants(oracle):
     # zero tensor: the norm test keeps it untouched
     z = np.zeros(8, F)
     assert oracle.rescale_clip(z, 1.0, 0.0) == 0.0 and not z.any()
+
+
+def test_detections_hand_computed(oracle):
+    """addDetects on a 2x2 head with one anchor and two classes, values worked out by hand."""
+    W = H = 2; K = 2
+    cfg, keep = oracle.yolo_cfg(1, W, H, K, [0], [16, 16], 64, 64)
+    p = np.zeros((1, K + 5, H, W), F)
+    # cell (row 0, col 1): centre offsets 0.5, log-sizes 0, objectness 0.9, class probabilities 0.8 / 0.5
+    p[0, 0, 0, 1] = 0.5; p[0, 1, 0, 1] = 0.5; p[0, 4, 0, 1] = 0.9; p[0, 5, 0, 1] = 0.8; p[0, 6, 0, 1] = 0.5
+    # cell (row 1, col 0): objectness below the threshold; cell (1, 1): objectness passes, no class does
+    p[0, 4, 1, 0] = 0.49; p[0, 5, 1, 0] = 1.0
+    p[0, 4, 1, 1] = 0.6; p[0, 5, 1, 1] = 0.8
+    rec, found = oracle.yolo_detections(cfg, p, 0.5, 16)
+    assert found == 1 and len(rec) == 1
+    r = rec[0]
+    # x = (1 + .5)/2 = .75, y = (0 + .5)/2 = .25, w = h = exp(0)*16/64 = .25 -> left .625, top .125
+    assert (r["x"], r["y"], r["w"], r["h"]) == (0.625, 0.125, 0.25, 0.25)
+    assert r["class_index"] == 0 and r["batch"] == 0 and abs(r["prob"] - 0.72) < 1e-7
+    assert r["order"] == (0 * 4 + 1) * 1 * K + 0
+    # a 128 x 64 image letterboxed into 64 x 64: newW 64, newH 32; x stays .75, y -> (.25 - .25)/.5 = 0,
+    # w .25, h .25 * 2 = .5 -> left int(.625*128) = 80, right int(.875*128) = 112, top max(0, int(-.25*64)) = 0,
+    # bottom int(.25*64) = 16
+    rec, found = oracle.yolo_detections(cfg, p, 0.5, 16, image_width=128, image_height=64)
+    assert found == 1
+    r = rec[0]
+    assert (r["x"], r["y"], r["w"], r["h"]) == (80.0, 0.0, 32.0, 16.0)
+    # a lower threshold lets the other class and the other cells in, in cell / mask / class order
+    rec, found = oracle.yolo_detections(cfg, p, 0.4, 16)
+    assert found == 4
+    assert list(rec["order"]) == [2, 3, 4, 6] and list(rec["class_index"]) == [0, 1, 0, 0]
+    # capacity smaller than the number found: the count still says how many there are
+    rec, found = oracle.yolo_detections(cfg, p, 0.4, 2)
+    assert found == 4 and len(rec) == 2
