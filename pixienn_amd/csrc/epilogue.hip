@@ -635,10 +635,19 @@ struct ResidentFwdArgs {
     ResidentGeom g;
 };
 
-// V = 4 needs spatial % 4 == 0 and 16-byte aligned tensors.  R vectors per thread at most.
-template<int ACT, int V, int R>
+// A thread keeps R vectors in registers and L more in LDS (dynamic, L * kResidentThreads vectors:
+// thread-major, so every access is the conflict-free 128-bit one).
+template<int V, int R>
+__device__ __forceinline__ Pack<V>* resident_lds_slot(float* lds, int r)
+{
+    return reinterpret_cast<Pack<V>*>(lds) + static_cast<size_t>(r - R) * kResidentThreads + threadIdx.x;
+}
+
+// V = 4 needs spatial % 4 == 0 and 16-byte aligned tensors.  R + L vectors per thread at most.
+template<int ACT, int V, int R, int L>
 __global__ __launch_bounds__(kResidentThreads) void bn_resident_fwd_kernel(ResidentFwdArgs a)
 {
+    extern __shared__ __align__(16) float resident_lds[];
     __shared__ double slots[2][kResidentWaves];
     __shared__ FoldCoef shared_coef;
     const uint32_t c = blockIdx.x;
@@ -646,21 +655,21 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_fwd_kernel(Resid
     // issued now, needed after the reduction
     const float rm_in = a.rolling_mean[c], rv_in = a.rolling_var[c], scale_in = a.scale[c], bias_in = a.bias[c];
     Pack<V> v[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
-        if (e < a.g.per_channel) v[r] = ld<V, false>(a.x, a.g.at(c, e));
-    }
     float a1 = 0.0f, a2 = 0.0f;
+    // the LDS part first: its registers are free again before the register part is loaded
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        if ((r * kResidentThreads + threadIdx.x) * V < a.g.per_channel) {
+    for (int r = R + L - 1; r >= 0; --r) {
+        const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+        if (e < a.g.per_channel) {
+            const Pack<V> t = ld<V, false>(a.x, a.g.at(c, e));
 #pragma unroll
             for (int k = 0; k < V; ++k) {
-                const float d = v[r].v[k] - shift;
+                const float d = t.v[k] - shift;
                 a1 += d;
                 a2 += d * d;
             }
+            if (r < R) v[r < R ? r : 0] = t;
+            else *resident_lds_slot<V, R>(resident_lds, r) = t;
         }
     }
     double s1 = static_cast<double>(a1), s2 = static_cast<double>(a2);
@@ -676,18 +685,19 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_fwd_kernel(Resid
     __syncthreads();
     const FoldCoef k = shared_coef;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
+    for (int r = 0; r < R + L; ++r) {
         const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
         if (e < a.g.per_channel) {
             const size_t where = a.g.at(c, e);
+            const Pack<V> t = r < R ? v[r < R ? r : 0] : *resident_lds_slot<V, R>(resident_lds, r);
             Pack<V> xn, pre, out;
 #pragma unroll
             for (int q = 0; q < V; ++q) {
-                xn.v[q] = normalize(v[r].v[q], k);
+                xn.v[q] = normalize(t.v[q], k);
                 pre.v[q] = affine(xn.v[q], k);
                 out.v[q] = act_apply<ACT>(pre.v[q]);
             }
-            if (a.x_saved) st<V, false>(a.x_saved, where, v[r]);
+            if (a.x_saved) st<V, false>(a.x_saved, where, t);
             if (a.x_norm) st<V, false>(a.x_norm, where, xn);
             if (a.pre) st<V, false>(a.pre, where, pre);
             st<V, false>(a.y, where, out);
@@ -704,11 +714,12 @@ struct ResidentBwdArgs {
     ResidentGeom g;
 };
 
-// The workgroup keeps d' = delta * act'(pre) in registers; x is read again for the dx phase
+// The workgroup keeps d' = delta * act'(pre) (registers + LDS); x is read again for the dx phase
 // (it is still in the cache: one channel's slice is a few hundred KB).
-template<int ACT, int V, int R>
+template<int ACT, int V, int R, int L>
 __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(ResidentBwdArgs a)
 {
+    extern __shared__ __align__(16) float resident_lds[];
     __shared__ double slots[2][kResidentWaves];
     __shared__ DxCoef shared_coef;
     const uint32_t c = blockIdx.x;
@@ -717,11 +728,11 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
     Pack<V> d[R];
     float fa = 0.0f, fb = 0.0f;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
+    for (int r = R + L - 1; r >= 0; --r) {
         const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
         if (e < a.g.per_channel) {
             const size_t where = a.g.at(c, e);
-            d[r] = ld<V, false>(a.b.delta, where);
+            Pack<V> dv = ld<V, false>(a.b.delta, where);
             const Pack<V> xv = ld<V, false>(a.b.x, where);
             Pack<V> pv;
             if constexpr (ACT != PXH_LINEAR) {
@@ -729,17 +740,19 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
             }
 #pragma unroll
             for (int q = 0; q < V; ++q) {
-                float dv = d[r].v[q];
+                float t = dv.v[q];
                 if constexpr (ACT != PXH_LINEAR) {
                     float pre;
                     if (recompute) pre = affine(normalize(xv.v[q], k), k);
                     else pre = pv.v[q];
-                    dv = dv * act_grad<ACT>(pre);
-                    d[r].v[q] = dv;
+                    t = t * act_grad<ACT>(pre);
+                    dv.v[q] = t;
                 }
-                fa += dv;
-                fb += dv * (xv.v[q] - k.mean);
+                fa += t;
+                fb += t * (xv.v[q] - k.mean);
             }
+            if (r < R) d[r < R ? r : 0] = dv;
+            else *resident_lds_slot<V, R>(resident_lds, r) = dv;
         }
     }
     double sa = static_cast<double>(fa), sb = static_cast<double>(fb);
@@ -750,14 +763,15 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
     __syncthreads();
     const DxCoef kd = shared_coef;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
+    for (int r = 0; r < R + L; ++r) {
         const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
         if (e < a.g.per_channel) {
             const size_t where = a.g.at(c, e);
             const Pack<V> xv = ld<V, false>(a.b.x, where);
+            const Pack<V> dv = r < R ? d[r < R ? r : 0] : *resident_lds_slot<V, R>(resident_lds, r);
             Pack<V> out;
 #pragma unroll
-            for (int q = 0; q < V; ++q) out.v[q] = dx_value<PXH_LINEAR>(d[r].v[q], xv.v[q], 0.0f, false, kd);
+            for (int q = 0; q < V; ++q) out.v[q] = dx_value<PXH_LINEAR>(dv.v[q], xv.v[q], 0.0f, false, kd);
             st<V, false>(a.b.delta, where, out);
         }
     }
@@ -766,8 +780,11 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
 // Vectors per thread the resident kernels are built for, and whether a shape takes that path:
 // the channel slice must fit, and there must be enough channels to occupy the machine.  (Measured
 // with 24 vectors per thread: the registers spill and 128 workgroups of 16x128x76^2 are slower than
-// the three launches.)
+// the three launches; with a third of them in LDS they do not.)
 constexpr int kResidentVectors = 8;
+// the large form (128-bit vectors only): 16 vectors in registers + 8 in LDS (128 KB of the CU's 160)
+constexpr int kResidentLargeRegs = 16, kResidentLargeLds = 8;
+constexpr size_t kResidentLargeLdsBytes = static_cast<size_t>(kResidentLargeLds) * kResidentThreads * 16;
 
 int resident_vectors(int batch, int channels, int spatial, bool vec)
 {
@@ -775,7 +792,21 @@ int resident_vectors(int batch, int channels, int spatial, bool vec)
     const size_t per_channel = static_cast<size_t>(batch) * spatial;
     const size_t vectors = (per_channel + (vec ? 3 : 0)) / (vec ? 4 : 1);
     const size_t per_thread = (vectors + kResidentThreads - 1) / kResidentThreads;
-    return per_thread <= kResidentVectors ? kResidentVectors : 0;
+    if (per_thread <= kResidentVectors) return kResidentVectors;
+    if (vec && per_thread <= kResidentLargeRegs + kResidentLargeLds) return kResidentLargeRegs + kResidentLargeLds;
+    return 0;
+}
+
+// A kernel that asks for more than 64 KB of dynamic LDS has to be allowed to, once.
+int allow_large_lds(const void* kernel)
+{
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             static_cast<int>(kResidentLargeLdsBytes));
+    if (e != hipSuccess) {
+        set_error("hipFuncSetAttribute(max dynamic LDS %zu): %s", kResidentLargeLdsBytes, hipGetErrorString(e));
+        return static_cast<int>(e);
+    }
+    return PXH_OK;
 }
 
 ResidentGeom resident_geom(int batch, int channels, int spatial)
@@ -942,11 +973,21 @@ int pxh_bn_train_act_forward(const float* x, float* y, float* pre_activation, fl
             const ResidentFwdArgs r{ x, y, pre_activation, x_saved, x_norm, mean, var, rolling_mean, rolling_var,
                                      scale, bias, resident_geom(batch, channels, spatial) };
             const dim3 grid(channels), block(kResidentThreads);
+            int large_lds_rc = PXH_OK;
             const bool known = dispatch_activation(activation, [&]<int ACT>() {
-                if (vec) hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 4, kResidentVectors>), grid, block, 0, s, r);
-                else hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 1, kResidentVectors>), grid, block, 0, s, r);
+                if (per_thread > kResidentVectors) {
+                    auto kernel = bn_resident_fwd_kernel<ACT, 4, kResidentLargeRegs, kResidentLargeLds>;
+                    large_lds_rc = allow_large_lds(reinterpret_cast<const void*>(kernel));
+                    if (large_lds_rc == PXH_OK)
+                        hipLaunchKernelGGL(kernel, grid, block, kResidentLargeLdsBytes, s, r);
+                } else if (vec) {
+                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 4, kResidentVectors, 0>), grid, block, 0, s, r);
+                } else {
+                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 1, kResidentVectors, 0>), grid, block, 0, s, r);
+                }
             });
             if (!known) return fail_invalid("pxh_bn_train_act_forward: unknown activation %d", activation);
+            if (large_lds_rc) return large_lds_rc;
             return check_launch("pxh_bn_train_act_forward");
         }
     }
@@ -981,11 +1022,21 @@ int pxh_bn_act_backward(float* delta, const float* x, const float* pre_activatio
             const ResidentBwdArgs r{ BackwardArgs{ delta, x, pre_activation, mean, var, scale, bias }, scale_updates,
                                      bias_updates, mean_delta, var_delta, resident_geom(batch, channels, spatial) };
             const dim3 grid(channels), block(kResidentThreads);
+            int large_lds_rc = PXH_OK;
             const bool known = dispatch_activation(activation, [&]<int ACT>() {
-                if (rvec) hipLaunchKernelGGL((bn_resident_bwd_kernel<ACT, 4, kResidentVectors>), grid, block, 0, s, r);
-                else hipLaunchKernelGGL((bn_resident_bwd_kernel<ACT, 1, kResidentVectors>), grid, block, 0, s, r);
+                if (per_thread > kResidentVectors) {
+                    auto kernel = bn_resident_bwd_kernel<ACT, 4, kResidentLargeRegs, kResidentLargeLds>;
+                    large_lds_rc = allow_large_lds(reinterpret_cast<const void*>(kernel));
+                    if (large_lds_rc == PXH_OK)
+                        hipLaunchKernelGGL(kernel, grid, block, kResidentLargeLdsBytes, s, r);
+                } else if (rvec) {
+                    hipLaunchKernelGGL((bn_resident_bwd_kernel<ACT, 4, kResidentVectors, 0>), grid, block, 0, s, r);
+                } else {
+                    hipLaunchKernelGGL((bn_resident_bwd_kernel<ACT, 1, kResidentVectors, 0>), grid, block, 0, s, r);
+                }
             });
             if (!known) return fail_invalid("pxh_bn_act_backward: unknown activation %d", activation);
+            if (large_lds_rc) return large_lds_rc;
             return check_launch("pxh_bn_act_backward");
         }
     }
