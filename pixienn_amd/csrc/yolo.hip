@@ -1,16 +1,19 @@
 // YOLO head for gfx950: logistic decode, and the training pass (decode + dense delta + cost +
 // statistics).
 //
-// Layout [batch][mask][5 + classes][area].  The training pass is two launches:
+// Layout [batch][mask][5 + classes][area].  The work of the training pass has two parts:
 //   head   one lane per slot (image, anchor, cell): the 5 box/objectness rows, the best-truth
 //          search against the image's truths staged in LDS, the decision what the slot is
 //          supervised with (one int per slot), box/objectness deltas, every statistic and the
-//          whole cost (the class rows of the few supervised slots are visited for it).  Latency
-//          bound: a few dependent memory round trips and ~20 IoU tests per lane, so the kernel is
-//          written for instruction-level parallelism rather than for occupancy.
-//   class  streams the class rows, 94 % of the tensor: logit -> probability -> `out`, and the
-//          dense class delta from the slots' decisions, 12 bytes per element.  Its first
-//          workgroups also add up the per-workgroup sums of the head kernel in a fixed order.
+//          whole cost (the class rows of the few supervised slots are visited for it).
+//          Instruction and latency bound: ~1000 vector instructions per wave.
+//   class  the class rows, 94 % of the tensor: logit -> probability -> `out`, and the dense class
+//          delta.  Bandwidth bound, 12 bytes per element.
+// From raw logits (pxh_yolo_forward_train) both run in ONE grid, persistent head workgroups beside
+// the class stream, followed by a small kernel that writes the class delta of the supervised
+// slots and adds up the sums in a fixed order.  From an already decoded head with host-assigned
+// positives (pxh_yolo_loss, the reference's argument list) a head kernel is followed by a class
+// kernel that takes the decisions.  pxh_yolo_detections is the inference-side compaction.
 // Box arithmetic follows the CPU layer (include/YoloLayer.h, src/DarkBox.cpp of the reference).
 #include "stream.h"
 
@@ -551,8 +554,7 @@ struct ClassSpace {
 
 // ---- class sweep: decode + dense class delta; the first workgroups add up the head sums --------
 struct ClassArgs {
-    const float* in;       // FUSED: raw logits; otherwise the decoded head
-    float* out;            // FUSED only
+    const float* in;       // the decoded head
     float* delta;
     const int* decision;
     const double* partial;
@@ -591,8 +593,9 @@ __device__ __forceinline__ void finish_statistic(int k, const ClassArgs& a, doub
     }
 }
 
+// The decoded-input form: dense class delta from the slots' decisions.
 // V = 4 needs area % 4 == 0 (a vector then never leaves its row) and 16-byte aligned tensors.
-template<bool FUSED, int V, bool NT>
+template<int V, bool NT>
 __global__ __launch_bounds__(kBlock) void yolo_class_kernel(ClassArgs a)
 {
     __shared__ double slots[kBlock / kWave];
@@ -603,21 +606,13 @@ __global__ __launch_bounds__(kBlock) void yolo_class_kernel(ClassArgs a)
     a.space.locate(e, bn, c, cell);
     const size_t at = a.space.offset(bn, c, cell);
     const IPack<V> cls = ldi<V, false>(a.decision, static_cast<size_t>(bn) * a.space.area + cell);
-    Pack<V> prob, d;
-    if constexpr (FUSED) {
-        const Pack<V> x = ld<V, NT>(a.in, at);
-#pragma unroll
-        for (int k = 0; k < V; ++k) prob.v[k] = sigmoid_fast(x.v[k]);
-        st<V, NT>(a.out, at, prob);
-    }
+    Pack<V> d;
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         d.v[k] = 0.0f;
         if (cls.v[k] >= 0) {      // rare: a supervised slot
             const float t = (static_cast<int>(c) == cls.v[k]) ? 1.0f : 0.0f;
-            float pr;
-            if constexpr (FUSED) pr = prob.v[k]; else pr = a.in[at + k];
-            d.v[k] = a.class_scale * (t - pr);
+            d.v[k] = a.class_scale * (t - a.in[at + k]);
         }
     }
     st<V, NT>(a.delta, at, d);
@@ -625,8 +620,8 @@ __global__ __launch_bounds__(kBlock) void yolo_class_kernel(ClassArgs a)
 
 // ---- fused pass: persistent head workgroups + class decode stream in one grid ------------------
 // The head tiles are instruction bound and the class stream is bandwidth bound, so they run side
-// by side: the first `head_workers` workgroups of the grid (dispatched first, about two per
-// compute unit) walk the head tiles with a stride, every other workgroup decodes one vector per
+// by side: the first `head_workers` workgroups of the grid (dispatched first, a few per compute
+// unit) walk the head tiles with a stride, every other workgroup decodes one vector per
 // lane of the class rows and writes a zero class delta.  The few supervised slots get their class
 // delta from yolo_patch_kernel afterwards, so nothing in this grid waits for anything else in it.
 struct FusedArgs {
@@ -913,7 +908,6 @@ int run_training_pass(const char* who, const float* in, float* out, float* delta
 
     ClassArgs ca{};
     ca.in = FUSED ? out : in;      // the decoded head
-    ca.out = nullptr;
     ca.delta = delta;
     ca.decision = w.decision;
     ca.partial = w.partial;
@@ -946,9 +940,9 @@ int run_training_pass(const char* who, const float* in, float* out, float* delta
         if (rc) return rc;
         const uint32_t grid = class_blocks < 13 ? 13 : class_blocks;
         const bool nt = static_cast<size_t>(space.elems) * 4 >= kStreamingBytes;
-        if (vec && nt) hipLaunchKernelGGL((yolo_class_kernel<false, 4, true>), dim3(grid), dim3(kBlock), 0, s, ca);
-        else if (vec) hipLaunchKernelGGL((yolo_class_kernel<false, 4, false>), dim3(grid), dim3(kBlock), 0, s, ca);
-        else hipLaunchKernelGGL((yolo_class_kernel<false, 1, false>), dim3(grid), dim3(kBlock), 0, s, ca);
+        if (vec && nt) hipLaunchKernelGGL((yolo_class_kernel<4, true>), dim3(grid), dim3(kBlock), 0, s, ca);
+        else if (vec) hipLaunchKernelGGL((yolo_class_kernel<4, false>), dim3(grid), dim3(kBlock), 0, s, ca);
+        else hipLaunchKernelGGL((yolo_class_kernel<1, false>), dim3(grid), dim3(kBlock), 0, s, ca);
         return check_launch(who);
     }
 }
