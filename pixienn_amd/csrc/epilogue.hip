@@ -9,6 +9,9 @@
 // equals the rounded double quotient except in about 1e-7 of the elements (1 ulp there).
 #include "stream.h"
 
+#include <mutex>
+#include <vector>
+
 namespace pxh {
 namespace {
 
@@ -800,12 +803,18 @@ int resident_vectors(int batch, int channels, int spatial, bool vec)
 // A kernel that asks for more than 64 KB of dynamic LDS has to be allowed to, once.
 int allow_large_lds(const void* kernel)
 {
+    static std::mutex mutex;
+    static std::vector<const void*> allowed;
+    std::lock_guard<std::mutex> lock(mutex);
+    for (const void* k: allowed)
+        if (k == kernel) return PXH_OK;
     const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                              static_cast<int>(kResidentLargeLdsBytes));
     if (e != hipSuccess) {
         set_error("hipFuncSetAttribute(max dynamic LDS %zu): %s", kResidentLargeLdsBytes, hipGetErrorString(e));
         return static_cast<int>(e);
     }
+    allowed.push_back(kernel);
     return PXH_OK;
 }
 

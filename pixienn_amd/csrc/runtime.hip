@@ -58,7 +58,9 @@ void* library_workspace(size_t bytes)
         s.ptr = nullptr;
         s.bytes = 0;
     }
-    size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+    // 16 MB covers every shape of a YOLOv3-sized network, so the buffer rarely grows after the first
+    // call (growing synchronises the device, which a call inside a graph capture must not do)
+    size_t want = bytes < (16u << 20) ? (16u << 20) : bytes;
     if (hipMalloc(&s.ptr, want) != hipSuccess) {
         s.ptr = nullptr;
         return nullptr;

@@ -12,7 +12,9 @@
 
 #include <algorithm>
 #include <cmath>
+#include <istream>
 #include <map>
+#include <ostream>
 #include <memory>
 #include <string>
 #include <variant>
@@ -174,6 +176,11 @@ public:
     }
 
     virtual void update() {}
+
+    // Optimizer moments for the checkpoint sidecar; bytes written / read (reference:
+    // Layer<D>::saveOptimizer / loadOptimizer, include/Layer.h:59-60).  Nothing by default.
+    virtual std::streamoff saveOptimizer(std::ostream& /*os*/) { return 0; }
+    virtual std::streamoff loadOptimizer(std::istream& /*is*/) { return 0; }
 
     virtual bool hasCost() const noexcept { return false; }
     float cost() const noexcept { return cost_; }

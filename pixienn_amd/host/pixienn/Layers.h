@@ -45,6 +45,17 @@ public:
         const int ow = props.get<int>("out_width", width());
         setOutput(filters_, oh, ow);
 
+        // The weights live here so that update() and the optimizer sidecar cover the whole layer;
+        // their values and gradients are the delegated convolution's business ("weights": count).
+        const auto nweights = static_cast<std::size_t>(props.get<int>("weights", 0));
+        if (nweights) {
+            weights_ = V(nweights, 0.0f);
+            if (training()) {
+                weightUpdates_ = V(nweights, 0.0f);
+                weightM_ = V(nweights, 0.0f);
+                weightV_ = V(nweights, 0.0f);
+            }
+        }
         const auto f = static_cast<std::size_t>(filters_);
         biases_ = V(f, 0.0f);
         if (batchNorm_) {
@@ -146,9 +157,13 @@ public:
         const auto& c = context();
         if (c.adamEnabled) {
             const Adam adam(c);
+            if (!weights_.empty()) adam.update(weights_, weightUpdates_, weightM_, weightV_, true);
             adam.update(biases_, biasUpdates_, biasM_, biasV_, false);
             if (batchNorm_) adam.update(scales_, scaleUpdates_, scaleM_, scaleV_, false);
         } else {
+            if (!weights_.empty())
+                PX_HIP_CHECK(pxh_sgd_update(weights_.size(), weights_.data(), weightUpdates_.data(), c.updateBatch,
+                                            c.learningRate, c.momentum, c.decay, 1, stream()));
             PX_HIP_CHECK(pxh_sgd_update(biases_.size(), biases_.data(), biasUpdates_.data(), c.updateBatch,
                                         c.learningRate, c.momentum, c.decay, 0, stream()));
             if (batchNorm_)
@@ -158,6 +173,32 @@ public:
         foldedValid_ = false;
     }
 
+    // m, v, bias_m, bias_v, scale_m, scale_v as raw fp32 (reference: include/cuda/ConvLayer.h:228-264)
+    std::streamoff saveOptimizer(std::ostream& os) override
+    {
+        const auto start = os.tellp();
+        for (const V* t: { &weightM_, &weightV_, &biasM_, &biasV_, &scaleM_, &scaleV_ }) {
+            const std::vector<float> host = t->asVector();
+            os.write(reinterpret_cast<const char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
+        }
+        PX_CHECK(os.good(), "Could not write convolution optimizer state");
+        return os.tellp() - start;
+    }
+
+    std::streamoff loadOptimizer(std::istream& is) override
+    {
+        const auto start = is.tellg();
+        for (V* t: { &weightM_, &weightV_, &biasM_, &biasV_, &scaleM_, &scaleV_ }) {
+            std::vector<float> host(t->size());
+            is.read(reinterpret_cast<char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
+            PX_CHECK(is.good() || host.empty(), "Could not read convolution optimizer state");
+            t->copyHost(host);
+        }
+        return is.tellg() - start;
+    }
+
+    V& weights() noexcept { return weights_; }
+    V& weightUpdates() noexcept { return weightUpdates_; }
     const V& biases() const noexcept { return biases_; }
     const V& scales() const noexcept { return scales_; }
     const V& rollingMean() const noexcept { return rollingMean_; }
@@ -188,6 +229,7 @@ private:
     const float* x_ = nullptr;      // conv result of the last forward (borrowed)
     V biases_, scales_, rollingMean_, rollingVar_, mean_, var_, folded_;
     V biasUpdates_, scaleUpdates_, biasM_, biasV_, scaleM_, scaleV_;
+    V weights_, weightUpdates_, weightM_, weightV_;
     V result_, pre_;
     Convolve convolve_;
     ConvolveBackward convolveBackward_;

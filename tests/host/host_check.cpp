@@ -14,7 +14,10 @@
 #include <string>
 #include <vector>
 
+#include <sstream>
+
 #include "pixienn/Layers.h"
+#include "pixienn/OptimizerState.h"
 #include "px_oracle.h"
 
 using namespace px::hip;
@@ -95,6 +98,13 @@ void expectClose(const std::string& what, const Host& got, const Host& want, dou
     char buf[64];
     std::snprintf(buf, sizeof buf, "max rel %.2e", worst);
     report(what, ok, buf);
+}
+
+Host readFloats(const std::string& bytes, size_t offset, size_t count)
+{
+    Host v(count);
+    std::memcpy(v.data(), bytes.data() + offset, count * sizeof(float));
+    return v;
 }
 
 template<typename F>
@@ -464,6 +474,39 @@ void trainingChecks()
         net.conv2->update();
         expectClose("conv2 Adam update of the scales", net.conv2->scales().asVector(), w, 1e-6, 1e-3);
         expectExact("conv2 scale updates consumed", net.conv2->scaleUpdates().asVector(), Host(C, 0.0f));
+    }
+
+    // ---- optimizer sidecar: layout, round trip, stale file
+    {
+        const std::vector<Layer::Ptr> layers{ net.conv0, net.pool1, net.conv2, net.short3, net.conv6 };
+        std::stringstream file(std::ios::in | std::ios::out | std::ios::binary);
+        saveOptimizerState(file, OptimizerHeader{ 6400, 400, true }, layers);
+        const std::string bytes = file.str();
+        // header 4 + 8 + 8, conv0 and conv2: (bias m,v + scale m,v) * C floats, conv6: bias m,v * 2C floats
+        const size_t expect = 20 + 2 * (4 * C) * 4 + (2 * 2 * C) * 4;
+        report("optimizer sidecar size", bytes.size() == expect, std::to_string(bytes.size()) + " bytes");
+        std::uint32_t magic = 0;
+        std::memcpy(&magic, bytes.data(), 4);
+        report("optimizer sidecar magic", magic == 0x50584f32);
+        // conv2's scale moments sit after conv0's block and conv2's bias moments
+        const Host scaleM = readFloats(bytes, 20 + (4 * C) * 4 + (2 * C) * 4, C);
+        Host w = net.scale2, d = net.conv2->scaleUpdates().asVector();
+        (void) w; (void) d;
+        bool moved = false;
+        for (float v: scaleM) moved = moved || v != 0.0f;
+        report("conv2 scale moments are in their place", moved);
+
+        Net fresh(true);
+        const std::vector<Layer::Ptr> freshLayers{ fresh.conv0, fresh.pool1, fresh.conv2, fresh.short3, fresh.conv6 };
+        OptimizerHeader h;
+        std::stringstream again(bytes, std::ios::in | std::ios::binary);
+        report("sidecar of other weights is refused", !loadOptimizerState(again, 1234, h, freshLayers));
+        std::stringstream third(bytes, std::ios::in | std::ios::binary);
+        const bool loaded = loadOptimizerState(third, 6400, h, freshLayers);
+        report("sidecar header round trip", loaded && h.seen == 6400 && h.step == 400);
+        std::stringstream out(std::ios::in | std::ios::out | std::ios::binary);
+        saveOptimizerState(out, h, freshLayers);
+        report("sidecar round trip is byte identical", out.str() == bytes);
     }
 }
 
