@@ -1,0 +1,110 @@
+"""Seeded random geometries for the index-work kernels, bit for bit against the CPU checker:
+whatever kernel, stride, padding, size, channel mismatch or pointer alignment a model file can
+ask for has to give the CPU layer's result, not only the shapes of the shipped networks."""
+import numpy as np
+import pytest
+
+from pixienn_amd import workloads as wl
+from util import F, assert_bit_exact, gpu, host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from pixienn_amd import ops as o
+    return o
+
+
+def test_maxpool_random_geometries(ops, oracle):
+    import torch
+    r = np.random.default_rng(101)
+    done = 0
+    while done < 60:
+        k = int(r.integers(1, 5)); s = int(r.integers(1, 4)); p = int(r.integers(0, k + 1))
+        H = int(r.integers(1, 24)); W = int(r.integers(1, 24)); N = int(r.integers(1, 4)); C = int(r.integers(1, 6))
+        oh = oracle.maxpool_out_dim(H, k, s, p); ow = oracle.maxpool_out_dim(W, k, s, p)
+        if oh <= 0 or ow <= 0:
+            continue
+        done += 1
+        x = wl.normal(5000 + done, (N, C, H, W))
+        if done % 5 == 0:
+            x = np.round(x)            # ties: the first maximum in window order must win
+        want = np.empty((N, C, oh, ow), F); widx = np.empty((N, C, oh, ow), np.int32)
+        oracle.maxpool_forward(x, want, widx, N, C, H, W, oh, ow, k, s, p)
+        out = torch.full((N, C, oh, ow), 9.0, device="cuda")
+        idx = torch.full((N, C, oh, ow), -9, device="cuda", dtype=torch.int32)
+        ops.maxpool_forward(gpu(x), out, idx, k, s, p)
+        what = "maxpool %s k%d s%d p%d" % ((N, C, H, W), k, s, p)
+        assert_bit_exact(host(out), want, what + " values")
+        assert_bit_exact(host(idx), widx, what + " indexes")
+        delta = wl.normal(5100 + done, want.shape); grad0 = wl.normal(5200 + done, x.shape)
+        gw = grad0.copy()
+        oracle.maxpool_backward(delta, widx, gw)
+        gg = gpu(grad0)
+        ops.maxpool_backward(gpu(delta), idx, gg, k, s, p)
+        assert_bit_exact(host(gg), gw, what + " backward")
+
+
+def test_upsample_random_geometries(ops, oracle):
+    import torch
+    r = np.random.default_rng(102)
+    for case in range(40):
+        stride = int(r.integers(1, 5)); H = int(r.integers(1, 20)); W = int(r.integers(1, 20))
+        N = int(r.integers(1, 4)); C = int(r.integers(1, 6)); scale = float(r.choice([1.0, 0.5, 2.0, -1.25]))
+        x = wl.normal(5300 + case, (N, C, H, W))
+        want = np.empty((N, C, H * stride, W * stride), F)
+        oracle.upsample(x, W, H, C, N, stride, True, scale, None, want)
+        out = torch.full(want.shape, 7.0, device="cuda")
+        ops.upsample_forward(gpu(x), out, stride, scale)
+        what = "upsample %s stride %d scale %g" % ((N, C, H, W), stride, scale)
+        assert_bit_exact(host(out), want, what)
+        d = wl.normal(5400 + case, want.shape); acc0 = wl.normal(5500 + case, x.shape)
+        aw = acc0.copy()
+        oracle.upsample(None, W, H, C, N, stride, False, scale, aw, d.copy())
+        ga = gpu(acc0)
+        ops.upsample_backward(gpu(d), ga, stride, scale)
+        assert_bit_exact(host(ga), aw, what + " backward")
+
+
+def test_shortcut_random_shape_pairs(ops, oracle):
+    """shortcutGpu's index map: integer stride (out smaller than add's source) or sample (larger)."""
+    r = np.random.default_rng(103)
+    done = 0
+    while done < 40:
+        N = int(r.integers(1, 3)); h2 = int(r.integers(1, 7)); w2 = int(r.integers(1, 7))
+        f = int(r.integers(1, 4)); grow = bool(r.integers(0, 2))
+        w1, h1 = (w2 * f, h2 * f) if grow else (w2, h2)
+        w2, h2 = (w2, h2) if grow else (w2 * f, h2 * f)
+        c1 = int(r.integers(1, 6)); c2 = int(r.integers(1, 6))
+        add = wl.normal(5600 + done, (N, c1, h1, w1)); out0 = wl.normal(5700 + done, (N, c2, h2, w2))
+        want = out0.copy()
+        if oracle.shortcut(N, w1, h1, c1, add, w2, h2, c2, 0.75, 1.5, want) != 0:
+            continue
+        done += 1
+        g = gpu(out0)
+        ops.shortcut(N, w1, h1, c1, gpu(add), w2, h2, c2, 0.75, 1.5, g)
+        assert_bit_exact(host(g), want, "shortcut %s into %s" % ((N, c1, h1, w1), (N, c2, h2, w2)))
+
+
+def test_streaming_kernels_with_unaligned_views(ops, oracle):
+    """Pointers 4, 8 and 12 bytes off a 16-byte boundary take the scalar kernels: same bits."""
+    import torch
+    n = 4099
+    for off in (1, 2, 3):
+        a = wl.normal(5800 + off, n + off); b = wl.normal(5810 + off, n + off)
+        ga = gpu(a)[off:]; gb = gpu(b)[off:]
+        out = torch.zeros(n + off, device="cuda")[off:]
+        ops.shortcut_forward(ga.view(1, 1, 1, n), gb.view(1, 1, 1, n), out.view(1, 1, 1, n), "leaky")
+        want = np.empty(n, F); pre = np.empty(n, F)
+        oracle.shortcut_forward("leaky", 1, n, 1, 1, a[off:].copy(), b[off:].copy(), 1.0, 1.0, want, pre)
+        assert_bit_exact(host(out), want, "shortcut forward at offset %d" % off)
+        w = a[off:].copy(); d = b[off:].copy()
+        oracle.sgd_update(w, d, 4, 1e-2, 0.9, 1e-3, True)
+        gw = gpu(a)[off:]; gd = gpu(b)[off:]
+        ops.sgd_update(gw, gd, 4, 1e-2, 0.9, 1e-3, True)
+        assert np.allclose(host(gw), w, rtol=1e-6, atol=1e-7) and np.allclose(host(gd), d, rtol=1e-6, atol=1e-7)
+        route = torch.full((2, 3 * n), -1.0, device="cuda")
+        src = gpu(np.stack([a[off:], b[off:]]))
+        ops.route_forward(src, route, n + 1)           # an odd offset inside the concatenation
+        assert torch.equal(route[:, n + 1:2 * n + 1], src) and float(route[:, :n + 1].max()) == -1.0
