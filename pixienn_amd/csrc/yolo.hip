@@ -250,8 +250,9 @@ __device__ __forceinline__ TruthSlot make_truth_slot(const float* __restrict__ g
 
 // probability of class row `c` of the slot at `base`, exactly as the class sweep computes it
 template<bool FUSED>
-__device__ __forceinline__ float class_prob(const float* in, size_t base, int c, int area)
+__device__ __forceinline__ float class_prob(const float* in, size_t base, int c, int area, int classes)
 {
+    if (c < 0 || c >= classes) return 0.0f;      // a label outside the class range reads nothing
     const float v = in[base + (5 + static_cast<size_t>(c)) * area];
     if constexpr (FUSED) return sigmoid_fast(v);
     else return v;
@@ -301,7 +302,8 @@ __device__ __forceinline__ double head_tile(const uint32_t head_block, const Hea
     const size_t base = (static_cast<size_t>(bn) * entries) * area + (live ? cell : 0);
 
     // issued first, used last: the truth count and this lane's truth do not depend on each other
-    const int count = a.truth_counts[b];
+    // a count beyond the table's rows must not read past them
+    const int count = min(a.truth_counts[b], p.max_truth);
     const float* image_truths = a.truths + static_cast<size_t>(b) * p.max_truth * 5;
 
     int mask_anchor;
@@ -402,7 +404,7 @@ __device__ __forceinline__ double head_tile(const uint32_t head_block, const Hea
                             const TruthSlot& ts = tile[k0 + u];
                             pos_cls = ts.cls;
                             pos_box = Box{ ts.x, ts.y, ts.w, ts.h };
-                            st_cat += fminf(1.0f, class_prob<FUSED>(in, base, ts.cls, area));
+                            st_cat += fminf(1.0f, class_prob<FUSED>(in, base, ts.cls, area, p.classes));
                             st_iou += iou[u];
                             if (iou[u] > .5f) st_r50 += 1.0f;
                             if (iou[u] > .75f) st_r75 += 1.0f;
@@ -431,7 +433,7 @@ __device__ __forceinline__ double head_tile(const uint32_t head_block, const Hea
                 st_r75 = iou > .75f ? 1.0f : 0.0f;
                 st_obj = so;
                 st_count = 1.0f;
-                st_cat = fminf(1.0f, class_prob<FUSED>(in, base, acls, area));
+                st_cat = fminf(1.0f, class_prob<FUSED>(in, base, acls, area, p.classes));
             }
         }
     }
@@ -450,7 +452,7 @@ __device__ __forceinline__ double head_tile(const uint32_t head_block, const Hea
             cls = static_cast<int>(g[4]);
             bd = box_delta(Box{ g[0], g[1], g[2], g[3] }, sx, sy, rw, rh, i, j, aw, ah, p);
             // deltaYoloClass also feeds the class-probability statistic on this path
-            if constexpr (FUSED) st_cat += fminf(1.0f, class_prob<FUSED>(in, base, cls, area));
+            if constexpr (FUSED) st_cat += fminf(1.0f, class_prob<FUSED>(in, base, cls, area, p.classes));
         }
         if (pos_cls >= 0) {
             float paw = aw, pah = ah;
