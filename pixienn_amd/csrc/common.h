@@ -127,11 +127,12 @@ __device__ __forceinline__ float act_apply(float x)
     if constexpr (ACT == PXH_LEAKY) return x > 0.0f ? x : 0.1f * x;
     else if constexpr (ACT == PXH_LINEAR) return x;
     else if constexpr (ACT == PXH_LOGGY) return 2.0f / (1.0f + expf(-x)) - 1.0f;
-    else if constexpr (ACT == PXH_LOGISTIC) return 1.0f / (1.0f + expf(-x));
+    // logistic and swish: the accurate exp, then a hardware reciprocal (1 ulp) in place of the division
+    else if constexpr (ACT == PXH_LOGISTIC) return __builtin_amdgcn_rcpf(1.0f + expf(-x));
     else if constexpr (ACT == PXH_MISH) return mish_apply(x);
     else if constexpr (ACT == PXH_RELU) return x > 0.0f ? x : 0.0f;
     else if constexpr (ACT == PXH_SOFTPLUS) return softplus_apply(x);
-    else if constexpr (ACT == PXH_SWISH) return x / (1.0f + expf(-1.0f * x));
+    else if constexpr (ACT == PXH_SWISH) return x * __builtin_amdgcn_rcpf(1.0f + expf(-1.0f * x));
     else return tanhf(x);
 }
 
