@@ -9,11 +9,12 @@
 //          Instruction and latency bound: ~1000 vector instructions per wave.
 //   class  the class rows, 94 % of the tensor: logit -> probability -> `out`, and the dense class
 //          delta.  Bandwidth bound, 12 bytes per element.
-// From raw logits (pxh_yolo_forward_train) both run in ONE grid, persistent head workgroups beside
-// the class stream, followed by a small kernel that writes the class delta of the supervised
-// slots and adds up the sums in a fixed order.  From an already decoded head with host-assigned
-// positives (pxh_yolo_loss, the reference's argument list) a head kernel is followed by a class
-// kernel that takes the decisions.  pxh_yolo_detections is the inference-side compaction.
+// Both run in ONE grid, persistent head workgroups beside the class stream, followed by a small
+// kernel that writes the class delta of the supervised slots and adds up the sums in a fixed order.
+// pxh_yolo_forward_train starts from raw logits and assigns the positives on the device;
+// pxh_yolo_loss (the reference's argument list) starts from a decoded head and host-assigned
+// positives, its class stream only writes the zero delta.  pxh_yolo_detections is the
+// inference-side compaction.
 // Box arithmetic follows the CPU layer (include/YoloLayer.h, src/DarkBox.cpp of the reference).
 #include "stream.h"
 
@@ -525,16 +526,6 @@ __device__ __forceinline__ double head_tile(const uint32_t head_block, const Hea
     return total;
 }
 
-// One workgroup per head tile (the decoded-input form of the reference's signature).
-template<bool FUSED>
-__global__ __launch_bounds__(kBlock) void yolo_head_kernel(HeadArgs a, YoloParams p, YoloTables tb)
-{
-    __shared__ TruthSlot tile[kTruthTile];
-    __shared__ double wave_sums[kSums][kWaves];
-    const double total = head_tile<FUSED>(blockIdx.x, a, p, tb, tile, wave_sums);
-    if (threadIdx.x < kSums) a.partial[static_cast<size_t>(threadIdx.x) * gridDim.x + blockIdx.x] = total;   // [12][n]
-}
-
 // The class rows as a flat index space over [batch*mask][classes][area] (the 5 head rows of every
 // anchor are skipped).
 struct ClassSpace {
@@ -595,31 +586,6 @@ __device__ __forceinline__ void finish_statistic(int k, const ClassArgs& a, doub
     }
 }
 
-// The decoded-input form: dense class delta from the slots' decisions.
-// V = 4 needs area % 4 == 0 (a vector then never leaves its row) and 16-byte aligned tensors.
-template<int V, bool NT>
-__global__ __launch_bounds__(kBlock) void yolo_class_kernel(ClassArgs a)
-{
-    __shared__ double slots[kBlock / kWave];
-    if (blockIdx.x < 13) finish_statistic(blockIdx.x, a, slots);
-    const uint32_t e = (blockIdx.x * kBlock + threadIdx.x) * V;
-    if (e >= a.space.elems) return;
-    uint32_t bn, c, cell;
-    a.space.locate(e, bn, c, cell);
-    const size_t at = a.space.offset(bn, c, cell);
-    const IPack<V> cls = ldi<V, false>(a.decision, static_cast<size_t>(bn) * a.space.area + cell);
-    Pack<V> d;
-#pragma unroll
-    for (int k = 0; k < V; ++k) {
-        d.v[k] = 0.0f;
-        if (cls.v[k] >= 0) {      // rare: a supervised slot
-            const float t = (static_cast<int>(c) == cls.v[k]) ? 1.0f : 0.0f;
-            d.v[k] = a.class_scale * (t - a.in[at + k]);
-        }
-    }
-    st<V, NT>(a.delta, at, d);
-}
-
 // ---- fused pass: persistent head workgroups + class decode stream in one grid ------------------
 // The head tiles are instruction bound and the class stream is bandwidth bound, so they run side
 // by side: the first `head_workers` workgroups of the grid (dispatched first, a few per compute
@@ -632,8 +598,10 @@ struct FusedArgs {
     uint32_t head_workers;
 };
 
+// FUSED: raw logits in, the class stream decodes them.  !FUSED (the reference's yoloLossGpu
+// argument list): the head is already decoded and the class stream only writes the zero delta.
 // Eight waves per SIMD (at most 64 vector registers): the class stream needs the occupancy.
-template<int V, bool NT>
+template<bool FUSED, int V, bool NT>
 __global__ __launch_bounds__(kBlock, 8) void yolo_fused_kernel(FusedArgs a, YoloParams p, YoloTables tb)
 {
     __shared__ TruthSlot tile[kTruthTile];
@@ -642,7 +610,7 @@ __global__ __launch_bounds__(kBlock, 8) void yolo_fused_kernel(FusedArgs a, Yolo
         // one sum per worker and statistic, over its tiles in walking order
         double total = 0.0;
         for (uint32_t t = blockIdx.x; t < p.blocks; t += a.head_workers) {
-            total += head_tile<true>(t, a.head, p, tb, tile, wave_sums);
+            total += head_tile<FUSED>(t, a.head, p, tb, tile, wave_sums);
             __syncthreads();      // wave_sums is read by the first lanes until here
         }
         if (threadIdx.x < kSums)
@@ -654,14 +622,16 @@ __global__ __launch_bounds__(kBlock, 8) void yolo_fused_kernel(FusedArgs a, Yolo
     uint32_t bn, c, cell;
     a.space.locate(e, bn, c, cell);
     const size_t at = a.space.offset(bn, c, cell);
-    const Pack<V> x = ld<V, NT>(a.head.in, at);
-    Pack<V> prob, zero;
+    Pack<V> zero;
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-        prob.v[k] = sigmoid_fast(x.v[k]);
-        zero.v[k] = 0.0f;
+    for (int k = 0; k < V; ++k) zero.v[k] = 0.0f;
+    if constexpr (FUSED) {
+        const Pack<V> x = ld<V, NT>(a.head.in, at);
+        Pack<V> prob;
+#pragma unroll
+        for (int k = 0; k < V; ++k) prob.v[k] = sigmoid_fast(x.v[k]);
+        st<V, NT>(a.head.out, at, prob);
     }
-    st<V, NT>(a.head.out, at, prob);
     st<V, NT>(a.head.delta, at, zero);
 }
 
@@ -921,32 +891,21 @@ int run_training_pass(const char* who, const float* in, float* out, float* delta
     ca.accumulate = accumulate;
     const HeadArgs ha{ in, out, delta, truths, truth_counts, w.decision, w.partial };
 
-    if constexpr (FUSED) {
-        const double stream_us = static_cast<double>(space.elems) * 12.0 / 6.0e6;   // class stream at 6 TB/s
-        FusedArgs fa{ ha, space, head_workers(p.blocks, stream_us) };
-        ca.head_blocks = fa.head_workers;      // one partial sum per worker
-        const uint32_t grid = fa.head_workers + class_blocks;
-        const bool nt = static_cast<size_t>(space.elems) * 12 >= kStreamingBytes;
-        if (vec && nt) hipLaunchKernelGGL((yolo_fused_kernel<4, true>), dim3(grid), dim3(kBlock), 0, s, fa, p, tb);
-        else if (vec) hipLaunchKernelGGL((yolo_fused_kernel<4, false>), dim3(grid), dim3(kBlock), 0, s, fa, p, tb);
-        else hipLaunchKernelGGL((yolo_fused_kernel<1, false>), dim3(grid), dim3(kBlock), 0, s, fa, p, tb);
-        int rc = check_launch(who);
-        if (rc) return rc;
-        PatchArgs pa{ ca, static_cast<uint32_t>(p.batch) * p.mask_count * p.area, p.classes };
-        const uint32_t pgrid = grid_for(pa.slots, kBlock);
-        hipLaunchKernelGGL(yolo_patch_kernel, dim3(pgrid < 13 ? 13 : pgrid), dim3(kBlock), 0, s, pa);
-        return check_launch(who);
-    } else {
-        hipLaunchKernelGGL((yolo_head_kernel<false>), dim3(p.blocks), dim3(kBlock), 0, s, ha, p, tb);
-        int rc = check_launch(who);
-        if (rc) return rc;
-        const uint32_t grid = class_blocks < 13 ? 13 : class_blocks;
-        const bool nt = static_cast<size_t>(space.elems) * 4 >= kStreamingBytes;
-        if (vec && nt) hipLaunchKernelGGL((yolo_class_kernel<4, true>), dim3(grid), dim3(kBlock), 0, s, ca);
-        else if (vec) hipLaunchKernelGGL((yolo_class_kernel<4, false>), dim3(grid), dim3(kBlock), 0, s, ca);
-        else hipLaunchKernelGGL((yolo_class_kernel<1, false>), dim3(grid), dim3(kBlock), 0, s, ca);
-        return check_launch(who);
-    }
+    const int stream_bytes = FUSED ? 12 : 4;      // per class element: read + decode + zero delta, or the zero delta alone
+    const double stream_us = static_cast<double>(space.elems) * stream_bytes / 6.0e6;   // at 6 TB/s
+    FusedArgs fa{ ha, space, head_workers(p.blocks, stream_us) };
+    ca.head_blocks = fa.head_workers;      // one partial sum per worker
+    const uint32_t grid = fa.head_workers + class_blocks;
+    const bool nt = static_cast<size_t>(space.elems) * stream_bytes >= kStreamingBytes;
+    if (vec && nt) hipLaunchKernelGGL((yolo_fused_kernel<FUSED, 4, true>), dim3(grid), dim3(kBlock), 0, s, fa, p, tb);
+    else if (vec) hipLaunchKernelGGL((yolo_fused_kernel<FUSED, 4, false>), dim3(grid), dim3(kBlock), 0, s, fa, p, tb);
+    else hipLaunchKernelGGL((yolo_fused_kernel<FUSED, 1, false>), dim3(grid), dim3(kBlock), 0, s, fa, p, tb);
+    int rc = check_launch(who);
+    if (rc) return rc;
+    PatchArgs pa{ ca, static_cast<uint32_t>(p.batch) * p.mask_count * p.area, p.classes };
+    const uint32_t pgrid = grid_for(pa.slots, kBlock);
+    hipLaunchKernelGGL(yolo_patch_kernel, dim3(pgrid < 13 ? 13 : pgrid), dim3(kBlock), 0, s, pa);
+    return check_launch(who);
 }
 
 }  // namespace
