@@ -239,6 +239,16 @@ def measure_extras(torch, ops, wl, timer, capi):
             cost, NB, 80, s, s, 608, 608, 0.7, 1.0, 1.0, 2.0, 0.1, 1.0), 20, rotate=rot)
         add("yolo_decode+delta+cost", "%dx255x%d^2" % (NB, s), 12 * e, ms_t, "fused 12B/elem")
         head_ms[s] = (ms_d, ms_t)
+        # the reference's own split: loss from the decoded head with host-assigned positives
+        acls, aanc, abox = wl.yolo_assign_targets(truths_np, counts_np, wl.YOLOV3_MASKS[s], wl.YOLOV3_ANCHORS, s, s,
+                                                  608, 608)
+        tabs = [torch.from_numpy(t).to(dev) for t in (acls, aanc, abox)]
+        gmasks = torch.tensor(wl.YOLOV3_MASKS[s], device=dev, dtype=torch.int32)
+        ganch = torch.tensor(wl.YOLOV3_ANCHORS, device=dev, dtype=torch.float32)
+        ms_l = timer.time(lambda i: ops.yolo_loss(out[i], dl[i], truths, counts, truths.shape[1], tabs[0], tabs[1],
+                                                  tabs[2], gmasks, ganch, stats, cost, NB, 9, 80, s, s, 608, 608,
+                                                  0.7, 1.0, 1.0, 2.0, 0.1, 1.0), 20, rotate=rot)
+        add("yolo_delta+cost", "%dx255x%d^2" % (NB, s), (4 + 4 * 5 / 85) * e, ms_l, "decoded input, 4.24B/elem")
         if s == 76:
             # detections of the decoded head at a confidence threshold of 0.5: the objectness row of every
             # slot, the box and class rows of the slots that pass (about half of them on these logits)

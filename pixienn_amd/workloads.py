@@ -61,3 +61,37 @@ def yolo_truths(seed, batch, max_boxes=20, classes=80):
         truths[b, :k, 2:4] = np.exp(g.uniform(np.log(0.02), np.log(0.9), (k, 2)))
         truths[b, :k, 4] = g.integers(0, classes, k)
     return truths, counts
+
+
+def yolo_assign_targets(truths, counts, masks, anchors, width, height, net_width, net_height):
+    """Host-side positive assignment for the decoded-input loss entry point, as the reference's
+    target builder does it (src/YoloTargetBuilder.cpp:21-62): every truth goes to the anchor whose
+    origin-centred box overlaps its own best; if this head owns that anchor, the slot at the
+    truth's cell takes its class, anchor and box (a later truth overwrites an earlier one).
+    Returns (classes[slots], anchors[slots], boxes[slots, 4]) with slots = batch * masks * area."""
+    batch = truths.shape[0]
+    area = width * height
+    slots = batch * len(masks) * area
+    cls = np.full(slots, -1, np.int32)
+    anc = np.full(slots, -1, np.int32)
+    box = np.zeros((slots, 4), np.float32)
+    aw = np.asarray(anchors[0::2], np.float32) / np.float32(net_width)
+    ah = np.asarray(anchors[1::2], np.float32) / np.float32(net_height)
+    for b in range(batch):
+        for t in range(int(counts[b])):
+            x, y, w, h, c = truths[b, t]
+            if w <= 0 or h <= 0:
+                continue
+            inter = np.minimum(aw, w) * np.minimum(ah, h)
+            iou = inter / (aw * ah + w * h - inter)
+            best = int(np.argmax(iou))
+            if best not in masks:
+                continue
+            n = list(masks).index(best)
+            i = min(width - 1, max(0, int(x * width)))
+            j = min(height - 1, max(0, int(y * height)))
+            s = (b * len(masks) + n) * area + j * width + i
+            cls[s] = int(c)
+            anc[s] = best
+            box[s] = (x, y, w, h)
+    return cls, anc, box
