@@ -394,6 +394,9 @@ def main():
         sys.exit(2)
     import torch
     from pixienn_amd import capi, ops, workloads as wl
+    if not os.path.exists(capi.LIB_PATH):
+        from pixienn_amd import build
+        build.build_library()      # nothing built yet: build; there is no other path
     capi.load()      # fails loudly when the HIP library is missing
     assert torch.cuda.is_available(), "no GPU visible"
     torch.cuda.set_device(0)

@@ -13,6 +13,14 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """The tests load what is built; only when nothing is built do they build it."""
+    from pixienn_amd import capi
+    if not os.path.exists(capi.LIB_PATH):
+        from pixienn_amd import build
+        build.build_library()
+
+
 @pytest.fixture(scope="session")
 def kats():
     with open(os.path.join(ROOT, "tests", "golden", "reference_kats.json")) as f:
