@@ -189,6 +189,14 @@ int pxh_maxpool_backward_scatter(const float* delta, const int* indexes, float* 
  * ---------------------------------------------------------------------- */
 int pxh_upsample(const float* in, int w, int h, int c, int batch, int stride, int forward,
                  float scale, float* acc, float* out, void* stream);
+/* The same with the large tensor (`out`) being a channel slice of a wider one: image n of it starts at
+ * out + n * out_image_stride (elements, >= c*h*w*stride^2).  With `out` pointing at a channel offset
+ * inside the buffer of the route layer that follows (include/RouteLayer.h:91-137), the upsampled
+ * tensor lands directly in the concatenation and the route copy of this source is not needed;
+ * backward reads the route's delta slice in place. */
+int pxh_upsample_strided(const float* in, int w, int h, int c, int batch, int stride, int forward,
+                         float scale, float* acc, float* out, long long out_image_stride,
+                         void* stream);
 
 /* ------------------------------------------------------------------------
  * Shortcut.  include/ShortcutKernel.cuh:21-22, CPU semantics include/ShortcutLayer.h:84-141.

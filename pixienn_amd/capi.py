@@ -17,6 +17,7 @@ P = ctypes.c_void_p
 I = ctypes.c_int
 F = ctypes.c_float
 Z = ctypes.c_size_t
+L = ctypes.c_longlong
 
 # name -> argument types (every function returns int unless listed in _OTHER_RETURNS)
 SIGNATURES = {
@@ -43,6 +44,7 @@ SIGNATURES = {
     "pxh_maxpool_backward": [P, P, P, I, I, I, I, I, I, I, I, I, P],
     "pxh_maxpool_backward_scatter": [P, P, P, I, P],
     "pxh_upsample": [P, I, I, I, I, I, I, F, P, P, P],
+    "pxh_upsample_strided": [P, I, I, I, I, I, I, F, P, P, L, P],
     "pxh_shortcut": [I, I, I, I, P, I, I, I, F, F, P, P],
     "pxh_shortcut_forward": [P, P, P, P, Z, F, F, I, P],
     "pxh_shortcut_backward": [P, P, P, P, Z, F, F, I, P],

@@ -251,11 +251,20 @@ __global__ __launch_bounds__(kBlock) void maxpool_bwd_scatter_kernel(const float
 }
 
 // ------------------------------------------------------------------ upsample
+// The large tensor may be a channel slice of a wider one (a concatenation buffer): image n then
+// starts `extra` elements later than in a dense tensor, for every image before it.
+struct ImageGap {
+    FastDiv by_channels;
+    uint32_t extra;     // image stride of the large tensor minus channels * its plane size
+    __device__ uint32_t of_plane(uint32_t plane) const { return extra ? by_channels.div(plane) * extra : 0u; }
+};
+
 // stride 2: VX inputs per lane; forward writes the 2 x (2*VX) block, backward folds it into the
 // input cell as (((acc + s*o00) + s*o01) + s*o10) + s*o11, the raster order of the CPU loop.
 template<int VX, bool FORWARD>
 __global__ __launch_bounds__(kBlock) void upsample2_kernel(const float* in, float* acc, float* out, uint32_t units,
-                                                           int w, float scale, FastDiv by_wv, FastDiv by_h)
+                                                           int w, float scale, FastDiv by_wv, FastDiv by_h,
+                                                           ImageGap gap)
 {
     const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
     if (t >= units) return;
@@ -265,7 +274,7 @@ __global__ __launch_bounds__(kBlock) void upsample2_kernel(const float* in, floa
     const uint32_t x = xv * VX;
     const uint32_t ii = rows * w + x;                                   // rows = plane*h + y
     const uint32_t ow = 2 * w;
-    const uint32_t oi = (2 * rows) * ow + 2 * x;                        // (plane*2h + 2y)*2w + 2x
+    const uint32_t oi = (2 * rows) * ow + 2 * x + gap.of_plane(plane);  // (plane*2h + 2y)*2w + 2x
     if constexpr (FORWARD) {
         const Pack<VX> v = ld<VX>(in, ii);
         Pack<2 * VX> o;
@@ -302,14 +311,15 @@ __global__ __launch_bounds__(kBlock) void upsample2_kernel(const float* in, floa
 template<bool FORWARD>
 __global__ __launch_bounds__(kBlock) void upsample_generic_kernel(const float* in, float* acc, float* out,
                                                                   uint32_t total, int w, int stride, float scale,
-                                                                  FastDiv by_w)
+                                                                  FastDiv by_w, FastDiv by_h, ImageGap gap)
 {
     const uint32_t cell = blockIdx.x * kBlock + threadIdx.x;
     if (cell >= total) return;
-    uint32_t rows, x;
+    uint32_t rows, x, plane, y;
     by_w.divmod(cell, rows, x);
+    by_h.divmod(rows, plane, y);
     const size_t ow = static_cast<size_t>(w) * stride;
-    const size_t o0 = static_cast<size_t>(rows) * stride * ow + static_cast<size_t>(x) * stride;
+    const size_t o0 = static_cast<size_t>(rows) * stride * ow + static_cast<size_t>(x) * stride + gap.of_plane(plane);
     if constexpr (FORWARD) {
         const float s = scale * in[cell];
         for (int dy = 0; dy < stride; ++dy)
@@ -451,28 +461,32 @@ int pxh_maxpool_backward_scatter(const float* delta, const int* indexes, float* 
     return check_launch("pxh_maxpool_backward_scatter");
 }
 
-int pxh_upsample(const float* in, int w, int h, int c, int batch, int stride, int forward, float scale, float* acc,
-                 float* out, void* stream)
+int pxh_upsample_strided(const float* in, int w, int h, int c, int batch, int stride, int forward, float scale,
+                         float* acc, float* out, long long out_image_stride, void* stream)
 {
     if (w <= 0 || h <= 0 || c <= 0 || batch <= 0 || stride <= 0)
         return fail_invalid("pxh_upsample: dimensions and stride must be positive");
     if (!out || (forward && !in) || (!forward && !acc)) return fail_invalid("pxh_upsample: null pointer");
-    const unsigned long long out_total = 1ull * batch * c * h * w * stride * stride;
-    if (out_total >= (1ull << 31)) {
+    const unsigned long long image = 1ull * c * h * w * stride * stride;
+    if (out_image_stride < 0 || static_cast<unsigned long long>(out_image_stride) < image)
+        return fail_invalid("pxh_upsample: image stride %lld is smaller than one upsampled image (%llu)",
+                            out_image_stride, image);
+    if (1ull * batch * static_cast<unsigned long long>(out_image_stride) >= (1ull << 31)) {
         set_error("pxh_upsample: tensors of 2^31 elements or more are not supported");
         return PXH_ERR_UNSUPPORTED;
     }
     hipStream_t s = as_stream(stream);
     const uint32_t total = static_cast<uint32_t>(batch) * c * h * w;
+    const ImageGap gap{ FastDiv(c), static_cast<uint32_t>(static_cast<unsigned long long>(out_image_stride) - image) };
     const float* small = forward ? in : acc;
-    if (stride == 2 && aligned16(small) && aligned16(out)) {
+    if (stride == 2 && aligned16(small) && aligned16(out) && gap.extra % 4 == 0) {
         // VX inputs per lane; the input vector needs 4*VX-byte alignment of every row start
         const int vx = (w % 4 == 0) ? 4 : (w % 2 == 0 ? 2 : 1);
         const uint32_t units = total / vx;
         const dim3 grid(grid_for(units, kBlock));
 #define PXH_UPSAMPLE2(VX, FWD)                                                                              \
         hipLaunchKernelGGL((upsample2_kernel<VX, FWD>), grid, dim3(kBlock), 0, s, in, acc, out, units, w, \
-                           scale, FastDiv(w / VX), FastDiv(h))
+                           scale, FastDiv(w / VX), FastDiv(h), gap)
         if (forward) {
             if (vx == 4) PXH_UPSAMPLE2(4, true); else if (vx == 2) PXH_UPSAMPLE2(2, true); else PXH_UPSAMPLE2(1, true);
         } else {
@@ -484,12 +498,21 @@ int pxh_upsample(const float* in, int w, int h, int c, int batch, int stride, in
     const dim3 grid(grid_for(total, kBlock));
     if (forward) {
         hipLaunchKernelGGL((upsample_generic_kernel<true>), grid, dim3(kBlock), 0, s, in, acc, out, total, w, stride,
-                           scale, FastDiv(w));
+                           scale, FastDiv(w), FastDiv(h), gap);
     } else {
         hipLaunchKernelGGL((upsample_generic_kernel<false>), grid, dim3(kBlock), 0, s, in, acc, out, total, w, stride,
-                           scale, FastDiv(w));
+                           scale, FastDiv(w), FastDiv(h), gap);
     }
     return check_launch("pxh_upsample");
+}
+
+int pxh_upsample(const float* in, int w, int h, int c, int batch, int stride, int forward, float scale, float* acc,
+                 float* out, void* stream)
+{
+    if (w <= 0 || h <= 0 || c <= 0 || batch <= 0 || stride <= 0)
+        return fail_invalid("pxh_upsample: dimensions and stride must be positive");
+    return pxh_upsample_strided(in, w, h, c, batch, stride, forward, scale, acc, out,
+                                1ll * c * h * w * stride * stride, stream);
 }
 
 }

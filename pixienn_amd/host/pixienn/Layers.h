@@ -298,6 +298,11 @@ public:
     {
         Layer::forward(input);
         checkInput(input, "UpsampleLayer");
+        if (outSlice_) {
+            PX_HIP_CHECK(pxh_upsample_strided(input.data(), width(), height(), channels(), batch(), stride_, 1, scale_,
+                                              nullptr, outSlice_, imageStride_, stream()));
+            return;
+        }
         PX_HIP_CHECK(pxh_upsample(input.data(), width(), height(), channels(), batch(), stride_, 1, scale_, nullptr,
                                   output_.data(), stream()));
     }
@@ -306,13 +311,37 @@ public:
     {
         Layer::backward(input, grad);
         if (grad == nullptr) return;
+        if (outSlice_) {
+            PX_HIP_CHECK(pxh_upsample_strided(nullptr, width(), height(), channels(), batch(), stride_, 0, scale_,
+                                              grad->data(), deltaSlice_, imageStride_, stream()));
+            return;
+        }
         PX_HIP_CHECK(pxh_upsample(nullptr, width(), height(), channels(), batch(), stride_, 0, scale_, grad->data(),
                                   delta_.data(), stream()));
     }
 
+    // The route layer that is this layer's only consumer hands over the channel slice of its own
+    // buffers where the upsampled tensor belongs (image n at slice + n * imageStride): forward
+    // writes there, backward reads the delta there, and this layer's own tensors are released.
+    void writeInto(float* outSlice, float* deltaSlice, long long imageStride)
+    {
+        PX_CHECK(outSlice != nullptr && imageStride >= outputs(), "upsample: bad slice to write into");
+        PX_CHECK(!training() || deltaSlice != nullptr, "upsample: a training layer needs the delta slice too");
+        outSlice_ = outSlice;
+        deltaSlice_ = deltaSlice;
+        imageStride_ = imageStride;
+        output_ = V();
+        delta_ = V();
+    }
+
+    bool writesIntoConsumer() const noexcept { return outSlice_ != nullptr; }
+
 private:
     int stride_ = 2;
     float scale_ = 1.0f;
+    float* outSlice_ = nullptr;
+    float* deltaSlice_ = nullptr;
+    long long imageStride_ = 0;
 };
 
 // ---------------------------------------------------------------- shortcut
@@ -396,15 +425,32 @@ public:
             outChannels += layer->outChannels();
         }
         setOutput(outChannels, oh, ow);
+        // "absorb_upsample": an upsample layer among the sources, read by no other layer, writes
+        // straight into its channel slice here, which saves its copy in both directions.  The
+        // caller vouches for "no other reader"; the reference's graphs (yolov3.yml, yolov3-tiny.yml)
+        // meet it: every upsample is followed by the route that reads it.
+        absorbed_.assign(layers_.size(), false);
+        if (props.get<bool>("absorb_upsample", false)) {
+            int offset = 0;
+            for (std::size_t i = 0; i < layers_.size(); ++i) {
+                if (auto* up = dynamic_cast<UpsampleLayer*>(layers_[i].get())) {
+                    up->writeInto(output_.data() + offset, training() ? delta_.data() + offset : nullptr, outputs());
+                    absorbed_[i] = true;
+                }
+                offset += layers_[i]->outputs();
+            }
+        }
     }
 
     void forward(const V& input) override
     {
         Layer::forward(input);
         int offset = 0;
-        for (const auto& layer: layers_) {
-            PX_HIP_CHECK(pxh_route_forward(layer->output().data(), output_.data(), batch(), layer->outputs(),
-                                           outputs(), offset, stream()));
+        for (std::size_t i = 0; i < layers_.size(); ++i) {
+            const auto& layer = layers_[i];
+            if (!absorbed_[i])
+                PX_HIP_CHECK(pxh_route_forward(layer->output().data(), output_.data(), batch(), layer->outputs(),
+                                               outputs(), offset, stream()));
             offset += layer->outputs();
         }
     }
@@ -413,15 +459,18 @@ public:
     {
         Layer::backward(input, grad);
         int offset = 0;
-        for (const auto& layer: layers_) {
-            PX_HIP_CHECK(pxh_route_backward(delta_.data(), layer->delta().data(), batch(), layer->outputs(),
-                                            outputs(), offset, stream()));
+        for (std::size_t i = 0; i < layers_.size(); ++i) {
+            const auto& layer = layers_[i];
+            if (!absorbed_[i])
+                PX_HIP_CHECK(pxh_route_backward(delta_.data(), layer->delta().data(), batch(), layer->outputs(),
+                                                outputs(), offset, stream()));
             offset += layer->outputs();
         }
     }
 
 private:
     std::vector<Layer::Ptr> layers_;
+    std::vector<bool> absorbed_;
 };
 
 // ---------------------------------------------------------------- detections

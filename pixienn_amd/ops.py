@@ -228,6 +228,32 @@ def upsample_backward(delta, grad, stride=2, scale=1.0):
     call("pxh_upsample", None, w, h, c, n, stride, 0, float(scale), ptr(grad), ptr(delta), _stream())
 
 
+def upsample_forward_into(x, buffer, channel_offset, stride=2, scale=1.0):
+    """Upsample x straight into channels [channel_offset, channel_offset + C) of a wider NCHW buffer."""
+    _chk_all(x, buffer)
+    n, c, h, w = x.shape
+    plane = buffer.shape[2] * buffer.shape[3]
+    if buffer.shape[0] != n or buffer.shape[2] != h * stride or buffer.shape[3] != w * stride \
+            or channel_offset < 0 or channel_offset + c > buffer.shape[1]:
+        raise ValueError("buffer %s cannot hold %s upsampled by %d at channel %d"
+                         % (tuple(buffer.shape), tuple(x.shape), stride, channel_offset))
+    call("pxh_upsample_strided", ptr(x), w, h, c, n, stride, 1, float(scale), None,
+         ptr(buffer) + 4 * channel_offset * plane, buffer.shape[1] * plane, _stream())
+
+
+def upsample_backward_from(buffer_delta, channel_offset, grad, stride=2, scale=1.0):
+    """Backward of upsample_forward_into: reads the delta slice of the wider buffer in place."""
+    _chk_all(buffer_delta, grad)
+    n, c, h, w = grad.shape
+    plane = buffer_delta.shape[2] * buffer_delta.shape[3]
+    if buffer_delta.shape[0] != n or buffer_delta.shape[2] != h * stride or buffer_delta.shape[3] != w * stride \
+            or channel_offset < 0 or channel_offset + c > buffer_delta.shape[1]:
+        raise ValueError("buffer %s does not hold %s upsampled by %d at channel %d"
+                         % (tuple(buffer_delta.shape), tuple(grad.shape), stride, channel_offset))
+    call("pxh_upsample_strided", None, w, h, c, n, stride, 0, float(scale), ptr(grad),
+         ptr(buffer_delta) + 4 * channel_offset * plane, buffer_delta.shape[1] * plane, _stream())
+
+
 def shortcut(batch, w1, h1, c1, add, w2, h2, c2, s1, s2, out):
     _chk_all(add, out)
     call("pxh_shortcut", batch, w1, h1, c1, ptr(add), w2, h2, c2, float(s1), float(s2), ptr(out), _stream())

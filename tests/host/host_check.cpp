@@ -510,6 +510,54 @@ void trainingChecks()
     }
 }
 
+// An upsample layer absorbed by the route that reads it gives the same tensors as the two-step form.
+void absorbedUpsampleChecks()
+{
+    struct Pair {
+        Context ctx;
+        std::shared_ptr<UpsampleLayer> up;
+        std::shared_ptr<MaxPoolLayer> pool;
+        std::shared_ptr<RouteLayer> route;
+        explicit Pair(bool absorb)
+        {
+            ctx.training = true;
+            up = std::make_shared<UpsampleLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S / 2 },
+                                                                  { "width", S / 2 }, { "stride", 2 },
+                                                                  { "scale", 0.5f } });
+            pool = std::make_shared<MaxPoolLayer>(ctx, Properties{ { "batch", N }, { "channels", 3 }, { "height", 2 * S },
+                                                                   { "width", 2 * S }, { "kernel", 2 }, { "stride", 2 } });
+            route = std::make_shared<RouteLayer>(ctx, Properties{ { "batch", N }, { "channels", C + 3 }, { "height", S },
+                                                                  { "width", S }, { "absorb_upsample", absorb } },
+                                                 std::vector<Layer::Ptr>{ pool, up });
+        }
+    };
+    Pair plain(false), fused(true);
+    report("absorbed upsample releases its own tensors",
+           fused.up->writesIntoConsumer() && fused.up->output().empty() && !plain.up->writesIntoConsumer());
+    const FloatVector small(normals(301, size_t(N) * C * (S / 2) * (S / 2)));
+    const FloatVector large(normals(302, size_t(N) * 3 * 2 * S * 2 * S));
+    const Host routeDelta = normals(303, size_t(N) * (C + 3) * S * S);
+    const Host grad0 = normals(304, small.size());
+    Host out[2], upGrad[2], poolDelta[2];
+    int k = 0;
+    for (Pair* net: { &plain, &fused }) {
+        net->pool->forward(large);
+        net->up->forward(small);
+        net->route->forward(net->up->output());
+        out[k] = net->route->output().asVector();
+        net->route->delta().copyHost(routeDelta);
+        FloatVector grad(grad0);
+        net->route->backward(net->up->output(), nullptr);
+        net->up->backward(small, &grad);
+        upGrad[k] = grad.asVector();
+        poolDelta[k] = net->pool->delta().asVector();
+        ++k;
+    }
+    expectExact("route output with an absorbed upsample", out[1], out[0]);
+    expectExact("upsample backward from the route's delta slice", upGrad[1], upGrad[0]);
+    expectExact("other route source's delta unchanged", poolDelta[1], poolDelta[0]);
+}
+
 }   // namespace
 
 int main(int argc, char** argv)
@@ -525,6 +573,7 @@ int main(int argc, char** argv)
             }
             inferenceChecks();
             trainingChecks();
+            absorbedUpsampleChecks();
         }
     } catch (const std::exception& e) {
         std::printf("unexpected exception: %s\n", e.what());

@@ -68,6 +68,8 @@ def test_rejects_bad_arguments_without_launching():
     assert "equal in x and y" in capi.last_error()
     assert capi.call_raw("pxh_adam_update", 8, p, p, p, p, 0, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 0, None) == inv
     assert capi.call_raw("pxh_adam_update", 8, p, p, p, p, 1, 0, 1e-3, 0.9, 0.999, 1e-8, 0.0, 0, None) == inv
+    assert capi.call_raw("pxh_upsample_strided", p, 4, 4, 2, 1, 2, 1, 1.0, None, p, 100, None) == inv
+    assert "image stride" in capi.last_error()
     # tensors of 2^31 elements or more are refused, not mis-indexed
     assert capi.call_raw("pxh_bn_infer_act_forward", p, p, None, p, p, p, p, 1024, 1024, 4096, 0, None, 0, None) == -2
     with pytest.raises(capi.PxError):

@@ -114,6 +114,38 @@ def test_upsample_forward_backward(ops, oracle, shape, stride):
         assert_bit_exact(host(gg), grad_w, "upsample bwd %s s%d scale %g" % (shape, stride, scale))
 
 
+@pytest.mark.parametrize("shape,stride,other,offset", [((2, 8, 19, 19), 2, 16, 0), ((2, 8, 19, 19), 2, 16, 16),
+                                                       ((3, 4, 8, 12), 2, 5, 5), ((2, 3, 5, 7), 2, 3, 0),
+                                                       ((2, 3, 5, 7), 3, 2, 2), ((1, 2, 4, 4), 2, 1, 1)])
+def test_upsample_into_concatenation_buffer(ops, oracle, shape, stride, other, offset):
+    """The strided form writes (and, backward, reads) a channel slice of a wider tensor: the result
+    equals the dense upsample followed by the route copy, and the other channels stay untouched."""
+    import torch
+    N, C, H, W = shape
+    OH, OW = H * stride, W * stride
+    x = wl.normal(1650 + H + offset, shape)
+    dense = np.zeros((N, C, OH, OW), F)
+    oracle.upsample(x, W, H, C, N, stride, True, 0.75, None, dense)
+    buf0 = wl.normal(1651 + W, (N, C + other, OH, OW))
+    expect = buf0.copy()
+    expect[:, offset:offset + C] = dense
+    gbuf = gpu(buf0)
+    ops.upsample_forward_into(gpu(x), gbuf, offset, stride, 0.75)
+    assert_bit_exact(host(gbuf), expect, "upsample into buffer %s +%d" % (shape, offset))
+    delta_buf = wl.normal(1652 + W, (N, C + other, OH, OW))
+    grad0 = wl.normal(1653 + W, shape)
+    grad_w = grad0.copy()
+    oracle.upsample(None, W, H, C, N, stride, False, 0.75, grad_w,
+                    np.ascontiguousarray(delta_buf[:, offset:offset + C]))
+    gg = gpu(grad0)
+    gdelta = gpu(delta_buf)
+    ops.upsample_backward_from(gdelta, offset, gg, stride, 0.75)
+    assert_bit_exact(host(gg), grad_w, "upsample from buffer %s +%d" % (shape, offset))
+    assert_bit_exact(host(gdelta), delta_buf, "delta buffer untouched")
+    with pytest.raises(ValueError):
+        ops.upsample_forward_into(gpu(x), gbuf, other + 1, stride, 0.75)
+
+
 @pytest.mark.parametrize("act", ["linear", "leaky"])
 @pytest.mark.parametrize("shape", [(2, 8, 38, 38), (3, 5, 19, 19), (1, 1, 1, 3), (2, 3, 64, 64)])
 def test_shortcut_forward_backward(ops, oracle, shape, act):
