@@ -161,23 +161,23 @@ def measure_extras(torch, ops, wl, timer, capi):
         return torch.randn(shape, device=dev)
 
     N = 16
-    # ---- route concat of YOLOv3 @608: 256x38^2 (upsampled) ++ 512x38^2, and 128x76^2 ++ 256x76^2
+    # ---- route concat of YOLOv3 @608: 256x38^2 (upsampled) ++ 512x38^2, and 128x76^2 ++ 256x76^2.
+    # The upsample in front writes its channels straight into the concat buffer (timed below, same
+    # bytes as the dense form), so the route moves the other source only.
     for (c1, c2, s) in [(256, 512, 38), (128, 256, 76)]:
-        a = randn(N, c1, s, s); b = randn(N, c2, s, s)
+        b = randn(N, c2, s, s)
         r = torch.empty((N, c1 + c2, s, s), device=dev)
-
-        def concat(i):
-            ops.route_forward(a, r, 0)
-            ops.route_forward(b, r, c1 * s * s)
-
-        def split(i):
-            ops.route_backward(r, a, 0)
-            ops.route_backward(r, b, c1 * s * s)
-
-        e = N * (c1 + c2) * s * s
-        add("route_fwd", "%dx(%d+%d)x%d^2" % (N, c1, c2, s), 8 * e, timer.time(concat, 20), "2 launches, 8B/elem")
-        add("route_bwd", "%dx(%d+%d)x%d^2" % (N, c1, c2, s), 12 * e, timer.time(split, 20), "2 launches, 12B/elem")
-        del a, b, r
+        e = N * c2 * s * s
+        ms = timer.time(lambda i: ops.route_forward(b, r, c1 * s * s), 20)
+        add("route_fwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), 8 * e, ms, "the %d-channel source, 8B/elem" % c2)
+        ms = timer.time(lambda i: ops.route_backward(r, b, c1 * s * s), 20)
+        add("route_bwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), 12 * e, ms, "the %d-channel source, 12B/elem" % c2)
+        x = randn(N, c1, s // 2, s // 2)
+        e_up = N * c1 * s * s
+        ms = timer.time(lambda i: ops.upsample_forward_into(x, r, 0, 2, 1.0), 20)
+        add("upsample_fwd(into route)", "%dx%dx%d^2" % (N, c1, s // 2), 5 * e_up, ms, "same bytes as upsample_fwd; "
+            "not in ms/batch twice")
+        del b, r, x
     # ---- max-pool 2x2 s2 forward + backward (config 2)
     for c, s in wl.YOLOV3_MAXPOOL_SHAPES:
         e_in = N * c * s * s
@@ -342,7 +342,7 @@ def measure_extras(torch, ops, wl, timer, capi):
     for key, (f, b, count) in shortcut_ms.items():
         total += (f + b) * count
     for r in rows:
-        if r["kernel"].startswith(("upsample", "maxpool", "route_fwd", "route_bwd")):
+        if r["kernel"] in ("upsample_fwd", "upsample_bwd", "maxpool_fwd", "maxpool_bwd", "route_fwd", "route_bwd"):
             total += r["ms"]
     for s, (ms_d, ms_t) in head_ms.items():
         total += ms_t * N / NB
