@@ -314,6 +314,17 @@ DETECTION_DTYPE = np.dtype([("x", "f4"), ("y", "f4"), ("w", "f4"), ("h", "f4"), 
                             ("class_index", "i4"), ("order", "u4")])
 
 
+def nms(records, threshold):
+    """src/Box.cpp nms on an array of DETECTION_DTYPE records (their sequence is the input order)."""
+    records = np.ascontiguousarray(records, DETECTION_DTYPE)
+    out = np.zeros(max(1, len(records)), DETECTION_DTYPE)
+    fn = lib().pxo_nms
+    fn.restype = _c_int
+    kept = fn(records.ctypes.data_as(ctypes.c_void_p), int(len(records)), _c_float(threshold),
+              out.ctypes.data_as(ctypes.c_void_p))
+    return out[:kept]
+
+
 def yolo_detections(cfg, predictions, threshold, capacity, image_width=0, image_height=0):
     """Returns (records in the reference's emission order, total number found)."""
     out = np.zeros(max(1, capacity), DETECTION_DTYPE)

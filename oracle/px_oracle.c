@@ -30,6 +30,10 @@
  *   Adam             parity unpinned by reference tests (the reference has
  *                    no CPU Adam and no numeric Adam test); pinned by the
  *                    t=1 closed form and an fp64 Adam-with-L2 recurrence
+ *   SGD, rescale +   parity unpinned by reference tests; closed forms,
+ *   clip, detections invariants and hand-computed cases (see px_oracle.h)
+ *   nms              reference known-answer tests (tests/src/box.cpp),
+ *                    hand-worked scenarios, an independent restatement
  */
 #include "px_oracle.h"
 
@@ -1073,4 +1077,117 @@ int pxo_yolo_detections(const pxo_yolo_cfg* g, const float* predictions, float t
             }
         }
     return found;
+}
+
+/* ------------------------------------------------------------------ */
+/* non-maximum suppression -- src/Box.cpp                              */
+/* ------------------------------------------------------------------ */
+
+/* Box.cpp:47-54 */
+static rect_f nms_normalized_rect(const pxo_detection* d)
+{
+    const float xe = d->x + d->w, ye = d->y + d->h;
+    const float x1 = d->x < xe ? d->x : xe, y1 = d->y < ye ? d->y : ye;
+    const float x2 = d->x < xe ? xe : d->x, y2 = d->y < ye ? ye : d->y;
+    rect_f r;
+    r.x = x1; r.y = y1;
+    r.w = x2 - x1 > 0.0f ? x2 - x1 : 0.0f;
+    r.h = y2 - y1 > 0.0f ? y2 - y1 : 0.0f;
+    return r;
+}
+
+/* Box.cpp:25-45: areas and overlap are floats, the union is clamped at zero, and a quotient that is
+ * not finite counts as no overlap */
+static float nms_iou(rect_f a, rect_f b)
+{
+    const float inter = rect_intersection_area(a, b);
+    float uni = a.w * a.h + b.w * b.h - inter;
+    if (!(0.0f < uni)) uni = 0.0f;
+    const float q = inter / uni;
+    if (isnan(q) || isinf(q)) return 0.0f;
+    return q;
+}
+
+typedef struct nms_item {
+    const pxo_detection* det;
+    int position;           /* place in the input sequence */
+} nms_item;
+
+static int nms_by_prob(const void* pa, const void* pb)
+{
+    const nms_item* a = (const nms_item*) pa;
+    const nms_item* b = (const nms_item*) pb;
+    if (a->det->prob > b->det->prob) return -1;
+    if (b->det->prob > a->det->prob) return 1;
+    return a->position < b->position ? -1 : (a->position > b->position ? 1 : 0);   /* stable */
+}
+
+typedef struct nms_member {
+    unsigned long long key;     /* image << 32 | class */
+    int sorted;                 /* place in the sequence sorted by probability */
+} nms_member;
+
+static int nms_by_group(const void* pa, const void* pb)
+{
+    const nms_member* a = (const nms_member*) pa;
+    const nms_member* b = (const nms_member*) pb;
+    if (a->key != b->key) return a->key < b->key ? -1 : 1;
+    return a->sorted < b->sorted ? -1 : (a->sorted > b->sorted ? 1 : 0);
+}
+
+/* Box.cpp:56-147.  The reference finds the earlier boxes of a group through an R-tree query for
+ * intersecting rectangles and then tests their overlap ratio; a ratio above a non-negative
+ * threshold implies a positive overlap, so testing every earlier kept box of the group decides the
+ * same.  Only the first 1024 members of a group (in sorted order, counting those the first pass
+ * discarded) are visited; later ones stay. */
+int pxo_nms(const pxo_detection* detections, int count, float threshold, pxo_detection* out)
+{
+    if (count <= 0) return 0;
+    nms_item* items = (nms_item*) malloc(sizeof(nms_item) * (size_t) count);
+    rect_f* rects = (rect_f*) malloc(sizeof(rect_f) * (size_t) count);
+    char* discard = (char*) calloc((size_t) count, 1);
+    nms_member* members = (nms_member*) malloc(sizeof(nms_member) * (size_t) count);
+    int* kept = (int*) malloc(sizeof(int) * 1024);
+    for (int i = 0; i < count; ++i) { items[i].det = detections + i; items[i].position = i; }
+    qsort(items, (size_t) count, sizeof(nms_item), nms_by_prob);
+    for (int i = 0; i < count; ++i) rects[i] = nms_normalized_rect(items[i].det);
+
+    /* near-identical boxes of different classes in one image: the strongest stays (65-88) */
+    for (int i = 0; i < count; ++i)
+        for (int j = 0; j < i; ++j) {
+            if (discard[j] || items[i].det->batch != items[j].det->batch ||
+                items[i].det->class_index == items[j].det->class_index)
+                continue;
+            if (nms_iou(rects[i], rects[j]) > 0.9f) { discard[i] = 1; break; }
+        }
+
+    /* greedy suppression inside each (image, class) group (90-136) */
+    for (int i = 0; i < count; ++i) {
+        members[i].key = ((unsigned long long) (unsigned) items[i].det->batch << 32) |
+                         (unsigned) items[i].det->class_index;
+        members[i].sorted = i;
+    }
+    qsort(members, (size_t) count, sizeof(nms_member), nms_by_group);
+    for (int start = 0; start < count;) {
+        int end = start;
+        while (end < count && members[end].key == members[start].key) ++end;
+        const int visit = end - start < 1024 ? end - start : 1024;
+        int n_kept = 0;
+        for (int p = 0; p < visit; ++p) {
+            const int i = members[start + p].sorted;
+            if (discard[i]) continue;
+            int suppressed = 0;
+            for (int k = 0; k < n_kept && !suppressed; ++k)
+                if (nms_iou(rects[i], rects[kept[k]]) > threshold) suppressed = 1;
+            if (suppressed) discard[i] = 1;
+            else kept[n_kept++] = i;
+        }
+        start = end;
+    }
+
+    int n_out = 0;
+    for (int i = 0; i < count; ++i)
+        if (!discard[i]) out[n_out++] = *items[i].det;
+    free(items); free(rects); free(discard); free(members); free(kept);
+    return n_out;
 }

@@ -154,6 +154,13 @@ typedef struct pxo_detection {
 int pxo_yolo_detections(const pxo_yolo_cfg* cfg, const float* predictions, float threshold,
                         int image_width, int image_height, pxo_detection* out, int capacity);
 
+/* ---- nms, src/Box.cpp:56-147: stable sort by probability (descending), near-identical boxes
+ * (overlap ratio > 0.9) of different classes in one image keep the strongest, then greedy
+ * suppression above `threshold` (>= 0) inside each (image, class) group over its first 1024
+ * members.  `out` needs room for `count` records; returns the number kept, in sorted order.
+ * Pinned by the reference's tests/src/box.cpp:25-101 and by brute-force restatements. */
+int pxo_nms(const pxo_detection* detections, int count, float threshold, pxo_detection* out);
+
 /* ---- SGD with momentum: include/ConvLayer.h:309-311.  Parity unpinned by reference tests (no
  * numeric test of update() exists); pinned by the closed form of one step and an fp64 recurrence. */
 void pxo_sgd_update(size_t n, float* w, float* d, int batch, float lr, float momentum, float decay,

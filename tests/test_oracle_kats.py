@@ -608,3 +608,150 @@ def test_detections_hand_computed(oracle):
     # capacity smaller than the number found: the count still says how many there are
     rec, found = oracle.yolo_detections(cfg, p, 0.4, 2)
     assert found == 4 and len(rec) == 2
+
+
+def _records(oracle, rows):
+    """rows of [left, top, width, height, batch, class, prob] -> detection records in that order."""
+    rec = np.zeros(len(rows), oracle.DETECTION_DTYPE)
+    for i, (x, y, w, h, b, c, p) in enumerate(rows):
+        rec[i] = (x, y, w, h, p, b, c, i)
+    return rec
+
+
+def test_nms_kats(oracle, kats):
+    """tests/src/box.cpp:25-101."""
+    for case in kats["nms"]["cases"]:
+        out = oracle.nms(_records(oracle, case["detections"]), case["threshold"])
+        if "expected_boxes" in case:
+            got = [[float(r["x"]), float(r["y"]), float(r["w"]), float(r["h"])] for r in out]
+            assert got == [[float(v) for v in b] for b in case["expected_boxes"]], case["name"]
+        if "expected_count" in case:
+            assert len(out) == case["expected_count"], case["name"]
+        if "expected_classes" in case:
+            assert list(out["class_index"]) == case["expected_classes"], case["name"]
+        if "expected_probs" in case:
+            assert np.allclose(out["prob"], case["expected_probs"], rtol=1e-7), case["name"]
+
+
+def test_nms_hand_worked_scenarios(oracle):
+    """Cases whose answer follows from src/Box.cpp:56-147 by hand."""
+    X = [0, 0, 100, 100]
+    Y = [0, 0, 100, 70]          # overlap ratio with X: 0.7
+    # a box discarded as a cross-class duplicate never suppresses a weaker box of its own class
+    out = oracle.nms(_records(oracle, [X + [0, 1, 0.9], X + [0, 2, 0.8], Y + [0, 2, 0.7]]), 0.5)
+    assert [(int(r["class_index"]), float(r["h"])) for r in out] == [(1, 100.0), (2, 70.0)]
+    # ... and does not discard a near-identical box of a third class either (it is skipped, 76-79)
+    A = [0, 0, 100, 100]; A1 = [0, 0, 100, 95]; A2 = [0, 0, 100, 89]      # A/A1 .95, A1/A2 .937, A/A2 .89
+    out = oracle.nms(_records(oracle, [A + [0, 1, 0.9], A1 + [0, 2, 0.8], A2 + [0, 3, 0.7]]), 0.5)
+    assert list(out["class_index"]) == [1, 3]
+    # equal probabilities keep their input order (stable sort): the first of two twins survives
+    out = oracle.nms(_records(oracle, [X + [0, 1, 0.5], X + [0, 1, 0.5]]), 0.5)
+    assert len(out) == 1 and out[0]["order"] == 0
+    # the output is sorted by probability whatever the input order, across images
+    out = oracle.nms(_records(oracle, [X + [1, 1, 0.2], X + [0, 1, 0.9], X + [2, 1, 0.5]]), 0.5)
+    assert list(out["batch"]) == [0, 2, 1]
+    # negative extents are normalised (47-54): (100,100,-100,-100) is X
+    out = oracle.nms(_records(oracle, [X + [0, 1, 0.9], [100, 100, -100, -100, 0, 1, 0.8]]), 0.5)
+    assert len(out) == 1
+    # empty boxes have no overlap ratio (0/0 counts as none): both stay
+    Z = [5, 5, 0, 0]
+    out = oracle.nms(_records(oracle, [Z + [0, 1, 0.9], Z + [0, 1, 0.8]]), 0.0)
+    assert len(out) == 2
+    # exactly at the threshold is not above it
+    out = oracle.nms(_records(oracle, [[0, 0, 100, 100, 0, 1, 0.9], [0, 0, 100, 50, 0, 1, 0.8]]), 0.5)
+    assert len(out) == 2
+    # only the first 1024 members of a group are visited; the rest stay whatever they overlap
+    rows = [X + [0, 1, 1.0 - i * 1e-4] for i in range(1100)]
+    out = oracle.nms(_records(oracle, rows), 0.5)
+    assert len(out) == 1 + (1100 - 1024)
+    assert list(out["order"]) == [0] + list(range(1024, 1100))
+    # members that the duplicate pass discarded still use up places among the 1024
+    rows = [X + [0, 2, 1.0]] + [X + [0, 1, 0.9 - i * 1e-4] for i in range(1100)]
+    out = oracle.nms(_records(oracle, rows), 0.5)        # all of class 1 are duplicates of the class-2 box
+    assert len(out) == 1 and out[0]["class_index"] == 2
+    assert len(oracle.nms(_records(oracle, []), 0.5)) == 0
+
+
+def nms_by_the_book(rec, threshold):
+    """src/Box.cpp:56-147 restated with Python containers and numpy float32 arithmetic, written
+    independently of the C checker (dictionary groups, lists of kept boxes)."""
+    f = np.float32
+
+    def norm(r):
+        x, y, w, h = f(r["x"]), f(r["y"]), f(r["w"]), f(r["h"])
+        x1, y1 = min(x, f(x + w)), min(y, f(y + h))
+        x2, y2 = max(x, f(x + w)), max(y, f(y + h))
+        return x1, y1, max(f(0), f(x2 - x1)), max(f(0), f(y2 - y1))
+
+    def iou(a, b):
+        if a[2] <= 0 or a[3] <= 0 or b[2] <= 0 or b[3] <= 0:
+            inter = f(0)
+        else:
+            xl, xh = (a, b) if a[0] < b[0] else (b, a)
+            yl, yh = (a, b) if a[1] < b[1] else (b, a)
+            if (xl[0] < 0 and f(xl[0] + xl[2]) < xh[0]) or (yl[1] < 0 and f(yl[1] + yl[3]) < yh[1]):
+                inter = f(0)
+            else:
+                iw = min(f(xl[2] - f(xh[0] - xl[0])), xh[2])
+                ih = min(f(yl[3] - f(yh[1] - yl[1])), yh[3])
+                inter = f(iw * ih) if iw > 0 and ih > 0 else f(0)
+        uni = max(f(0), f(f(f(a[2] * a[3]) + f(b[2] * b[3])) - inter))
+        with np.errstate(divide="ignore", invalid="ignore"):
+            q = inter / uni
+        return f(0) if not np.isfinite(q) else q
+
+    order = sorted(range(len(rec)), key=lambda i: -float(rec[i]["prob"]))      # sorted() is stable
+    boxes = [norm(rec[i]) for i in order]
+    discard = [False] * len(order)
+    for i in range(len(order)):
+        for j in range(i):
+            a, b = rec[order[i]], rec[order[j]]
+            if discard[j] or a["batch"] != b["batch"] or a["class_index"] == b["class_index"]:
+                continue
+            if iou(boxes[i], boxes[j]) > f(0.9):
+                discard[i] = True
+                break
+    groups = {}
+    for i in range(len(order)):
+        groups.setdefault((int(rec[order[i]]["batch"]), int(rec[order[i]]["class_index"])), []).append(i)
+    for members in groups.values():
+        kept = []
+        for i in members[:1024]:
+            if discard[i]:
+                continue
+            if any(iou(boxes[i], boxes[j]) > f(threshold) for j in kept):
+                discard[i] = True
+            else:
+                kept.append(i)
+    return rec[[order[i] for i in range(len(order)) if not discard[i]]]
+
+
+def random_detections(oracle, seed, n, batch, classes, clusters, spread=6.0):
+    """Boxes scattered around a few centres per image so that many overlap, with tied probabilities."""
+    g = np.random.Generator(np.random.Philox(key=seed))
+    rec = np.zeros(n, oracle.DETECTION_DTYPE)
+    centre = g.uniform(50, 400, (batch, clusters, 2))
+    size = g.uniform(20, 120, (batch, clusters, 2))
+    b = g.integers(0, batch, n)
+    k = g.integers(0, clusters, n)
+    rec["batch"] = b
+    rec["class_index"] = g.integers(0, classes, n)
+    jitter = g.normal(0, spread, (n, 4)).astype(F)
+    rec["w"] = np.maximum(1, size[b, k, 0] + jitter[:, 2])
+    rec["h"] = np.maximum(1, size[b, k, 1] + jitter[:, 3])
+    rec["x"] = centre[b, k, 0] + jitter[:, 0] - rec["w"] / 2
+    rec["y"] = centre[b, k, 1] + jitter[:, 1] - rec["h"] / 2
+    rec["prob"] = np.round(g.uniform(0.05, 1.0, n), 2).astype(F)         # two decimals: plenty of ties
+    rec["order"] = np.arange(n)
+    return rec
+
+
+@pytest.mark.parametrize("seed,n,batch,classes,clusters,thr", [(1, 300, 2, 3, 3, 0.45), (2, 500, 1, 2, 2, 0.3),
+                                                               (3, 400, 3, 5, 1, 0.6), (4, 64, 1, 1, 1, 0.0)])
+def test_nms_matches_the_book_on_random_clusters(oracle, seed, n, batch, classes, clusters, thr):
+    rec = random_detections(oracle, seed, n, batch, classes, clusters, spread=3.0 if seed == 3 else 6.0)
+    want = nms_by_the_book(rec, thr)
+    got = oracle.nms(rec, thr)
+    assert len(got) == len(want) and 0 < len(got) < n
+    assert list(got["order"]) == list(want["order"])
+    assert got.tobytes() == want.tobytes()
