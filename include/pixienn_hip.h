@@ -261,6 +261,31 @@ int pxh_yolo_detections(const float* predictions, int batch, const int* host_mas
                         const int* host_anchors, int anchor_count, int classes, int width, int height,
                         int net_width, int net_height, int image_width, int image_height,
                         float threshold, pxh_detection* out, int capacity, int* count, void* stream);
+/* The same without clearing *count: the records of this head go behind those already there, and
+ * `order_base` is added to their `order` -- with the number of (slot, class) pairs of the heads
+ * before it, the orders of a model's heads continue as in Model::detections (include/Model.h:
+ * 1078-1088), which asks one YOLO layer after the other. */
+int pxh_yolo_detections_append(const float* predictions, int batch, const int* host_masks,
+                               int mask_count, const int* host_anchors, int anchor_count, int classes,
+                               int width, int height, int net_width, int net_height, int image_width,
+                               int image_height, float threshold, unsigned order_base,
+                               pxh_detection* out, int capacity, int* count, void* stream);
+
+/* nms (src/Box.cpp:56-147) on records that never leave the device.  The input sequence of the
+ * reference is the records' `order` (unique; ties in probability keep it, as its stable sort does).
+ * *count (device) says how many of records[capacity] are there (more than capacity = capacity).
+ * Records must name images in [0, batch) and classes in [0, classes).  kept[capacity] receives the
+ * survivors sorted by descending probability, *kept_count (device) their number.  threshold >= 0.
+ * Steps: near-identical boxes (overlap ratio > 0.9) of different classes in one image keep the
+ * strongest; then greedy suppression above `threshold` inside each (image, class) group over its
+ * first 1024 members.  Workspace: pxh_nms_workspace_bytes(capacity), or NULL for the library's. */
+size_t pxh_nms_workspace_bytes(int capacity);
+int pxh_nms(const pxh_detection* records, const int* count, int capacity, int batch, int classes,
+            float threshold, pxh_detection* kept, int* kept_count, void* workspace,
+            size_t workspace_bytes, void* stream);
+/* Test hook: number (1..6) of whole-array sweeps of the duplicate step before the per-image loop
+ * finishes what they left; returns the previous value.  Results do not depend on it. */
+int pxh_debug_nms_sweeps(int sweeps);
 
 size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int width, int height,
                                 int max_truth);

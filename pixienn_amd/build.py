@@ -10,7 +10,7 @@ CSRC = os.path.join(PKG, "csrc")
 OBJ = os.path.join(PKG, "build")
 LIB = os.path.join(PKG, "libpixienn_hip.so")
 
-SOURCES = ["runtime.hip", "epilogue.hip", "elementwise.hip", "pool.hip", "yolo.hip"]
+SOURCES = ["runtime.hip", "epilogue.hip", "elementwise.hip", "pool.hip", "yolo.hip", "nms.hip"]
 
 # -ffp-contract=off: the bit-exact kernels must not fuse a*b+c; packed fp32 VALU forms are
 # switched off for every kernel.

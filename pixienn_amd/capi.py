@@ -18,6 +18,7 @@ I = ctypes.c_int
 F = ctypes.c_float
 Z = ctypes.c_size_t
 L = ctypes.c_longlong
+U = ctypes.c_uint
 
 # name -> argument types (every function returns int unless listed in _OTHER_RETURNS)
 SIGNATURES = {
@@ -54,6 +55,9 @@ SIGNATURES = {
     "pxh_sgd_update": [Z, P, P, I, F, F, F, I, P],
     "pxh_rescale_clip": [P, Z, F, F, P, P, Z, P],
     "pxh_yolo_detections": [P, I, P, I, P, I, I, I, I, I, I, I, I, F, P, I, P, P],
+    "pxh_yolo_detections_append": [P, I, P, I, P, I, I, I, I, I, I, I, I, F, U, P, I, P, P],
+    "pxh_nms": [P, P, I, I, I, F, P, P, P, Z, P],
+    "pxh_debug_nms_sweeps": [I],
     "pxh_adam": [I, P, P, P, F, F, F, F, I, P],
     "pxh_adam_update": [Z, P, P, P, P, I, I, F, F, F, F, F, I, P],
 }
@@ -64,6 +68,7 @@ _OTHER_RETURNS = {
     "pxh_bn_folded_bytes": (Z, [I]),
     "pxh_rescale_workspace_bytes": (Z, []),
     "pxh_yolo_workspace_bytes": (Z, [I, I, I, I, I, I]),
+    "pxh_nms_workspace_bytes": (Z, [I]),
     "pxh_debug_fastdiv": (ctypes.c_uint, [ctypes.c_uint, ctypes.c_uint]),
 }
 

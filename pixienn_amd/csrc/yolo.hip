@@ -680,6 +680,7 @@ struct DetectArgs {
     float threshold;
     int image_width, image_height;    // > 0: letterbox-corrected pixel boxes
     uint32_t slots;                   // batch * masks * area
+    uint32_t order_base;              // added to every record's emission order
     FastDiv by_area;
 };
 
@@ -789,7 +790,7 @@ __global__ __launch_bounds__(kBlock) void yolo_detect_kernel(DetectArgs a, YoloP
                     d.prob = objectness * rows[static_cast<size_t>(j) * area];
                     d.batch = static_cast<int>(b);
                     d.class_index = j;
-                    d.order = order0 + j;
+                    d.order = a.order_base + order0 + j;
                     a.out[at] = d;
                 }
                 ++at;
@@ -930,10 +931,10 @@ int pxh_yolo_activate(const float* input, float* output, int batch, int masks, i
     return launch_stream("pxh_yolo_activate", static_cast<size_t>(total), vec, 8, op, as_stream(stream));
 }
 
-int pxh_yolo_detections(const float* predictions, int batch, const int* host_masks, int mask_count,
-                        const int* host_anchors, int anchor_count, int classes, int width, int height,
-                        int net_width, int net_height, int image_width, int image_height, float threshold,
-                        pxh_detection* out, int capacity, int* count, void* stream)
+int pxh_yolo_detections_append(const float* predictions, int batch, const int* host_masks, int mask_count,
+                               const int* host_anchors, int anchor_count, int classes, int width, int height,
+                               int net_width, int net_height, int image_width, int image_height, float threshold,
+                               unsigned order_base, pxh_detection* out, int capacity, int* count, void* stream)
 {
     if (!predictions || !host_masks || !host_anchors || !count || (!out && capacity > 0))
         return fail_invalid("pxh_yolo_detections: null pointer");
@@ -948,16 +949,33 @@ int pxh_yolo_detections(const float* predictions, int batch, const int* host_mas
         p.masks[m] = host_masks[m];
     }
     for (int a = 0; a < 2 * anchor_count; ++a) p.anchors[a] = static_cast<float>(host_anchors[a]);
+    const unsigned long long orders = 1ull * batch * mask_count * p.area * classes;
+    if (orders + order_base > 0xFFFFFFFFull) {
+        set_error("pxh_yolo_detections: emission orders past 2^32 (base %u + %llu)", order_base, orders);
+        return PXH_ERR_UNSUPPORTED;
+    }
     hipStream_t s = as_stream(stream);
-    rc = pxh_fill_i32(count, 1, 0, stream);
-    if (rc) return rc;
     DetectArgs a{};
     a.pred = predictions; a.out = out; a.count = count; a.capacity = capacity; a.threshold = threshold;
     a.image_width = image_width; a.image_height = image_height;
     a.slots = static_cast<uint32_t>(batch) * mask_count * p.area;
+    a.order_base = order_base;
     a.by_area = FastDiv(p.area);
     hipLaunchKernelGGL(yolo_detect_kernel, dim3(grid_for(a.slots, kBlock)), dim3(kBlock), 0, s, a, p);
     return check_launch("pxh_yolo_detections");
+}
+
+int pxh_yolo_detections(const float* predictions, int batch, const int* host_masks, int mask_count,
+                        const int* host_anchors, int anchor_count, int classes, int width, int height,
+                        int net_width, int net_height, int image_width, int image_height, float threshold,
+                        pxh_detection* out, int capacity, int* count, void* stream)
+{
+    if (!count) return fail_invalid("pxh_yolo_detections: null pointer");
+    const int rc = pxh_fill_i32(count, 1, 0, stream);
+    if (rc) return rc;
+    return pxh_yolo_detections_append(predictions, batch, host_masks, mask_count, host_anchors, anchor_count, classes,
+                                      width, height, net_width, net_height, image_width, image_height, threshold, 0u,
+                                      out, capacity, count, stream);
 }
 
 size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int width, int height, int max_truth)

@@ -351,3 +351,50 @@ def yolo_detections(predictions, batch, masks, anchors, classes, width, height, 
     found = int(count.item())
     rec = out[:min(found, capacity)].cpu().numpy().view(DETECTION_DTYPE).reshape(-1)
     return rec[np.argsort(rec["order"], kind="stable")], found
+
+
+def yolo_detections_append(predictions, batch, masks, anchors, classes, width, height, net_width, net_height,
+                           threshold, order_base, records, count, image_width=0, image_height=0):
+    """Adds the detections of one more head behind those already in `records` (an int32 tensor
+    [capacity, 8] on the device); `count` is the device counter both heads share."""
+    _chk_all(predictions)
+    _chk(records, torch.int32, "records")
+    _chk(count, torch.int32, "count")
+    m = np.ascontiguousarray(masks, dtype=np.int32)
+    a = np.ascontiguousarray(anchors, dtype=np.int32)
+    call("pxh_yolo_detections_append", ptr(predictions), batch, m.ctypes.data, len(m), a.ctypes.data, len(a) // 2,
+         classes, width, height, net_width, net_height, int(image_width), int(image_height), float(threshold),
+         int(order_base), ptr(records), int(records.shape[0]), ptr(count), _stream())
+
+
+def nms(records, count, batch, classes, threshold, workspace=None):
+    """src/Box.cpp nms on device-resident records (int32 tensor [capacity, 8] viewed as detection
+    records, device counter `count`).  Returns (kept records tensor, device counter of the kept)."""
+    _chk(records, torch.int32, "records")
+    _chk(count, torch.int32, "count")
+    capacity = int(records.shape[0])
+    kept = torch.empty_like(records)
+    kept_count = torch.empty(1, device=records.device, dtype=torch.int32)
+    ws_ptr, ws_bytes = (ptr(workspace), workspace.numel() * workspace.element_size()) if workspace is not None \
+        else (None, 0)
+    call("pxh_nms", ptr(records), ptr(count), capacity, int(batch), int(classes), float(threshold), ptr(kept),
+         ptr(kept_count), ws_ptr, ws_bytes, _stream())
+    return kept, kept_count
+
+
+def nms_to_host(kept, kept_count):
+    """Blocking copy of the survivors as a numpy structured array."""
+    torch.cuda.current_stream().synchronize()
+    n = int(kept_count.item())
+    return kept[:n].cpu().numpy().view(DETECTION_DTYPE).reshape(-1)
+
+
+def records_to_device(rec, capacity=None, device="cuda"):
+    """numpy detection records -> (int32 tensor [capacity, 8], device counter)."""
+    rec = np.ascontiguousarray(rec, DETECTION_DTYPE)
+    capacity = max(1, len(rec)) if capacity is None else capacity
+    t = torch.zeros((capacity, 8), dtype=torch.int32, device=device)
+    if len(rec):
+        t[:len(rec)] = torch.from_numpy(rec.view(np.int32).reshape(-1, 8)).to(device)
+    count = torch.tensor([len(rec)], dtype=torch.int32, device=device)
+    return t, count

@@ -7,6 +7,8 @@ import os
 import numpy as np
 import pytest
 
+from util import detection_records, random_detections
+
 F = np.float32
 
 
@@ -610,18 +612,10 @@ def test_detections_hand_computed(oracle):
     assert found == 4 and len(rec) == 2
 
 
-def _records(oracle, rows):
-    """rows of [left, top, width, height, batch, class, prob] -> detection records in that order."""
-    rec = np.zeros(len(rows), oracle.DETECTION_DTYPE)
-    for i, (x, y, w, h, b, c, p) in enumerate(rows):
-        rec[i] = (x, y, w, h, p, b, c, i)
-    return rec
-
-
 def test_nms_kats(oracle, kats):
     """tests/src/box.cpp:25-101."""
     for case in kats["nms"]["cases"]:
-        out = oracle.nms(_records(oracle, case["detections"]), case["threshold"])
+        out = oracle.nms(detection_records(oracle, case["detections"]), case["threshold"])
         if "expected_boxes" in case:
             got = [[float(r["x"]), float(r["y"]), float(r["w"]), float(r["h"])] for r in out]
             assert got == [[float(v) for v in b] for b in case["expected_boxes"]], case["name"]
@@ -638,38 +632,38 @@ def test_nms_hand_worked_scenarios(oracle):
     X = [0, 0, 100, 100]
     Y = [0, 0, 100, 70]          # overlap ratio with X: 0.7
     # a box discarded as a cross-class duplicate never suppresses a weaker box of its own class
-    out = oracle.nms(_records(oracle, [X + [0, 1, 0.9], X + [0, 2, 0.8], Y + [0, 2, 0.7]]), 0.5)
+    out = oracle.nms(detection_records(oracle, [X + [0, 1, 0.9], X + [0, 2, 0.8], Y + [0, 2, 0.7]]), 0.5)
     assert [(int(r["class_index"]), float(r["h"])) for r in out] == [(1, 100.0), (2, 70.0)]
     # ... and does not discard a near-identical box of a third class either (it is skipped, 76-79)
     A = [0, 0, 100, 100]; A1 = [0, 0, 100, 95]; A2 = [0, 0, 100, 89]      # A/A1 .95, A1/A2 .937, A/A2 .89
-    out = oracle.nms(_records(oracle, [A + [0, 1, 0.9], A1 + [0, 2, 0.8], A2 + [0, 3, 0.7]]), 0.5)
+    out = oracle.nms(detection_records(oracle, [A + [0, 1, 0.9], A1 + [0, 2, 0.8], A2 + [0, 3, 0.7]]), 0.5)
     assert list(out["class_index"]) == [1, 3]
     # equal probabilities keep their input order (stable sort): the first of two twins survives
-    out = oracle.nms(_records(oracle, [X + [0, 1, 0.5], X + [0, 1, 0.5]]), 0.5)
+    out = oracle.nms(detection_records(oracle, [X + [0, 1, 0.5], X + [0, 1, 0.5]]), 0.5)
     assert len(out) == 1 and out[0]["order"] == 0
     # the output is sorted by probability whatever the input order, across images
-    out = oracle.nms(_records(oracle, [X + [1, 1, 0.2], X + [0, 1, 0.9], X + [2, 1, 0.5]]), 0.5)
+    out = oracle.nms(detection_records(oracle, [X + [1, 1, 0.2], X + [0, 1, 0.9], X + [2, 1, 0.5]]), 0.5)
     assert list(out["batch"]) == [0, 2, 1]
     # negative extents are normalised (47-54): (100,100,-100,-100) is X
-    out = oracle.nms(_records(oracle, [X + [0, 1, 0.9], [100, 100, -100, -100, 0, 1, 0.8]]), 0.5)
+    out = oracle.nms(detection_records(oracle, [X + [0, 1, 0.9], [100, 100, -100, -100, 0, 1, 0.8]]), 0.5)
     assert len(out) == 1
     # empty boxes have no overlap ratio (0/0 counts as none): both stay
     Z = [5, 5, 0, 0]
-    out = oracle.nms(_records(oracle, [Z + [0, 1, 0.9], Z + [0, 1, 0.8]]), 0.0)
+    out = oracle.nms(detection_records(oracle, [Z + [0, 1, 0.9], Z + [0, 1, 0.8]]), 0.0)
     assert len(out) == 2
     # exactly at the threshold is not above it
-    out = oracle.nms(_records(oracle, [[0, 0, 100, 100, 0, 1, 0.9], [0, 0, 100, 50, 0, 1, 0.8]]), 0.5)
+    out = oracle.nms(detection_records(oracle, [[0, 0, 100, 100, 0, 1, 0.9], [0, 0, 100, 50, 0, 1, 0.8]]), 0.5)
     assert len(out) == 2
     # only the first 1024 members of a group are visited; the rest stay whatever they overlap
     rows = [X + [0, 1, 1.0 - i * 1e-4] for i in range(1100)]
-    out = oracle.nms(_records(oracle, rows), 0.5)
+    out = oracle.nms(detection_records(oracle, rows), 0.5)
     assert len(out) == 1 + (1100 - 1024)
     assert list(out["order"]) == [0] + list(range(1024, 1100))
     # members that the duplicate pass discarded still use up places among the 1024
     rows = [X + [0, 2, 1.0]] + [X + [0, 1, 0.9 - i * 1e-4] for i in range(1100)]
-    out = oracle.nms(_records(oracle, rows), 0.5)        # all of class 1 are duplicates of the class-2 box
+    out = oracle.nms(detection_records(oracle, rows), 0.5)        # all of class 1 are duplicates of the class-2 box
     assert len(out) == 1 and out[0]["class_index"] == 2
-    assert len(oracle.nms(_records(oracle, []), 0.5)) == 0
+    assert len(oracle.nms(detection_records(oracle, []), 0.5)) == 0
 
 
 def nms_by_the_book(rec, threshold):
@@ -724,26 +718,6 @@ def nms_by_the_book(rec, threshold):
             else:
                 kept.append(i)
     return rec[[order[i] for i in range(len(order)) if not discard[i]]]
-
-
-def random_detections(oracle, seed, n, batch, classes, clusters, spread=6.0):
-    """Boxes scattered around a few centres per image so that many overlap, with tied probabilities."""
-    g = np.random.Generator(np.random.Philox(key=seed))
-    rec = np.zeros(n, oracle.DETECTION_DTYPE)
-    centre = g.uniform(50, 400, (batch, clusters, 2))
-    size = g.uniform(20, 120, (batch, clusters, 2))
-    b = g.integers(0, batch, n)
-    k = g.integers(0, clusters, n)
-    rec["batch"] = b
-    rec["class_index"] = g.integers(0, classes, n)
-    jitter = g.normal(0, spread, (n, 4)).astype(F)
-    rec["w"] = np.maximum(1, size[b, k, 0] + jitter[:, 2])
-    rec["h"] = np.maximum(1, size[b, k, 1] + jitter[:, 3])
-    rec["x"] = centre[b, k, 0] + jitter[:, 0] - rec["w"] / 2
-    rec["y"] = centre[b, k, 1] + jitter[:, 1] - rec["h"] / 2
-    rec["prob"] = np.round(g.uniform(0.05, 1.0, n), 2).astype(F)         # two decimals: plenty of ties
-    rec["order"] = np.arange(n)
-    return rec
 
 
 @pytest.mark.parametrize("seed,n,batch,classes,clusters,thr", [(1, 300, 2, 3, 3, 0.45), (2, 500, 1, 2, 2, 0.3),
