@@ -241,25 +241,30 @@ __device__ __forceinline__ float4 normalized_rect(const pxh_detection& d)
     return make_float4(x1, y1, fmaxf(0.0f, x2 - x1), fmaxf(0.0f, y2 - y1));
 }
 
-// boxIoU, src/Box.cpp:25-45, with cv::Rect2f's operator& (OpenCV >= 4.5.4): an empty operand or a
-// non-positive extent gives no overlap; the extent along an axis is
-// min(lo.size - (hi.origin - lo.origin), hi.size) with lo/hi ordered by origin.
-__device__ __forceinline__ float overlap_ratio(const float4 a, const float4 b)
+// boxIoU(a, b) > threshold, src/Box.cpp:25-45, with cv::Rect2f's operator& (OpenCV >= 4.5.4): an
+// empty operand or a non-positive extent gives no overlap; the extent along an axis is
+// min(lo.size - (hi.origin - lo.origin), hi.size) with lo/hi ordered by origin.  threshold >= 0, so
+// no overlap can never be above it; and the union is at least the larger area, so an overlap well
+// below threshold * that area is decided without the division (the margin of a tenth is far more
+// than all rounding involved).  Everything else takes the reference's own operations.
+__device__ __forceinline__ bool overlaps_above(const float4 a, const float4 b, float threshold)
 {
-    float inter = 0.0f;
-    if (!(a.z <= 0.0f || a.w <= 0.0f || b.z <= 0.0f || b.w <= 0.0f)) {
-        const bool ax = a.x < b.x, ay = a.y < b.y;
-        const float xlo = ax ? a.x : b.x, xlo_w = ax ? a.z : b.z, xhi = ax ? b.x : a.x, xhi_w = ax ? b.z : a.z;
-        const float ylo = ay ? a.y : b.y, ylo_h = ay ? a.w : b.w, yhi = ay ? b.y : a.y, yhi_h = ay ? b.w : a.w;
-        const bool apart = (xlo < 0.0f && xlo + xlo_w < xhi) || (ylo < 0.0f && ylo + ylo_h < yhi);
-        const float iw = fminf(xlo_w - (xhi - xlo), xhi_w);
-        const float ih = fminf(ylo_h - (yhi - ylo), yhi_h);
-        if (!apart && iw > 0.0f && ih > 0.0f) inter = iw * ih;
-    }
-    float uni = a.z * a.w + b.z * b.w - inter;
+    if (a.z <= 0.0f || a.w <= 0.0f || b.z <= 0.0f || b.w <= 0.0f) return false;
+    const bool ax = a.x < b.x, ay = a.y < b.y;
+    const float xlo = ax ? a.x : b.x, xlo_w = ax ? a.z : b.z, xhi = ax ? b.x : a.x, xhi_w = ax ? b.z : a.z;
+    const float ylo = ay ? a.y : b.y, ylo_h = ay ? a.w : b.w, yhi = ay ? b.y : a.y, yhi_h = ay ? b.w : a.w;
+    if ((xlo < 0.0f && xlo + xlo_w < xhi) || (ylo < 0.0f && ylo + ylo_h < yhi)) return false;
+    const float iw = fminf(xlo_w - (xhi - xlo), xhi_w);
+    const float ih = fminf(ylo_h - (yhi - ylo), yhi_h);
+    if (!(iw > 0.0f && ih > 0.0f)) return false;
+    const float inter = iw * ih;
+    const float area_a = a.z * a.w, area_b = b.z * b.w;
+    if (inter < 0.9f * threshold * fmaxf(area_a, area_b)) return false;
+    float uni = area_a + area_b - inter;
     if (!(0.0f < uni)) uni = 0.0f;
     const float q = inter / uni;
-    return (isnan(q) || isinf(q)) ? 0.0f : q;
+    if (isnan(q) || isinf(q)) return false;          // counts as no overlap: 0 > threshold is false
+    return q > threshold;
 }
 
 struct Segments {
@@ -277,7 +282,9 @@ struct NmsArgs {
     Segments* seg;             // per place
     uint32_t* state;           // per place, duplicate pass
     uint32_t* keep;            // per rank
-    uint32_t* counters;        // undecided records left after each sweep
+    uint32_t* resume;          // per place: where the next sweep of the duplicate pass continues
+    uint32_t* counters;        // [k] != 0: sweep k left records undecided
+    uint32_t waves;            // waves of a duplicate sweep's grid
 };
 
 __global__ __launch_bounds__(kBlock) void nms_gather_kernel(NmsArgs a)
@@ -295,72 +302,62 @@ __global__ __launch_bounds__(kBlock) void nms_gather_kernel(NmsArgs a)
     s.group_end = lower_bound(a.group_key, n, key + 1ull);
     a.seg[p] = s;
     a.state[p] = kUndecided;
+    a.resume[p] = s.image_begin;
 }
 
 // ---------------------------------------------------------------- duplicate pass
 // src/Box.cpp:65-88: a record is dropped when an earlier KEPT record of the same image and another
-// class overlaps it by more than 0.9.  One lane per undecided record; the candidates (all places of
-// the images this workgroup touches) pass through LDS a tile at a time.
-__global__ __launch_bounds__(kBlock) void nms_duplicate_sweep_kernel(NmsArgs a, int sweep)
+// class overlaps it by more than 0.9.  One WAVE per undecided record, its lanes side by side over
+// the other places of the image (the record's own class group is stepped over).  Outcome for the
+// record at place p: 1 = dropped, 0 = kept, 2 = still waiting for an undecided earlier record, in
+// which case resume[p] is the first such place: everything before it that conflicts is dropped for
+// good and need not be looked at again.
+__device__ __forceinline__ int duplicate_scan(const NmsArgs& a, uint32_t p, int lane)
 {
-    __shared__ float4 tile_box[kBlock];
-    __shared__ uint32_t tile_rank[kBlock];
-    __shared__ uint32_t tile_state[kBlock];
-    const uint32_t n = live_count(a.count, a.capacity);
-    if (blockIdx.x * kBlock >= n) return;
-    if (sweep > 0 && a.counters[sweep - 1] == 0) return;
-    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
-    const bool valid = p < n;
-    const bool mine = valid && load_state(a.state + p) == kUndecided;
-    if (!__syncthreads_or(mine)) return;
-    Segments s{ 0, 0, 0, 0 };
-    float4 box = make_float4(0, 0, 0, 0);
-    uint32_t rank = 0;
-    if (valid) {
-        s = a.seg[p];
-        box = a.box[p];
-        rank = a.rank[p];
-    }
-    const uint32_t last = min(n, (blockIdx.x + 1) * kBlock) - 1;
-    const uint32_t q_begin = a.seg[blockIdx.x * kBlock].image_begin;
-    const uint32_t q_end = a.seg[last].image_end;
-    bool drop = false, pending = false;
-    for (uint32_t q0 = q_begin; q0 < q_end; q0 += kBlock) {
-        const uint32_t q = q0 + threadIdx.x;
-        if (q < q_end) {
-            tile_box[threadIdx.x] = a.box[q];
-            tile_rank[threadIdx.x] = a.rank[q];
-            tile_state[threadIdx.x] = load_state(a.state + q);
+    const Segments s = a.seg[p];
+    const float4 box = a.box[p];
+    const uint32_t rank = a.rank[p];
+    uint32_t first_pending = 0xFFFFFFFFu;
+    uint32_t q0 = a.resume[p];
+    while (q0 < s.image_end) {
+        if (q0 >= s.group_begin && q0 < s.group_end) {          // the same class: not compared
+            q0 = s.group_end;
+            continue;
         }
-        __syncthreads();
-        if (mine && !drop) {
-            const uint32_t m = min(static_cast<uint32_t>(kBlock), q_end - q0);
-            for (uint32_t k = 0; k < m; ++k) {
-                const uint32_t place = q0 + k;
-                if (place < s.image_begin || place >= s.image_end) continue;       // another image
-                if (place >= s.group_begin && place < s.group_end) continue;       // the same class
-                if (tile_rank[k] >= rank) continue;                                // not earlier
-                const uint32_t st = tile_state[k];
-                if (st == kDropped) continue;
-                if (overlap_ratio(box, tile_box[k]) > kDuplicateOverlap) {
-                    if (st == kKept) {
-                        drop = true;
-                        break;
-                    }
-                    pending = true;
-                }
+        const uint32_t stop = q0 < s.group_begin ? s.group_begin : s.image_end;
+        const uint32_t q = q0 + lane;
+        bool kept_hit = false, waiting = false;
+        if (q < stop && a.rank[q] < rank) {
+            const uint32_t st = load_state(a.state + q);
+            if (st != kDropped && overlaps_above(box, a.box[q], kDuplicateOverlap)) {
+                kept_hit = st == kKept;
+                waiting = st == kUndecided;
             }
         }
-        __syncthreads();
+        if (__ballot(kept_hit)) return 1;
+        const uint64_t w = __ballot(waiting);
+        if (w && first_pending == 0xFFFFFFFFu) first_pending = q0 + __builtin_ctzll(w);
+        q0 = min(q0 + kWave, stop);
     }
-    bool still = false;
-    if (mine) {
-        if (drop) store_state(a.state + p, kDropped);
-        else if (!pending) store_state(a.state + p, kKept);
-        else still = true;
+    if (first_pending == 0xFFFFFFFFu) return 0;
+    if (lane == 0) a.resume[p] = first_pending;
+    return 2;
+}
+
+__global__ __launch_bounds__(kBlock) void nms_duplicate_sweep_kernel(NmsArgs a, int sweep)
+{
+    const uint32_t n = live_count(a.count, a.capacity);
+    if (sweep > 0 && a.counters[sweep - 1] == 0) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) / kWave;
+    bool left = false;
+    for (uint32_t p = wave; p < n; p += a.waves) {
+        if (load_state(a.state + p) != kUndecided) continue;
+        const int outcome = duplicate_scan(a, p, lane);
+        if (outcome == 2) left = true;
+        else if (lane == 0) store_state(a.state + p, outcome == 1 ? kDropped : kKept);
     }
-    const int left = __syncthreads_count(still);
-    if (threadIdx.x == 0 && left) atomicAdd(a.counters + sweep, static_cast<uint32_t>(left));
+    if (left && lane == 0) store_state(a.counters + sweep, 1u);
 }
 
 // What the sweeps left undecided (long chains of conflicts): one workgroup per image repeats the
@@ -373,35 +370,20 @@ __global__ __launch_bounds__(kWide) void nms_duplicate_finish_kernel(NmsArgs a, 
     const uint64_t image = static_cast<uint64_t>(blockIdx.x) << 32;
     const uint32_t begin = lower_bound(a.group_key, n, image);
     const uint32_t end = lower_bound(a.group_key, n, image + 0x100000000ull);
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x / kWave;
     // one repetition per record is the most the argument above allows; the bound makes the exit
     // unconditional
     for (uint32_t repetition = 0; repetition <= end - begin; ++repetition) {
         int left = 0;
-        for (uint32_t p = begin + threadIdx.x; p < end; p += kWide) {
+        for (uint32_t p = begin + wave; p < end; p += kWide / kWave) {
             if (load_state(a.state + p) != kUndecided) continue;
-            const Segments s = a.seg[p];
-            const float4 box = a.box[p];
-            const uint32_t rank = a.rank[p];
-            bool drop = false, pending = false;
-            for (uint32_t q = begin; q < end && !drop; ++q) {
-                if (q == s.group_begin) {                                           // skip the own class
-                    q = s.group_end - 1;
-                    continue;
-                }
-                if (a.rank[q] >= rank) continue;
-                const uint32_t st = load_state(a.state + q);
-                if (st == kDropped) continue;
-                if (overlap_ratio(box, a.box[q]) > kDuplicateOverlap) {
-                    if (st == kKept) drop = true;
-                    else pending = true;
-                }
-            }
-            if (drop) store_state(a.state + p, kDropped);
-            else if (!pending) store_state(a.state + p, kKept);
-            else ++left;
+            const int outcome = duplicate_scan(a, p, lane);
+            if (outcome == 2) left = 1;
+            else if (lane == 0) store_state(a.state + p, outcome == 1 ? kDropped : kKept);
         }
         __threadfence();
-        if (__syncthreads_count(left) == 0) break;
+        if (__syncthreads_or(left) == 0) break;
     }
 }
 
@@ -444,7 +426,7 @@ __global__ __launch_bounds__(kWide) void nms_group_kernel(NmsArgs a, float thres
             for (uint32_t j = from; j < t; ++j) {
                 const uint32_t st = states[j];
                 if (st == kAbsent || st == kDropped) continue;
-                if (overlap_ratio(box, group_box[j]) > threshold) {
+                if (overlaps_above(box, group_box[j], threshold)) {
                     if (st == kKept) {
                         drop = true;
                         break;
@@ -534,6 +516,7 @@ struct Workspace {
     Segments* seg;
     uint32_t* state;
     uint32_t* keep;
+    uint32_t* resume;
     uint32_t* hist;
     uint32_t* tile_kept;
     uint32_t* counters;
@@ -561,6 +544,7 @@ Workspace carve(void* base, int capacity)
     w.seg = reinterpret_cast<Segments*>(take(cap * sizeof(Segments)));
     w.state = reinterpret_cast<uint32_t*>(take(cap * 4));
     w.keep = reinterpret_cast<uint32_t*>(take(cap * 4));
+    w.resume = reinterpret_cast<uint32_t*>(take(cap * 4));
     w.hist = reinterpret_cast<uint32_t*>(take(tiles * kDigits * 4));
     w.tile_kept = reinterpret_cast<uint32_t*>(take(tiles * 4));
     w.counters = reinterpret_cast<uint32_t*>(take(8 * 4));
@@ -568,7 +552,7 @@ Workspace carve(void* base, int capacity)
     return w;
 }
 
-int g_sweeps = 3;      // parallel sweeps of the duplicate pass before the per-image loop takes over
+int g_sweeps = 6;      // parallel sweeps of the duplicate pass before the per-image loop takes over
 
 }  // namespace
 }  // namespace pxh
@@ -633,10 +617,14 @@ int pxh_nms(const pxh_detection* records, const int* count, int capacity, int ba
     NmsArgs a{};
     a.records = records; a.count = count; a.capacity = capacity; a.perm = w.perm;
     a.group_key = w.keys[from]; a.rank = w.vals[from];
-    a.box = w.box; a.seg = w.seg; a.state = w.state; a.keep = w.keep; a.counters = w.counters;
+    a.box = w.box; a.seg = w.seg; a.state = w.state; a.keep = w.keep; a.resume = w.resume; a.counters = w.counters;
     hipLaunchKernelGGL(nms_gather_kernel, per_record, lanes, 0, s, a);
     const int sweeps = g_sweeps;
-    for (int k = 0; k < sweeps; ++k) hipLaunchKernelGGL(nms_duplicate_sweep_kernel, per_record, lanes, 0, s, a, k);
+    // one wave per record, at most 64 Ki workgroups (the rest of a longer list comes round again)
+    const unsigned sweep_blocks = grid_for(capacity, kBlock / kWave) < 65536u ? grid_for(capacity, kBlock / kWave) : 65536u;
+    a.waves = sweep_blocks * (kBlock / kWave);
+    for (int k = 0; k < sweeps; ++k)
+        hipLaunchKernelGGL(nms_duplicate_sweep_kernel, dim3(sweep_blocks), lanes, 0, s, a, k);
     hipLaunchKernelGGL(nms_duplicate_finish_kernel, dim3(batch), wide, 0, s, a, sweeps - 1);
     hipLaunchKernelGGL(nms_group_kernel, dim3(static_cast<unsigned>(batch) * classes), wide, 0, s, a, threshold,
                        FastDiv(classes));
