@@ -278,7 +278,8 @@ int pxh_yolo_detections_append(const float* predictions, int batch, const int* h
  * survivors sorted by descending probability, *kept_count (device) their number.  threshold >= 0.
  * Steps: near-identical boxes (overlap ratio > 0.9) of different classes in one image keep the
  * strongest; then greedy suppression above `threshold` inside each (image, class) group over its
- * first 1024 members.  Workspace: pxh_nms_workspace_bytes(capacity), or NULL for the library's. */
+ * first 1024 members.  Workspace: pxh_nms_workspace_bytes(capacity), or NULL for the library's.
+ * A capacity of at most 512 (an inference pass) runs as one launch and needs no workspace. */
 size_t pxh_nms_workspace_bytes(int capacity);
 int pxh_nms(const pxh_detection* records, const int* count, int capacity, int batch, int classes,
             float threshold, pxh_detection* kept, int* kept_count, void* workspace,

@@ -506,6 +506,102 @@ __global__ __launch_bounds__(kBlock) void nms_write_kept_kernel(NmsArgs a, const
     }
 }
 
+// ---------------------------------------------------------------- short lists in one workgroup
+// Up to 512 records (what an inference pass leaves): everything above in ONE launch, with the
+// records in LDS.  Ranks come from counting the smaller keys.  Both passes take one wave per record,
+// lanes side by side over the records of lower rank, and the waves walk the ranks in ascending
+// order, so nearly every record finds the ones it depends on already decided; the few that do not
+// are taken again.  No group can reach the 1024-place limit.
+constexpr int kSmall = 512;
+
+// One pass over the ranks: `same_class` false = duplicates across classes (src/Box.cpp:65-88), true =
+// greedy suppression inside (image, class) (src/Box.cpp:104-136).
+__device__ __forceinline__ void small_pass(uint32_t n, bool same_class, float threshold, const float4* ranked_box,
+                                           const uint2* ranked_group, uint32_t* state)
+{
+    const volatile uint32_t* states = state;
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x / kWave;
+    // a repetition decides at least the undecided record of lowest rank; the bound makes the exit
+    // unconditional
+    for (uint32_t repetition = 0; repetition <= n; ++repetition) {
+        int left = 0;
+        for (uint32_t t = wave; t < n; t += kWide / kWave) {
+            if (states[t] != kUndecided) continue;
+            const float4 box = ranked_box[t];
+            const uint2 group = ranked_group[t];
+            bool drop = false, pending = false;
+            for (uint32_t j0 = 0; j0 < t && !drop; j0 += kWave) {
+                const uint32_t j = j0 + lane;
+                bool hit = false, wait = false;
+                if (j < t) {
+                    const uint2 other = ranked_group[j];
+                    if (other.x == group.x && (other.y == group.y) == same_class) {
+                        const uint32_t st = states[j];
+                        if ((st == kKept || st == kUndecided) && overlaps_above(box, ranked_box[j], threshold)) {
+                            hit = st == kKept;
+                            wait = st == kUndecided;
+                        }
+                    }
+                }
+                drop = __ballot(hit) != 0;
+                pending = pending || __ballot(wait) != 0;
+            }
+            if (drop || !pending) {
+                if (lane == 0) state[t] = drop ? kDropped : kKept;
+            } else {
+                left = 1;
+            }
+        }
+        if (__syncthreads_or(left) == 0) break;
+    }
+}
+
+__global__ __launch_bounds__(kWide) void nms_small_kernel(const pxh_detection* records, const int* count, int capacity,
+                                                          int batch, int classes, float threshold,
+                                                          pxh_detection* kept, int* kept_count)
+{
+    __shared__ uint64_t key[kSmall];
+    __shared__ float4 ranked_box[kSmall];
+    __shared__ uint2 ranked_group[kSmall];       // image, class
+    __shared__ uint32_t source[kSmall];
+    __shared__ uint32_t state[kSmall];
+    __shared__ uint32_t scan_lds[kWide / kWave + 1];
+    const uint32_t n = live_count(count, capacity);
+    const uint32_t t = threadIdx.x;
+    const bool valid = t < n;
+    pxh_detection d{};
+    if (valid) {
+        d = records[t];
+        key[t] = (static_cast<uint64_t>(descending_bits(d.prob)) << 32) | d.order;
+    }
+    __syncthreads();
+    if (valid) {
+        const uint64_t mine = key[t];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < n; ++j) {
+            const uint64_t k = key[j];
+            rank += (k < mine || (k == mine && j < t)) ? 1u : 0u;
+        }
+        ranked_box[rank] = normalized_rect(d);
+        ranked_group[rank] = make_uint2(static_cast<uint32_t>(min(max(d.batch, 0), batch - 1)),
+                                        static_cast<uint32_t>(min(max(d.class_index, 0), classes - 1)));
+        source[rank] = t;
+        state[rank] = kUndecided;
+    }
+    __syncthreads();
+    small_pass(n, false, kDuplicateOverlap, ranked_box, ranked_group, state);
+    // survivors of the first pass enter the second; the dropped ones are absent from it
+    if (valid) state[t] = state[t] == kKept ? kUndecided : kAbsent;
+    __syncthreads();
+    small_pass(n, true, threshold, ranked_box, ranked_group, state);
+    const bool take = valid && state[t] == kKept;
+    uint32_t total;
+    const uint32_t at = wide_exclusive_scan(take ? 1u : 0u, scan_lds, total);
+    if (take) kept[at] = records[source[t]];
+    if (t == 0) *kept_count = static_cast<int>(total);
+}
+
 size_t align256(size_t b) { return (b + 255) & ~static_cast<size_t>(255); }
 
 struct Workspace {
@@ -587,6 +683,11 @@ int pxh_nms(const pxh_detection* records, const int* count, int capacity, int ba
     }
     if (records == kept && capacity > 0) return fail_invalid("pxh_nms: records and kept must be distinct buffers");
     if (capacity == 0) return pxh_fill_i32(kept_count, 1, 0, stream);
+    if (capacity <= kSmall) {
+        hipLaunchKernelGGL(nms_small_kernel, dim3(1), dim3(kWide), 0, as_stream(stream), records, count, capacity,
+                           batch, classes, threshold, kept, kept_count);
+        return check_launch("pxh_nms");
+    }
     void* ws;
     int rc = resolve_workspace(workspace, workspace_bytes, carve(nullptr, capacity).bytes, &ws);
     if (rc) return rc;
