@@ -271,6 +271,27 @@ def measure_extras(torch, ops, wl, timer, capi):
                 ms_det, "%d records; %.0f%% of the slots pass" % (found, 100 * passing))
             del rec
         del xin, out, dl
+    # ---- non-maximum suppression of device-resident records: an inference-sized list (one image, one
+    # launch) and a validation-sized one (64 images, low confidence threshold).  Not a streaming kernel:
+    # the time is comparisons between records, the bytes column is just the records read and written.
+    for n_rec, images, clusters, cap in [(100, 1, 6, 512), (100000, 64, 8, 1 << 17)]:
+        recs_np = wl.detection_clusters(7, n_rec, images, 80, clusters)
+        recs = torch.zeros((cap, 8), dtype=torch.int32, device=dev)
+        recs[:n_rec] = torch.from_numpy(recs_np.view(np.int32).reshape(-1, 8)).to(dev)
+        cnt = torch.tensor([n_rec], dtype=torch.int32, device=dev)
+        kept = torch.empty_like(recs)
+        kept_cnt = torch.zeros(1, dtype=torch.int32, device=dev)
+        ws_bytes = int(capi.load().pxh_nms_workspace_bytes(cap))
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+
+        def suppress(i):
+            capi.call("pxh_nms", recs.data_ptr(), cnt.data_ptr(), cap, images, 80, 0.45, kept.data_ptr(),
+                      kept_cnt.data_ptr(), ws.data_ptr(), ws_bytes, torch.cuda.current_stream().cuda_stream)
+
+        ms = timer.time(suppress, 10)
+        add("nms(thr .45)", "%d records, %d image%s" % (n_rec, images, "s" if images > 1 else ""), 64 * n_rec, ms,
+            "%d kept; not bandwidth bound" % int(kept_cnt.item()))
+        del recs, kept, ws
     # ---- BN training forward / backward (config 4): batch 16 @608, 13 shapes
     bn_ms = {}
     for (c, s), count in zip(wl.YOLOV3_BN_SHAPES, wl.YOLOV3_BN_COUNTS):

@@ -485,6 +485,71 @@ struct Detection
 
 using Detections = std::vector<Detection>;
 
+// Detections that stay on the device: the YOLO layers of a pass append their records to one list
+// (Model::detections walks the layers the same way, include/Model.h:1078-1109), nms() runs on it in
+// place, and only the survivors cross to the host.  A list of at most 512 records (an inference
+// pass) is suppressed in a single launch.
+class DeviceDetections
+{
+public:
+    explicit DeviceDetections(int capacity) : capacity_(capacity)
+    {
+        PX_CHECK(capacity > 0, "a detection list needs a positive capacity");
+        static_assert(sizeof(pxh_detection) == 8 * sizeof(int), "record layout");
+        records_ = IntVector(static_cast<std::size_t>(capacity) * 8);
+        spare_ = IntVector(static_cast<std::size_t>(capacity) * 8);
+        count_ = IntVector(1, 0);
+        spareCount_ = IntVector(1, 0);
+    }
+
+    int capacity() const noexcept { return capacity_; }
+    pxh_detection* records() noexcept { return reinterpret_cast<pxh_detection*>(records_.data()); }
+    int* count() noexcept { return count_.data(); }
+
+    // Empties the list (ordered on `stream`).
+    void clear(hipStream_t stream = nullptr)
+    {
+        count_.fill(0, stream);
+        nextOrder_ = 0;
+    }
+
+    // The emission order of the next head's first record, and its advance by that head's pairs of
+    // (slot, class).
+    unsigned nextOrder() const noexcept { return nextOrder_; }
+    void advanceOrder(unsigned pairs) noexcept { nextOrder_ += pairs; }
+
+    // nms, src/Box.cpp:56-147, on the device; the list then holds the survivors by descending
+    // probability.  `batch` and `classes` bound the image and class numbers of the records.
+    void nms(int batch, int classes, float threshold, hipStream_t stream = nullptr)
+    {
+        PX_HIP_CHECK(pxh_nms(records(), count_.data(), capacity_, batch, classes, threshold,
+                             reinterpret_cast<pxh_detection*>(spare_.data()), spareCount_.data(), nullptr, 0, stream));
+        std::swap(records_, spare_);
+        std::swap(count_, spareCount_);
+    }
+
+    // Blocking copy to the host, in the list's order.  A list that overflowed holds `capacity` records.
+    Detections toHost(hipStream_t stream = nullptr)
+    {
+        PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(stream));
+        const int found = std::min(std::max(count_.asVector()[0], 0), capacity_);
+        const std::vector<int> raw = records_.asVector();
+        Detections out;
+        out.reserve(static_cast<std::size_t>(found));
+        for (int i = 0; i < found; ++i) {
+            pxh_detection r;
+            std::memcpy(&r, raw.data() + static_cast<std::size_t>(i) * 8, sizeof(r));
+            out.push_back(Detection{ r.x, r.y, r.w, r.h, r.batch, r.class_index, r.prob });
+        }
+        return out;
+    }
+
+private:
+    int capacity_;
+    IntVector records_, spare_, count_, spareCount_;
+    unsigned nextOrder_ = 0;
+};
+
 // ---------------------------------------------------------------- YOLO head
 // reference: include/YoloLayer.h:115-239, 390-547, include/cuda/YoloLayer.h:70-166.
 // The reference assigns the positive slots on the host and uploads them on every training
@@ -573,6 +638,20 @@ public:
             }
             growDetections(found);
         }
+    }
+
+    // The same onto a device-resident list, without synchronising: the records go behind those of
+    // the YOLO layers asked before, with emission orders that continue theirs.
+    void addDetects(DeviceDetections& list, int width, int height, float threshold)
+    {
+        const auto& c = context();
+        PX_HIP_CHECK(pxh_yolo_detections_append(output_.data(), batch(), mask_.data(), static_cast<int>(mask_.size()),
+                                                anchors_.data(), numAnchors_, c.classes, this->width(),
+                                                this->height(), c.width, c.height, width, height, threshold,
+                                                list.nextOrder(), list.records(), list.capacity(), list.count(),
+                                                stream()));
+        list.advanceOrder(static_cast<unsigned>(batch()) * static_cast<unsigned>(mask_.size()) *
+                          static_cast<unsigned>(this->width() * this->height()) * static_cast<unsigned>(c.classes));
     }
 
     // Blocking: cost = sum(delta^2) / max(1, batch) (reference: include/cuda/YoloLayer.h:132).

@@ -6,7 +6,7 @@ Tensors must be fp32 (int32 for indices), contiguous and on a HIP device.
 import numpy as np
 import torch
 
-from . import capi
+from . import capi, workloads
 from .capi import PxError, act_id, call, ptr
 
 
@@ -331,8 +331,7 @@ def rescale_clip(x, threshold=0.0, clip=0.0, norm_out=None):
     call("pxh_rescale_clip", ptr(x), x.numel(), float(threshold), float(clip), ptr(norm_out), None, 0, _stream())
 
 
-DETECTION_DTYPE = np.dtype([("x", "f4"), ("y", "f4"), ("w", "f4"), ("h", "f4"), ("prob", "f4"), ("batch", "i4"),
-                            ("class_index", "i4"), ("order", "u4")])
+DETECTION_DTYPE = workloads.DETECTION_DTYPE
 
 
 def yolo_detections(predictions, batch, masks, anchors, classes, width, height, net_width, net_height, threshold,

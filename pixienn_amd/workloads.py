@@ -95,3 +95,30 @@ def yolo_assign_targets(truths, counts, masks, anchors, width, height, net_width
             anc[s] = best
             box[s] = (x, y, w, h)
     return cls, anc, box
+
+
+# one detection record of the C ABI (struct pxh_detection): left, top, width, height, probability,
+# image, class, position in the reference's emission order
+DETECTION_DTYPE = np.dtype([("x", "f4"), ("y", "f4"), ("w", "f4"), ("h", "f4"), ("prob", "f4"), ("batch", "i4"),
+                            ("class_index", "i4"), ("order", "u4")])
+
+
+def detection_clusters(seed, n, batch, classes, clusters, spread=6.0):
+    """n detection records scattered around a few centres per image, so that many overlap, with
+    probabilities rounded to two decimals (plenty of ties) -- input for non-maximum suppression."""
+    g = rng(seed)
+    rec = np.zeros(n, DETECTION_DTYPE)
+    centre = g.uniform(50, 400, (batch, clusters, 2))
+    size = g.uniform(20, 120, (batch, clusters, 2))
+    b = g.integers(0, batch, n)
+    k = g.integers(0, clusters, n)
+    rec["batch"] = b
+    rec["class_index"] = g.integers(0, classes, n)
+    jitter = g.normal(0, spread, (n, 4)).astype(np.float32)
+    rec["w"] = np.maximum(1, size[b, k, 0] + jitter[:, 2])
+    rec["h"] = np.maximum(1, size[b, k, 1] + jitter[:, 3])
+    rec["x"] = centre[b, k, 0] + jitter[:, 0] - rec["w"] / 2
+    rec["y"] = centre[b, k, 1] + jitter[:, 1] - rec["h"] / 2
+    rec["prob"] = np.round(g.uniform(0.05, 1.0, n), 2).astype(np.float32)
+    rec["order"] = np.arange(n)
+    return rec

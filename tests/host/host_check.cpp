@@ -299,6 +299,46 @@ void inferenceChecks()
             // integer pixel boxes may differ by one where a last-place difference in exp moves a truncation
             expectClose(std::string("yolo7 detection boxes") + (scaled ? " (pixel boxes)" : ""), gb, wb,
                         scaled ? 1.0 / 320.0 : 1e-5, scaled ? 320.0 : 4.0);
+            // the same records kept on the device, the head asked twice (as two YOLO layers would be),
+            // then nms there; the checker's nms runs on the host copies of the device's own records
+            for (int capacity: { 512, 16384 }) {         // one-launch form and sorting form
+                // the short list needs a confidence that leaves at most 256 records per head
+                float confidence = 0.3f;
+                Detections once;
+                for (float c: { 0.3f, 0.8f, 0.9f, 0.95f, 0.98f }) {
+                    confidence = c;
+                    once.clear();
+                    net.yolo7->addDetects(once, iw, ih, confidence);
+                    if (2 * static_cast<int>(once.size()) <= capacity) break;
+                }
+                const int each = static_cast<int>(once.size());
+                DeviceDetections list(capacity);
+                list.clear();
+                net.yolo7->addDetects(list, iw, ih, confidence);
+                net.yolo7->addDetects(list, iw, ih, confidence);
+                const Detections both = list.toHost();
+                std::vector<pxo_detection> input;
+                for (int pass = 0; pass < 2; ++pass)
+                    for (const auto& d: once)
+                        input.push_back(pxo_detection{ d.x, d.y, d.w, d.h, d.prob, d.batchId, d.classIndex,
+                                                       static_cast<unsigned>(input.size()) });
+                const bool fits = each > 0 && 2 * each <= capacity;
+                report("two heads append " + std::to_string(both.size()) + " records into a list of " +
+                       std::to_string(capacity), fits && static_cast<int>(both.size()) == 2 * each);
+                if (!fits) continue;
+                std::vector<pxo_detection> kept(input.size());
+                const int keptCount = pxo_nms(input.data(), static_cast<int>(input.size()), 0.45f, kept.data());
+                list.nms(N, CLASSES, 0.45f);
+                const Detections survivors = list.toHost();
+                bool equal = static_cast<int>(survivors.size()) == keptCount && keptCount > 0 && keptCount <= each;
+                for (int k = 0; equal && k < keptCount; ++k)
+                    equal = survivors[k].x == kept[k].x && survivors[k].y == kept[k].y && survivors[k].w == kept[k].w &&
+                            survivors[k].h == kept[k].h && survivors[k].prob == kept[k].prob &&
+                            survivors[k].batchId == kept[k].batch && survivors[k].classIndex == kept[k].class_index;
+                report(std::string("nms on the device list") + (scaled ? " (pixel boxes)" : "") + ", capacity " +
+                       std::to_string(capacity), equal, std::to_string(keptCount) + " of " +
+                       std::to_string(input.size()) + " kept");
+            }
         }
     }
 }

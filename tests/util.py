@@ -78,20 +78,7 @@ def detection_records(oracle, rows):
 
 
 def random_detections(oracle, seed, n, batch, classes, clusters, spread=6.0):
-    """Boxes scattered around a few centres per image so that many overlap, with tied probabilities."""
-    g = np.random.Generator(np.random.Philox(key=seed))
-    rec = np.zeros(n, oracle.DETECTION_DTYPE)
-    centre = g.uniform(50, 400, (batch, clusters, 2))
-    size = g.uniform(20, 120, (batch, clusters, 2))
-    b = g.integers(0, batch, n)
-    k = g.integers(0, clusters, n)
-    rec["batch"] = b
-    rec["class_index"] = g.integers(0, classes, n)
-    jitter = g.normal(0, spread, (n, 4)).astype(F)
-    rec["w"] = np.maximum(1, size[b, k, 0] + jitter[:, 2])
-    rec["h"] = np.maximum(1, size[b, k, 1] + jitter[:, 3])
-    rec["x"] = centre[b, k, 0] + jitter[:, 0] - rec["w"] / 2
-    rec["y"] = centre[b, k, 1] + jitter[:, 1] - rec["h"] / 2
-    rec["prob"] = np.round(g.uniform(0.05, 1.0, n), 2).astype(F)         # two decimals: plenty of ties
-    rec["order"] = np.arange(n)
-    return rec
+    """Overlapping boxes around a few centres per image (pixienn_amd.workloads.detection_clusters)."""
+    from pixienn_amd import workloads
+    assert workloads.DETECTION_DTYPE == oracle.DETECTION_DTYPE
+    return workloads.detection_clusters(seed, n, batch, classes, clusters, spread)
