@@ -23,7 +23,7 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x2 __attribute__((ext_vector_type(2)));
 
 // A launch that touches at least this many bytes streams past the last-level cache.
-constexpr size_t kStreamingBytes = 192u << 20;
+constexpr size_t kStreamingBytes = 128u << 20;
 
 // V consecutive 32-bit values, aligned for the widest single access (128 bits).
 template<int V>
