@@ -115,14 +115,35 @@ __global__ __launch_bounds__(kBlock) void epilogue_fwd_kernel(EpilogueArgs a)
     a.by_channels.divmod(plane, q, c);
     const FoldCoef k0 = fetch_coef<BN>(a, c);
     Pack<4> yo, po, no;
-    if (r + 3 < hw) {
+    const bool crosses = !(r + 3 < hw);
+    if (!__ballot(crosses)) {
+        // no lane of the wave touches a plane boundary (the common case for large planes)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             po.v[j] = pre_value<BN>(xin.v[j], k0, no.v[j]);
             yo.v[j] = act_apply<ACT>(po.v[j]);
         }
+    } else if (hw >= 4) {
+        // some lane's vector runs into the next plane (at most one boundary per vector): the
+        // elements past it take the next channel's constants.  Selecting the constants per element
+        // keeps ONE copy of the arithmetic for the whole wave; a per-lane branch would make a wave
+        // that holds a boundary (every wave, for a 13 x 13 plane) run the activation twice.
+        FoldCoef k1 = k0;
+        if (crosses) k1 = fetch_coef<BN>(a, c + 1 == a.by_channels.d ? 0 : c + 1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool here = r + j < hw;
+            FoldCoef k;
+            k.mean = here ? k0.mean : k1.mean;
+            k.r_hi = here ? k0.r_hi : k1.r_hi;
+            k.r_lo = here ? k0.r_lo : k1.r_lo;
+            k.scale = here ? k0.scale : k1.scale;
+            k.bias = here ? k0.bias : k1.bias;
+            po.v[j] = pre_value<BN>(xin.v[j], k, no.v[j]);
+            yo.v[j] = act_apply<ACT>(po.v[j]);
+        }
     } else {
-        // crosses into the next plane(s): walk element by element
+        // planes of fewer than 4 elements: several boundaries per vector, walk element by element
         FoldCoef k = k0;
         uint32_t rr = r, cc = c;
 #pragma unroll
@@ -543,10 +564,31 @@ __global__ __launch_bounds__(kBlock) void bn_dx_kernel(DxArgs a)
     a.by_spatial.divmod(e, plane, r);
     a.by_channels.divmod(plane, q, c);
     Pack<4> out;
-    if (r + 3 < hw) {
+    const bool crosses = !(r + 3 < hw);
+    if (!__ballot(crosses)) {
         const DxCoef k = a.coef[c];
 #pragma unroll
         for (int j = 0; j < 4; ++j) out.v[j] = dx_value<ACT>(din.v[j], xin.v[j], pin.v[j], recompute, k);
+    } else if (hw >= 4) {
+        // one boundary per vector at most: constants selected per element, one copy of the arithmetic
+        // for the wave (see epilogue_fwd_kernel)
+        const DxCoef k0 = a.coef[c];
+        DxCoef k1 = k0;
+        if (crosses) k1 = a.coef[c + 1 == a.by_channels.d ? 0 : c + 1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool here = r + j < hw;
+            DxCoef k;
+            k.f.mean = here ? k0.f.mean : k1.f.mean;
+            k.f.r_hi = here ? k0.f.r_hi : k1.f.r_hi;
+            k.f.r_lo = here ? k0.f.r_lo : k1.f.r_lo;
+            k.f.scale = here ? k0.f.scale : k1.f.scale;
+            k.f.bias = here ? k0.f.bias : k1.f.bias;
+            k.rroot = here ? k0.rroot : k1.rroot;
+            k.c2 = here ? k0.c2 : k1.c2;
+            k.md_term = here ? k0.md_term : k1.md_term;
+            out.v[j] = dx_value<ACT>(din.v[j], xin.v[j], pin.v[j], recompute, k);
+        }
     } else {
         uint32_t rr = r, cc = c;
 #pragma unroll
