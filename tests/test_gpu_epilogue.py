@@ -129,7 +129,9 @@ TRAIN_SHAPES = [(4, 8, 52 * 52), (3, 16, 361), (16, 5, 169), (2, 3, 4096 + 512),
                 (1, 3, 37), (6, 9, 8), (3, 5, 7),
                 # 96 channels and more with a channel slice that fits one workgroup: the single-launch path,
                 # scalar and 128-bit; then the same channel counts with slices that do not fit
-                (3, 96, 361), (2, 100, 1444), (16, 128, 1444), (4, 96, 2047), (4, 96, 5001), (16, 97, 76 * 76)]
+                (3, 96, 361), (2, 100, 1444), (16, 128, 1444), (4, 96, 2047), (4, 96, 5001), (16, 97, 76 * 76),
+                # the large single-launch form (part of the slice in LDS), above and below 128 channels
+                (8, 192, 4800), (9, 100, 4096 + 8)]
 
 
 @pytest.mark.parametrize("act", ["leaky", "mish", "linear"])
