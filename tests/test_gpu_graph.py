@@ -70,3 +70,68 @@ def test_layer_sequence_in_a_graph_matches_eager():
         for k in buf:
             assert torch.equal(buf[k], eager[k]), "replay %d differs from eager in %s" % (step, k)
     assert float(buf["stats"][6]) > 0 and float(buf["norm"][0]) > 50.0
+
+
+@pytest.mark.parametrize("capacity", [512, 1 << 14], ids=["one-workgroup", "sorted"])
+def test_inference_postprocessing_in_a_graph_matches_eager(capacity):
+    """decode -> detections of two heads into one list -> nms, captured once and replayed on new
+    logits: the counter is cleared by a kernel, the record count never leaves the device."""
+    import torch
+    from pixienn_amd import ops
+    N, K = 2, 5
+    heads = [(13, [3, 4, 5]), (26, [0, 1, 2])]
+    thr = 0.9 if capacity == 512 else 0.3
+    dev = "cuda"
+    logits = [torch.zeros((N, 3 * (K + 5), W, W), device=dev) for W, _ in heads]
+
+    def make():
+        return dict(decoded=[torch.empty_like(l) for l in logits],
+                    records=torch.zeros((capacity, 8), dtype=torch.int32, device=dev),
+                    count=torch.zeros(1, dtype=torch.int32, device=dev),
+                    kept=torch.zeros((capacity, 8), dtype=torch.int32, device=dev),
+                    kept_count=torch.zeros(1, dtype=torch.int32, device=dev),
+                    ws=torch.empty(max(256, int(ops.capi.load().pxh_nms_workspace_bytes(capacity))), dtype=torch.uint8,
+                                   device=dev))
+
+    def sequence(b):
+        b["count"].zero_()
+        base = 0
+        for (W, mask), raw, dec in zip(heads, logits, b["decoded"]):
+            ops.yolo_activate(raw, dec, N, 3, K, W * W)
+            ops.yolo_detections_append(dec, N, mask, wl.TINY_ANCHORS, K, W, W, 416, 416, thr, base, b["records"],
+                                       b["count"], image_width=640, image_height=480)
+            base += N * 3 * W * W * K
+        ops.capi.call("pxh_nms", b["records"].data_ptr(), b["count"].data_ptr(), capacity, N, K, 0.45,
+                      b["kept"].data_ptr(), b["kept_count"].data_ptr(), b["ws"].data_ptr(),
+                      b["ws"].numel(), torch.cuda.current_stream().cuda_stream)
+
+    def load(step):
+        for i, l in enumerate(logits):
+            l.copy_(gpu(wl.normal(9400 + 10 * step + i, tuple(l.shape), std=1.5)))
+
+    def survivors(b):
+        n = int(b["kept_count"].item())
+        return n, b["kept"][:n].clone()
+
+    load(0)
+    static, eager = make(), make()
+    sequence(eager)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sequence(static)
+    seen = set()
+    for step in range(1, 4):
+        load(step)
+        graph.replay()
+        torch.cuda.synchronize()
+        sequence(eager)
+        torch.cuda.synchronize()
+        n_graph, kept_graph = survivors(static)
+        n_eager, kept_eager = survivors(eager)
+        # a list that overflows keeps whichever records came first: the case must fit
+        assert 0 < int(static["count"].item()) == int(eager["count"].item()) <= capacity, (step, static["count"])
+        assert 0 < n_graph == n_eager, (step, n_graph, n_eager)
+        assert torch.equal(kept_graph, kept_eager), "replay %d differs from eager" % step
+        seen.add(n_graph)
+    assert len(seen) > 1, "the replays must have seen different data"
