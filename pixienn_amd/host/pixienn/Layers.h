@@ -528,6 +528,14 @@ public:
         std::swap(count_, spareCount_);
     }
 
+    // Blocking: how many records the YOLO layers found.  More than capacity() means the list overflowed
+    // and holds whichever records arrived first; the caller then repeats the pass with a larger list.
+    int found(hipStream_t stream = nullptr)
+    {
+        PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(stream));
+        return count_.asVector()[0];
+    }
+
     // Blocking copy to the host, in the list's order.  A list that overflowed holds `capacity` records.
     Detections toHost(hipStream_t stream = nullptr)
     {
