@@ -4,6 +4,7 @@
 #pragma once
 
 #include <cstddef>
+#include <initializer_list>
 #include <type_traits>
 #include <utility>
 #include <vector>
@@ -32,6 +33,8 @@ public:
     }
 
     explicit DeviceVector(const std::vector<T>& host) : DeviceVector(host.data(), host.data() + host.size()) {}
+
+    DeviceVector(std::initializer_list<T> host) : DeviceVector(host.begin(), host.end()) {}
 
     DeviceVector(const DeviceVector&) = delete;
     DeviceVector& operator=(const DeviceVector&) = delete;
@@ -78,6 +81,14 @@ public:
 
     void copyHost(const std::vector<T>& host) { copyHost(host.data(), host.size()); }
 
+    // Device -> device copy of n elements from a raw device pointer, ordered on `stream`.
+    void copyDevice(const T* device, size_type n, hipStream_t stream = nullptr)
+    {
+        PX_CHECK(n <= size_, "device source larger than the device vector");
+        if (n == 0) return;
+        PX_HIP_RUNTIME_CHECK(hipMemcpyAsync(data_, device, n * sizeof(T), hipMemcpyDeviceToDevice, stream));
+    }
+
     // Blocking device -> host copy (waits for all work queued before it on the null stream).
     std::vector<T> asVector() const
     {
@@ -86,18 +97,19 @@ public:
         return host;
     }
 
-private:
-    void allocate(size_type n)
-    {
-        size_ = n;
-        if (n) PX_HIP_RUNTIME_CHECK(hipMalloc(reinterpret_cast<void**>(&data_), n * sizeof(T)));
-    }
-
+    // Frees the buffer now (the destructor does the same).
     void release() noexcept
     {
         if (data_) (void) hipFree(data_);
         data_ = nullptr;
         size_ = 0;
+    }
+
+private:
+    void allocate(size_type n)
+    {
+        size_ = n;
+        if (n) PX_HIP_RUNTIME_CHECK(hipMalloc(reinterpret_cast<void**>(&data_), n * sizeof(T)));
     }
 
     void swap(DeviceVector& rhs) noexcept

@@ -223,6 +223,30 @@ void convForwardCheck(const std::string& name, ConvLayer& layer, const Host& inp
     if (varOut) *varOut = var;
 }
 
+// the device vector's contract (reference: tests/src/vector.cpp -- fill, initializer list, copies)
+void deviceVectorChecks()
+{
+    FloatVector filled(7, 7.0f);
+    report("vector(count, value) fills", filled.asVector() == Host(7, 7.0f));
+    const FloatVector listed{ 1.0f, 2.0f, 3.0f, 4.0f };
+    report("vector from an initializer list", listed.size() == 4 && listed.asVector() == Host{ 1, 2, 3, 4 });
+    IntVector ints{ 1, 2, 3 };
+    report("int vector", ints.asVector() == std::vector<int>{ 1, 2, 3 });
+    FloatVector copy(4);
+    copy.copy(listed);
+    report("device to device copy", copy.asVector() == Host{ 1, 2, 3, 4 });
+    FloatVector part(6, 0.0f);
+    part.copyDevice(listed.data() + 1, 3);
+    report("copy from a raw device pointer", part.asVector() == Host{ 2, 3, 4, 0, 0, 0 });
+    part.copyHost(Host{ 9, 8 });
+    report("copy from the host", part.asVector() == Host{ 9, 8, 4, 0, 0, 0 });
+    FloatVector moved(std::move(part));
+    report("move leaves the source empty", part.empty() && moved.size() == 6);
+    moved.release();
+    report("release frees", moved.empty() && moved.data() == nullptr);
+    expectThrows("copy between different sizes is refused", [&] { copy.copy(filled); }, "different sizes");
+}
+
 void inferenceChecks()
 {
     Net net(false);
@@ -611,6 +635,7 @@ int main(int argc, char** argv)
                 std::printf("no GPU visible\n");
                 return 2;
             }
+            deviceVectorChecks();
             inferenceChecks();
             trainingChecks();
             absorbedUpsampleChecks();
