@@ -235,6 +235,114 @@ private:
     ConvolveBackward convolveBackward_;
 };
 
+// ---------------------------------------------------------------- stand-alone batch norm
+// reference: include/BatchNormLayer.h:39-183, include/cuda/BatchNormLayer.h:59-137.  The layer's
+// input is read again in backward (the reference keeps copies x_ and xNorm_ of it instead), so it
+// must be unchanged between the two calls, as it is when a model drives the layers in order.
+class BatchNormLayer : public Layer
+{
+public:
+    BatchNormLayer(Context& context, const Properties& props) : Layer(context, props)
+    {
+        setOutput(channels(), height(), width());
+        const auto c = static_cast<std::size_t>(channels());
+        biases_ = V(c, 0.0f);
+        scales_ = V(c, 1.0f);
+        rollingMean_ = V(c, 0.0f);
+        rollingVar_ = V(c, 0.0f);
+        folded_ = V(pxh_bn_folded_bytes(channels()) / sizeof(float));
+        if (training()) {
+            mean_ = V(c, 0.0f);
+            var_ = V(c, 0.0f);
+            biasUpdates_ = V(c, 0.0f);
+            scaleUpdates_ = V(c, 0.0f);
+        }
+    }
+
+    void forward(const V& input) override
+    {
+        Layer::forward(input);
+        checkInput(input, "BatchNormLayer");
+        const int spatial = outHeight() * outWidth();
+        if (training()) {
+            PX_HIP_CHECK(pxh_bn_train_act_forward(input.data(), output_.data(), nullptr, nullptr, nullptr, mean_.data(),
+                                                  var_.data(), rollingMean_.data(), rollingVar_.data(),
+                                                  scales_.data(), biases_.data(), batch(), channels(), spatial,
+                                                  PXH_LINEAR, nullptr, 0, stream()));
+            foldedValid_ = false;
+            return;
+        }
+        if (!foldedValid_) {
+            PX_HIP_CHECK(pxh_bn_fold(rollingMean_.data(), rollingVar_.data(), scales_.data(), biases_.data(),
+                                     channels(), folded_.data(), stream()));
+            foldedValid_ = true;
+        }
+        PX_HIP_CHECK(pxh_bn_folded_act_forward(input.data(), output_.data(), nullptr, folded_.data(), batch(),
+                                               channels(), spatial, PXH_LINEAR, stream()));
+    }
+
+    void backward(const V& input, V* grad) override
+    {
+        Layer::backward(input, grad);
+        PX_CHECK(training(), "BatchNormLayer: backward needs a training context");
+        checkInput(input, "BatchNormLayer");
+        PX_HIP_CHECK(pxh_bn_act_backward(delta_.data(), input.data(), nullptr, mean_.data(), var_.data(),
+                                         scales_.data(), biases_.data(), scaleUpdates_.data(), biasUpdates_.data(),
+                                         nullptr, nullptr, batch(), channels(), outHeight() * outWidth(), PXH_LINEAR,
+                                         nullptr, 0, stream()));
+        if (grad) PX_HIP_CHECK(pxh_axpy(delta_.size(), 1.0f, delta_.data(), grad->data(), stream()));
+    }
+
+    // plain momentum steps on biases and scales, no weight decay (include/BatchNormLayer.h:166-181)
+    void update() override
+    {
+        const auto& c = context();
+        PX_HIP_CHECK(pxh_sgd_update(biases_.size(), biases_.data(), biasUpdates_.data(), c.updateBatch, c.learningRate,
+                                    c.momentum, 0.0f, 0, stream()));
+        PX_HIP_CHECK(pxh_sgd_update(scales_.size(), scales_.data(), scaleUpdates_.data(), c.updateBatch,
+                                    c.learningRate, c.momentum, 0.0f, 0, stream()));
+        foldedValid_ = false;
+    }
+
+    // biases, scales, rolling mean, rolling variance as raw fp32 (include/BatchNormLayer.h:72-113)
+    std::streamoff loadWeights(std::istream& is)
+    {
+        const auto start = is.tellg();
+        for (V* t: { &biases_, &scales_, &rollingMean_, &rollingVar_ }) {
+            std::vector<float> host(t->size());
+            is.read(reinterpret_cast<char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
+            PX_CHECK(is.good(), "Could not read batch normalize parameters");
+            t->copyHost(host);
+        }
+        foldedValid_ = false;
+        return is.tellg() - start;
+    }
+
+    std::streamoff saveWeights(std::ostream& os)
+    {
+        const auto start = os.tellp();
+        for (const V* t: { &biases_, &scales_, &rollingMean_, &rollingVar_ }) {
+            const std::vector<float> host = t->asVector();
+            os.write(reinterpret_cast<const char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
+        }
+        PX_CHECK(os.good(), "Could not write batch normalize parameters");
+        return os.tellp() - start;
+    }
+
+    const V& biases() const noexcept { return biases_; }
+    const V& scales() const noexcept { return scales_; }
+    const V& rollingMean() const noexcept { return rollingMean_; }
+    const V& rollingVariance() const noexcept { return rollingVar_; }
+    const V& mean() const noexcept { return mean_; }
+    const V& variance() const noexcept { return var_; }
+    const V& biasUpdates() const noexcept { return biasUpdates_; }
+    const V& scaleUpdates() const noexcept { return scaleUpdates_; }
+
+private:
+    bool foldedValid_ = false;
+    V biases_, scales_, rollingMean_, rollingVar_, mean_, var_, folded_, biasUpdates_, scaleUpdates_;
+};
+
 // ---------------------------------------------------------------- max-pool
 // reference: include/MaxPoolLayer.h:50-158, include/cuda/MaxPoolLayer.h
 class MaxPoolLayer : public Layer

@@ -574,6 +574,76 @@ void trainingChecks()
     }
 }
 
+// The stand-alone batch-norm layer: inference, training forward/backward/update and the weight file
+// section, against the checker's batchNormForward / batchNormBackward.
+void batchNormLayerChecks()
+{
+    const int BC = 6, BS = 12;
+    const size_t total = size_t(N) * BC * BS * BS;
+    const Host x = normals(401, total, 1.5f, 0.3f);
+    const Host biases = normals(402, BC, 0.2f), scales = uniforms(403, BC, 0.5f, 1.5f);
+    const Host rmean = normals(404, BC, 0.1f), rvar = uniforms(405, BC, 0.5f, 1.5f);
+    std::stringstream file(std::ios::in | std::ios::out | std::ios::binary);
+    for (const Host* t: { &biases, &scales, &rmean, &rvar })
+        file.write(reinterpret_cast<const char*>(t->data()), std::streamsize(t->size() * sizeof(float)));
+    const Properties props{ { "batch", N }, { "channels", BC }, { "height", BS }, { "width", BS } };
+    const FloatVector input(x);
+    {
+        Context ctx;
+        ctx.training = false;
+        BatchNormLayer layer(ctx, props);
+        file.seekg(0);
+        const auto bytes = layer.loadWeights(file);
+        report("batchnorm weight section is 4 x channels floats", bytes == std::streamoff(4 * BC * sizeof(float)));
+        layer.forward(input);
+        Host want(total), m(BC), v(BC), rm = rmean, rv = rvar;
+        pxo_batchnorm_forward(0, N, BC, BS, BS, x.data(), want.data(), m.data(), v.data(), rm.data(), rv.data(),
+                              scales.data(), biases.data(), nullptr, nullptr, 0);
+        expectClose("batchnorm layer, inference", layer.output().asVector(), want, 1e-5, 1.0);
+        std::stringstream out(std::ios::in | std::ios::out | std::ios::binary);
+        layer.saveWeights(out);
+        report("batchnorm weights round trip", out.str() == file.str());
+    }
+    Context ctx;
+    ctx.training = true;
+    ctx.updateBatch = N;
+    ctx.learningRate = 0.01f;
+    ctx.momentum = 0.9f;
+    BatchNormLayer layer(ctx, props);
+    file.clear();
+    file.seekg(0);
+    layer.loadWeights(file);
+    layer.forward(input);
+    Host want(total), mean(BC), var(BC), rm = rmean, rv = rvar, xs(total), xn(total);
+    pxo_batchnorm_forward(1, N, BC, BS, BS, x.data(), want.data(), mean.data(), var.data(), rm.data(), rv.data(),
+                          scales.data(), biases.data(), xs.data(), xn.data(), 0);
+    expectClose("batchnorm layer, training forward", layer.output().asVector(), want, 1e-5, 4.0);
+    expectClose("batchnorm layer, rolling mean", layer.rollingMean().asVector(), rm, 1e-5, 0.05);
+    expectClose("batchnorm layer, rolling variance", layer.rollingVariance().asVector(), rv, 1e-5, 1.0);
+    Host delta = normals(406, total);
+    const Host grad0 = normals(407, total);
+    layer.delta().copyHost(delta);
+    FloatVector grad(grad0);
+    layer.backward(input, &grad);
+    Host md(BC), vd(BC), su(BC, 0.0f), bu(BC, 0.0f);
+    pxo_batchnorm_backward(N, BC, BS, BS, delta.data(), mean.data(), var.data(), md.data(), vd.data(), scales.data(),
+                           su.data(), bu.data(), xs.data(), xn.data(), 0);
+    Host wantGrad = grad0;
+    for (size_t i = 0; i < total; ++i) wantGrad[i] = wantGrad[i] + delta[i];
+    expectClose("batchnorm layer, backward delta", layer.delta().asVector(), delta, 1e-5, 2.0);
+    expectClose("batchnorm layer, backward into grad", grad.asVector(), wantGrad, 1e-5, 2.0);
+    expectClose("batchnorm layer, scale updates", layer.scaleUpdates().asVector(), su, 1e-5, 30.0);
+    expectClose("batchnorm layer, bias updates", layer.biasUpdates().asVector(), bu, 1e-5, 30.0);
+    layer.update();
+    Host wb = biases, ws = scales, dsu = layer.scaleUpdates().asVector(), dbu = layer.biasUpdates().asVector();
+    // the layer's own updates before the step were su / bu up to rounding; use the checker's
+    pxo_sgd_update(BC, wb.data(), bu.data(), N, 0.01f, 0.9f, 0.0f, 0);
+    pxo_sgd_update(BC, ws.data(), su.data(), N, 0.01f, 0.9f, 0.0f, 0);
+    expectClose("batchnorm layer, biases after update", layer.biases().asVector(), wb, 1e-5, 1.0);
+    expectClose("batchnorm layer, scales after update", layer.scales().asVector(), ws, 1e-5, 1.0);
+    expectClose("batchnorm layer, momentum kept in the updates", dbu, bu, 1e-5, 30.0);
+}
+
 // An upsample layer absorbed by the route that reads it gives the same tensors as the two-step form.
 void absorbedUpsampleChecks()
 {
@@ -639,6 +709,7 @@ int main(int argc, char** argv)
             inferenceChecks();
             trainingChecks();
             absorbedUpsampleChecks();
+            batchNormLayerChecks();
         }
     } catch (const std::exception& e) {
         std::printf("unexpected exception: %s\n", e.what());
