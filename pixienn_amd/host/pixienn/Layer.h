@@ -177,6 +177,11 @@ public:
 
     virtual void update() {}
 
+    // This layer's section of a weight file; bytes read / written (reference: Layer<D>::loadWeights /
+    // saveWeights, include/Layer.h:57-58).  Layers without parameters have none.
+    virtual std::streamoff loadWeights(std::istream& /*is*/) { return 0; }
+    virtual std::streamoff saveWeights(std::ostream& /*os*/) { return 0; }
+
     // Optimizer moments for the checkpoint sidecar; bytes written / read (reference:
     // Layer<D>::saveOptimizer / loadOptimizer, include/Layer.h:59-60).  Nothing by default.
     virtual std::streamoff saveOptimizer(std::ostream& /*os*/) { return 0; }

@@ -173,6 +173,32 @@ public:
         foldedValid_ = false;
     }
 
+    // biases [, scales, rolling mean, rolling variance], weights as raw fp32 (reference:
+    // include/ConvLayer.h:132-171)
+    std::streamoff loadWeights(std::istream& is) override
+    {
+        const auto start = is.tellg();
+        for (V* t: weightFileOrder()) {
+            std::vector<float> host(t->size());
+            is.read(reinterpret_cast<char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
+            PX_CHECK(is.good() || host.empty(), "Could not read weights");
+            t->copyHost(host);
+        }
+        foldedValid_ = false;
+        return is.tellg() - start;
+    }
+
+    std::streamoff saveWeights(std::ostream& os) override
+    {
+        const auto start = os.tellp();
+        for (const V* t: weightFileOrder()) {
+            const std::vector<float> host = t->asVector();
+            os.write(reinterpret_cast<const char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
+        }
+        PX_CHECK(os.good(), "Could not write weights");
+        return os.tellp() - start;
+    }
+
     // m, v, bias_m, bias_v, scale_m, scale_v as raw fp32 (reference: include/cuda/ConvLayer.h:228-264)
     std::streamoff saveOptimizer(std::ostream& os) override
     {
@@ -209,6 +235,12 @@ public:
     const V& scaleUpdates() const noexcept { return scaleUpdates_; }
 
 private:
+    std::vector<V*> weightFileOrder()
+    {
+        if (batchNorm_) return { &biases_, &scales_, &rollingMean_, &rollingVar_, &weights_ };
+        return { &biases_, &weights_ };
+    }
+
     void load(V& dst, const std::vector<float>& src)
     {
         PX_CHECK(dst.size() == src.size(), "ConvLayer: parameter vector of the wrong size");
@@ -305,7 +337,7 @@ public:
     }
 
     // biases, scales, rolling mean, rolling variance as raw fp32 (include/BatchNormLayer.h:72-113)
-    std::streamoff loadWeights(std::istream& is)
+    std::streamoff loadWeights(std::istream& is) override
     {
         const auto start = is.tellg();
         for (V* t: { &biases_, &scales_, &rollingMean_, &rollingVar_ }) {
@@ -318,7 +350,7 @@ public:
         return is.tellg() - start;
     }
 
-    std::streamoff saveWeights(std::ostream& os)
+    std::streamoff saveWeights(std::ostream& os) override
     {
         const auto start = os.tellp();
         for (const V* t: { &biases_, &scales_, &rollingMean_, &rollingVar_ }) {

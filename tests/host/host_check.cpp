@@ -604,6 +604,36 @@ void batchNormLayerChecks()
         layer.saveWeights(out);
         report("batchnorm weights round trip", out.str() == file.str());
     }
+    {   // a conv layer's section: biases, scales, rolling mean, rolling variance, then the weights
+        Context ctx;
+        ctx.training = false;
+        const int weights = BC * BC * 9;
+        ConvLayer conv(ctx, Properties{ { "batch", N }, { "channels", BC }, { "height", BS }, { "width", BS },
+                                         { "filters", BC }, { "batch_normalize", true }, { "weights", weights },
+                                         { "activation", std::string("leaky") } });
+        const Host w = normals(408, weights, 0.02f);
+        std::stringstream section(std::ios::in | std::ios::out | std::ios::binary);
+        for (const Host* t: { &biases, &scales, &rmean, &rvar, &w })
+            section.write(reinterpret_cast<const char*>(t->data()), std::streamsize(t->size() * sizeof(float)));
+        const auto bytes = conv.loadWeights(section);
+        report("conv weight section: 4 x filters + weights floats",
+               bytes == std::streamoff((4 * BC + weights) * sizeof(float)) && conv.weights().asVector() == w &&
+               conv.scales().asVector() == scales && conv.rollingVariance().asVector() == rvar);
+        std::stringstream out(std::ios::in | std::ios::out | std::ios::binary);
+        conv.saveWeights(out);
+        report("conv weights round trip", out.str() == section.str());
+        ConvLayer plain(ctx, Properties{ { "batch", N }, { "channels", BC }, { "height", BS }, { "width", BS },
+                                          { "filters", BC }, { "weights", weights } });
+        std::stringstream two(std::ios::in | std::ios::out | std::ios::binary);
+        for (const Host* t: { &biases, &w })
+            two.write(reinterpret_cast<const char*>(t->data()), std::streamsize(t->size() * sizeof(float)));
+        report("conv without batch norm: biases, then weights",
+               plain.loadWeights(two) == std::streamoff((BC + weights) * sizeof(float)) &&
+               plain.biases().asVector() == biases && plain.weights().asVector() == w);
+        std::stringstream shortFile(std::string(10, 'x'), std::ios::in | std::ios::binary);
+        expectThrows("a truncated weight section is refused", [&] { plain.loadWeights(shortFile); },
+                     "Could not read weights");
+    }
     Context ctx;
     ctx.training = true;
     ctx.updateBatch = N;
