@@ -294,12 +294,15 @@ struct SgdUpdateOp {
 constexpr int kNormBlocks = 2048;     // 8 per compute unit: full occupancy
 constexpr int kNormLoads = 4;      // 128-bit loads in flight per lane
 
+// Per workgroup: the sum of squares and the largest magnitude (NaN-free; a NaN shows in the sum).
 template<int V, bool NT>
-__global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, size_t n_vec, double* partial)
+__global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, size_t n_vec, double2* partial)
 {
     __shared__ double slots[kBlock / kWave];
+    __shared__ float peaks[kBlock / kWave];
     const size_t per_step = static_cast<size_t>(kBlock) * V * kNormLoads;
     double s = 0.0;
+    float peak = 0.0f;
     for (size_t base = static_cast<size_t>(blockIdx.x) * per_step; base < n_vec;
          base += static_cast<size_t>(gridDim.x) * per_step) {
         Pack<V> v[kNormLoads];
@@ -314,40 +317,67 @@ __global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, s
             const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
             if (e < n_vec) {
 #pragma unroll
-                for (int k = 0; k < V; ++k) a += v[u].v[k] * v[u].v[k];
+                for (int k = 0; k < V; ++k) {
+                    a += v[u].v[k] * v[u].v[k];
+                    peak = fmaxf(peak, fabsf(v[u].v[k]));
+                }
             }
         }
         s += static_cast<double>(a);
     }
-    const double total = block_sum(s, slots);
-    if (threadIdx.x == 0) partial[blockIdx.x] = total;
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) peak = fmaxf(peak, __shfl_xor(peak, off, kWave));
+    if ((threadIdx.x & (kWave - 1)) == 0) peaks[threadIdx.x / kWave] = peak;
+    const double total = block_sum(s, slots);       // synchronises the workgroup twice
+    if (threadIdx.x == 0) {
+        float top = peaks[0];
+#pragma unroll
+        for (int w = 1; w < kBlock / kWave; ++w) top = fmaxf(top, peaks[w]);
+        partial[blockIdx.x] = make_double2(total, static_cast<double>(top));
+    }
 }
 
-// One workgroup: the norm from the partial sums, and the factor the rewrite applies.
-__global__ __launch_bounds__(kBlock) void rescale_factor_kernel(const double* partial, int partials, float threshold,
-                                                                float* factor_out, float* norm_out)
+// One workgroup: the norm from the partial sums, the factor the rewrite applies, and whether the
+// rewrite has anything to do: a factor other than 1, or a value that the clamp would move.  The
+// scaled magnitudes are at most fl(factor * peak) (rounding is monotonic), so a peak within the
+// clamp after scaling means no element changes; a NaN anywhere (it shows in the sum) or an
+// infinite peak keeps the rewrite, which treats them as the CPU loop does.
+__global__ __launch_bounds__(kBlock) void rescale_factor_kernel(const double2* partial, int partials, float threshold,
+                                                                float clip, float* factor_out, float* norm_out)
 {
     __shared__ double slots[kBlock / kWave];
-    double s = 0.0;
-    for (int j = threadIdx.x; j < partials; j += kBlock) s += partial[j];
+    __shared__ double tops[kBlock / kWave];
+    double s = 0.0, top = 0.0;
+    for (int j = threadIdx.x; j < partials; j += kBlock) {
+        const double2 p = partial[j];
+        s += p.x;
+        top = fmax(top, p.y);
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) top = fmax(top, __shfl_xor(top, off, kWave));
+    if ((threadIdx.x & (kWave - 1)) == 0) tops[threadIdx.x / kWave] = top;
     const double total = block_sum(s, slots);
     if (threadIdx.x == 0) {
+        float peak = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kBlock / kWave; ++w) peak = fmaxf(peak, static_cast<float>(tops[w]));
         const float norm = static_cast<float>(sqrt(total));
         if (norm_out) *norm_out = norm;
         float factor = 1.0f;
         if (threshold > 0.0f && norm > 0.0f && norm > threshold) factor = threshold / norm;
-        *factor_out = factor;
+        factor_out[0] = factor;
+        const bool clamps = clip > 0.0f && (!(factor * peak <= clip) || total != total);
+        factor_out[1] = (factor != 1.0f || clamps) ? 1.0f : 0.0f;
     }
 }
 
-// x = clamp(factor * x); leaves without touching the tensor when there is nothing to do.
-// factor_in == nullptr: no rescaling was asked for.
+// x = clamp(factor * x); leaves without touching the tensor when there is nothing to do
+// (plan[0] = factor, plan[1] = 0 when no element would change).
 template<int V, bool NT>
-__global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n_vec, const float* factor_in,
-                                                              float clip)
+__global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n_vec, const float* plan, float clip)
 {
-    const float factor = factor_in ? *factor_in : 1.0f;
-    if (factor == 1.0f && !(clip > 0.0f)) return;
+    const float factor = plan[0];
+    if (plan[1] == 0.0f) return;
     // kNormLoads vectors per lane: a quarter of the workgroups to dispatch when there is nothing to do
     const size_t base = static_cast<size_t>(blockIdx.x) * kBlock * V * kNormLoads;
     Pack<V> v[kNormLoads];
@@ -616,7 +646,7 @@ int pxh_sgd_update(size_t n, float* w, float* d, int batch, float lr, float mome
 
 size_t pxh_rescale_workspace_bytes(void)
 {
-    return kNormBlocks * sizeof(double) + 256;      // partial sums, then the factor
+    return kNormBlocks * sizeof(double2) + 256;      // partial sums and peaks, then factor and flag
 }
 
 int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* norm_out, void* workspace,
@@ -629,33 +659,31 @@ int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* nor
     void* ws = nullptr;
     int rc = resolve_workspace(workspace, workspace_bytes, pxh_rescale_workspace_bytes(), &ws);
     if (rc) return rc;
-    double* partial = static_cast<double*>(ws);
-    float* factor = reinterpret_cast<float*>(partial + kNormBlocks);
+    double2* partial = static_cast<double2*>(ws);
+    float* plan = reinterpret_cast<float*>(partial + kNormBlocks);
     hipStream_t s = as_stream(stream);
     const bool vec = aligned16(x) && n % 4 == 0;
     const int v = vec ? 4 : 1;
     // a tensor past the last-level cache gains nothing from being kept for the next pass
     const bool nt = vec && n * 4 >= kStreamingBytes;
-    if (rescale) {
-        const size_t per_step = static_cast<size_t>(kBlock) * v * kNormLoads;
-        const size_t want = (n + per_step - 1) / per_step;
-        const int blocks = static_cast<int>(want < static_cast<size_t>(kNormBlocks) ? want : kNormBlocks);
-        if (nt) hipLaunchKernelGGL((sumsq_partial_kernel<4, true>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
-        else if (vec) hipLaunchKernelGGL((sumsq_partial_kernel<4, false>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
-        else hipLaunchKernelGGL((sumsq_partial_kernel<1, false>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
-        rc = check_launch("pxh_rescale_clip");
-        if (rc) return rc;
-        hipLaunchKernelGGL(rescale_factor_kernel, dim3(1), dim3(kBlock), 0, s, partial, blocks, threshold, factor,
-                           norm_out);
-        rc = check_launch("pxh_rescale_clip");
-        if (rc) return rc;
-        if (!(threshold > 0.0f) && !(clip > 0.0f)) return PXH_OK;      // only the norm was asked for
-    }
-    const float* factor_in = threshold > 0.0f ? factor : nullptr;
+    // the reduction also finds the largest magnitude, which tells whether the clamp can move anything
+    const size_t per_step = static_cast<size_t>(kBlock) * v * kNormLoads;
+    const size_t want = (n + per_step - 1) / per_step;
+    const int blocks = static_cast<int>(want < static_cast<size_t>(kNormBlocks) ? want : kNormBlocks);
+    if (nt) hipLaunchKernelGGL((sumsq_partial_kernel<4, true>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
+    else if (vec) hipLaunchKernelGGL((sumsq_partial_kernel<4, false>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
+    else hipLaunchKernelGGL((sumsq_partial_kernel<1, false>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
+    rc = check_launch("pxh_rescale_clip");
+    if (rc) return rc;
+    hipLaunchKernelGGL(rescale_factor_kernel, dim3(1), dim3(kBlock), 0, s, partial, blocks, threshold, clip, plan,
+                       norm_out);
+    rc = check_launch("pxh_rescale_clip");
+    if (rc) return rc;
+    if (!(threshold > 0.0f) && !(clip > 0.0f)) return PXH_OK;      // only the norm was asked for
     const dim3 grid(grid_for(n, static_cast<size_t>(kBlock) * v * kNormLoads));
-    if (nt) hipLaunchKernelGGL((rescale_clip_kernel<4, true>), grid, dim3(kBlock), 0, s, x, n, factor_in, clip);
-    else if (vec) hipLaunchKernelGGL((rescale_clip_kernel<4, false>), grid, dim3(kBlock), 0, s, x, n, factor_in, clip);
-    else hipLaunchKernelGGL((rescale_clip_kernel<1, false>), grid, dim3(kBlock), 0, s, x, n, factor_in, clip);
+    if (nt) hipLaunchKernelGGL((rescale_clip_kernel<4, true>), grid, dim3(kBlock), 0, s, x, n, plan, clip);
+    else if (vec) hipLaunchKernelGGL((rescale_clip_kernel<4, false>), grid, dim3(kBlock), 0, s, x, n, plan, clip);
+    else hipLaunchKernelGGL((rescale_clip_kernel<1, false>), grid, dim3(kBlock), 0, s, x, n, plan, clip);
     return check_launch("pxh_rescale_clip");
 }
 

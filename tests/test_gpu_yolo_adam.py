@@ -330,6 +330,37 @@ def test_rescale_clip_matches_oracle(ops, oracle, n, mode):
     assert_bit_exact(host(gy), host(gx), "with and without norm_out")
 
 
+def test_rescale_clip_edges_of_the_no_work_shortcut(ops, oracle):
+    """The rewrite is skipped when the largest magnitude stays inside the clamp: exactly at the clamp
+    is inside, one value beyond it (anywhere in the tensor) is not, and a NaN or an infinity keeps
+    the rewrite, which maps them as the CPU loop's min/max do."""
+    n = 70001
+    base = np.clip(wl.normal(3450, n), -0.9, 0.9).astype(F)
+    for where in (0, 12345, n - 1):
+        for value in (1.0, -1.0):                     # at the clamp: unchanged
+            x0 = base.copy(); x0[where] = value
+            gx = gpu(x0)
+            ops.rescale_clip(gx, 0.0, 1.0)
+            assert_bit_exact(host(gx), x0, "peak at the clamp")
+        for value in (np.nextafter(F(1.0), F(2.0)), F(-3.5), F(np.inf), F(-np.inf), F(np.nan)):
+            x0 = base.copy(); x0[where] = value
+            want = x0.copy()
+            oracle.rescale_clip(want, 0.0, 1.0)
+            gx = gpu(x0)
+            ops.rescale_clip(gx, 0.0, 1.0)
+            assert_bit_exact(host(gx), want, "one value %r beyond the clamp at %d" % (value, where))
+            assert np.isfinite(host(gx)).all() and np.abs(host(gx)).max() <= 1.0
+    # rescaling pulls the peak inside the clamp: scaled, not clamped
+    x0 = (4.0 * base).astype(F)
+    norm = float(np.sqrt(np.square(x0.astype(np.float64)).sum()))
+    want = x0.copy()
+    oracle.rescale_clip(want, 0.2 * norm, 1.0)
+    gx = gpu(x0)
+    ops.rescale_clip(gx, 0.2 * norm, 1.0)
+    assert_close(host(gx), want, 1e-6, 1e-6, "rescaled below the clamp")
+    assert np.abs(want).max() < 1.0
+
+
 # ---------------------------------------------------------------- detections (device-side compaction)
 @pytest.mark.parametrize("case", [(2, 3, 80, 19, 0.5), (4, 3, 80, 38, 0.4), (1, 2, 5, 7, 0.1), (3, 3, 20, 13, 0.9)])
 @pytest.mark.parametrize("image", [(0, 0), (640, 480), (333, 500)])
