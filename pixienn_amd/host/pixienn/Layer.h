@@ -167,15 +167,12 @@ public:
     // into *grad (nullptr for the first layer).
     // First the reference's two helpers on delta_ (include/Layer.h:385-397): rescale to a norm
     // threshold, then clamp; one fused call here.
-    virtual void backward(const V& /*input*/, V* /*grad*/)
-    {
-        if (gradientRescaling_ || gradientClipping_)
-            PX_HIP_CHECK(pxh_rescale_clip(delta_.data(), delta_.size(), gradientRescaling_ ? gradientThreshold_ : 0.0f,
-                                          gradientClipping_ ? gradientClipValue_ : 0.0f, nullptr, nullptr, 0,
-                                          stream()));
-    }
+    virtual void backward(const V& /*input*/, V* /*grad*/) { rescaleAndClip(delta_); }
 
-    virtual void update() {}
+    // The reference's update() runs the same two helpers once more, through the hooks that layers
+    // with parameters extend to their update buffers (include/Layer.h:400-411, 473-493).  Derived
+    // classes call this first, then rescaleAndClip() on each of their update tensors.
+    virtual void update() { rescaleAndClip(delta_); }
 
     // This layer's section of a weight file; bytes read / written (reference: Layer<D>::loadWeights /
     // saveWeights, include/Layer.h:57-58).  Layers without parameters have none.
@@ -220,6 +217,15 @@ protected:
         PX_CHECK(n < (std::size_t(1) << 31), "tensors of 2^31 elements or more are not supported");
         output_ = V(n);
         if (context_.training) delta_ = V(n);
+    }
+
+    // scaleTensor then constrain on one tensor, when the layer's flags ask for them; one fused call
+    // that reads the tensor once and rewrites it only if some value has to change.
+    void rescaleAndClip(V& tensor)
+    {
+        if (tensor.empty() || !(gradientRescaling_ || gradientClipping_)) return;
+        PX_HIP_CHECK(pxh_rescale_clip(tensor.data(), tensor.size(), gradientRescaling_ ? gradientThreshold_ : 0.0f,
+                                      gradientClipping_ ? gradientClipValue_ : 0.0f, nullptr, nullptr, 0, stream()));
     }
 
     void checkInput(const V& input, const char* who) const

@@ -155,6 +155,11 @@ public:
     void update() override
     {
         const auto& c = context();
+        // the reference's scaleGradients / clipGradients hooks (include/ConvLayer.h:323-340)
+        Layer::update();
+        rescaleAndClip(weightUpdates_);
+        rescaleAndClip(biasUpdates_);
+        rescaleAndClip(scaleUpdates_);
         if (c.adamEnabled) {
             const Adam adam(c);
             if (!weights_.empty()) adam.update(weights_, weightUpdates_, weightM_, weightV_, true);
@@ -329,6 +334,10 @@ public:
     void update() override
     {
         const auto& c = context();
+        // scaleGradients / clipGradients (include/BatchNormLayer.h:160-176)
+        Layer::update();
+        rescaleAndClip(biasUpdates_);
+        rescaleAndClip(scaleUpdates_);
         PX_HIP_CHECK(pxh_sgd_update(biases_.size(), biases_.data(), biasUpdates_.data(), c.updateBatch, c.learningRate,
                                     c.momentum, 0.0f, 0, stream()));
         PX_HIP_CHECK(pxh_sgd_update(scales_.size(), scales_.data(), scaleUpdates_.data(), c.updateBatch,

@@ -672,6 +672,29 @@ void batchNormLayerChecks()
     expectClose("batchnorm layer, biases after update", layer.biases().asVector(), wb, 1e-5, 1.0);
     expectClose("batchnorm layer, scales after update", layer.scales().asVector(), ws, 1e-5, 1.0);
     expectClose("batchnorm layer, momentum kept in the updates", dbu, bu, 1e-5, 30.0);
+
+    // the same step with the gradient helpers switched on: update() rescales and clamps the update
+    // buffers before it applies them (include/BatchNormLayer.h:160-176)
+    BatchNormLayer guarded(ctx, props);
+    file.clear();
+    file.seekg(0);
+    guarded.loadWeights(file);
+    guarded.forward(input);
+    guarded.delta().copyHost(normals(406, total));
+    guarded.backward(input, nullptr);
+    Host gsu = guarded.scaleUpdates().asVector(), gbu = guarded.biasUpdates().asVector();
+    const float thr = 0.5f * pxo_rescale_clip(gsu.data(), gsu.size(), 0.0f, 0.0f);
+    guarded.setGradientRescaling(true, thr);
+    guarded.setGradientClipping(true, 0.4f * thr);
+    guarded.update();
+    pxo_rescale_clip(gsu.data(), gsu.size(), thr, 0.4f * thr);
+    pxo_rescale_clip(gbu.data(), gbu.size(), thr, 0.4f * thr);
+    Host gb = biases, gs = scales;
+    pxo_sgd_update(BC, gb.data(), gbu.data(), N, 0.01f, 0.9f, 0.0f, 0);
+    pxo_sgd_update(BC, gs.data(), gsu.data(), N, 0.01f, 0.9f, 0.0f, 0);
+    expectClose("guarded update: scales", guarded.scales().asVector(), gs, 1e-5, 1.0);
+    expectClose("guarded update: biases", guarded.biases().asVector(), gb, 1e-5, 1.0);
+    expectClose("guarded update: clamped scale updates", guarded.scaleUpdates().asVector(), gsu, 1e-5, 1.0);
 }
 
 // An upsample layer absorbed by the route that reads it gives the same tensors as the two-step form.
