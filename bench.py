@@ -68,9 +68,13 @@ class Timer:
         self.trials = 5
         self.last_min = 0.0
 
-    def time(self, fn, reps, warm=2, rotate=1):
-        """fn(i) launches one repetition using buffer set i % rotate.  Returns ms per repetition."""
+    def time(self, fn, reps, warm=2, rotate=1, prepare=None):
+        """fn(i) launches one repetition using buffer set i % rotate.  Returns ms per repetition.
+        prepare() runs untimed before every trial (for a kernel that changes what it will do next
+        time on the same data)."""
         t = self.torch
+        if prepare:
+            prepare()
         for i in range(max(warm, rotate)):
             fn(i % rotate)
         t.cuda.synchronize()
@@ -91,6 +95,9 @@ class Timer:
         # several trials of the whole repetition sequence: the median is reported, the minimum kept
         samples = []
         for _ in range(self.trials):
+            if prepare:
+                prepare()
+                t.cuda.synchronize()
             start = t.cuda.Event(enable_timing=True)
             stop = t.cuda.Event(enable_timing=True)
             start.record()
@@ -152,6 +159,118 @@ def run_epilogue_step(ops, shapes, events=None, torch=None, raw=False):
         if events is not None:
             b.record()
             events.append((act, a, b))
+
+
+def measure_model_order(torch, ops, wl, timer, N=16):
+    """One training step of YOLOv3 @608 at batch N with every non-convolution kernel launched in the
+    model's own layer order on tensors of their own (21 GB): forward (per layer the delta zero-fill
+    of Layer::forward, then the layer), backward in reverse (per layer the gradient rescale + clip
+    of Layer::backward with the thresholds of yolov3.yml, 100 and 10, then the layer), update (the
+    same helpers once more per layer and on the update buffer, then Adam on the flat parameters).
+    The convolutions' GEMMs are not run: a conv layer reads a resident conv result and its input
+    gradient goes nowhere.  Each phase is timed as one HIP graph."""
+    dev = torch.device("cuda")
+    layers = wl.yolov3_layers(608)
+    T = []
+    for l in layers:
+        shape = (N, l["c"], l["s"], l["s"])
+        t = dict(y=torch.empty(shape, device=dev), d=torch.zeros(shape, device=dev))
+        if l["type"] == "conv":
+            t["x"] = torch.randn(shape, device=dev)
+            c = l["c"]
+            t["bias"] = torch.zeros(c, device=dev); t["bu"] = torch.zeros(c, device=dev)
+            if l["bn"]:
+                scale, bias, rmean, rvar = (torch.from_numpy(a).to(dev) for a in wl.bn_params(2000 + len(T), c))
+                t.update(scale=scale, bias=bias, rmean=rmean, rvar=rvar, mean=torch.zeros(c, device=dev),
+                         var=torch.zeros(c, device=dev), su=torch.zeros(c, device=dev))
+        elif l["type"] == "yolo":
+            t["stats"] = torch.zeros(12, device=dev); t["cost"] = torch.zeros(1, device=dev)
+        T.append(t)
+    truths_np, counts_np = wl.yolo_truths(5100, N)
+    truths = torch.from_numpy(truths_np).to(dev); counts = torch.from_numpy(counts_np).to(dev)
+    P = wl.YOLOV3_PARAMS
+    w = 0.02 * torch.randn(P, device=dev); g = 1e-3 * torch.randn(P, device=dev)
+    m = torch.zeros(P, device=dev); v = torch.zeros(P, device=dev)
+    launches = dict(forward=0, backward=0, update=0)
+
+    def absorbed(i):            # an upsample writes into (and reads its delta from) the route that follows
+        return layers[i]["type"] == "upsample"
+
+    def forward(_):
+        n = 0
+        for i, (l, t) in enumerate(zip(layers, T)):
+            if not absorbed(i):
+                ops.fill(t["d"], 0.0); n += 1
+            kind = l["type"]
+            if kind == "conv" and l["bn"]:
+                ops.bn_train_act_forward(t["x"], t["y"], t["mean"], t["var"], t["rmean"], t["rvar"], t["scale"],
+                                         t["bias"], "leaky")
+            elif kind == "conv":
+                ops.bias_act_forward(t["x"], t["y"], t["bias"], "linear")
+            elif kind == "shortcut":
+                ops.shortcut_forward(T[i - 1]["y"], T[l["frm"]]["y"], t["y"], "linear")
+            elif kind == "upsample":
+                ops.upsample_forward_into(T[i - 1]["y"], T[i + 1]["y"], 0, 2, 1.0)
+            elif kind == "route" and len(l["sources"]) == 1:
+                ops.route_forward(T[l["sources"][0]]["y"], t["y"], 0)
+            elif kind == "route":
+                up, other = l["sources"]
+                ops.route_forward(T[other]["y"], t["y"], layers[up]["c"] * l["s"] * l["s"])
+            elif kind == "yolo":
+                ops.yolo_forward_train(T[i - 1]["y"], t["y"], t["d"], truths, counts, truths.shape[1], l["mask"],
+                                       wl.YOLOV3_ANCHORS, t["stats"], t["cost"], N, 80, l["s"], l["s"], 608, 608,
+                                       0.7, 1.0, 1.0, 1.0, 1.0, 1.0)
+            n += 1
+        launches["forward"] = n
+
+    def backward(_):
+        n = 0
+        for i in reversed(range(len(layers))):
+            l, t = layers[i], T[i]
+            kind = l["type"]
+            if not absorbed(i):
+                ops.rescale_clip(t["d"], 100.0, 10.0); n += 1
+            if kind == "yolo":
+                ops.axpy(1.0, t["d"], T[i - 1]["d"])
+            elif kind == "conv" and l["bn"]:
+                ops.bn_act_backward(t["d"], t["x"], t["mean"], t["var"], t["scale"], t["bias"], t["su"], t["bu"],
+                                    "leaky")
+            elif kind == "conv":
+                ops.bias_act_backward(t["d"], None, t["bu"], "linear")
+            elif kind == "shortcut":
+                ops.shortcut_backward(t["d"], T[l["frm"]]["d"], T[i - 1]["d"], "linear")
+            elif kind == "upsample":
+                ops.upsample_backward_from(T[i + 1]["d"], 0, T[i - 1]["d"], 2, 1.0)
+            elif kind == "route" and len(l["sources"]) == 1:
+                ops.route_backward(t["d"], T[l["sources"][0]]["d"], 0)
+            elif kind == "route":
+                up, other = l["sources"]
+                ops.route_backward(t["d"], T[other]["d"], layers[up]["c"] * l["s"] * l["s"])
+            n += 1
+        launches["backward"] = n
+
+    def update(_, touch_delta=True):
+        n = 0
+        if touch_delta:         # the reference's update() passes every delta through the helpers once more
+            for i, t in enumerate(T):
+                if not absorbed(i):
+                    ops.rescale_clip(t["d"], 100.0, 10.0); n += 1
+        ops.rescale_clip(g, 100.0, 10.0)
+        ops.adam_update(w, g, m, v, N, 1, 1e-3, decay=5e-4, apply_decay=True)
+        launches["update"] = n + 2
+
+    out = {}
+    for name, fn in (("forward", forward), ("backward", backward), ("update", update)):
+        out[name + "_ms"] = round(timer.time(fn, 3, warm=1), 3)
+    out["total_ms"] = round(out["forward_ms"] + out["backward_ms"] + out["update_ms"], 3)
+    # nothing reads a delta after backward: the pass over them in update() is dead work that a host
+    # may drop (Context::helpersTouchDeltaInUpdate of the C++ layer interface)
+    out["calls"] = dict(launches)
+    out["update_without_delta_pass_ms"] = round(timer.time(lambda i: update(i, False), 3, warm=1), 3)
+    out["elements_per_tensor_kind"] = int(sum(N * l["c"] * l["s"] * l["s"] for l in layers))
+    del T, w, g, m, v
+    torch.cuda.empty_cache()
+    return out
 
 
 def measure_extras(torch, ops, wl, timer, capi):
@@ -358,8 +477,13 @@ def measure_extras(torch, ops, wl, timer, capi):
         e = N * c * s_ * s_
         rot = rotation_for(12 * e)
         xs = [randn(N, c, s_, s_) for _ in range(rot)]
-        # a threshold far below the norm: every call rescales and clamps
-        ms = timer.time(lambda i: ops.rescale_clip(xs[i], 1e-3, 1e-6), 10, rotate=rot)
+        # fresh values before every trial and one call per buffer: a second call on the same data
+        # would find nothing left to change and skip the rewrite
+        def refill():
+            for x in xs:
+                x.normal_()
+
+        ms = timer.time(lambda i: ops.rescale_clip(xs[i], 1e-3, 1e-6), rot, warm=0, rotate=rot, prepare=refill)
         add("rescale_clip", "%dx%dx%d^2" % (N, c, s_), 12 * e, ms, "norm 4B + rewrite 8B per elem")
         ms = timer.time(lambda i: ops.rescale_clip(xs[i], 1e30, 0.0), 10, rotate=rot)
         add("rescale_clip(no-op)", "%dx%dx%d^2" % (N, c, s_), 4 * e, ms, "below the threshold: norm only, 4B/elem")
@@ -502,13 +626,15 @@ def main():
     copy_row = calibration_copy(torch, ops, timer)
     log("plain copy of 2 x 512 MiB: %.4f ms %.1f GB/s" % (copy_row["ms"], copy_row["GBps"]))
 
-    extras, ms_batch = (None, None)
+    extras, ms_batch, model_order = (None, None, None)
     if not args.no_extras:
         extras, ms_batch = measure_extras(torch, ops, wl, timer, capi)
         for r in extras:
             log("%-24s %-18s %9.1f MB %8.4f ms %8.1f GB/s  %4.1f%%  %s"
                 % (r["kernel"], r["shape"], r["MB"], r["ms"], r["GBps"], 100 * r["frac"], r["note"]))
         log("non-conv ms/batch, YOLOv3 @608, batch 16, training step: %.3f" % ms_batch)
+        model_order = measure_model_order(torch, ops, wl, timer)
+        log("the same step in model order, with the Layer base's fills and gradient helpers:", model_order)
 
     cpu = None
     if not args.no_cpu:
@@ -536,6 +662,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "noconv_ms_per_batch_yolov3_608": None if ms_batch is None else round(ms_batch, 3),
+        "noconv_step_in_model_order_yolov3_608": model_order,
         "value_folding_every_call": round(value_raw, 1),
         "plain_copy": copy_row,
         "per_activation": per_act,

@@ -102,6 +102,11 @@ public:
     int timeStep = 1;               // Adam's t
     int updateBatch = 1;            // images a parameter update averages over (batch * subdivisions)
 
+    // The reference's update() rescales and clamps every layer's delta once more.  By then backward
+    // has consumed it and the next forward clears it, so nothing reads the result; switching this
+    // off drops one pass over every activation-sized tensor per step and changes no trained value.
+    bool helpersTouchDeltaInUpdate = true;
+
     // Uploads the ground truth of the current batch: [batch][maxTruth][5] floats + counts.
     void setGroundTruth(const std::vector<GroundTruthVec>& batchTruth)
     {
@@ -172,7 +177,10 @@ public:
     // The reference's update() runs the same two helpers once more, through the hooks that layers
     // with parameters extend to their update buffers (include/Layer.h:400-411, 473-493).  Derived
     // classes call this first, then rescaleAndClip() on each of their update tensors.
-    virtual void update() { rescaleAndClip(delta_); }
+    virtual void update()
+    {
+        if (context_.helpersTouchDeltaInUpdate) rescaleAndClip(delta_);
+    }
 
     // This layer's section of a weight file; bytes read / written (reference: Layer<D>::loadWeights /
     // saveWeights, include/Layer.h:57-58).  Layers without parameters have none.

@@ -122,3 +122,45 @@ def detection_clusters(seed, n, batch, classes, clusters, spread=6.0):
     rec["prob"] = np.round(g.uniform(0.05, 1.0, n), 2).astype(np.float32)
     rec["order"] = np.arange(n)
     return rec
+
+
+def yolov3_layers(size=608):
+    """The 107 layers of the reference's resources/models/yolov3.yml as dictionaries with the output
+    shape filled in: conv (filters, stride, bn), shortcut (from), route (layers), upsample, yolo (mask).
+    Keys: type, c, s (output channels and height == width), plus the type's own."""
+    layers = []
+
+    def conv(filters, stride=1, bn=True):
+        prev = layers[-1] if layers else dict(c=3, s=size)
+        layers.append(dict(type="conv", c=filters, s=prev["s"] // stride, bn=bn))
+
+    def shortcut():
+        layers.append(dict(type="shortcut", c=layers[-1]["c"], s=layers[-1]["s"], frm=len(layers) - 3))
+
+    def residual(narrow, wide, times):
+        for _ in range(times):
+            conv(narrow)
+            conv(wide)
+            shortcut()
+
+    conv(32)
+    conv(64, 2); residual(32, 64, 1)
+    conv(128, 2); residual(64, 128, 2)
+    conv(256, 2); residual(128, 256, 8)
+    conv(512, 2); residual(256, 512, 8)
+    conv(1024, 2); residual(512, 1024, 4)
+    for head, (narrow, wide, mask, joins) in enumerate([(512, 1024, [6, 7, 8], None), (256, 512, [3, 4, 5], 61),
+                                                        (128, 256, [0, 1, 2], 36)]):
+        if joins is not None:
+            src = len(layers) - 4
+            layers.append(dict(type="route", c=layers[src]["c"], s=layers[src]["s"], sources=[src]))
+            conv(narrow)
+            layers.append(dict(type="upsample", c=narrow, s=2 * layers[-1]["s"]))
+            up = len(layers) - 1
+            layers.append(dict(type="route", c=narrow + layers[joins]["c"], s=layers[up]["s"], sources=[up, joins]))
+        for _ in range(3):
+            conv(narrow)
+            conv(wide)
+        conv(255, bn=False)
+        layers.append(dict(type="yolo", c=255, s=layers[-1]["s"], mask=mask))
+    return layers

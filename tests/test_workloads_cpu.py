@@ -1,0 +1,37 @@
+"""The synthetic workloads: the YOLOv3 layer list that the benchmark walks must have the inventory of
+the reference's resources/models/yolov3.yml (107 layers: 72 batch-normalised convs with the shape
+counts of the BN table, 3 linear head convs, 23 shortcuts, 2 upsamples, 4 routes, 3 heads)."""
+from collections import Counter
+
+from pixienn_amd import workloads as wl
+
+
+def test_yolov3_layer_inventory():
+    layers = wl.yolov3_layers(608)
+    kinds = Counter(l["type"] for l in layers)
+    assert len(layers) == 107
+    assert kinds == {"conv": 75, "shortcut": 23, "route": 4, "upsample": 2, "yolo": 3}
+    bn = Counter((l["c"], l["s"]) for l in layers if l["type"] == "conv" and l["bn"])
+    assert bn == dict(zip(wl.YOLOV3_BN_SHAPES, wl.YOLOV3_BN_COUNTS))
+    assert sorted((l["c"], l["s"]) for l in layers if l["type"] == "conv" and not l["bn"]) == \
+        sorted(wl.YOLOV3_HEAD_CONV_SHAPES)
+    shortcuts = Counter((l["c"], l["s"]) for l in layers if l["type"] == "shortcut")
+    assert shortcuts == {(c, s): n for c, s, n in wl.YOLOV3_SHORTCUT_SHAPES}
+    for i, l in enumerate(layers):
+        if l["type"] == "shortcut":
+            assert l["frm"] == i - 3 and (layers[l["frm"]]["c"], layers[l["frm"]]["s"]) == (l["c"], l["s"])
+        if l["type"] == "route":
+            assert l["c"] == sum(layers[j]["c"] for j in l["sources"])
+            assert all(layers[j]["s"] == l["s"] for j in l["sources"])
+        if l["type"] == "yolo":
+            assert l["mask"] == wl.YOLOV3_MASKS[l["s"]]
+    # the two concatenations read layers 61 and 36, as the model file says
+    assert [l["sources"] for l in layers if l["type"] == "route"] == [[79], [85, 61], [91], [97, 36]]
+
+
+def test_detection_clusters_are_reproducible():
+    a = wl.detection_clusters(3, 500, 4, 7, 3)
+    b = wl.detection_clusters(3, 500, 4, 7, 3)
+    assert a.tobytes() == b.tobytes() and a.dtype == wl.DETECTION_DTYPE
+    assert a["batch"].max() < 4 and a["class_index"].max() < 7 and (a["w"] >= 1).all()
+    assert len(set(a["prob"])) < 120          # two decimals: ties
