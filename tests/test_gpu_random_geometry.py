@@ -108,3 +108,43 @@ def test_streaming_kernels_with_unaligned_views(ops, oracle):
         src = gpu(np.stack([a[off:], b[off:]]))
         ops.route_forward(src, route, n + 1)           # an odd offset inside the concatenation
         assert torch.equal(route[:, n + 1:2 * n + 1], src) and float(route[:, :n + 1].max()) == -1.0
+
+
+def test_yolo_training_pass_random_heads(ops, oracle):
+    """Rectangular heads, 1 to 200 classes, any subset of the anchors as mask, truth tables with
+    empty rows, truths outside the image, empty or inverted boxes and labels outside the class
+    range: delta support, cost and statistics must follow the CPU layer."""
+    from test_gpu_yolo_adam import compare_head, gpu_head, oracle_head
+    r = np.random.default_rng(107)
+    for case in range(40):
+        W = int(r.integers(1, 30)); H = int(r.integers(1, 30)); K = int(r.choice([1, 2, 3, 7, 20, 64, 80, 129, 200]))
+        total_anchors = int(r.integers(1, 10)); masks = int(r.integers(1, min(total_anchors, 5) + 1))
+        mask = sorted(r.choice(total_anchors, masks, replace=False).tolist())
+        anchors = [int(v) for v in r.integers(2, 300, 2 * total_anchors)]
+        N = int(r.integers(1, 5)); net = int(r.choice([32, 96, 416, 608]))
+        max_truth = int(r.choice([1, 3, 20, 90]))
+        x = wl.normal(7000 + case, (N, masks * (K + 5), H, W), std=float(r.choice([0.5, 2.0, 4.0])))
+        truths = np.zeros((N, max_truth, 5), F)
+        truths[..., 0:2] = r.uniform(-0.1, 1.1, (N, max_truth, 2))
+        truths[..., 2:4] = np.exp(r.uniform(np.log(0.01), np.log(1.2), (N, max_truth, 2)))
+        truths[..., 4] = r.integers(0, K, (N, max_truth))
+        for _ in range(int(r.integers(0, 4))):
+            b = int(r.integers(0, N)); t = int(r.integers(0, max_truth))
+            kind = int(r.integers(0, 4))
+            if kind == 0:
+                truths[b, t, 2] = 0.0
+            elif kind == 1:
+                truths[b, t, 3] = -0.2
+            elif kind == 2:
+                truths[b, t, 0:2] = [1.0, 0.0]
+            else:
+                truths[b, t, 4] = K + 3
+        counts = r.integers(0, max_truth + 1, N).astype(np.int32)
+        kw = dict(ignore_thresh=float(r.choice([0.3, 0.5, 0.7])), truth_thresh=float(r.choice([1.0, 1.0, 0.4])),
+                  coord_scale=float(r.choice([1.0, 1.5])), object_scale=float(r.choice([1.0, 2.0])),
+                  noobject_scale=float(r.choice([1.0, 0.1])), class_scale=float(r.choice([1.0, 0.7])))
+        what = "case %d: N%d %dx%d K%d mask %s of %d net %d counts %s" % (case, N, W, H, K, mask, total_anchors, net,
+                                                                           counts.tolist())
+        want = oracle_head(oracle, x, truths, counts, W, H, K, mask, anchors, net, **kw)
+        got = gpu_head(ops, x, truths, counts, W, H, K, mask, anchors, net, **kw)
+        compare_head(got, want, what, sum_rtol=5e-5)
