@@ -148,3 +148,37 @@ def test_yolo_training_pass_random_heads(ops, oracle):
         want = oracle_head(oracle, x, truths, counts, W, H, K, mask, anchors, net, **kw)
         got = gpu_head(ops, x, truths, counts, W, H, K, mask, anchors, net, **kw)
         compare_head(got, want, what, sum_rtol=5e-5)
+
+
+def test_yolo_detections_random_heads(ops, oracle):
+    """Detection extraction on rectangular heads and class counts on either side of the kernel's
+    32- and 128-class steps: the same records, in the same emission order, as the CPU layer."""
+    r = np.random.default_rng(108)
+    for case in range(24):
+        W = int(r.integers(1, 40)); H = int(r.integers(1, 40))
+        K = int(r.choice([1, 2, 31, 32, 33, 80, 127, 128, 129, 300]))
+        total_anchors = int(r.integers(1, 8)); masks = int(r.integers(1, min(total_anchors, 4) + 1))
+        mask = sorted(r.choice(total_anchors, masks, replace=False).tolist())
+        anchors = [int(v) for v in r.integers(2, 300, 2 * total_anchors)]
+        N = int(r.integers(1, 4)); net = (int(r.choice([96, 416, 608])), int(r.choice([96, 416, 608])))
+        thr = float(r.choice([0.05, 0.3, 0.6]))
+        image = [(0, 0), (640, 480), (333, 500), (100, 1000)][case % 4]
+        logits = wl.normal(8000 + case, (N, masks * (K + 5), H, W), std=2.0)
+        cfg, keep = oracle.yolo_cfg(N, W, H, K, mask, anchors, net[0], net[1])
+        decoded = np.zeros_like(logits)
+        oracle.yolo_decode(cfg, logits, decoded)
+        cap = 1 << 21
+        want, found_w = oracle.yolo_detections(cfg, decoded, thr, cap, image_width=image[0], image_height=image[1])
+        got, found_g = ops.yolo_detections(gpu(decoded), N, mask, anchors, K, W, H, net[0], net[1], thr, cap,
+                                           image_width=image[0], image_height=image[1])
+        what = "case %d: N%d %dx%d K%d mask %s net %s thr %g image %s" % (case, N, W, H, K, mask, net, thr, image)
+        assert found_g == found_w <= cap, what
+        for k in ("order", "batch", "class_index"):
+            assert np.array_equal(got[k], want[k]), (what, k)
+        assert_bit_exact(got["prob"], want["prob"], what + " probabilities")
+        for k in "xywh":
+            d = np.abs(got[k].astype(np.float64) - want[k])
+            # pixel boxes: a last-place difference in exp may move a truncation by one pixel; relative boxes:
+            # left/top are differences of the centre and half the size
+            bound = 1.0 if image[0] else 1e-5 * np.maximum(1.0, np.abs(want[k]) + np.abs(want["w"]) + np.abs(want["h"]))
+            assert np.all(d <= bound), (what, k, float(d.max()))
