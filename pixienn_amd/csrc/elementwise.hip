@@ -342,25 +342,38 @@ __global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, s
 // scaled magnitudes are at most fl(factor * peak) (rounding is monotonic), so a peak within the
 // clamp after scaling means no element changes; a NaN anywhere (it shows in the sum) or an
 // infinite peak keeps the rewrite, which treats them as the CPU loop does.
-__global__ __launch_bounds__(kBlock) void rescale_factor_kernel(const double2* partial, int partials, float threshold,
-                                                                float clip, float* factor_out, float* norm_out)
+constexpr int kFactorLanes = 1024;      // two partials per lane at most: one trip to memory
+
+__global__ __launch_bounds__(kFactorLanes) void rescale_factor_kernel(const double2* partial, int partials,
+                                                                      float threshold, float clip, float* factor_out,
+                                                                      float* norm_out)
 {
-    __shared__ double slots[kBlock / kWave];
-    __shared__ double tops[kBlock / kWave];
+    __shared__ double sums[kFactorLanes / kWave];
+    __shared__ double tops[kFactorLanes / kWave];
     double s = 0.0, top = 0.0;
-    for (int j = threadIdx.x; j < partials; j += kBlock) {
+    for (int j = threadIdx.x; j < partials; j += kFactorLanes) {
         const double2 p = partial[j];
         s += p.x;
         top = fmax(top, p.y);
     }
 #pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) top = fmax(top, __shfl_xor(top, off, kWave));
-    if ((threadIdx.x & (kWave - 1)) == 0) tops[threadIdx.x / kWave] = top;
-    const double total = block_sum(s, slots);
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        s += __shfl_xor(s, off, kWave);
+        top = fmax(top, __shfl_xor(top, off, kWave));
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        sums[threadIdx.x / kWave] = s;
+        tops[threadIdx.x / kWave] = top;
+    }
+    __syncthreads();
     if (threadIdx.x == 0) {
+        double total = 0.0;
         float peak = 0.0f;
 #pragma unroll
-        for (int w = 0; w < kBlock / kWave; ++w) peak = fmaxf(peak, static_cast<float>(tops[w]));
+        for (int w = 0; w < kFactorLanes / kWave; ++w) {
+            total += sums[w];
+            peak = fmaxf(peak, static_cast<float>(tops[w]));
+        }
         const float norm = static_cast<float>(sqrt(total));
         if (norm_out) *norm_out = norm;
         float factor = 1.0f;
@@ -378,25 +391,29 @@ __global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n
 {
     const float factor = plan[0];
     if (plan[1] == 0.0f) return;
-    // kNormLoads vectors per lane: a quarter of the workgroups to dispatch when there is nothing to do
-    const size_t base = static_cast<size_t>(blockIdx.x) * kBlock * V * kNormLoads;
-    Pack<V> v[kNormLoads];
+    // kNormLoads vectors per lane and step; the grid is capped (a launch that finds nothing to do
+    // should cost a few hundred workgroups, not one per 16 KB of tensor) and strides over the rest
+    const size_t per_step = static_cast<size_t>(kBlock) * V * kNormLoads;
+    for (size_t base = static_cast<size_t>(blockIdx.x) * per_step; base < n_vec;
+         base += static_cast<size_t>(gridDim.x) * per_step) {
+        Pack<V> v[kNormLoads];
 #pragma unroll
-    for (int u = 0; u < kNormLoads; ++u) {
-        const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
-        if (e < n_vec) v[u] = ld<V, NT>(x, e);
-    }
+        for (int u = 0; u < kNormLoads; ++u) {
+            const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
+            if (e < n_vec) v[u] = ld<V, NT>(x, e);
+        }
 #pragma unroll
-    for (int u = 0; u < kNormLoads; ++u) {
-        const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
-        if (e < n_vec) {
+        for (int u = 0; u < kNormLoads; ++u) {
+            const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
+            if (e < n_vec) {
 #pragma unroll
-            for (int k = 0; k < V; ++k) {
-                float t = factor == 1.0f ? v[u].v[k] : factor * v[u].v[k];
-                if (clip > 0.0f) t = fminf(clip, fmaxf(-clip, t));
-                v[u].v[k] = t;
+                for (int k = 0; k < V; ++k) {
+                    float t = factor == 1.0f ? v[u].v[k] : factor * v[u].v[k];
+                    if (clip > 0.0f) t = fminf(clip, fmaxf(-clip, t));
+                    v[u].v[k] = t;
+                }
+                st<V, NT>(x, e, v[u]);
             }
-            st<V, NT>(x, e, v[u]);
         }
     }
 }
@@ -675,12 +692,12 @@ int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* nor
     else hipLaunchKernelGGL((sumsq_partial_kernel<1, false>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
     rc = check_launch("pxh_rescale_clip");
     if (rc) return rc;
-    hipLaunchKernelGGL(rescale_factor_kernel, dim3(1), dim3(kBlock), 0, s, partial, blocks, threshold, clip, plan,
+    hipLaunchKernelGGL(rescale_factor_kernel, dim3(1), dim3(kFactorLanes), 0, s, partial, blocks, threshold, clip, plan,
                        norm_out);
     rc = check_launch("pxh_rescale_clip");
     if (rc) return rc;
     if (!(threshold > 0.0f) && !(clip > 0.0f)) return PXH_OK;      // only the norm was asked for
-    const dim3 grid(grid_for(n, static_cast<size_t>(kBlock) * v * kNormLoads));
+    const dim3 grid(static_cast<unsigned>(blocks));      // the same capped grid as the reduction
     if (nt) hipLaunchKernelGGL((rescale_clip_kernel<4, true>), grid, dim3(kBlock), 0, s, x, n, plan, clip);
     else if (vec) hipLaunchKernelGGL((rescale_clip_kernel<4, false>), grid, dim3(kBlock), 0, s, x, n, plan, clip);
     else hipLaunchKernelGGL((rescale_clip_kernel<1, false>), grid, dim3(kBlock), 0, s, x, n, plan, clip);
