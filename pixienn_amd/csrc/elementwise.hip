@@ -291,8 +291,8 @@ struct SgdUpdateOp {
 // Pass 1: a fixed number of workgroups walk the tensor and leave one partial sum of squares each;
 // pass 2: every workgroup adds up those partials (the same order everywhere), derives the factor
 // and rewrites its part of the tensor; when nothing is to be done it leaves without touching it.
-constexpr int kNormBlocks = 2048;     // 8 per compute unit: full occupancy
-constexpr int kNormLoads = 4;      // 128-bit loads in flight per lane
+constexpr int kNormBlocks = 1024;     // 4 per compute unit; every workgroup of pass 2 re-adds this many partials
+constexpr int kNormLoads = 8;         // 128-bit loads in flight per lane
 
 // Per workgroup: the sum of squares and the largest magnitude (NaN-free; a NaN shows in the sum).
 template<int V, bool NT>
@@ -337,21 +337,23 @@ __global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, s
     }
 }
 
-// One workgroup: the norm from the partial sums, the factor the rewrite applies, and whether the
-// rewrite has anything to do: a factor other than 1, or a value that the clamp would move.  The
-// scaled magnitudes are at most fl(factor * peak) (rounding is monotonic), so a peak within the
-// clamp after scaling means no element changes; a NaN anywhere (it shows in the sum) or an
-// infinite peak keeps the rewrite, which treats them as the CPU loop does.
-constexpr int kFactorLanes = 1024;      // two partials per lane at most: one trip to memory
+// The plan of the rewrite, formed by every workgroup for itself from the same partials in the same
+// order (so all arrive at the same one): the norm, the factor, and whether anything can change -- a
+// factor other than 1, or a value that the clamp would move.  The scaled magnitudes are at most
+// fl(factor * peak) (rounding is monotonic), so a peak within the clamp after scaling means no
+// element changes; a NaN anywhere (it shows in the sum) or an infinite peak keeps the rewrite, which
+// treats them as the CPU loop does.
+struct RescalePlan {
+    float norm, factor;
+    bool work;
+};
 
-__global__ __launch_bounds__(kFactorLanes) void rescale_factor_kernel(const double2* partial, int partials,
-                                                                      float threshold, float clip, float* factor_out,
-                                                                      float* norm_out)
+__device__ __forceinline__ RescalePlan rescale_plan(const double2* partial, int partials, float threshold, float clip)
 {
-    __shared__ double sums[kFactorLanes / kWave];
-    __shared__ double tops[kFactorLanes / kWave];
+    __shared__ double sums[kBlock / kWave];
+    __shared__ double tops[kBlock / kWave];
     double s = 0.0, top = 0.0;
-    for (int j = threadIdx.x; j < partials; j += kFactorLanes) {
+    for (int j = threadIdx.x; j < partials; j += kBlock) {
         const double2 p = partial[j];
         s += p.x;
         top = fmax(top, p.y);
@@ -366,33 +368,33 @@ __global__ __launch_bounds__(kFactorLanes) void rescale_factor_kernel(const doub
         tops[threadIdx.x / kWave] = top;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        double total = 0.0;
-        float peak = 0.0f;
+    double total = 0.0;
+    float peak = 0.0f;
 #pragma unroll
-        for (int w = 0; w < kFactorLanes / kWave; ++w) {
-            total += sums[w];
-            peak = fmaxf(peak, static_cast<float>(tops[w]));
-        }
-        const float norm = static_cast<float>(sqrt(total));
-        if (norm_out) *norm_out = norm;
-        float factor = 1.0f;
-        if (threshold > 0.0f && norm > 0.0f && norm > threshold) factor = threshold / norm;
-        factor_out[0] = factor;
-        const bool clamps = clip > 0.0f && (!(factor * peak <= clip) || total != total);
-        factor_out[1] = (factor != 1.0f || clamps) ? 1.0f : 0.0f;
+    for (int w = 0; w < kBlock / kWave; ++w) {
+        total += sums[w];
+        peak = fmaxf(peak, static_cast<float>(tops[w]));
     }
+    RescalePlan plan;
+    plan.norm = static_cast<float>(sqrt(total));
+    plan.factor = 1.0f;
+    if (threshold > 0.0f && plan.norm > 0.0f && plan.norm > threshold) plan.factor = threshold / plan.norm;
+    const bool clamps = clip > 0.0f && (!(plan.factor * peak <= clip) || total != total);
+    plan.work = plan.factor != 1.0f || clamps;
+    return plan;
 }
 
-// x = clamp(factor * x); leaves without touching the tensor when there is nothing to do
-// (plan[0] = factor, plan[1] = 0 when no element would change).
+// x = clamp(factor * x); leaves without touching the tensor when there is nothing to do.  The grid
+// is the reduction's capped one and strides over the tensor.
 template<int V, bool NT>
-__global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n_vec, const float* plan, float clip)
+__global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n_vec, const double2* partial,
+                                                              int partials, float threshold, float clip,
+                                                              float* norm_out)
 {
-    const float factor = plan[0];
-    if (plan[1] == 0.0f) return;
-    // kNormLoads vectors per lane and step; the grid is capped (a launch that finds nothing to do
-    // should cost a few hundred workgroups, not one per 16 KB of tensor) and strides over the rest
+    const RescalePlan plan = rescale_plan(partial, partials, threshold, clip);
+    if (norm_out && blockIdx.x == 0 && threadIdx.x == 0) *norm_out = plan.norm;
+    if (!plan.work) return;
+    const float factor = plan.factor;
     const size_t per_step = static_cast<size_t>(kBlock) * V * kNormLoads;
     for (size_t base = static_cast<size_t>(blockIdx.x) * per_step; base < n_vec;
          base += static_cast<size_t>(gridDim.x) * per_step) {
@@ -663,7 +665,7 @@ int pxh_sgd_update(size_t n, float* w, float* d, int batch, float lr, float mome
 
 size_t pxh_rescale_workspace_bytes(void)
 {
-    return kNormBlocks * sizeof(double2) + 256;      // partial sums and peaks, then factor and flag
+    return kNormBlocks * sizeof(double2);      // partial sums and peaks
 }
 
 int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* norm_out, void* workspace,
@@ -677,7 +679,6 @@ int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* nor
     int rc = resolve_workspace(workspace, workspace_bytes, pxh_rescale_workspace_bytes(), &ws);
     if (rc) return rc;
     double2* partial = static_cast<double2*>(ws);
-    float* plan = reinterpret_cast<float*>(partial + kNormBlocks);
     hipStream_t s = as_stream(stream);
     const bool vec = aligned16(x) && n % 4 == 0;
     const int v = vec ? 4 : 1;
@@ -692,15 +693,14 @@ int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* nor
     else hipLaunchKernelGGL((sumsq_partial_kernel<1, false>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
     rc = check_launch("pxh_rescale_clip");
     if (rc) return rc;
-    hipLaunchKernelGGL(rescale_factor_kernel, dim3(1), dim3(kFactorLanes), 0, s, partial, blocks, threshold, clip, plan,
-                       norm_out);
-    rc = check_launch("pxh_rescale_clip");
-    if (rc) return rc;
-    if (!(threshold > 0.0f) && !(clip > 0.0f)) return PXH_OK;      // only the norm was asked for
-    const dim3 grid(static_cast<unsigned>(blocks));      // the same capped grid as the reduction
-    if (nt) hipLaunchKernelGGL((rescale_clip_kernel<4, true>), grid, dim3(kBlock), 0, s, x, n, plan, clip);
-    else if (vec) hipLaunchKernelGGL((rescale_clip_kernel<4, false>), grid, dim3(kBlock), 0, s, x, n, plan, clip);
-    else hipLaunchKernelGGL((rescale_clip_kernel<1, false>), grid, dim3(kBlock), 0, s, x, n, plan, clip);
+    // only the norm asked for: one workgroup adds up the partials and writes it
+    const dim3 grid(threshold > 0.0f || clip > 0.0f ? static_cast<unsigned>(blocks) : 1u);
+    if (nt) hipLaunchKernelGGL((rescale_clip_kernel<4, true>), grid, dim3(kBlock), 0, s, x, n, partial, blocks,
+                               threshold, clip, norm_out);
+    else if (vec) hipLaunchKernelGGL((rescale_clip_kernel<4, false>), grid, dim3(kBlock), 0, s, x, n, partial, blocks,
+                                     threshold, clip, norm_out);
+    else hipLaunchKernelGGL((rescale_clip_kernel<1, false>), grid, dim3(kBlock), 0, s, x, n, partial, blocks,
+                            threshold, clip, norm_out);
     return check_launch("pxh_rescale_clip");
 }
 
