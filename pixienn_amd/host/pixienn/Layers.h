@@ -228,6 +228,14 @@ public:
         return is.tellg() - start;
     }
 
+    // Clears the accumulated parameter updates and the optimizer moments (a fresh start of training).
+    void zeroUpdates()
+    {
+        for (V* t: { &weightUpdates_, &biasUpdates_, &scaleUpdates_, &weightM_, &weightV_, &biasM_, &biasV_, &scaleM_,
+                     &scaleV_ })
+            if (!t->empty()) t->fill(0.0f, stream());
+    }
+
     V& weights() noexcept { return weights_; }
     V& weightUpdates() noexcept { return weightUpdates_; }
     const V& biases() const noexcept { return biases_; }

@@ -17,6 +17,7 @@
 #include <sstream>
 
 #include "pixienn/Layers.h"
+#include "pixienn/CapturedSequence.h"
 #include "pixienn/OptimizerState.h"
 #include "px_oracle.h"
 
@@ -697,6 +698,84 @@ void batchNormLayerChecks()
     expectClose("guarded update: clamped scale updates", guarded.scaleUpdates().asVector(), gsu, 1e-5, 1.0);
 }
 
+// The whole training step of the mini network (forward, backward, update) recorded as one HIP graph
+// and replayed on new inputs: every tensor must be what the same calls give when issued one by one.
+void capturedSequenceChecks()
+{
+    hipStream_t stream = nullptr;
+    PX_HIP_RUNTIME_CHECK(hipStreamCreate(&stream));
+    {
+        Net eager(true), captured(true);
+        eager.ctx.stream = stream;
+        captured.ctx.stream = stream;
+        const auto truth = makeTruth();
+        eager.ctx.setGroundTruth(truth);
+        captured.ctx.setGroundTruth(truth);
+        FloatVector inputEager(size_t(N) * C * S * S), inputCaptured(size_t(N) * C * S * S);
+        auto step = [](Net& net, const FloatVector& input) {
+            net.conv0->forward(input);
+            net.pool1->forward(net.conv0->output());
+            net.conv2->forward(net.pool1->output());
+            net.short3->forward(net.conv2->output());
+            net.up4->forward(net.short3->output());
+            net.route5->forward(net.up4->output());
+            net.conv6->forward(net.route5->output());
+            net.yolo7->forward(net.conv6->output());
+            net.yolo7->backward(net.conv6->output(), &net.conv6->delta());
+            net.conv6->backward(net.route5->output(), &net.route5->delta());
+            net.route5->backward(net.up4->output(), &net.up4->delta());
+            net.up4->backward(net.short3->output(), &net.short3->delta());
+            net.short3->backward(net.conv2->output(), &net.conv2->delta());
+            net.conv2->backward(net.pool1->output(), &net.pool1->delta());
+            net.pool1->backward(net.conv0->output(), &net.conv0->delta());
+            net.conv0->backward(input, nullptr);
+            for (Layer* l: std::initializer_list<Layer*>{ net.conv0.get(), net.conv2.get(), net.conv6.get() }) l->update();
+        };
+        inputCaptured.copyHost(normals(500, inputCaptured.size()));
+        step(captured, inputCaptured);                 // eager once: the library sizes its workspace
+        PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(stream));
+        CapturedSequence graph;
+        graph.capture(stream, [&] { step(captured, inputCaptured); });
+        report("a training step is captured as one graph", graph.captured());
+        // bring both networks to the same state: the capture run and the warm-up moved `captured` only
+        Net* nets[2] = { &eager, &captured };
+        bool same = true;
+        for (int round = 1; round <= 3; ++round) {
+            const Host in = normals(500 + round, inputEager.size());
+            inputEager.copyHost(in);
+            inputCaptured.copyHost(in);
+            if (round == 1) {
+                // parameters and rolling statistics back to the initial ones on both sides
+                for (Net* n: nets) {
+                    n->conv0->copyScales(n->scale0); n->conv0->copyBiases(n->bias0);
+                    n->conv0->copyRollingMean(normals(16, C, 0.1f));
+                    n->conv0->copyRollingVariance(uniforms(17, C, 0.5f, 1.5f));
+                    n->conv2->copyScales(n->scale2); n->conv2->copyBiases(n->bias2);
+                    n->conv2->copyRollingMean(normals(18, C, 0.1f));
+                    n->conv2->copyRollingVariance(uniforms(19, C, 0.5f, 1.5f));
+                    n->conv6->copyBiases(n->bias6);
+                    n->conv0->zeroUpdates(); n->conv2->zeroUpdates(); n->conv6->zeroUpdates();
+                }
+            }
+            graph.replay(stream);
+            step(eager, inputEager);
+            PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(stream));
+            same = same && captured.yolo7->delta().asVector() == eager.yolo7->delta().asVector() &&
+                   captured.conv0->delta().asVector() == eager.conv0->delta().asVector() &&
+                   captured.conv0->scales().asVector() == eager.conv0->scales().asVector() &&
+                   captured.conv2->biases().asVector() == eager.conv2->biases().asVector() &&
+                   captured.conv0->rollingVariance().asVector() == eager.conv0->rollingVariance().asVector() &&
+                   captured.yolo7->fetchStats() == eager.yolo7->fetchStats();
+            report("replay " + std::to_string(round) + " equals the eager step", same);
+        }
+        expectThrows("capture on the null stream is refused", [&] {
+            CapturedSequence g;
+            g.capture(nullptr, [] {});
+        }, "null stream");
+    }
+    PX_HIP_RUNTIME_CHECK(hipStreamDestroy(stream));
+}
+
 // An upsample layer absorbed by the route that reads it gives the same tensors as the two-step form.
 void absorbedUpsampleChecks()
 {
@@ -763,6 +842,7 @@ int main(int argc, char** argv)
             trainingChecks();
             absorbedUpsampleChecks();
             batchNormLayerChecks();
+            capturedSequenceChecks();
         }
     } catch (const std::exception& e) {
         std::printf("unexpected exception: %s\n", e.what());
