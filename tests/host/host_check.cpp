@@ -19,6 +19,7 @@
 #include "pixienn/Layers.h"
 #include "pixienn/CapturedSequence.h"
 #include "pixienn/OptimizerState.h"
+#include "pixienn/WeightsFile.h"
 #include "px_oracle.h"
 
 using namespace px::hip;
@@ -776,6 +777,56 @@ void capturedSequenceChecks()
     PX_HIP_RUNTIME_CHECK(hipStreamDestroy(stream));
 }
 
+// A model's weights file: header of either seen-width, every layer's section in network order, exact length.
+void weightsFileChecks()
+{
+    auto build = [](Context& ctx) {
+        std::vector<Layer::Ptr> layers;
+        layers.push_back(std::make_shared<ConvLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S },
+                                                                      { "width", S }, { "filters", C }, { "weights", 27 * C },
+                                                                      { "batch_normalize", true } }));
+        layers.push_back(std::make_shared<MaxPoolLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S },
+                                                                         { "width", S }, { "kernel", 2 }, { "stride", 2 } }));
+        layers.push_back(std::make_shared<BatchNormLayer>(ctx, Properties{ { "batch", N }, { "channels", C },
+                                                                           { "height", S / 2 }, { "width", S / 2 } }));
+        layers.push_back(std::make_shared<ConvLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S / 2 },
+                                                                      { "width", S / 2 }, { "filters", 5 },
+                                                                      { "weights", 5 * C } }));
+        return layers;
+    };
+    Context ctx;
+    auto source = build(ctx);
+    auto* conv = static_cast<ConvLayer*>(source[0].get());
+    conv->copyBiases(normals(601, C, 0.1f)); conv->copyScales(uniforms(602, C, 0.5f, 1.5f));
+    conv->copyRollingMean(normals(603, C, 0.1f)); conv->copyRollingVariance(uniforms(604, C, 0.5f, 1.5f));
+    conv->weights().copyHost(normals(605, 27 * C, 0.02f));
+    auto* last = static_cast<ConvLayer*>(source[3].get());
+    last->copyBiases(normals(606, 5, 0.1f));
+    last->weights().copyHost(normals(607, 5 * C, 0.02f));
+    for (const bool wide: { false, true }) {
+        WeightsHeader h;
+        if (wide) { h.major = 0; h.minor = 2; }
+        h.seen = wide ? 0x123456789aull : 64000u;
+        std::stringstream file(std::ios::in | std::ios::out | std::ios::binary);
+        saveWeightsFile(file, h, source);
+        const size_t floats = (4 * C + 27 * C) + 4 * C + (5 + 5 * C);
+        report(std::string("weights file length, ") + (wide ? "64-bit" : "32-bit") + " seen",
+               file.str().size() == 12 + (wide ? 8 : 4) + floats * sizeof(float));
+        auto target = build(ctx);
+        const WeightsHeader back = loadWeightsFile(file, target);
+        report("weights file header round trip", back.major == h.major && back.minor == h.minor && back.seen == h.seen);
+        report("weights file restores every layer",
+               static_cast<ConvLayer*>(target[0].get())->weights().asVector() == conv->weights().asVector() &&
+               static_cast<ConvLayer*>(target[0].get())->rollingVariance().asVector() == conv->rollingVariance().asVector() &&
+               static_cast<ConvLayer*>(target[3].get())->biases().asVector() == last->biases().asVector() &&
+               static_cast<ConvLayer*>(target[3].get())->weights().asVector() == last->weights().asVector());
+        std::stringstream longer(file.str() + "tail", std::ios::in | std::ios::binary);
+        expectThrows("trailing bytes are refused", [&] { loadWeightsFile(longer, target); }, "Did not fully read");
+        std::stringstream shorter(file.str().substr(0, file.str().size() - 8), std::ios::in | std::ios::binary);
+        expectThrows("a truncated file is refused", [&] { loadWeightsFile(shorter, target); }, "Could not read");
+    }
+}
+
 // An upsample layer absorbed by the route that reads it gives the same tensors as the two-step form.
 void absorbedUpsampleChecks()
 {
@@ -842,6 +893,7 @@ int main(int argc, char** argv)
             trainingChecks();
             absorbedUpsampleChecks();
             batchNormLayerChecks();
+            weightsFileChecks();
             capturedSequenceChecks();
         }
     } catch (const std::exception& e) {
