@@ -50,6 +50,8 @@ def parse_args():
     ap.add_argument("--no-extras", action="store_true", help="skip the other kernels of the path")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-batch", type=int, default=64, help="images per shape in the CPU sample")
+    ap.add_argument("--only-model-order", action="store_true",
+                    help="run only the YOLOv3 training step in model order (for a kernel trace of that step)")
     return ap.parse_args()
 
 
@@ -558,6 +560,10 @@ def main():
     assert torch.cuda.is_available(), "no GPU visible"
     torch.cuda.set_device(0)
     timer = Timer(torch)
+    if args.only_model_order:
+        print(json.dumps({"noconv_step_in_model_order_yolov3_608": measure_model_order(torch, ops, wl, timer)}),
+              flush=True)
+        return
 
     shapes = epilogue_workload(torch, wl)
     fold_weights(ops, shapes)
