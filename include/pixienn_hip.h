@@ -215,6 +215,17 @@ int pxh_shortcut_forward(const float* input, const float* from_output, float* ou
  *   from_delta = 1*from_delta + beta*delta;  grad += alpha*delta (grad nullable). */
 int pxh_shortcut_backward(float* delta, const float* pre_activation, float* from_delta, float* grad,
                           size_t n, float alpha, float beta, int activation, void* stream);
+/* The same for the call that is the FIRST in a backward pass to write both targets: they are
+ * overwritten (from_delta = beta*delta', grad = alpha*delta') instead of accumulated into, which is
+ * what accumulating into cleared tensors gives (up to the sign of a zero), so neither needs the
+ * zero-fill of Layer::forward (include/Layer.h:378-383) and neither is read: 12 B per element
+ * instead of 20 + 8.  In a residual block the shortcut is that call for the delta of the layer in
+ * front of it and of its `from` layer (the only other reader of the latter comes earlier in the
+ * network, so later in the backward pass).  No counterpart in the reference, which always clears
+ * and accumulates; the caller vouches for the order. */
+int pxh_shortcut_backward_first(float* delta, const float* pre_activation, float* from_delta,
+                                float* grad, size_t n, float alpha, float beta, int activation,
+                                void* stream);
 
 /* ------------------------------------------------------------------------
  * YOLO head.  include/YoloKernels.cuh:7-17, CPU semantics include/YoloLayer.h:164-239, 390-547.

@@ -49,6 +49,7 @@ SIGNATURES = {
     "pxh_shortcut": [I, I, I, I, P, I, I, I, F, F, P, P],
     "pxh_shortcut_forward": [P, P, P, P, Z, F, F, I, P],
     "pxh_shortcut_backward": [P, P, P, P, Z, F, F, I, P],
+    "pxh_shortcut_backward_first": [P, P, P, P, Z, F, F, I, P],
     "pxh_yolo_activate": [P, P, I, I, I, I, P],
     "pxh_yolo_loss": [P, P, P, P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, F, F, F, F, F, P, Z, P],
     "pxh_yolo_forward_train": [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, F, F, F, F, P, Z, P],

@@ -196,8 +196,10 @@ struct ShortcutForwardOp {
     }
 };
 
-// delta *= act'(pre); from_delta = 1*from_delta + beta*delta; grad += alpha*delta
-template<int ACT>
+// delta *= act'(pre); from_delta = 1*from_delta + beta*delta; grad += alpha*delta.
+// FIRST: this call is the first to write both targets in this backward pass, so they need not have
+// been cleared: from_delta = beta*delta, grad = alpha*delta (what accumulating into zeros gives).
+template<int ACT, bool FIRST = false>
 struct ShortcutBackwardOp {
     float* delta;
     const float* pre;
@@ -209,8 +211,10 @@ struct ShortcutBackwardOp {
     {
         r.d = ld<V, NT>(delta, e);
         if constexpr (ACT != PXH_LINEAR) r.p = ld<V, NT>(pre, e);
-        r.f = ld<V, NT>(from_delta, e);
-        if (grad) r.g = ld<V, NT>(grad, e);
+        if constexpr (!FIRST) {
+            r.f = ld<V, NT>(from_delta, e);
+            if (grad) r.g = ld<V, NT>(grad, e);
+        }
     }
     template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
     {
@@ -218,12 +222,15 @@ struct ShortcutBackwardOp {
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             if constexpr (ACT != PXH_LINEAR) d.v[k] = d.v[k] * act_grad<ACT>(r.p.v[k]);
-            const float keep = 1.0f * r.f.v[k];
             const float add = beta * d.v[k];
-            f.v[k] = keep + add;
-            if (grad) {
-                const float ga = alpha * d.v[k];
-                g.v[k] = r.g.v[k] + ga;
+            const float ga = alpha * d.v[k];
+            if constexpr (FIRST) {
+                f.v[k] = add;
+                g.v[k] = ga;
+            } else {
+                const float keep = 1.0f * r.f.v[k];
+                f.v[k] = keep + add;
+                if (grad) g.v[k] = r.g.v[k] + ga;
             }
         }
         if constexpr (ACT != PXH_LINEAR) st<V, NT>(delta, e, d);
@@ -650,6 +657,25 @@ int pxh_shortcut_backward(float* delta, const float* pre_activation, float* from
                            as_stream(stream));
     });
     if (!known) return fail_invalid("pxh_shortcut_backward: unknown activation %d", activation);
+    return rc;
+}
+
+int pxh_shortcut_backward_first(float* delta, const float* pre_activation, float* from_delta, float* grad, size_t n,
+                                float alpha, float beta, int activation, void* stream)
+{
+    if ((!delta || !from_delta) && n) return fail_invalid("pxh_shortcut_backward_first: null pointer");
+    if (activation != PXH_LINEAR && !pre_activation && n)
+        return fail_invalid("pxh_shortcut_backward_first: pre_activation is required for a non-linear activation");
+    if (from_delta == grad && n)
+        return fail_invalid("pxh_shortcut_backward_first: from_delta and grad must be distinct when both are overwritten");
+    int rc = PXH_OK;
+    const bool vec = aligned16(delta) && aligned16(pre_activation) && aligned16(from_delta) && aligned16(grad);
+    const bool known = dispatch_activation(activation, [&]<int ACT>() {
+        rc = launch_stream("pxh_shortcut_backward_first", n, vec, grad ? 12 : 8,
+                           ShortcutBackwardOp<ACT, true>{ delta, pre_activation, from_delta, grad, alpha, beta },
+                           as_stream(stream));
+    });
+    if (!known) return fail_invalid("pxh_shortcut_backward_first: unknown activation %d", activation);
     return rc;
 }
 

@@ -164,7 +164,7 @@ public:
     // (include/Layer.h:377-383), then write output_.
     virtual void forward(const V& /*input*/)
     {
-        if (training() && !delta_.empty()) delta_.fill(0.0f, stream());
+        if (training() && !delta_.empty() && !firstConsumerOverwrites_) delta_.fill(0.0f, stream());
         cost_ = 0.0f;
     }
 
@@ -208,6 +208,12 @@ public:
 
     const V& output() const noexcept { return output_; }
     V& delta() noexcept { return delta_; }
+
+    // A layer whose delta is OVERWRITTEN by the first of its readers to run backward (a shortcut with
+    // "first_writer") needs no zero-fill in forward.  Whoever sets this vouches that every backward
+    // pass starts with that reader.
+    void setFirstConsumerOverwrites(bool on) noexcept { firstConsumerOverwrites_ = on; }
+    bool firstConsumerOverwrites() const noexcept { return firstConsumerOverwrites_; }
 
     void setGradientClipping(bool on, float value) { gradientClipping_ = on; gradientClipValue_ = value; }
     void setGradientRescaling(bool on, float threshold) { gradientRescaling_ = on; gradientThreshold_ = threshold; }
@@ -257,7 +263,7 @@ private:
     Properties props_;
     int batch_, channels_, height_, width_, index_, inputs_;
     int outChannels_ = 0, outHeight_ = 0, outWidth_ = 0, outputs_ = 0;
-    bool gradientClipping_ = false, gradientRescaling_ = false;
+    bool gradientClipping_ = false, gradientRescaling_ = false, firstConsumerOverwrites_ = false;
     float gradientClipValue_ = 1.0f, gradientThreshold_ = 0.0f;
 };
 

@@ -518,6 +518,13 @@ public:
         sameShape_ = from_->outChannels() == outChannels() && from_->outHeight() == outHeight() &&
                      from_->outWidth() == outWidth();
         if (training() && (activation_ != PXH_LINEAR || !sameShape_)) preActivation_ = V(output_.size());
+        // "first_writer": in the backward pass this shortcut runs before every other reader of the
+        // layer in front of it and of its `from` layer (true of a residual block: the block's first
+        // conv reads `from` too, but comes earlier in the network).  It then overwrites both deltas
+        // instead of adding to them, and neither needs clearing: the `from` layer is told here, the
+        // layer in front by whoever builds the network (setFirstConsumerOverwrites).
+        firstWriter_ = training() && sameShape_ && props.get<bool>("first_writer", false);
+        if (firstWriter_) from_->setFirstConsumerOverwrites(true);
     }
 
     void forward(const V& input) override
@@ -543,6 +550,12 @@ public:
     {
         Layer::backward(input, grad);
         const float* pre = preActivation_.empty() ? nullptr : preActivation_.data();
+        if (firstWriter_) {
+            PX_CHECK(grad != nullptr, "a first-writer shortcut needs the delta of the layer in front of it");
+            PX_HIP_CHECK(pxh_shortcut_backward_first(delta_.data(), pre, from_->delta().data(), grad->data(),
+                                                     delta_.size(), alpha_, beta_, activation_, stream()));
+            return;
+        }
         if (sameShape_) {
             PX_HIP_CHECK(pxh_shortcut_backward(delta_.data(), pre, from_->delta().data(),
                                                grad ? grad->data() : nullptr, delta_.size(), alpha_, beta_,
@@ -561,7 +574,7 @@ private:
     Layer::Ptr from_;
     int activation_ = PXH_LINEAR;
     float alpha_ = 1.0f, beta_ = 1.0f;
-    bool sameShape_ = true;
+    bool sameShape_ = true, firstWriter_ = false;
     V preActivation_;
 };
 

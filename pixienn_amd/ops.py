@@ -271,6 +271,14 @@ def shortcut_backward(delta, from_delta, grad=None, activation="linear", alpha=1
          float(alpha), float(beta), act_id(activation), _stream())
 
 
+def shortcut_backward_first(delta, from_delta, grad=None, activation="linear", alpha=1.0, beta=1.0,
+                            pre_activation=None):
+    """shortcut_backward for the first writer of both targets: overwrites instead of accumulating."""
+    _chk_all(delta, from_delta, grad, pre_activation)
+    call("pxh_shortcut_backward_first", ptr(delta), ptr(pre_activation), ptr(from_delta), ptr(grad), delta.numel(),
+         float(alpha), float(beta), act_id(activation), _stream())
+
+
 # ---------------------------------------------------------------- YOLO head
 def yolo_activate(inp, out, batch, masks, classes, area):
     _chk_all(inp, out)

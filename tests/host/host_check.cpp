@@ -777,6 +777,60 @@ void capturedSequenceChecks()
     PX_HIP_RUNTIME_CHECK(hipStreamDestroy(stream));
 }
 
+// A residual block whose shortcut overwrites the two deltas it is the first to write: the same
+// gradients as the clearing-and-accumulating form, with the two zero-fills gone.
+void firstWriterShortcutChecks()
+{
+    struct Block {
+        Context ctx;
+        std::shared_ptr<ConvLayer> a, b, c;
+        std::shared_ptr<ShortcutLayer> add;
+        explicit Block(bool firstWriter)
+        {
+            ctx.training = true;
+            const Properties conv{ { "batch", N }, { "channels", C }, { "height", S }, { "width", S }, { "filters", C },
+                                   { "batch_normalize", true }, { "activation", std::string("leaky") } };
+            a = std::make_shared<ConvLayer>(ctx, conv);
+            b = std::make_shared<ConvLayer>(ctx, conv);
+            c = std::make_shared<ConvLayer>(ctx, conv);
+            add = std::make_shared<ShortcutLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S },
+                                                                   { "width", S }, { "first_writer", firstWriter } }, a);
+            if (firstWriter) c->setFirstConsumerOverwrites(true);
+        }
+        void step(const FloatVector& input, const Host& outDelta)
+        {
+            a->forward(input);
+            b->forward(a->output());
+            c->forward(b->output());
+            add->forward(c->output());
+            add->delta().copyHost(outDelta);
+            add->backward(c->output(), &c->delta());
+            c->backward(b->output(), &b->delta());
+            b->backward(a->output(), &a->delta());
+            a->backward(input, nullptr);
+        }
+    };
+    Block plain(false), first(true);
+    report("the shortcut marks its from layer", first.a->firstConsumerOverwrites() && !plain.a->firstConsumerOverwrites() &&
+                                                !first.b->firstConsumerOverwrites());
+    const FloatVector input(normals(701, size_t(N) * C * S * S));
+    for (int round = 0; round < 2; ++round) {
+        const Host outDelta = normals(702 + round, size_t(N) * C * S * S);
+        // stale values where the fill used to be: they must not survive
+        first.a->delta().fill(std::nanf(""));
+        first.c->delta().fill(std::nanf(""));
+        plain.step(input, outDelta);
+        first.step(input, outDelta);
+        const std::string tag = " (step " + std::to_string(round + 1) + ")";
+        expectClose("first-writer block: delta of the layer in front" + tag, first.c->delta().asVector(),
+                    plain.c->delta().asVector(), 0.0, 1.0);
+        expectClose("first-writer block: delta of the from layer" + tag, first.a->delta().asVector(),
+                    plain.a->delta().asVector(), 0.0, 1.0);
+        expectClose("first-writer block: scale updates of the from layer" + tag, first.a->scaleUpdates().asVector(),
+                    plain.a->scaleUpdates().asVector(), 0.0, 1.0);
+    }
+}
+
 // A model's weights file: header of either seen-width, every layer's section in network order, exact length.
 void weightsFileChecks()
 {
@@ -894,6 +948,7 @@ int main(int argc, char** argv)
             absorbedUpsampleChecks();
             batchNormLayerChecks();
             weightsFileChecks();
+            firstWriterShortcutChecks();
             capturedSequenceChecks();
         }
     } catch (const std::exception& e) {

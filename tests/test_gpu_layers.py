@@ -147,6 +147,36 @@ def test_upsample_into_concatenation_buffer(ops, oracle, shape, stride, other, o
 
 
 @pytest.mark.parametrize("act", ["linear", "leaky"])
+@pytest.mark.parametrize("shape", [(2, 8, 38, 38), (3, 5, 19, 19), (1, 1, 1, 3), (4, 64, 76, 76)])
+def test_shortcut_backward_as_first_writer(ops, oracle, shape, act):
+    """The overwriting form gives what the CPU layer's accumulation into cleared tensors gives, and
+    reads neither target: they start as NaN here."""
+    import torch
+    N, C, H, W = shape
+    for alpha, beta in ((1.0, 1.0), (0.5, 1.25)):
+        pre = wl.normal(1820 + W, shape)
+        d0 = wl.normal(1821 + W, shape)
+        d0[0, 0, 0, 0] = 0.0                                  # a zero delta: -0 * beta stays a zero of either sign
+        d_w, fd_w, g_w = d0.copy(), np.zeros(shape, F), np.zeros(shape, F)
+        oracle.shortcut_backward(act, N, W, H, C, d_w, pre, fd_w, g_w, alpha, beta)
+        gd = gpu(d0)
+        gfd = torch.full(shape, float("nan"), device="cuda"); gg = torch.full(shape, float("nan"), device="cuda")
+        ops.shortcut_backward_first(gd, gfd, gg, act, alpha, beta, pre_activation=gpu(pre))
+        what = "first-writer shortcut %s %s a=%g b=%g" % (shape, act, alpha, beta)
+        assert_bit_exact(host(gd), d_w, what + " delta")
+        for got, want, name in ((host(gfd), fd_w, "from delta"), (host(gg), g_w, "grad")):
+            assert np.array_equal(got, want), what + " " + name                       # equal as numbers
+            nonzero = want != 0
+            assert_bit_exact(got[nonzero], want[nonzero], what + " " + name)         # and bit for bit off zero
+        # without a grad target only from_delta is written
+        gfd2 = torch.full(shape, float("nan"), device="cuda")
+        ops.shortcut_backward_first(gpu(d0), gfd2, None, act, alpha, beta, pre_activation=gpu(pre))
+        assert np.array_equal(host(gfd2), fd_w), what + " from delta alone"
+    with pytest.raises(ops.capi.PxError):
+        ops.shortcut_backward_first(gd, gfd, gfd, act, 1.0, 1.0, pre_activation=gpu(pre))
+
+
+@pytest.mark.parametrize("act", ["linear", "leaky"])
 @pytest.mark.parametrize("shape", [(2, 8, 38, 38), (3, 5, 19, 19), (1, 1, 1, 3), (2, 3, 64, 64)])
 def test_shortcut_forward_backward(ops, oracle, shape, act):
     import torch
