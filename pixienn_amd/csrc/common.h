@@ -59,11 +59,64 @@ struct FastDiv {
 
 // ---------------------------------------------------------------- activations (device)
 // The arithmetic follows the CPU functors operation by operation (fp32, no contraction).
+// exp(x) to about a unit in the last place around the hardware's exp2: x * log2(e) is formed to twice
+// the working precision (the fma recovers the product's rounding error, a second term carries the low
+// bits of log2(e)), split into its integer part and a fraction in [-0.5, 0.5], and only the fraction
+// goes through exp2.  No range checks: ldexp saturates to 0 and infinity by itself.
+__device__ __forceinline__ float exp_by_exp2(float x)
+{
+    const float hi = 0x1.715476p+0f, lo = 0x1.4ae0c0p-26f;      // log2(e) = hi + lo
+    const float p = x * hi;
+    const float err = fmaf(x, lo, fmaf(x, hi, -p));
+    const float n = rintf(p);
+    const float f = (p - n) + err;
+    return ldexpf(__builtin_amdgcn_exp2f(f), static_cast<int>(n));
+}
+
+// exp(x) rounded to nearest, through a double-precision evaluation (argument reduction by ln 2,
+// Taylor polynomial of degree 10 on |r| <= 0.35: 2.4e-13 relative, so the conversion to float rounds
+// as the exact value would except within 2e-6 of a tie).
+__device__ __forceinline__ float exp_nearest(float x)
+{
+    const double xd = static_cast<double>(x);
+    const double k = rint(xd * 1.4426950408889634);
+    double r = fma(-k, 0.6931471805599453, xd);
+    r = fma(-k, 2.3190468138462996e-17, r);
+    double p = 1.0 / 3628800.0;
+    p = fma(p, r, 1.0 / 362880.0);
+    p = fma(p, r, 1.0 / 40320.0);
+    p = fma(p, r, 1.0 / 5040.0);
+    p = fma(p, r, 1.0 / 720.0);
+    p = fma(p, r, 1.0 / 120.0);
+    p = fma(p, r, 1.0 / 24.0);
+    p = fma(p, r, 1.0 / 6.0);
+    p = fma(p, r, 0.5);
+    p = fma(p, r, 1.0);
+    p = fma(p, r, 1.0);
+    return static_cast<float>(ldexp(p, static_cast<int>(k)));
+}
+
+// e = exp(x) for the chains that go on with u = float(e + 1) (softplus and everything built on it).
+// Below x = -4.4 (e < 0.012) one unit of u = 1.2e-7 is more than 1e-5 of e, and the CPU result moves
+// by that whole unit -- up to 0.4 % of its value -- when e is one unit in ITS last place off: there e
+// has to be the correctly rounded value the host's libm returns (measured with a 1-ulp exp: 25
+// elements per million of x in [-10.5, -4.4] off by up to 1e-3).  Such arguments are rare in a network
+// (a pre-activation 4 sigma below zero), so the double-precision path costs a wave only now and
+// then; elsewhere one unit in the last place is plenty and the short form is used.
+__device__ __forceinline__ bool one_plus_exp_is_sensitive(float x) { return x < -4.4f && x >= -20.0f; }
+
+__device__ __forceinline__ float exp_before_one_plus(float x)
+{
+    float e = exp_by_exp2(x);
+    if (one_plus_exp_is_sensitive(x)) e = exp_nearest(x);
+    return e;
+}
+
 __device__ __forceinline__ float softplus_apply(float x)
 {
     if (x > 20.0f) return x;
     if (x < -20.0f) return expf(x);
-    return logf(expf(x) + 1.0f);
+    return logf(exp_before_one_plus(x) + 1.0f);
 }
 
 __device__ __forceinline__ float softplus_grad(float x)
@@ -87,16 +140,15 @@ __device__ __forceinline__ float tanh_softplus_from_exp(float e)
 
 __device__ __forceinline__ float tanh_softplus_mid(float x)
 {
-    return tanh_softplus_from_exp(expf(x));
+    return tanh_softplus_from_exp(exp_before_one_plus(x));
 }
 
-// Forward mish without branches.  exp stays the accurate one: u = fl(exp(x) + 1) is where the CPU
-// chain loses its bits for negative x, so a last-place difference in exp(x) can show as 1e-5 of
-// the result (measured with the hardware exp2: 3 elements per million beyond 1e-5).  The division
-// is a hardware reciprocal and a multiply, 2 ulp.
+// Forward mish: one exp (see exp_before_one_plus), the division as a hardware reciprocal and a
+// multiply (2 ulp), the two tails by selection.
+template<bool QUICK = false>
 __device__ __forceinline__ float mish_apply(float x)
 {
-    const float e = expf(x);
+    const float e = QUICK ? exp_by_exp2(x) : exp_before_one_plus(x);
     const float u = e + 1.0f;
     const float num = (u - 1.0f) * (u + 1.0f);
     const float den = u * u + 1.0f;
@@ -129,11 +181,35 @@ __device__ __forceinline__ float act_apply(float x)
     else if constexpr (ACT == PXH_LOGGY) return 2.0f / (1.0f + expf(-x)) - 1.0f;
     // logistic and swish: the accurate exp, then a hardware reciprocal (1 ulp) in place of the division
     else if constexpr (ACT == PXH_LOGISTIC) return __builtin_amdgcn_rcpf(1.0f + expf(-x));
-    else if constexpr (ACT == PXH_MISH) return mish_apply(x);
+    else if constexpr (ACT == PXH_MISH) return mish_apply<false>(x);
     else if constexpr (ACT == PXH_RELU) return x > 0.0f ? x : 0.0f;
     else if constexpr (ACT == PXH_SOFTPLUS) return softplus_apply(x);
     else if constexpr (ACT == PXH_SWISH) return x * __builtin_amdgcn_rcpf(1.0f + expf(-1.0f * x));
     else return tanhf(x);
+}
+
+// V values at once.  For mish the short exp goes everywhere first and the values whose argument is
+// in the sensitive range are redone, behind ONE branch for the whole wave instead of one per value:
+// the same results as act_apply value by value.
+template<int ACT, int V>
+__device__ __forceinline__ void act_apply_n(const float (&pre)[V], float (&out)[V])
+{
+    if constexpr (ACT == PXH_MISH) {
+        bool any = false;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            out[k] = mish_apply<true>(pre[k]);
+            any = any | one_plus_exp_is_sensitive(pre[k]);
+        }
+        if (__ballot(any)) {
+#pragma unroll
+            for (int k = 0; k < V; ++k)
+                if (one_plus_exp_is_sensitive(pre[k])) out[k] = mish_apply<false>(pre[k]);
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k) out[k] = act_apply<ACT>(pre[k]);
+    }
 }
 
 template<int ACT>

@@ -119,10 +119,8 @@ __global__ __launch_bounds__(kBlock) void epilogue_fwd_kernel(EpilogueArgs a)
     if (!__ballot(crosses)) {
         // no lane of the wave touches a plane boundary (the common case for large planes)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            po.v[j] = pre_value<BN>(xin.v[j], k0, no.v[j]);
-            yo.v[j] = act_apply<ACT>(po.v[j]);
-        }
+        for (int j = 0; j < 4; ++j) po.v[j] = pre_value<BN>(xin.v[j], k0, no.v[j]);
+        act_apply_n<ACT>(po.v, yo.v);
     } else if (hw >= 4) {
         // some lane's vector runs into the next plane (at most one boundary per vector): the
         // elements past it take the next channel's constants.  Selecting the constants per element
@@ -140,8 +138,8 @@ __global__ __launch_bounds__(kBlock) void epilogue_fwd_kernel(EpilogueArgs a)
             k.scale = here ? k0.scale : k1.scale;
             k.bias = here ? k0.bias : k1.bias;
             po.v[j] = pre_value<BN>(xin.v[j], k, no.v[j]);
-            yo.v[j] = act_apply<ACT>(po.v[j]);
         }
+        act_apply_n<ACT>(po.v, yo.v);
     } else {
         // planes of fewer than 4 elements: several boundaries per vector, walk element by element
         FoldCoef k = k0;

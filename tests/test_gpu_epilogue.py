@@ -291,6 +291,20 @@ def test_activation_kats_and_sweep(ops, oracle, kats, act):
     assert_close(host(v), want[:1000], RTOL, fl if np.isscalar(fl) else fl[:1000], act + " unaligned")
 
 
+@pytest.mark.parametrize("act", ["mish", "softplus"])
+def test_one_plus_exp_chain_follows_the_host_libm(ops, oracle, act):
+    """Between x = -17 and -4.4 the CPU formula's u = float(1 + exp(x)) keeps only a few bits of exp(x):
+    one unit in the last place of exp(x) can move u by a whole unit and the result by up to 0.4 %.
+    With a 1-ulp exp that shows in 25 elements per million; the kernels evaluate exp there rounded to
+    nearest, as the host's libm (nearly always) does, which leaves well under one per million."""
+    x = np.random.Generator(np.random.Philox(key=77)).uniform(-17.0, -3.0, 8_000_000).astype(F)
+    want = oracle.activate(act, x.copy())
+    got = host(ops.activate(act, gpu(x)))
+    rel = np.abs(got.astype(np.float64) - want) / np.maximum(np.abs(want), 1e-9)
+    off = int((rel > 1e-5).sum())
+    assert off <= 8, "%s: %d of %d elements moved by a unit of 1 + exp(x); worst %.3g" % (act, off, x.size, rel.max())
+
+
 def test_helper_kernels(ops, oracle):
     import torch
     x = wl.normal(900, 10007)
