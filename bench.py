@@ -311,19 +311,20 @@ def measure_extras(torch, ops, wl, timer, capi):
     # The upsample in front writes its channels straight into the concat buffer (timed below, same
     # bytes as the dense form), so the route moves the other source only.
     for (c1, c2, s) in [(256, 512, 38), (128, 256, 76)]:
-        b = randn(N, c2, s, s)
-        r = torch.empty((N, c1 + c2, s, s), device=dev)
         e = N * c2 * s * s
-        ms = timer.time(lambda i: ops.route_forward(b, r, c1 * s * s), 20)
-        add("route_fwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), 8 * e, ms, "the %d-channel source, 8B/elem" % c2)
-        ms = timer.time(lambda i: ops.route_backward(r, b, c1 * s * s), 20)
-        add("route_bwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), 12 * e, ms, "the %d-channel source, 12B/elem" % c2)
-        x = randn(N, c1, s // 2, s // 2)
         e_up = N * c1 * s * s
-        ms = timer.time(lambda i: ops.upsample_forward_into(x, r, 0, 2, 1.0), 20)
+        rot = rotation_for(5 * e_up)      # the smallest of the three launches sets the number of buffer sets
+        bs = [randn(N, c2, s, s) for _ in range(rot)]
+        rs = [torch.empty((N, c1 + c2, s, s), device=dev) for _ in range(rot)]
+        ms = timer.time(lambda i: ops.route_forward(bs[i], rs[i], c1 * s * s), 20, rotate=rot)
+        add("route_fwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), 8 * e, ms, "the %d-channel source, 8B/elem" % c2)
+        ms = timer.time(lambda i: ops.route_backward(rs[i], bs[i], c1 * s * s), 20, rotate=rot)
+        add("route_bwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), 12 * e, ms, "the %d-channel source, 12B/elem" % c2)
+        xs = [randn(N, c1, s // 2, s // 2) for _ in range(rot)]
+        ms = timer.time(lambda i: ops.upsample_forward_into(xs[i], rs[i], 0, 2, 1.0), 20, rotate=rot)
         add("upsample_fwd(into route)", "%dx%dx%d^2" % (N, c1, s // 2), 5 * e_up, ms, "same bytes as upsample_fwd; "
             "not in ms/batch twice")
-        del b, r, x
+        del bs, rs, xs
     # ---- max-pool 2x2 s2 forward + backward (config 2)
     for c, s in wl.YOLOV3_MAXPOOL_SHAPES:
         e_in = N * c * s * s
