@@ -94,3 +94,15 @@ def test_ops_refuse_cpu_tensors():
     x = torch.zeros(1, 2, 4, 4)
     with pytest.raises(capi.PxError):
         ops.activate("leaky", x)
+
+
+def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
+    """Nothing computes on the CPU in place of the kernels: without the built library every entry
+    point of the binding raises, naming the file and how to build it."""
+    monkeypatch.setattr(capi, "LIB_PATH", str(tmp_path / "libpixienn_hip.so"))
+    monkeypatch.setattr(capi, "_lib", None)
+    with pytest.raises(capi.PxError) as e:
+        capi.load()
+    assert "not built" in str(e.value) and "pixienn_amd.build" in str(e.value)
+    with pytest.raises(capi.PxError):
+        capi.call("pxh_abi_version")
