@@ -313,20 +313,32 @@ __global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, s
     for (size_t base = static_cast<size_t>(blockIdx.x) * per_step; base < n_vec;
          base += static_cast<size_t>(gridDim.x) * per_step) {
         Pack<V> v[kNormLoads];
-#pragma unroll
-        for (int u = 0; u < kNormLoads; ++u) {
-            const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
-            if (e < n_vec) v[u] = ld<V, NT>(x, e);
-        }
         float a = 0.0f;
+        // a whole step has no branch between its loads (behind one each load is waited for before the
+        // next goes out); only the last step of the tensor tests every vector
+        if (base + per_step <= n_vec) {
 #pragma unroll
-        for (int u = 0; u < kNormLoads; ++u) {
-            const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
-            if (e < n_vec) {
+            for (int u = 0; u < kNormLoads; ++u)
+                v[u] = ld<V, NT>(x, base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V);
+#pragma unroll
+            for (int u = 0; u < kNormLoads; ++u) {
 #pragma unroll
                 for (int k = 0; k < V; ++k) {
                     a += v[u].v[k] * v[u].v[k];
                     peak = fmaxf(peak, fabsf(v[u].v[k]));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < kNormLoads; ++u) {
+                const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
+                if (e < n_vec) {
+                    v[u] = ld<V, NT>(x, e);
+#pragma unroll
+                    for (int k = 0; k < V; ++k) {
+                        a += v[u].v[k] * v[u].v[k];
+                        peak = fmaxf(peak, fabsf(v[u].v[k]));
+                    }
                 }
             }
         }
@@ -406,22 +418,32 @@ __global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n
     for (size_t base = static_cast<size_t>(blockIdx.x) * per_step; base < n_vec;
          base += static_cast<size_t>(gridDim.x) * per_step) {
         Pack<V> v[kNormLoads];
+        const auto rewrite = [&](Pack<V>& p) {
 #pragma unroll
-        for (int u = 0; u < kNormLoads; ++u) {
-            const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
-            if (e < n_vec) v[u] = ld<V, NT>(x, e);
-        }
+            for (int k = 0; k < V; ++k) {
+                float t = factor == 1.0f ? p.v[k] : factor * p.v[k];
+                if (clip > 0.0f) t = fminf(clip, fmaxf(-clip, t));
+                p.v[k] = t;
+            }
+        };
+        if (base + per_step <= n_vec) {      // a whole step: no branch between its loads
 #pragma unroll
-        for (int u = 0; u < kNormLoads; ++u) {
-            const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
-            if (e < n_vec) {
+            for (int u = 0; u < kNormLoads; ++u)
+                v[u] = ld<V, NT>(x, base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V);
 #pragma unroll
-                for (int k = 0; k < V; ++k) {
-                    float t = factor == 1.0f ? v[u].v[k] : factor * v[u].v[k];
-                    if (clip > 0.0f) t = fminf(clip, fmaxf(-clip, t));
-                    v[u].v[k] = t;
+            for (int u = 0; u < kNormLoads; ++u) {
+                rewrite(v[u]);
+                st<V, NT>(x, base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V, v[u]);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < kNormLoads; ++u) {
+                const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
+                if (e < n_vec) {
+                    v[u] = ld<V, NT>(x, e);
+                    rewrite(v[u]);
+                    st<V, NT>(x, e, v[u]);
                 }
-                st<V, NT>(x, e, v[u]);
             }
         }
     }

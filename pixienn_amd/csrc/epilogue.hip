@@ -699,22 +699,41 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_fwd_kernel(Resid
     const float rm_in = a.rolling_mean[c], rv_in = a.rolling_var[c], scale_in = a.scale[c], bias_in = a.bias[c];
     Pack<V> v[R];
     float a1 = 0.0f, a2 = 0.0f;
-    // the LDS part first: its registers are free again before the register part is loaded
+    // No branch around a load: a lane past the end of the slice reads the slice's first vector and
+    // adds nothing, so that the loads of a lane are in flight together (behind a branch each one is
+    // waited for before the next is issued, and a wave then has one kilobyte on its way at a time).
+    const auto element = [&](int r) { return static_cast<uint32_t>(r * kResidentThreads + threadIdx.x) * V; };
+    const auto fetch = [&](int r) {
+        const uint32_t e = element(r);
+        return ld<V, false>(a.x, a.g.at(c, e < a.g.per_channel ? e : 0u));
+    };
+    const auto add = [&](int r, const Pack<V>& t) {
+        const bool valid = element(r) < a.g.per_channel;
 #pragma unroll
-    for (int r = R + L - 1; r >= 0; --r) {
-        const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
-        if (e < a.g.per_channel) {
-            const Pack<V> t = ld<V, false>(a.x, a.g.at(c, e));
-#pragma unroll
-            for (int k = 0; k < V; ++k) {
-                const float d = t.v[k] - shift;
-                a1 += d;
-                a2 += d * d;
-            }
-            if (r < R) v[r < R ? r : 0] = t;
-            else *resident_lds_slot<V, R>(resident_lds, r) = t;
+        for (int k = 0; k < V; ++k) {
+            const float d = t.v[k] - shift;
+            a1 += valid ? d : 0.0f;
+            a2 += valid ? d * d : 0.0f;
         }
+    };
+    // the LDS part first, all of it at once: its registers are free again before the register part
+    // is loaded, which lands where it stays
+    if constexpr (L > 0) {
+        Pack<V> stage[L];
+#pragma unroll
+        for (int r = R + L - 1; r >= R; --r) stage[r - R] = fetch(r);
+#pragma unroll
+        for (int r = R + L - 1; r >= R; --r) {
+            add(r, stage[r - R]);
+            *resident_lds_slot<V, R>(resident_lds, r) = stage[r - R];
+        }
+        // the sums as they stand, before the registers are handed to the second part
+        asm volatile("" : "+v"(a1), "+v"(a2));
     }
+#pragma unroll
+    for (int r = R - 1; r >= 0; --r) v[r] = fetch(r);
+#pragma unroll
+    for (int r = R - 1; r >= 0; --r) add(r, v[r]);
     double s1 = static_cast<double>(a1), s2 = static_cast<double>(a2);
     resident_sum2(s1, s2, slots);
     if (threadIdx.x == 0) {
@@ -770,32 +789,101 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
     const bool recompute = a.b.pre == nullptr;
     Pack<V> d[R];
     float fa = 0.0f, fb = 0.0f;
-#pragma unroll
-    for (int r = R + L - 1; r >= 0; --r) {
-        const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
-        if (e < a.g.per_channel) {
-            const size_t where = a.g.at(c, e);
-            Pack<V> dv = ld<V, false>(a.b.delta, where);
-            const Pack<V> xv = ld<V, false>(a.b.x, where);
-            Pack<V> pv;
-            if constexpr (ACT != PXH_LINEAR) {
-                if (!recompute) pv = ld<V, false>(a.b.pre, where);
-            }
+    // Two shapes of the same two passes.  The large form (part of the slice in LDS) is bound by its
+    // loads and takes them in groups with no branch in between; the small form does more arithmetic
+    // per byte than it waits, and is fastest when a step past the end of the slice is skipped outright.
+    // The large form: no branch around the loads (see the forward kernel), lanes past the end read the
+    // first vector; kGroup steps at a time, their loads go out together, then each is used as it arrives.
+    constexpr int kGroup = 4;
+    static_assert(L == 0 || (R % kGroup == 0 && L % kGroup == 0), "steps come in whole groups");
+    // `lane` is the thread index; the second pass takes it through an empty asm statement, so that
+    // its addresses are formed again there instead of being held in registers (48 of them) from the first
+    [[maybe_unused]] uint32_t lane = threadIdx.x;
+    [[maybe_unused]] const auto element = [&](int r) { return (static_cast<uint32_t>(r * kResidentThreads) + lane) * V; };
+    [[maybe_unused]] const auto place = [&](int r) {
+        const uint32_t e = element(r);
+        return a.g.at(c, e < a.g.per_channel ? e : 0u);
+    };
+    if constexpr (L > 0) {
+        // delta * f'(pre) in dv, and the step's share of the two sums
+        const auto take = [&](int r, Pack<V>& dv, const Pack<V>& xv, const Pack<V>& pv) {
+            const bool valid = element(r) < a.g.per_channel;
 #pragma unroll
             for (int q = 0; q < V; ++q) {
                 float t = dv.v[q];
                 if constexpr (ACT != PXH_LINEAR) {
-                    float pre;
-                    if (recompute) pre = affine(normalize(xv.v[q], k), k);
-                    else pre = pv.v[q];
-                    t = t * act_grad<ACT>(pre);
+                    t = t * act_grad<ACT>(pv.v[q]);
                     dv.v[q] = t;
                 }
-                fa += t;
-                fb += t * (xv.v[q] - k.mean);
+                fa += valid ? t : 0.0f;
+                fb += valid ? t * (xv.v[q] - k.mean) : 0.0f;
             }
-            if (r < R) d[r < R ? r : 0] = dv;
-            else *resident_lds_slot<V, R>(resident_lds, r) = dv;
+        };
+#pragma unroll
+        for (int top = R + L - 1; top >= 0; top -= kGroup) {
+            Pack<V> dv[kGroup], xv[kGroup], pv[kGroup];
+            size_t where[kGroup];
+#pragma unroll
+            for (int i = 0; i < kGroup; ++i) {
+                where[i] = place(top - i);
+                dv[i] = ld<V, false>(a.b.delta, where[i]);
+                xv[i] = ld<V, false>(a.b.x, where[i]);
+            }
+            // the pre-activation: the saved one, or formed again from x (one decision per group)
+            if constexpr (ACT != PXH_LINEAR) {
+                if (!recompute) {
+#pragma unroll
+                    for (int i = 0; i < kGroup; ++i) pv[i] = ld<V, false>(a.b.pre, where[i]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < kGroup; ++i) {
+#pragma unroll
+                        for (int q = 0; q < V; ++q) pv[i].v[q] = affine(normalize(xv[i].v[q], k), k);
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kGroup; ++i) {
+                const int r = top - i;
+                take(r, dv[i], xv[i], pv[i]);
+                if (r < R) d[r < R ? r : 0] = dv[i];
+                else *resident_lds_slot<V, R>(resident_lds, r) = dv[i];
+            }
+            // The group ends here for the compiler too: the sums are taken as they stand (otherwise it
+            // puts the additions off to the end of the pass and keeps every group's values until then),
+            // and the next group's loads stay behind this one's arithmetic -- either would need more
+            // registers than a lane has.
+            asm volatile("" : "+v"(fa), "+v"(fb));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+#pragma unroll
+        for (int r = R + L - 1; r >= 0; --r) {
+            const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+            if (e < a.g.per_channel) {
+                const size_t where = a.g.at(c, e);
+                Pack<V> dv = ld<V, false>(a.b.delta, where);
+                const Pack<V> xv = ld<V, false>(a.b.x, where);
+                Pack<V> pv;
+                if constexpr (ACT != PXH_LINEAR) {
+                    if (!recompute) pv = ld<V, false>(a.b.pre, where);
+                }
+#pragma unroll
+                for (int q = 0; q < V; ++q) {
+                    float t = dv.v[q];
+                    if constexpr (ACT != PXH_LINEAR) {
+                        float pre;
+                        if (recompute) pre = affine(normalize(xv.v[q], k), k);
+                        else pre = pv.v[q];
+                        t = t * act_grad<ACT>(pre);
+                        dv.v[q] = t;
+                    }
+                    fa += t;
+                    fb += t * (xv.v[q] - k.mean);
+                }
+                if (r < R) d[r < R ? r : 0] = dv;
+                else *resident_lds_slot<V, R>(resident_lds, r) = dv;
+            }
         }
     }
     double sa = static_cast<double>(fa), sb = static_cast<double>(fb);
@@ -805,21 +893,40 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
                                             a.b.bias, a.scale_updates, a.bias_updates, a.mean_delta, a.var_delta);
     __syncthreads();
     const DxCoef kd = shared_coef;
+    if constexpr (L > 0) {
+        asm volatile("" : "+v"(lane));
 #pragma unroll
-    for (int r = 0; r < R + L; ++r) {
-        const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
-        if (e < a.g.per_channel) {
-            const size_t where = a.g.at(c, e);
-            const Pack<V> xv = ld<V, false>(a.b.x, where);
-            const Pack<V> dv = r < R ? d[r < R ? r : 0] : *resident_lds_slot<V, R>(resident_lds, r);
-            Pack<V> out;
+        for (int first = 0; first < R + L; first += kGroup) {
+            Pack<V> xv[kGroup];
 #pragma unroll
-            for (int q = 0; q < V; ++q) out.v[q] = dx_value<PXH_LINEAR>(dv.v[q], xv.v[q], 0.0f, false, kd);
-            st<V, false>(a.b.delta, where, out);
+            for (int i = 0; i < kGroup; ++i) xv[i] = ld<V, false>(a.b.x, place(first + i));
+#pragma unroll
+            for (int i = 0; i < kGroup; ++i) {
+                const int r = first + i;
+                const Pack<V> dv = r < R ? d[r < R ? r : 0] : *resident_lds_slot<V, R>(resident_lds, r);
+                Pack<V> out;
+#pragma unroll
+                for (int q = 0; q < V; ++q) out.v[q] = dx_value<PXH_LINEAR>(dv.v[q], xv[i].v[q], 0.0f, false, kd);
+                if (element(r) < a.g.per_channel) st<V, false>(a.b.delta, place(r), out);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R + L; ++r) {
+            const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+            if (e < a.g.per_channel) {
+                const size_t where = a.g.at(c, e);
+                const Pack<V> xv = ld<V, false>(a.b.x, where);
+                const Pack<V> dv = r < R ? d[r < R ? r : 0] : *resident_lds_slot<V, R>(resident_lds, r);
+                Pack<V> out;
+#pragma unroll
+                for (int q = 0; q < V; ++q) out.v[q] = dx_value<PXH_LINEAR>(dv.v[q], xv.v[q], 0.0f, false, kd);
+                st<V, false>(a.b.delta, where, out);
+            }
         }
     }
 }
-
 // Vectors per thread the resident kernels are built for, and whether a shape takes that path:
 // the channel slice must fit, and there must be enough channels to occupy the machine.  (Measured
 // with 24 vectors per thread: the registers spill and 128 workgroups of 16x128x76^2 are slower than
