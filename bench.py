@@ -456,10 +456,20 @@ def measure_extras(torch, ops, wl, timer, capi):
         su = torch.zeros(c, device=dev); bu = torch.zeros(c, device=dev)
         ms_f = timer.time(lambda i: ops.bn_train_act_forward(x[i], y[i], mean, var, rmean, rvar, scale, bias, "leaky"),
                           10, rotate=rot)
-        add("bn_train_fwd(leaky)", "%dx%dx%d^2" % (N, c, s), 12 * e, ms_f, "stats 4B + apply 8B per elem; x kept")
+        # shapes whose channel slice fits one workgroup (and with 96 channels or more) run as ONE launch that
+        # reads x once: the same 12 / 20 B per element are charged, so that rows compare, and the note says so
+        vec = (s * s) % 4 == 0
+        vectors = -(-N * s * s // (4 if vec else 1))
+        per_thread = -(-vectors // 1024)
+        one_launch = c >= 96 and (per_thread <= 8 or (vec and per_thread <= 24))
+        add("bn_train_fwd(leaky)", "%dx%dx%d^2" % (N, c, s), 12 * e, ms_f,
+            "one launch, moves 8B per elem; priced as stats 4B + apply 8B" if one_launch
+            else "stats 4B + apply 8B per elem; x kept")
         ms_b = timer.time(lambda i: ops.bn_act_backward(d[i], x[i], mean, var, scale, bias, su, bu, "leaky"),
                           10, rotate=rot)
-        add("bn_bwd(leaky)", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_b, "sums 8B + dx 12B per elem; pre recomputed")
+        add("bn_bwd(leaky)", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_b,
+            "one launch, moves 16B per elem; priced as sums 8B + dx 12B" if one_launch
+            else "sums 8B + dx 12B per elem; pre recomputed")
         bn_ms[(c, s)] = (ms_f, ms_b, count)
         del x, y, d
     # ---- linear bias epilogue of the three head convs at batch 16
