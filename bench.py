@@ -457,18 +457,19 @@ def measure_extras(torch, ops, wl, timer, capi):
         ms_f = timer.time(lambda i: ops.bn_train_act_forward(x[i], y[i], mean, var, rmean, rvar, scale, bias, "leaky"),
                           10, rotate=rot)
         # shapes whose channel slice fits one workgroup (and with 96 channels or more) run as ONE launch that
-        # reads x once: the same 12 / 20 B per element are charged, so that rows compare, and the note says so
+        # reads x once: their rows count the bytes that launch moves (8 / 16 B per element), not the 12 / 20 of
+        # the three-launch form
         vec = (s * s) % 4 == 0
         vectors = -(-N * s * s // (4 if vec else 1))
         per_thread = -(-vectors // 1024)
         one_launch = c >= 96 and (per_thread <= 8 or (vec and per_thread <= 24))
-        add("bn_train_fwd(leaky)", "%dx%dx%d^2" % (N, c, s), 12 * e, ms_f,
-            "one launch, moves 8B per elem; priced as stats 4B + apply 8B" if one_launch
+        add("bn_train_fwd(leaky)", "%dx%dx%d^2" % (N, c, s), (8 if one_launch else 12) * e, ms_f,
+            "one launch: x read once, 8B per elem (three launches move 12)" if one_launch
             else "stats 4B + apply 8B per elem; x kept")
         ms_b = timer.time(lambda i: ops.bn_act_backward(d[i], x[i], mean, var, scale, bias, su, bu, "leaky"),
                           10, rotate=rot)
-        add("bn_bwd(leaky)", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_b,
-            "one launch, moves 16B per elem; priced as sums 8B + dx 12B" if one_launch
+        add("bn_bwd(leaky)", "%dx%dx%d^2" % (N, c, s), (16 if one_launch else 20) * e, ms_b,
+            "one launch: delta once, x twice, 16B per elem (three launches move 20)" if one_launch
             else "sums 8B + dx 12B per elem; pre recomputed")
         bn_ms[(c, s)] = (ms_f, ms_b, count)
         del x, y, d

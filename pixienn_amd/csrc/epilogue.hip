@@ -699,13 +699,16 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_fwd_kernel(Resid
     const float rm_in = a.rolling_mean[c], rv_in = a.rolling_var[c], scale_in = a.scale[c], bias_in = a.bias[c];
     Pack<V> v[R];
     float a1 = 0.0f, a2 = 0.0f;
+    // Every tensor here is touched once and goes past the caches (non-temporal: with the whole slice
+    // of every channel asked for at once, cached reads run at two thirds of the rate; the backward
+    // kernel keeps x cached, which it reads twice).
     // No branch around a load: a lane past the end of the slice reads the slice's first vector and
     // adds nothing, so that the loads of a lane are in flight together (behind a branch each one is
     // waited for before the next is issued, and a wave then has one kilobyte on its way at a time).
     const auto element = [&](int r) { return static_cast<uint32_t>(r * kResidentThreads + threadIdx.x) * V; };
     const auto fetch = [&](int r) {
         const uint32_t e = element(r);
-        return ld<V, false>(a.x, a.g.at(c, e < a.g.per_channel ? e : 0u));
+        return ld<V, true>(a.x, a.g.at(c, e < a.g.per_channel ? e : 0u));
     };
     const auto add = [&](int r, const Pack<V>& t) {
         const bool valid = element(r) < a.g.per_channel;
@@ -759,10 +762,10 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_fwd_kernel(Resid
                 pre.v[q] = affine(xn.v[q], k);
                 out.v[q] = act_apply<ACT>(pre.v[q]);
             }
-            if (a.x_saved) st<V, false>(a.x_saved, where, t);
-            if (a.x_norm) st<V, false>(a.x_norm, where, xn);
-            if (a.pre) st<V, false>(a.pre, where, pre);
-            st<V, false>(a.y, where, out);
+            if (a.x_saved) st<V, true>(a.x_saved, where, t);
+            if (a.x_norm) st<V, true>(a.x_norm, where, xn);
+            if (a.pre) st<V, true>(a.pre, where, pre);
+            st<V, true>(a.y, where, out);
         }
     }
 }
@@ -826,14 +829,14 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
 #pragma unroll
             for (int i = 0; i < kGroup; ++i) {
                 where[i] = place(top - i);
-                dv[i] = ld<V, false>(a.b.delta, where[i]);
+                dv[i] = ld<V, true>(a.b.delta, where[i]);
                 xv[i] = ld<V, false>(a.b.x, where[i]);
             }
             // the pre-activation: the saved one, or formed again from x (one decision per group)
             if constexpr (ACT != PXH_LINEAR) {
                 if (!recompute) {
 #pragma unroll
-                    for (int i = 0; i < kGroup; ++i) pv[i] = ld<V, false>(a.b.pre, where[i]);
+                    for (int i = 0; i < kGroup; ++i) pv[i] = ld<V, true>(a.b.pre, where[i]);
                 } else {
 #pragma unroll
                     for (int i = 0; i < kGroup; ++i) {
@@ -862,11 +865,11 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
             const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
             if (e < a.g.per_channel) {
                 const size_t where = a.g.at(c, e);
-                Pack<V> dv = ld<V, false>(a.b.delta, where);
+                Pack<V> dv = ld<V, true>(a.b.delta, where);
                 const Pack<V> xv = ld<V, false>(a.b.x, where);
                 Pack<V> pv;
                 if constexpr (ACT != PXH_LINEAR) {
-                    if (!recompute) pv = ld<V, false>(a.b.pre, where);
+                    if (!recompute) pv = ld<V, true>(a.b.pre, where);
                 }
 #pragma unroll
                 for (int q = 0; q < V; ++q) {
@@ -907,7 +910,7 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
                 Pack<V> out;
 #pragma unroll
                 for (int q = 0; q < V; ++q) out.v[q] = dx_value<PXH_LINEAR>(dv.v[q], xv[i].v[q], 0.0f, false, kd);
-                if (element(r) < a.g.per_channel) st<V, false>(a.b.delta, place(r), out);
+                if (element(r) < a.g.per_channel) st<V, true>(a.b.delta, place(r), out);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -922,7 +925,7 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
                 Pack<V> out;
 #pragma unroll
                 for (int q = 0; q < V; ++q) out.v[q] = dx_value<PXH_LINEAR>(dv.v[q], xv.v[q], 0.0f, false, kd);
-                st<V, false>(a.b.delta, where, out);
+                st<V, true>(a.b.delta, where, out);
             }
         }
     }

@@ -121,12 +121,14 @@ __global__ __launch_bounds__(kWave) void stream_tail_kernel(size_t begin, size_t
 }
 
 // Launches op over n elements.  `vector_ok`: every pointer the op touches is 16-byte aligned.
-// `bytes_per_elem`: bytes the op moves per element, which picks the non-temporal variant.
+// `bytes_per_elem`: bytes the op moves per element, which picks the non-temporal variant from
+// `streaming_from` bytes per launch on.
 template<typename Op>
-int launch_stream(const char* name, size_t n, bool vector_ok, int bytes_per_elem, const Op& op, hipStream_t stream)
+int launch_stream(const char* name, size_t n, bool vector_ok, int bytes_per_elem, const Op& op, hipStream_t stream,
+                  size_t streaming_from = kStreamingBytes)
 {
     if (n == 0) return PXH_OK;
-    const bool nt = n * static_cast<size_t>(bytes_per_elem) >= kStreamingBytes;
+    const bool nt = n * static_cast<size_t>(bytes_per_elem) >= streaming_from;
     if (vector_ok) {
         const size_t n4 = n & ~static_cast<size_t>(3);
         if (n4) {
