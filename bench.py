@@ -168,7 +168,8 @@ def measure_model_order(torch, ops, wl, timer, N=16):
     model's own layer order on tensors of their own (21 GB): forward (per layer the delta zero-fill
     of Layer::forward, then the layer), backward in reverse (per layer the gradient rescale + clip
     of Layer::backward with the thresholds of yolov3.yml, 100 and 10, then the layer), update (the
-    same helpers once more per layer and on the update buffer, then Adam on the flat parameters).
+    same helpers once more per layer and on each of the 222 update buffers, then Adam on the 222
+    parameter tensors, both through the entry points that take many tensors per launch).
     The convolutions' GEMMs are not run: a conv layer reads a resident conv result and its input
     gradient goes nowhere.  Each phase is timed as one HIP graph."""
     dev = torch.device("cuda")
@@ -190,9 +191,17 @@ def measure_model_order(torch, ops, wl, timer, N=16):
         T.append(t)
     truths_np, counts_np = wl.yolo_truths(5100, N)
     truths = torch.from_numpy(truths_np).to(dev); counts = torch.from_numpy(counts_np).to(dev)
-    P = wl.YOLOV3_PARAMS
-    w = 0.02 * torch.randn(P, device=dev); g = 1e-3 * torch.randn(P, device=dev)
-    m = torch.zeros(P, device=dev); v = torch.zeros(P, device=dev)
+    # the parameters as the engine holds them: 222 tensors (weights, biases, scales per convolution), here as
+    # 256-byte aligned views into one buffer per kind
+    sizes = wl.yolov3_parameter_tensors(608)
+    starts, at = [], 0
+    for n_, _ in sizes:
+        starts.append(at); at += (n_ + 63) // 64 * 64
+    w = 0.02 * torch.randn(at, device=dev); g = 1e-3 * torch.randn(at, device=dev)
+    m = torch.zeros(at, device=dev); v = torch.zeros(at, device=dev)
+    views = lambda flat: [flat[o:o + n_] for o, (n_, _) in zip(starts, sizes)]
+    pw, pg, pm, pv = views(w), views(g), views(m), views(v)
+    decayed = [d_ for _, d_ in sizes]
     launches = dict(forward=0, backward=0, update=0)
 
     def absorbed(i):            # an upsample writes into (and reads its delta from) the route that follows
@@ -266,8 +275,9 @@ def measure_model_order(torch, ops, wl, timer, N=16):
             for i, t in enumerate(T):
                 if not absorbed(i):
                     ops.rescale_clip(t["d"], 100.0, 10.0); n += 1
-        ops.rescale_clip(g, 100.0, 10.0)
-        ops.adam_update(w, g, m, v, N, 1, 1e-3, decay=5e-4, apply_decay=True)
+        # the hooks on every update buffer, each with its own norm, then Adam: every tensor in a few launches
+        ops.rescale_clip_multi(pg, 100.0, 10.0)
+        ops.adam_update_multi(pw, pg, pm, pv, N, 1, 1e-3, decay=5e-4, apply_decay=decayed)
         launches["update"] = n + 2
 
     out = {}
@@ -504,7 +514,38 @@ def measure_extras(torch, ops, wl, timer, capi):
     # ---- SGD with momentum over the same buffer (the optimiser of the shipped presets)
     ms_sgd = timer.time(lambda i: ops.sgd_update(w, d, 16, 1e-3, 0.9, 5e-4, True), 10)
     add("sgd_update", "%d params" % P, 16 * P, ms_sgd, "16B/param; not in ms/batch (Adam is)")
-    del w, g, m, v, d
+    # ---- the same parameters as the engine holds them: 222 tensors (three per convolution), updated through
+    # the entry points that take many tensors per launch, and one call per tensor beside it
+    sizes = wl.yolov3_parameter_tensors(608)
+    starts, at = [], 0
+    for n_, _ in sizes:
+        starts.append(at); at += (n_ + 63) // 64 * 64
+    assert at <= w.numel() + 64 * len(sizes)
+    big = [torch.zeros(at, device=dev) for _ in range(4)]
+    big[0].normal_(0, 0.02); big[1].normal_(0, 1e-3)
+    pw, pd, pm, pv = ([flat[o:o + n_] for o, (n_, _) in zip(starts, sizes)] for flat in big)
+    decayed = [d_ for _, d_ in sizes]
+    ms = timer.time(lambda i: ops.adam_update_multi(pw, pd, pm, pv, 16, 1, 1e-3, 0.9, 0.999, 1e-8, 5e-4, decayed), 10)
+    add("adam_update_multi", "%d tensors, %d params" % (len(sizes), P), 32 * P, ms, "7 launches; gradients already zero after the first")
+
+    def one_by_one(i):
+        for k in range(len(sizes)):
+            ops.adam_update(pw[k], pd[k], pm[k], pv[k], 16, 1, 1e-3, 0.9, 0.999, 1e-8, 5e-4, decayed[k])
+
+    ms = timer.time(one_by_one, 3)
+    add("adam_update x222", "%d tensors, %d params" % (len(sizes), P), 32 * P, ms, "one call per tensor, for comparison")
+    ms = timer.time(lambda i: ops.sgd_update_multi(pw, pd, 16, 1e-3, 0.9, 5e-4, decayed), 10)
+    add("sgd_update_multi", "%d tensors, %d params" % (len(sizes), P), 16 * P, ms, "7 launches")
+    ms = timer.time(lambda i: ops.rescale_clip_multi(pd, 100.0, 10.0), 10)
+    add("rescale_clip_multi(no-op)", "%d update buffers" % len(sizes), 4 * P, ms, "14 launches; norm only, 4B/param")
+
+    def hooks_one_by_one(i):
+        for k in range(len(sizes)):
+            ops.rescale_clip(pd[k], 100.0, 10.0)
+
+    ms = timer.time(hooks_one_by_one, 3)
+    add("rescale_clip x222(no-op)", "%d update buffers" % len(sizes), 4 * P, ms, "one call (two launches) per buffer, for comparison")
+    del w, g, m, v, d, big, pw, pd, pm, pv
     # ---- gradient rescale + clamp of a delta tensor: 4B/elem for the norm, 8B/elem to rewrite
     for c, s_ in [(256, 76), (64, 304)]:
         e = N * c * s_ * s_

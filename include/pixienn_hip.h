@@ -324,6 +324,12 @@ int pxh_yolo_forward_train(const float* input, float* output, float* delta, cons
 int pxh_sgd_update(size_t n, float* w, float* d, int batch, float lr, float momentum, float decay,
                    int apply_decay, void* stream);
 
+/* ... and for every parameter tensor of a model at once, as pxh_adam_update_multi does for Adam
+ * (SGD is the optimiser of every shipped preset). */
+int pxh_sgd_update_multi(int count, float* const* w, float* const* d, const size_t* n,
+                         const int* apply_decay, int batch, float lr, float momentum, float decay,
+                         void* stream);
+
 /* ------------------------------------------------------------------------
  * Gradient rescale and clip, the two helpers Layer::backward runs on delta before a layer's own
  * backward (include/Layer.h:385-397, 479-499; include/cuda/Layer.h:24-39: cublasSnrm2 +
@@ -338,6 +344,16 @@ size_t pxh_rescale_workspace_bytes(void);
 int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* norm_out,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same for many tensors in a few launches: Layer::update's hooks pass every update buffer of
+ * every layer through these helpers (include/Layer.h:400-411, ConvLayer.h:323-340: weights, biases,
+ * scales), each with its own norm.  x and n are HOST arrays of `count` device pointers / element
+ * counts; norms, if not NULL, is a DEVICE array of `count` floats that receives each tensor's norm
+ * (an empty tensor's entry is left alone).  Every tensor ends up exactly as pxh_rescale_clip leaves
+ * it.  Workspace: pxh_rescale_multi_workspace_bytes(), or NULL for the library's. */
+size_t pxh_rescale_multi_workspace_bytes(void);
+int pxh_rescale_clip_multi(int count, float* const* x, const size_t* n, float threshold, float clip,
+                           float* norms, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------
  * Adam.  include/Adam.cuh:21, include/cuda/Adam.h:49-90.
  * ---------------------------------------------------------------------- */
@@ -351,6 +367,15 @@ int pxh_adam(int n, float* x, const float* m, const float* v, float beta1, float
  * (L2 decay folded into the update before the moments, as the reference does; not decoupled.) */
 int pxh_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch, int t, float lr,
                     float beta1, float beta2, float eps, float decay, int apply_decay, void* stream);
+
+/* The same for every parameter tensor of a model in as few launches as possible (the engine updates
+ * its layers one by one, cuda/ConvLayer.h:370-386: three tensors per convolution, most of them a few
+ * hundred values).  w, d, m, v and n are HOST arrays of `count` device pointers / element counts;
+ * apply_decay is a host array of flags (weights: 1, biases and scales: 0) or NULL for none.  Each
+ * element gets exactly what pxh_adam_update gives it.  Tensors of length 0 are skipped. */
+int pxh_adam_update_multi(int count, float* const* w, float* const* d, float* const* m,
+                          float* const* v, const size_t* n, const int* apply_decay, int batch, int t,
+                          float lr, float beta1, float beta2, float eps, float decay, void* stream);
 
 #ifdef __cplusplus
 }

@@ -61,6 +61,9 @@ SIGNATURES = {
     "pxh_debug_nms_sweeps": [I],
     "pxh_adam": [I, P, P, P, F, F, F, F, I, P],
     "pxh_adam_update": [Z, P, P, P, P, I, I, F, F, F, F, F, I, P],
+    "pxh_adam_update_multi": [I, P, P, P, P, P, P, I, I, F, F, F, F, F, P],
+    "pxh_rescale_clip_multi": [I, P, P, F, F, P, P, Z, P],
+    "pxh_sgd_update_multi": [I, P, P, P, P, I, F, F, F, P],
 }
 _OTHER_RETURNS = {
     "pxh_last_error": (ctypes.c_char_p, []),
@@ -68,6 +71,7 @@ _OTHER_RETURNS = {
     "pxh_bn_workspace_bytes": (Z, [I, I, I]),
     "pxh_bn_folded_bytes": (Z, [I]),
     "pxh_rescale_workspace_bytes": (Z, []),
+    "pxh_rescale_multi_workspace_bytes": (Z, []),
     "pxh_yolo_workspace_bytes": (Z, [I, I, I, I, I, I]),
     "pxh_nms_workspace_bytes": (Z, [I]),
     "pxh_debug_fastdiv": (ctypes.c_uint, [ctypes.c_uint, ctypes.c_uint]),

@@ -307,16 +307,17 @@ constexpr int kNormBlocks = 1024;     // 4 per compute unit; every workgroup of 
 constexpr int kNormLoads = 8;         // 128-bit loads in flight per lane
 
 // Per workgroup: the sum of squares and the largest magnitude (NaN-free; a NaN shows in the sum).
+// (workgroup `block` of `blocks` that share the tensor; the result goes to *out)
 template<int V, bool NT>
-__global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, size_t n_vec, double2* partial)
+__device__ __forceinline__ void sumsq_walk(const float* x, size_t n_vec, uint32_t block, uint32_t blocks, double2* out)
 {
     __shared__ double slots[kBlock / kWave];
     __shared__ float peaks[kBlock / kWave];
     const size_t per_step = static_cast<size_t>(kBlock) * V * kNormLoads;
     double s = 0.0;
     float peak = 0.0f;
-    for (size_t base = static_cast<size_t>(blockIdx.x) * per_step; base < n_vec;
-         base += static_cast<size_t>(gridDim.x) * per_step) {
+    for (size_t base = static_cast<size_t>(block) * per_step; base < n_vec;
+         base += static_cast<size_t>(blocks) * per_step) {
         Pack<V> v[kNormLoads];
         float a = 0.0f;
         // a whole step has no branch between its loads (behind one each load is waited for before the
@@ -357,8 +358,14 @@ __global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, s
         float top = peaks[0];
 #pragma unroll
         for (int w = 1; w < kBlock / kWave; ++w) top = fmaxf(top, peaks[w]);
-        partial[blockIdx.x] = make_double2(total, static_cast<double>(top));
+        *out = make_double2(total, static_cast<double>(top));
     }
+}
+
+template<int V, bool NT>
+__global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, size_t n_vec, double2* partial)
+{
+    sumsq_walk<V, NT>(x, n_vec, blockIdx.x, gridDim.x, partial + blockIdx.x);
 }
 
 // The plan of the rewrite, formed by every workgroup for itself from the same partials in the same
@@ -411,17 +418,17 @@ __device__ __forceinline__ RescalePlan rescale_plan(const double2* partial, int 
 // x = clamp(factor * x); leaves without touching the tensor when there is nothing to do.  The grid
 // is the reduction's capped one and strides over the tensor.
 template<int V, bool NT>
-__global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n_vec, const double2* partial,
-                                                              int partials, float threshold, float clip,
-                                                              float* norm_out)
+__device__ __forceinline__ void rescale_walk(float* x, size_t n_vec, const double2* partial, int partials,
+                                             uint32_t block, uint32_t blocks, float threshold, float clip,
+                                             float* norm_out)
 {
     const RescalePlan plan = rescale_plan(partial, partials, threshold, clip);
-    if (norm_out && blockIdx.x == 0 && threadIdx.x == 0) *norm_out = plan.norm;
+    if (norm_out && block == 0 && threadIdx.x == 0) *norm_out = plan.norm;
     if (!plan.work) return;
     const float factor = plan.factor;
     const size_t per_step = static_cast<size_t>(kBlock) * V * kNormLoads;
-    for (size_t base = static_cast<size_t>(blockIdx.x) * per_step; base < n_vec;
-         base += static_cast<size_t>(gridDim.x) * per_step) {
+    for (size_t base = static_cast<size_t>(block) * per_step; base < n_vec;
+         base += static_cast<size_t>(blocks) * per_step) {
         Pack<V> v[kNormLoads];
         const auto rewrite = [&](Pack<V>& p) {
 #pragma unroll
@@ -452,6 +459,65 @@ __global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n
             }
         }
     }
+}
+
+template<int V, bool NT>
+__global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n_vec, const double2* partial,
+                                                              int partials, float threshold, float clip,
+                                                              float* norm_out)
+{
+    rescale_walk<V, NT>(x, n_vec, partial, partials, blockIdx.x, gridDim.x, threshold, clip, norm_out);
+}
+
+// The same two passes over up to kRescaleTensors tensors per launch (the update hooks of a model run
+// on every layer's update buffers, three per convolution).  Every tensor gets the workgroups, the
+// walk and therefore the sums of its single call: the results are the same bit for bit.
+constexpr int kRescaleTensors = 32;
+
+struct RescaleTable {
+    float* x[kRescaleTensors];
+    unsigned long long n[kRescaleTensors];
+    uint32_t first_block[kRescaleTensors + 1];     // also the tensor's first partial
+    uint32_t vector_mask;                          // bit i: 16-byte aligned and a multiple of 4 long
+    uint32_t past_cache_mask;
+    int count;
+    float* norms;                                  // nullable: norms[first_tensor + i]
+    int first_tensor;
+};
+
+__device__ __forceinline__ int tensor_of_block(const uint32_t* first_block, int count, uint32_t block)
+{
+    int lo = 0, hi = count - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (first_block[mid] <= block) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+
+__global__ __launch_bounds__(kBlock) void multi_sumsq_kernel(RescaleTable t, double2* partial)
+{
+    const int i = tensor_of_block(t.first_block, t.count, blockIdx.x);
+    const uint32_t block = blockIdx.x - t.first_block[i], blocks = t.first_block[i + 1] - t.first_block[i];
+    double2* out = partial + blockIdx.x;
+    if (!((t.vector_mask >> i) & 1u)) sumsq_walk<1, false>(t.x[i], t.n[i], block, blocks, out);
+    else if ((t.past_cache_mask >> i) & 1u) sumsq_walk<4, true>(t.x[i], t.n[i], block, blocks, out);
+    else sumsq_walk<4, false>(t.x[i], t.n[i], block, blocks, out);
+}
+
+__global__ __launch_bounds__(kBlock) void multi_rescale_kernel(RescaleTable t, const double2* partial, float threshold,
+                                                               float clip)
+{
+    const int i = tensor_of_block(t.first_block, t.count, blockIdx.x);
+    const uint32_t block = blockIdx.x - t.first_block[i], blocks = t.first_block[i + 1] - t.first_block[i];
+    const double2* mine = partial + t.first_block[i];
+    float* norm_out = t.norms ? t.norms + t.first_tensor + i : nullptr;
+    if (!((t.vector_mask >> i) & 1u))
+        rescale_walk<1, false>(t.x[i], t.n[i], mine, static_cast<int>(blocks), block, blocks, threshold, clip, norm_out);
+    else if ((t.past_cache_mask >> i) & 1u)
+        rescale_walk<4, true>(t.x[i], t.n[i], mine, static_cast<int>(blocks), block, blocks, threshold, clip, norm_out);
+    else
+        rescale_walk<4, false>(t.x[i], t.n[i], mine, static_cast<int>(blocks), block, blocks, threshold, clip, norm_out);
 }
 
 // ---------------------------------------------------------------- Adam
@@ -502,6 +568,117 @@ struct AdamUpdateOp {
         st<V, NT>(d, e, od);
     }
 };
+
+// ---------------------------------------------------------------- many parameter tensors, few launches
+// The engine keeps every layer's weights, biases and scales in buffers of their own and updates them
+// one by one (include/cuda/ConvLayer.h:370-413): 222 tensors for YOLOv3, two thirds of them smaller
+// than one workgroup's worth.  A launch here takes up to kMultiTensors of them: the table travels by
+// value, workgroup b finds its tensor by bisection over the first workgroup of each, and runs the
+// same per-element operation on 1024 elements of it.
+constexpr int kMultiTensors = 32;
+constexpr uint32_t kMultiPerBlock = kBlock * 4;
+
+struct MultiTable {
+    float* stream[4][kMultiTensors];               // the tensor's buffers, in the operation's own order
+    unsigned long long n[kMultiTensors];
+    uint32_t first_block[kMultiTensors + 1];
+    uint32_t decay_mask;                           // bit i: tensor i takes the weight decay
+    uint32_t past_cache_mask;                      // bit i: tensor i is too large to stay cached
+    uint32_t vector_mask;                          // bit i: all buffers of tensor i are 16-byte aligned
+    int count;
+};
+
+struct AdamMaker {
+    AdamUpdateOp base;
+    __device__ AdamUpdateOp operator()(const MultiTable& t, int i) const
+    {
+        AdamUpdateOp op = base;
+        op.w = t.stream[0][i]; op.d = t.stream[1][i]; op.m = t.stream[2][i]; op.v = t.stream[3][i];
+        op.apply_decay = (t.decay_mask >> i) & 1u;
+        return op;
+    }
+};
+
+struct SgdMaker {
+    SgdUpdateOp base;
+    __device__ SgdUpdateOp operator()(const MultiTable& t, int i) const
+    {
+        SgdUpdateOp op = base;
+        op.w = t.stream[0][i]; op.d = t.stream[1][i];
+        op.apply_decay = (t.decay_mask >> i) & 1u;
+        return op;
+    }
+};
+
+template<typename Maker>
+__global__ __launch_bounds__(kBlock) void multi_tensor_kernel(MultiTable t, Maker make)
+{
+    const int lo = tensor_of_block(t.first_block, t.count, blockIdx.x);
+    const auto op = make(t, lo);
+    const size_t n = t.n[lo];
+    const size_t e = (static_cast<size_t>(blockIdx.x - t.first_block[lo]) * kBlock + threadIdx.x) * 4;
+    if (e >= n) return;
+    using Op = decltype(make(t, 0));
+    if (((t.vector_mask >> lo) & 1u) && e + 4 <= n) {
+        typename Op::template Regs<4> r;
+        if ((t.past_cache_mask >> lo) & 1u) {
+            op.template load<4, true>(e, r);
+            op.template finish<4, true>(e, r);
+        } else {
+            op.template load<4, false>(e, r);
+            op.template finish<4, false>(e, r);
+        }
+    } else {
+        for (size_t k = e; k < n && k < e + 4; ++k) {
+            typename Op::template Regs<1> r;
+            op.template load<1, false>(k, r);
+            op.template finish<1, false>(k, r);
+        }
+    }
+}
+
+// Runs `make`'s operation over `count` tensors (host arrays of device pointers and sizes).
+template<int STREAMS, typename Maker>
+int launch_multi(const char* who, int count, float* const* const* buffers, const size_t* n, const int* apply_decay,
+                 int bytes_per_elem, const Maker& make, hipStream_t stream)
+{
+    for (int begin = 0; begin < count; begin += kMultiTensors) {
+        MultiTable t{};
+        const int part = count - begin < kMultiTensors ? count - begin : kMultiTensors;
+        unsigned long long blocks = 0;
+        int used = 0;
+        for (int i = 0; i < part; ++i) {
+            const size_t len = n[begin + i];
+            if (len == 0) continue;
+            bool aligned = true;
+            for (int k = 0; k < STREAMS; ++k) {
+                float* ptr = buffers[k][begin + i];
+                if (!ptr) return fail_invalid("%s: null pointer for tensor %d", who, begin + i);
+                aligned = aligned && aligned16(ptr);
+                t.stream[k][used] = ptr;
+            }
+            t.n[used] = len;
+            t.first_block[used] = static_cast<uint32_t>(blocks);
+            if (apply_decay && apply_decay[begin + i]) t.decay_mask |= 1u << used;
+            if (len * static_cast<size_t>(bytes_per_elem) >= kStreamingBytes) t.past_cache_mask |= 1u << used;
+            if (aligned) t.vector_mask |= 1u << used;
+            blocks += (len + kMultiPerBlock - 1) / kMultiPerBlock;
+            ++used;
+        }
+        if (used == 0) continue;
+        if (blocks > 0x7fffffffull) {
+            set_error("%s: more than 2^31 workgroups in one launch", who);
+            return PXH_ERR_UNSUPPORTED;
+        }
+        t.first_block[used] = static_cast<uint32_t>(blocks);
+        t.count = used;
+        hipLaunchKernelGGL((multi_tensor_kernel<Maker>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, t,
+                           make);
+        const int rc = check_launch(who);
+        if (rc) return rc;
+    }
+    return PXH_OK;
+}
 
 struct AdamStepOp {
     float* x;
@@ -757,6 +934,56 @@ int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* nor
     return check_launch("pxh_rescale_clip");
 }
 
+size_t pxh_rescale_multi_workspace_bytes(void)
+{
+    return static_cast<size_t>(kRescaleTensors) * kNormBlocks * sizeof(double2);
+}
+
+int pxh_rescale_clip_multi(int count, float* const* x, const size_t* n, float threshold, float clip, float* norms,
+                           void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (count < 0 || (count && (!x || !n))) return fail_invalid("pxh_rescale_clip_multi: bad argument");
+    const bool rescale = threshold > 0.0f || norms != nullptr;
+    if (!rescale && !(clip > 0.0f)) return PXH_OK;
+    void* ws = nullptr;
+    int rc = resolve_workspace(workspace, workspace_bytes, pxh_rescale_multi_workspace_bytes(), &ws);
+    if (rc) return rc;
+    double2* partial = static_cast<double2*>(ws);
+    hipStream_t s = as_stream(stream);
+    for (int begin = 0; begin < count; begin += kRescaleTensors) {
+        RescaleTable t{};
+        const int part = count - begin < kRescaleTensors ? count - begin : kRescaleTensors;
+        uint32_t blocks = 0;
+        for (int i = 0; i < part; ++i) {
+            // an empty tensor keeps its place in the table with no workgroup of its own (its norm stays unwritten)
+            float* ptr = x[begin + i];
+            const size_t len = n[begin + i];
+            if (!ptr && len) return fail_invalid("pxh_rescale_clip_multi: null pointer for tensor %d", begin + i);
+            const bool vec = aligned16(ptr) && len % 4 == 0;
+            const size_t per_step = static_cast<size_t>(kBlock) * (vec ? 4 : 1) * kNormLoads;
+            const size_t want = (len + per_step - 1) / per_step;
+            t.x[i] = ptr;
+            t.n[i] = len;
+            t.first_block[i] = blocks;
+            if (vec) t.vector_mask |= 1u << i;
+            if (vec && len * 4 >= kStreamingBytes) t.past_cache_mask |= 1u << i;
+            blocks += static_cast<uint32_t>(want < static_cast<size_t>(kNormBlocks) ? want : kNormBlocks);
+        }
+        t.first_block[part] = blocks;
+        t.count = part;
+        t.norms = norms;
+        t.first_tensor = begin;
+        if (blocks == 0) continue;
+        hipLaunchKernelGGL(multi_sumsq_kernel, dim3(blocks), dim3(kBlock), 0, s, t, partial);
+        rc = check_launch("pxh_rescale_clip_multi");
+        if (rc) return rc;
+        hipLaunchKernelGGL(multi_rescale_kernel, dim3(blocks), dim3(kBlock), 0, s, t, partial, threshold, clip);
+        rc = check_launch("pxh_rescale_clip_multi");
+        if (rc) return rc;
+    }
+    return PXH_OK;
+}
+
 int pxh_adam(int n, float* x, const float* m, const float* v, float beta1, float beta2, float rate, float eps, int t,
              void* stream)
 {
@@ -785,6 +1012,35 @@ int pxh_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch,
     op.lr = lr; op.eps = eps; op.apply_decay = apply_decay;
     return launch_stream("pxh_adam_update", n, aligned16(w) && aligned16(d) && aligned16(m) && aligned16(v), 32, op,
                          as_stream(stream));
+}
+
+int pxh_adam_update_multi(int count, float* const* w, float* const* d, float* const* m, float* const* v, const size_t* n,
+                          const int* apply_decay, int batch, int t, float lr, float beta1, float beta2, float eps,
+                          float decay, void* stream)
+{
+    if (count < 0 || (count && (!w || !d || !m || !v || !n))) return fail_invalid("pxh_adam_update_multi: bad argument");
+    if (batch <= 0) return fail_invalid("pxh_adam_update_multi: batch must be positive");
+    if (t < 1) return fail_invalid("pxh_adam_update_multi: t must be at least 1 (the update count is pre-incremented)");
+    AdamUpdateOp op{};
+    op.inv_batch = 1.0f / static_cast<float>(batch);
+    op.neg_decay = -decay;
+    op.beta1 = beta1; op.beta2 = beta2;
+    op.a1 = 1.0f - beta1; op.a2 = 1.0f - beta2;
+    op.c1 = 1.0f - powf(beta1, static_cast<float>(t));
+    op.c2 = 1.0f - powf(beta2, static_cast<float>(t));
+    op.lr = lr; op.eps = eps;
+    float* const* const buffers[4] = { w, d, m, v };
+    return launch_multi<4>("pxh_adam_update_multi", count, buffers, n, apply_decay, 32, AdamMaker{ op }, as_stream(stream));
+}
+
+int pxh_sgd_update_multi(int count, float* const* w, float* const* d, const size_t* n, const int* apply_decay, int batch,
+                         float lr, float momentum, float decay, void* stream)
+{
+    if (count < 0 || (count && (!w || !d || !n))) return fail_invalid("pxh_sgd_update_multi: bad argument");
+    if (batch <= 0) return fail_invalid("pxh_sgd_update_multi: batch must be positive");
+    const SgdUpdateOp op{ nullptr, nullptr, -decay * static_cast<float>(batch), lr / static_cast<float>(batch), momentum, 0 };
+    float* const* const buffers[4] = { w, d, nullptr, nullptr };
+    return launch_multi<2>("pxh_sgd_update_multi", count, buffers, n, apply_decay, 16, SgdMaker{ op }, as_stream(stream));
 }
 
 }

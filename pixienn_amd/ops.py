@@ -326,11 +326,59 @@ def adam_update(w, d, m, v, batch, t, lr, beta1=0.9, beta2=0.999, eps=1e-8, deca
          float(beta2), float(eps), float(decay), int(bool(apply_decay)), _stream())
 
 
+def _pointer_table(tensors):
+    import ctypes
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def _size_table(tensors):
+    import ctypes
+    return (ctypes.c_size_t * len(tensors))(*[t.numel() for t in tensors])
+
+
+def _flag_table(flags, count):
+    import ctypes
+    if flags is None:
+        return None
+    assert len(flags) == count
+    return (ctypes.c_int * count)(*[int(bool(f)) for f in flags])
+
+
+def adam_update_multi(ws, ds, ms, vs, batch, t, lr, beta1=0.9, beta2=0.999, eps=1e-8, decay=0.0, apply_decay=None):
+    """pxh_adam_update for lists of tensors (one entry per parameter tensor) in a few launches."""
+    _chk_all(*ws, *ds, *ms, *vs)
+    count = len(ws)
+    assert len(ds) == count and len(ms) == count and len(vs) == count
+    for group in zip(ws, ds, ms, vs):
+        assert len({x.numel() for x in group}) == 1
+    call("pxh_adam_update_multi", count, _pointer_table(ws), _pointer_table(ds), _pointer_table(ms), _pointer_table(vs),
+         _size_table(ws), _flag_table(apply_decay, count), int(batch), int(t), float(lr), float(beta1), float(beta2),
+         float(eps), float(decay), _stream())
+
+
+def sgd_update_multi(ws, ds, batch, lr, momentum, decay=0.0, apply_decay=None):
+    """pxh_sgd_update for lists of tensors in a few launches."""
+    _chk_all(*ws, *ds)
+    count = len(ws)
+    assert len(ds) == count
+    call("pxh_sgd_update_multi", count, _pointer_table(ws), _pointer_table(ds), _size_table(ws),
+         _flag_table(apply_decay, count), int(batch), float(lr), float(momentum), float(decay), _stream())
+
+
 def sgd_update(w, d, batch, lr, momentum, decay=0.0, apply_decay=False):
     """include/ConvLayer.h:309-311 of the reference for one parameter tensor."""
     _chk_all(w, d)
     call("pxh_sgd_update", w.numel(), ptr(w), ptr(d), int(batch), float(lr), float(momentum), float(decay),
          int(bool(apply_decay)), _stream())
+
+
+def rescale_clip_multi(xs, threshold=0.0, clip=0.0, norms=None):
+    """pxh_rescale_clip for a list of tensors in a few launches; `norms`: device float tensor, one per tensor."""
+    _chk_all(*xs, norms)
+    if norms is not None:
+        assert norms.numel() == len(xs)
+    call("pxh_rescale_clip_multi", len(xs), _pointer_table(xs), _size_table(xs), float(threshold), float(clip),
+         ptr(norms), None, 0, _stream())
 
 
 def rescale_clip(x, threshold=0.0, clip=0.0, norm_out=None):

@@ -126,20 +126,21 @@ def detection_clusters(seed, n, batch, classes, clusters, spread=6.0):
 
 def yolov3_layers(size=608):
     """The 107 layers of the reference's resources/models/yolov3.yml as dictionaries with the output
-    shape filled in: conv (filters, stride, bn), shortcut (from), route (layers), upsample, yolo (mask).
-    Keys: type, c, s (output channels and height == width), plus the type's own."""
+    shape filled in: conv (filters, stride, bn, kernel), shortcut (from), route (layers), upsample, yolo (mask).
+    Keys: type, c, s (output channels and height == width), plus the type's own (conv: bn, k = kernel
+    size, in_c = input channels)."""
     layers = []
 
-    def conv(filters, stride=1, bn=True):
+    def conv(filters, stride=1, bn=True, k=3):
         prev = layers[-1] if layers else dict(c=3, s=size)
-        layers.append(dict(type="conv", c=filters, s=prev["s"] // stride, bn=bn))
+        layers.append(dict(type="conv", c=filters, s=prev["s"] // stride, bn=bn, k=k, in_c=prev["c"]))
 
     def shortcut():
         layers.append(dict(type="shortcut", c=layers[-1]["c"], s=layers[-1]["s"], frm=len(layers) - 3))
 
     def residual(narrow, wide, times):
         for _ in range(times):
-            conv(narrow)
+            conv(narrow, k=1)
             conv(wide)
             shortcut()
 
@@ -154,13 +155,29 @@ def yolov3_layers(size=608):
         if joins is not None:
             src = len(layers) - 4
             layers.append(dict(type="route", c=layers[src]["c"], s=layers[src]["s"], sources=[src]))
-            conv(narrow)
+            conv(narrow, k=1)
             layers.append(dict(type="upsample", c=narrow, s=2 * layers[-1]["s"]))
             up = len(layers) - 1
             layers.append(dict(type="route", c=narrow + layers[joins]["c"], s=layers[up]["s"], sources=[up, joins]))
         for _ in range(3):
-            conv(narrow)
+            conv(narrow, k=1)
             conv(wide)
-        conv(255, bn=False)
+        conv(255, bn=False, k=1)
         layers.append(dict(type="yolo", c=255, s=layers[-1]["s"], mask=mask))
     return layers
+
+
+def yolov3_parameter_tensors(size=608):
+    """(elements, takes_weight_decay) of every parameter tensor of YOLOv3 in layer order, as the engine
+    holds them: per convolution the weights (filters x input channels x k x k, decayed), the biases and,
+    with batch norm, the scales (include/ConvLayer.h:96-115 of the reference).  222 tensors, YOLOV3_PARAMS
+    elements in all."""
+    tensors = []
+    for l in yolov3_layers(size):
+        if l["type"] != "conv":
+            continue
+        tensors.append((l["c"] * l["in_c"] * l["k"] * l["k"], True))
+        tensors.append((l["c"], False))
+        if l["bn"]:
+            tensors.append((l["c"], False))
+    return tensors

@@ -302,6 +302,117 @@ def test_sgd_update_matches_oracle(ops, oracle, n):
         assert_close(host(gd), d, 1e-6, 1e-3, "sgd updates n=%d decay=%s" % (n, apply_decay))
 
 
+# A model's parameter tensors as the engine holds them: many, mostly small, a few large, none related
+# to a workgroup's 1024 elements; one of them starts 4 bytes into its buffer (the scalar path).
+MULTI_SIZES = [32, 864, 32, 0, 1, 3, 4, 5, 255, 1023, 1024, 1025, 2048, 4097, 18432, 64, 64, 100003, 1 << 20, 7,
+               36864, 128, 128, 2_000_003, 255, 255, 9, 1024, 512, 512, 65536, 2, 6, 131, 4718592, 33, 1000, 1000]
+
+
+def _multi_tensors(seed, std, offset_one=True):
+    """Per size: (host array, device tensor); the sixth tensor is a view one element into its buffer."""
+    import torch
+    hosts, devs = [], []
+    for i, n in enumerate(MULTI_SIZES):
+        h = wl.normal(seed + i, n, std=std) if n else np.zeros(0, F)
+        if offset_one and i == 5:
+            buf = torch.zeros(n + 1, device="cuda")
+            buf[1:] = gpu(h)
+            t = buf[1:]
+            assert t.data_ptr() % 16 != 0
+        else:
+            t = gpu(h)
+        hosts.append(h); devs.append(t)
+    return hosts, devs
+
+
+def test_adam_update_multi_gives_every_tensor_what_the_single_call_gives(ops):
+    flags = [i % 3 == 0 for i in range(len(MULTI_SIZES))]
+    w0, gw = _multi_tensors(5000, 0.02)
+    d0, gd = _multi_tensors(5100, 1e-3)
+    m0, gm = _multi_tensors(5200, 1e-4)
+    v0, gv = _multi_tensors(5300, 1e-4)
+    gv = [t.abs_() for t in gv]
+    single = [[t.clone() for t in group] for group in (gw, gd, gm, gv)]
+    for step in (1, 2, 3):
+        ops.adam_update_multi(gw, gd, gm, gv, 16, step, 1e-3, 0.9, 0.999, 1e-8, 5e-4, flags)
+        for i in range(len(MULTI_SIZES)):
+            if MULTI_SIZES[i]:
+                ops.adam_update(single[0][i], single[1][i], single[2][i], single[3][i], 16, step, 1e-3, 0.9, 0.999, 1e-8,
+                                5e-4, flags[i])
+        for i in range(len(MULTI_SIZES)):      # a fresh gradient on both sides
+            if MULTI_SIZES[i]:
+                g = gpu(wl.normal(5400 + 10 * step + i, MULTI_SIZES[i], std=1e-3))
+                gd[i] += g; single[1][i] += g
+    for name, many, one in zip("wdmv", (gw, gd, gm, gv), single):
+        for i in range(len(MULTI_SIZES)):
+            assert_bit_exact(host(many[i]), host(one[i]), "adam multi %s[%d] n=%d" % (name, i, MULTI_SIZES[i]))
+    # the gradient buffers are cleared by the update, the weights moved
+    assert all(float(t.abs().max()) > 0 for t, n in zip(gw, MULTI_SIZES) if n)
+
+
+def test_sgd_update_multi_gives_every_tensor_what_the_single_call_gives(ops):
+    flags = [i % 2 == 0 for i in range(len(MULTI_SIZES))]
+    w0, gw = _multi_tensors(5600, 0.02)
+    d0, gd = _multi_tensors(5700, 0.5)
+    single = [[t.clone() for t in group] for group in (gw, gd)]
+    for step in range(2):
+        ops.sgd_update_multi(gw, gd, 16, 1e-3, 0.9, 5e-4, flags)
+        for i in range(len(MULTI_SIZES)):
+            if MULTI_SIZES[i]:
+                ops.sgd_update(single[0][i], single[1][i], 16, 1e-3, 0.9, 5e-4, flags[i])
+    for name, many, one in zip("wd", (gw, gd), single):
+        for i in range(len(MULTI_SIZES)):
+            assert_bit_exact(host(many[i]), host(one[i]), "sgd multi %s[%d] n=%d" % (name, i, MULTI_SIZES[i]))
+
+
+def test_update_multi_edge_cases(ops):
+    import torch
+    from pixienn_amd import capi
+    ops.adam_update_multi([], [], [], [], 16, 1, 1e-3)          # nothing to do
+    ops.sgd_update_multi([], [], 16, 1e-3, 0.9)
+    w = gpu(np.ones(8, F)); d = gpu(np.ones(8, F)); m = gpu(np.zeros(8, F)); v = gpu(np.zeros(8, F))
+    with pytest.raises(capi.PxError):
+        ops.adam_update_multi([w], [d], [m], [v], 0, 1, 1e-3)    # batch
+    with pytest.raises(capi.PxError):
+        ops.adam_update_multi([w], [d], [m], [v], 16, 0, 1e-3)   # t is pre-incremented
+    with pytest.raises(capi.PxError):
+        ops.sgd_update_multi([w], [d], 0, 1e-3, 0.9)
+    # more tensors than one launch takes, all tiny: every one is reached
+    many = [torch.full((3,), float(i), device="cuda") for i in range(100)]
+    grads = [torch.ones(3, device="cuda") for _ in range(100)]
+    ops.sgd_update_multi(many, grads, 1, 0.5, 0.0)
+    for i, t in enumerate(many):
+        assert host(t).tolist() == [i + 0.5] * 3
+    assert all(float(g.abs().max()) == 0.0 for g in grads)      # momentum 0 clears the update buffer
+
+
+@pytest.mark.parametrize("threshold,clip", [(0.5, 0.0), (0.0, 0.01), (3.0, 0.02), (1e9, 1e9), (0.0, 0.0)])
+def test_rescale_clip_multi_leaves_every_tensor_as_the_single_call_does(ops, threshold, clip):
+    """Tensors of a model's sizes with different scales, so that at one threshold some are rescaled,
+    some only clamped and some left alone."""
+    import torch
+    h, many = _multi_tensors(5800, 0.02)
+    for i, t in enumerate(many):
+        t *= float(1 + i % 5)
+    one = [t.clone() for t in many]
+    norms = torch.full((len(many),), -1.0, device="cuda")
+    ops.rescale_clip_multi(many, threshold, clip, norms)
+    want_norms = []
+    for t in one:
+        norm = torch.full((1,), -1.0, device="cuda")
+        if t.numel():
+            ops.rescale_clip(t, threshold, clip, norm)
+        want_norms.append(float(norm))
+    for i, (a_, b_) in enumerate(zip(many, one)):
+        assert_bit_exact(host(a_), host(b_), "rescale multi tensor %d n=%d" % (i, MULTI_SIZES[i]))
+    assert host(norms).tolist() == want_norms
+    # without the norms and with nothing asked for, nothing is touched
+    before = [t.clone() for t in many]
+    ops.rescale_clip_multi(many, 0.0, 0.0)
+    for a_, b_ in zip(many, before):
+        assert_bit_exact(host(a_), host(b_), "no-op")
+
+
 @pytest.mark.parametrize("n", [5, 1024, 4 * 1024 * 1024 + 4, 1234567])
 @pytest.mark.parametrize("mode", ["rescale", "clip", "both", "below", "none"])
 def test_rescale_clip_matches_oracle(ops, oracle, n, mode):

@@ -35,3 +35,11 @@ def test_detection_clusters_are_reproducible():
     assert a.tobytes() == b.tobytes() and a.dtype == wl.DETECTION_DTYPE
     assert a["batch"].max() < 4 and a["class_index"].max() < 7 and (a["w"] >= 1).all()
     assert len(set(a["prob"])) < 120          # two decimals: ties
+
+
+def test_yolov3_parameter_tensors_add_up_to_the_flat_count():
+    tensors = wl.yolov3_parameter_tensors(608)
+    assert len(tensors) == 222                      # 75 convolutions: weights + biases (+ scales with batch norm)
+    assert sum(n for n, _ in tensors) == wl.YOLOV3_PARAMS
+    assert sum(1 for _, decayed in tensors if decayed) == 75
+    assert max(n for n, _ in tensors) == 512 * 1024 * 9 and min(n for n, _ in tensors) == 32
