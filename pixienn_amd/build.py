@@ -60,7 +60,7 @@ def build_host(verbose=True):
     probe = os.path.join(OBJ, "host_headers.cpp")
     os.makedirs(OBJ, exist_ok=True)
     with open(probe, "w") as f:
-        f.write('#include "pixienn/Layers.h"\n#include "pixienn/OptimizerState.h"\n#include "pixienn/CapturedSequence.h"\n#include "pixienn/WeightsFile.h"\n#include "pixienn/DeviceTraits.h"\nstatic_assert(std::is_same_v<px::hip::DeviceTraits<px::hip::Device::HIP>::ValueType, float>);\nstatic_assert(px::hip::IsHipDevice<px::hip::Device::HIP>::value && !px::hip::IsHipDevice<px::hip::Device::CPU>::value);\nint pixienn_host_headers_compile() { return PXH_OK; }\n')
+        f.write('#include "pixienn/Layers.h"\n#include "pixienn/OptimizerState.h"\n#include "pixienn/CapturedSequence.h"\n#include "pixienn/ParameterSet.h"\n#include "pixienn/WeightsFile.h"\n#include "pixienn/DeviceTraits.h"\nstatic_assert(std::is_same_v<px::hip::DeviceTraits<px::hip::Device::HIP>::ValueType, float>);\nstatic_assert(px::hip::IsHipDevice<px::hip::Device::HIP>::value && !px::hip::IsHipDevice<px::hip::Device::CPU>::value);\nint pixienn_host_headers_compile() { return PXH_OK; }\n')
     obj = os.path.join(OBJ, "host_headers.o")
     cmd = [hipcc(), "-std=c++20", "-O1", "-Wall", "-Wextra", "-Wno-unused-parameter", "-I" + os.path.join(ROOT, "include"),
            "-I" + host, "-c", probe, "-o", obj]

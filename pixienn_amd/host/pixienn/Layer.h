@@ -141,6 +141,8 @@ private:
 };
 
 // ---------------------------------------------------------------- layer
+class ParameterSet;
+
 class Layer
 {
 public:
@@ -182,6 +184,11 @@ public:
         if (context_.helpersTouchDeltaInUpdate) rescaleAndClip(delta_);
     }
 
+    // For a model that updates all its parameter tensors together (ParameterSet.h): a layer with
+    // parameters adds them to the set, and is told when the set has stepped them.
+    virtual void collectParameters(ParameterSet& /*set*/) {}
+    virtual void parametersUpdated() {}
+
     // This layer's section of a weight file; bytes read / written (reference: Layer<D>::loadWeights /
     // saveWeights, include/Layer.h:57-58).  Layers without parameters have none.
     virtual std::streamoff loadWeights(std::istream& /*is*/) { return 0; }
@@ -216,6 +223,9 @@ public:
     bool firstConsumerOverwrites() const noexcept { return firstConsumerOverwrites_; }
 
     void setGradientClipping(bool on, float value) { gradientClipping_ = on; gradientClipValue_ = value; }
+    // thresholds of the two helpers as they apply to this layer's tensors; 0 = off
+    float rescaleThreshold() const noexcept { return gradientRescaling_ ? gradientThreshold_ : 0.0f; }
+    float clipValue() const noexcept { return gradientClipping_ ? gradientClipValue_ : 0.0f; }
     void setGradientRescaling(bool on, float threshold) { gradientRescaling_ = on; gradientThreshold_ = threshold; }
 
 protected:

@@ -8,6 +8,7 @@
 #include <functional>
 
 #include "Adam.h"
+#include "ParameterSet.h"
 
 namespace px::hip {
 
@@ -177,6 +178,24 @@ public:
         }
         foldedValid_ = false;
     }
+
+    // the same tensors, hooks and optimiser as update(), for a model that steps all layers together
+    void collectParameters(ParameterSet& set) override
+    {
+        if (!training()) return;
+        const ParameterSet::Hooks hooks{ rescaleThreshold(), clipValue() };
+        if (context().adamEnabled) {
+            set.addAdam(weights_, weightUpdates_, weightM_, weightV_, true, hooks);
+            set.addAdam(biases_, biasUpdates_, biasM_, biasV_, false, hooks);
+            if (batchNorm_) set.addAdam(scales_, scaleUpdates_, scaleM_, scaleV_, false, hooks);
+        } else {
+            set.addSgd(weights_, weightUpdates_, true, hooks);
+            set.addSgd(biases_, biasUpdates_, false, hooks);
+            if (batchNorm_) set.addSgd(scales_, scaleUpdates_, false, hooks);
+        }
+    }
+
+    void parametersUpdated() override { foldedValid_ = false; }
 
     // biases [, scales, rolling mean, rolling variance], weights as raw fp32 (reference:
     // include/ConvLayer.h:132-171)
@@ -352,6 +371,16 @@ public:
                                     c.learningRate, c.momentum, 0.0f, 0, stream()));
         foldedValid_ = false;
     }
+
+    void collectParameters(ParameterSet& set) override
+    {
+        if (!training()) return;
+        const ParameterSet::Hooks hooks{ rescaleThreshold(), clipValue() };
+        set.addSgd(biases_, biasUpdates_, false, hooks);
+        set.addSgd(scales_, scaleUpdates_, false, hooks);
+    }
+
+    void parametersUpdated() override { foldedValid_ = false; }
 
     // biases, scales, rolling mean, rolling variance as raw fp32 (include/BatchNormLayer.h:72-113)
     std::streamoff loadWeights(std::istream& is) override

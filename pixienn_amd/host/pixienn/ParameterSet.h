@@ -1,0 +1,114 @@
+// The parameter tensors of a model, gathered once, updated together.
+//
+// The reference updates layer by layer (Model<D>::update, include/Model.h:1786-1792): per convolution
+// the scaleGradients / clipGradients hooks on three update buffers and three optimiser calls
+// (include/ConvLayer.h:299-340, include/cuda/ConvLayer.h:362-413).  Most of those tensors are a few
+// hundred values, so on the GPU that loop is a thousand launches that each take longer to start than to
+// run.  A ParameterSet holds the same tensors and does the same arithmetic on each of them through the
+// entry points that take many tensors per launch:
+//
+//     ParameterSet params;
+//     for (auto& layer: layers) layer->collectParameters(params);      // once, after construction
+//     ...
+//     for (auto& layer: layers) layer->Layer::update();                // the helpers on the deltas
+//     params.update(context);                                          // hooks + optimiser, all tensors
+//     for (auto& layer: layers) layer->parametersUpdated();
+//
+// Every tensor ends up bit for bit as its layer's own update() leaves it.
+#pragma once
+
+#include <map>
+#include <utility>
+#include <vector>
+
+#include "Layer.h"
+
+namespace px::hip {
+
+class ParameterSet
+{
+public:
+    using V = FloatVector;
+
+    // thresholds of the two hooks for a tensor's update buffer; 0 = hook off
+    struct Hooks {
+        float rescaleThreshold = 0.0f, clipValue = 0.0f;
+    };
+
+    // values, their accumulated update, Adam's two moments; `decayed`: takes the weight decay
+    void addAdam(V& w, V& d, V& m, V& v, bool decayed, Hooks hooks)
+    {
+        if (w.empty()) return;
+        PX_CHECK(w.size() == d.size() && w.size() == m.size() && w.size() == v.size(),
+                 "ParameterSet: tensors of different sizes");
+        adam_.add(w, d, decayed);
+        adam_.m.push_back(m.data());
+        adam_.v.push_back(v.data());
+        hook(d, hooks);
+    }
+
+    // values and their accumulated update (which becomes the momentum term)
+    void addSgd(V& w, V& d, bool decayed, Hooks hooks)
+    {
+        if (w.empty()) return;
+        PX_CHECK(w.size() == d.size(), "ParameterSet: tensors of different sizes");
+        sgd_.add(w, d, decayed);
+        hook(d, hooks);
+    }
+
+    std::size_t tensors() const noexcept { return adam_.w.size() + sgd_.w.size(); }
+
+    void clear() { *this = ParameterSet(); }
+
+    // The hooks on every update buffer, then the optimiser step, with the context's settings.
+    void update(const Context& c) const
+    {
+        for (const auto& [key, group]: hooked_) {
+            PX_HIP_CHECK(pxh_rescale_clip_multi(static_cast<int>(group.x.size()), group.x.data(), group.n.data(),
+                                                key.first, key.second, nullptr, nullptr, 0, c.stream));
+        }
+        if (!adam_.w.empty()) {
+            PX_CHECK(c.updateBatch > 0 && c.timeStep > 0, "Adam needs batch > 0 and t > 0");
+            PX_HIP_CHECK(pxh_adam_update_multi(static_cast<int>(adam_.w.size()), adam_.w.data(), adam_.d.data(),
+                                               adam_.m.data(), adam_.v.data(), adam_.n.data(), adam_.decayed.data(),
+                                               c.updateBatch, c.timeStep, c.learningRate, c.adamBeta1, c.adamBeta2,
+                                               c.adamEpsilon, c.decay, c.stream));
+        }
+        if (!sgd_.w.empty()) {
+            PX_HIP_CHECK(pxh_sgd_update_multi(static_cast<int>(sgd_.w.size()), sgd_.w.data(), sgd_.d.data(),
+                                              sgd_.n.data(), sgd_.decayed.data(), c.updateBatch, c.learningRate,
+                                              c.momentum, c.decay, c.stream));
+        }
+    }
+
+private:
+    struct Group {
+        std::vector<float*> w, d, m, v;
+        std::vector<std::size_t> n;
+        std::vector<int> decayed;
+        void add(V& values, V& updates, bool decay)
+        {
+            w.push_back(values.data());
+            d.push_back(updates.data());
+            n.push_back(values.size());
+            decayed.push_back(decay ? 1 : 0);
+        }
+    };
+    struct Hooked {
+        std::vector<float*> x;
+        std::vector<std::size_t> n;
+    };
+
+    void hook(V& updates, Hooks h)
+    {
+        if (!(h.rescaleThreshold > 0.0f) && !(h.clipValue > 0.0f)) return;
+        Hooked& group = hooked_[{ h.rescaleThreshold, h.clipValue }];
+        group.x.push_back(updates.data());
+        group.n.push_back(updates.size());
+    }
+
+    Group adam_, sgd_;
+    std::map<std::pair<float, float>, Hooked> hooked_;     // update buffers by (threshold, clip)
+};
+
+}  // namespace px::hip

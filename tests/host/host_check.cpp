@@ -777,6 +777,71 @@ void capturedSequenceChecks()
     PX_HIP_RUNTIME_CHECK(hipStreamDestroy(stream));
 }
 
+// A model that steps all its parameter tensors together (ParameterSet) against the layer-by-layer
+// update(): the same values in every tensor, with Adam and with SGD, with the hooks on.
+void parameterSetChecks()
+{
+    for (const bool adam: { true, false }) {
+        Net byLayer(true), together(true);
+        const auto truth = makeTruth();
+        FloatVector input(size_t(N) * C * S * S);
+        input.copyHost(normals(900, input.size()));
+        Net* nets[2] = { &byLayer, &together };
+        for (Net* n: nets) {
+            n->ctx.adamEnabled = adam;
+            n->ctx.setGroundTruth(truth);
+            for (ConvLayer* l: { n->conv0.get(), n->conv2.get(), n->conv6.get() }) {
+                l->setGradientRescaling(true, 0.05f);      // small enough to bite on these update buffers
+                l->setGradientClipping(true, 0.01f);
+            }
+        }
+        ParameterSet params;
+        for (Layer* l: std::initializer_list<Layer*>{ together.conv0.get(), together.pool1.get(), together.conv2.get(),
+                                                      together.short3.get(), together.conv6.get(), together.yolo7.get() })
+            l->collectParameters(params);
+        report(std::string("parameter set: ") + (adam ? "Adam" : "SGD") + ": 5 tensors of three convolutions",
+               params.tensors() == 5);
+        bool same = true;
+        for (int step = 1; step <= 2; ++step) {
+            for (Net* n: nets) {
+                n->ctx.timeStep = step;
+                n->conv0->forward(input);
+                n->pool1->forward(n->conv0->output());
+                n->conv2->forward(n->pool1->output());
+                n->short3->forward(n->conv2->output());
+                n->up4->forward(n->short3->output());
+                n->route5->forward(n->up4->output());
+                n->conv6->forward(n->route5->output());
+                n->yolo7->forward(n->conv6->output());
+                n->yolo7->backward(n->conv6->output(), &n->conv6->delta());
+                n->conv6->backward(n->route5->output(), &n->route5->delta());
+                n->route5->backward(n->up4->output(), &n->up4->delta());
+                n->up4->backward(n->short3->output(), &n->short3->delta());
+                n->short3->backward(n->conv2->output(), &n->conv2->delta());
+                n->conv2->backward(n->pool1->output(), &n->pool1->delta());
+                n->pool1->backward(n->conv0->output(), &n->conv0->delta());
+                n->conv0->backward(input, nullptr);
+            }
+            for (Layer* l: std::initializer_list<Layer*>{ byLayer.conv0.get(), byLayer.conv2.get(), byLayer.conv6.get() })
+                l->update();
+            for (Layer* l: std::initializer_list<Layer*>{ together.conv0.get(), together.conv2.get(), together.conv6.get() })
+                l->Layer::update();
+            params.update(together.ctx);
+            for (Layer* l: std::initializer_list<Layer*>{ together.conv0.get(), together.conv2.get(), together.conv6.get() })
+                l->parametersUpdated();
+            same = same && together.conv0->scales().asVector() == byLayer.conv0->scales().asVector() &&
+                   together.conv0->biases().asVector() == byLayer.conv0->biases().asVector() &&
+                   together.conv2->scales().asVector() == byLayer.conv2->scales().asVector() &&
+                   together.conv2->biases().asVector() == byLayer.conv2->biases().asVector() &&
+                   together.conv6->biases().asVector() == byLayer.conv6->biases().asVector();
+            report(std::string("parameter set: ") + (adam ? "Adam" : "SGD") + " step " + std::to_string(step) +
+                   " leaves every tensor as the layers' own update does", same);
+        }
+        const Host moved = together.conv0->scales().asVector();
+        report(std::string("parameter set: ") + (adam ? "Adam" : "SGD") + ": the parameters moved", moved != together.scale0);
+    }
+}
+
 // A residual block whose shortcut overwrites the two deltas it is the first to write: the same
 // gradients as the clearing-and-accumulating form, with the two zero-fills gone.
 void firstWriterShortcutChecks()
@@ -950,6 +1015,7 @@ int main(int argc, char** argv)
             weightsFileChecks();
             firstWriterShortcutChecks();
             capturedSequenceChecks();
+            parameterSetChecks();
         }
     } catch (const std::exception& e) {
         std::printf("unexpected exception: %s\n", e.what());
