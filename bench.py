@@ -168,8 +168,8 @@ def measure_model_order(torch, ops, wl, timer, N=16):
     model's own layer order on tensors of their own (21 GB): forward (per layer the delta zero-fill
     of Layer::forward, then the layer), backward in reverse (per layer the gradient rescale + clip
     of Layer::backward with the thresholds of yolov3.yml, 100 and 10, then the layer), update (the
-    same helpers once more per layer and on each of the 222 update buffers, then Adam on the 222
-    parameter tensors, both through the entry points that take many tensors per launch).
+    same helpers once more on every layer's delta and on each of the 222 update buffers, then Adam
+    on the 222 parameter tensors, all through the entry points that take many tensors per launch).
     The convolutions' GEMMs are not run: a conv layer reads a resident conv result and its input
     gradient goes nowhere.  Each phase is timed as one HIP graph."""
     dev = torch.device("cuda")
@@ -272,9 +272,8 @@ def measure_model_order(torch, ops, wl, timer, N=16):
     def update(_, touch_delta=True):
         n = 0
         if touch_delta:         # the reference's update() passes every delta through the helpers once more
-            for i, t in enumerate(T):
-                if not absorbed(i):
-                    ops.rescale_clip(t["d"], 100.0, 10.0); n += 1
+            deltas = [t["d"] for i, t in enumerate(T) if not absorbed(i)]
+            ops.rescale_clip_multi(deltas, 100.0, 10.0); n += len(deltas)
         # the hooks on every update buffer, each with its own norm, then Adam: every tensor in a few launches
         ops.rescale_clip_multi(pg, 100.0, 10.0)
         ops.adam_update_multi(pw, pg, pm, pv, N, 1, 1e-3, decay=5e-4, apply_decay=decayed)

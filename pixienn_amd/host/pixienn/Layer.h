@@ -184,9 +184,10 @@ public:
         if (context_.helpersTouchDeltaInUpdate) rescaleAndClip(delta_);
     }
 
-    // For a model that updates all its parameter tensors together (ParameterSet.h): a layer with
-    // parameters adds them to the set, and is told when the set has stepped them.
-    virtual void collectParameters(ParameterSet& /*set*/) {}
+    // For a model that updates all its layers together (ParameterSet.h): a layer adds what its update()
+    // works on to the set -- its delta here, its parameter tensors in the classes that have them (which
+    // call this one first) -- and is told when the set has stepped them.
+    virtual void collectParameters(ParameterSet& set);
     virtual void parametersUpdated() {}
 
     // This layer's section of a weight file; bytes read / written (reference: Layer<D>::loadWeights /

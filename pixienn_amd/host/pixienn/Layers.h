@@ -183,6 +183,7 @@ public:
     void collectParameters(ParameterSet& set) override
     {
         if (!training()) return;
+        Layer::collectParameters(set);
         const ParameterSet::Hooks hooks{ rescaleThreshold(), clipValue() };
         if (context().adamEnabled) {
             set.addAdam(weights_, weightUpdates_, weightM_, weightV_, true, hooks);
@@ -375,6 +376,7 @@ public:
     void collectParameters(ParameterSet& set) override
     {
         if (!training()) return;
+        Layer::collectParameters(set);
         const ParameterSet::Hooks hooks{ rescaleThreshold(), clipValue() };
         set.addSgd(biases_, biasUpdates_, false, hooks);
         set.addSgd(scales_, scaleUpdates_, false, hooks);

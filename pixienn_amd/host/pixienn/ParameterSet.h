@@ -10,11 +10,11 @@
 //     ParameterSet params;
 //     for (auto& layer: layers) layer->collectParameters(params);      // once, after construction
 //     ...
-//     for (auto& layer: layers) layer->Layer::update();                // the helpers on the deltas
-//     params.update(context);                                          // hooks + optimiser, all tensors
+//     params.update(context);                  // instead of every layer's update(): hooks + optimiser
 //     for (auto& layer: layers) layer->parametersUpdated();
 //
-// Every tensor ends up bit for bit as its layer's own update() leaves it.
+// Every tensor ends up bit for bit as its layer's own update() leaves it -- the deltas included, which
+// the reference's update() passes through the two helpers once more (Context::helpersTouchDeltaInUpdate).
 #pragma once
 
 #include <map>
@@ -56,6 +56,13 @@ public:
         hook(d, hooks);
     }
 
+    // a layer's delta, for the helpers' pass over it in update()
+    void addDelta(V& delta, Hooks hooks)
+    {
+        if (!delta.empty()) hook(delta, hooks);
+    }
+
+    // parameter tensors held (deltas not counted)
     std::size_t tensors() const noexcept { return adam_.w.size() + sgd_.w.size(); }
 
     void clear() { *this = ParameterSet(); }
@@ -110,5 +117,11 @@ private:
     Group adam_, sgd_;
     std::map<std::pair<float, float>, Hooked> hooked_;     // update buffers by (threshold, clip)
 };
+
+// what Layer::update() does, as an entry of the set
+inline void Layer::collectParameters(ParameterSet& set)
+{
+    if (context_.helpersTouchDeltaInUpdate) set.addDelta(delta_, ParameterSet::Hooks{ rescaleThreshold(), clipValue() });
+}
 
 }  // namespace px::hip

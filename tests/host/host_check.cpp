@@ -158,6 +158,11 @@ struct Net {
     std::vector<int> mask{ 0, 2 }, anchors{ 10, 14, 23, 27, 37, 58 };
     Host scale0, bias0, scale2, bias2, bias6;
 
+    std::vector<Layer*> all() const
+    {
+        return { conv0.get(), pool1.get(), conv2.get(), short3.get(), up4.get(), route5.get(), conv6.get(), yolo7.get() };
+    }
+
     explicit Net(bool training)
     {
         ctx.training = training;
@@ -790,15 +795,13 @@ void parameterSetChecks()
         for (Net* n: nets) {
             n->ctx.adamEnabled = adam;
             n->ctx.setGroundTruth(truth);
-            for (ConvLayer* l: { n->conv0.get(), n->conv2.get(), n->conv6.get() }) {
+            for (Layer* l: n->all()) {
                 l->setGradientRescaling(true, 0.05f);      // small enough to bite on these update buffers
                 l->setGradientClipping(true, 0.01f);
             }
         }
         ParameterSet params;
-        for (Layer* l: std::initializer_list<Layer*>{ together.conv0.get(), together.pool1.get(), together.conv2.get(),
-                                                      together.short3.get(), together.conv6.get(), together.yolo7.get() })
-            l->collectParameters(params);
+        for (Layer* l: together.all()) l->collectParameters(params);
         report(std::string("parameter set: ") + (adam ? "Adam" : "SGD") + ": 5 tensors of three convolutions",
                params.tensors() == 5);
         bool same = true;
@@ -822,14 +825,14 @@ void parameterSetChecks()
                 n->pool1->backward(n->conv0->output(), &n->conv0->delta());
                 n->conv0->backward(input, nullptr);
             }
-            for (Layer* l: std::initializer_list<Layer*>{ byLayer.conv0.get(), byLayer.conv2.get(), byLayer.conv6.get() })
-                l->update();
-            for (Layer* l: std::initializer_list<Layer*>{ together.conv0.get(), together.conv2.get(), together.conv6.get() })
-                l->Layer::update();
+            for (Layer* l: byLayer.all()) l->update();
             params.update(together.ctx);
-            for (Layer* l: std::initializer_list<Layer*>{ together.conv0.get(), together.conv2.get(), together.conv6.get() })
-                l->parametersUpdated();
-            same = same && together.conv0->scales().asVector() == byLayer.conv0->scales().asVector() &&
+            for (Layer* l: together.all()) l->parametersUpdated();
+            // the deltas went through the helpers once more on both sides
+            same = same && together.conv0->delta().asVector() == byLayer.conv0->delta().asVector() &&
+                   together.short3->delta().asVector() == byLayer.short3->delta().asVector() &&
+                   together.yolo7->delta().asVector() == byLayer.yolo7->delta().asVector() &&
+                   together.conv0->scales().asVector() == byLayer.conv0->scales().asVector() &&
                    together.conv0->biases().asVector() == byLayer.conv0->biases().asVector() &&
                    together.conv2->scales().asVector() == byLayer.conv2->scales().asVector() &&
                    together.conv2->biases().asVector() == byLayer.conv2->biases().asVector() &&
