@@ -144,6 +144,10 @@ int pxh_backward_bias(float* bias_updates, const float* delta, int batch, int n,
                       void* workspace, size_t workspace_bytes, void* stream);
 /* include/CudaUtils.cuh:27-31 */
 int pxh_fill_f32(float* x, size_t n, float value, void* stream);
+/* pxh_fill_f32 for many tensors in a few launches (x, n: HOST arrays of `count` device pointers and
+ * element counts): the deltas of all layers, which Layer::forward clears one by one
+ * (include/Layer.h:378-383), at the start of a pass. */
+int pxh_fill_f32_multi(int count, float* const* x, const size_t* n, float value, void* stream);
 int pxh_fill_i32(int* x, size_t n, int value, void* stream);
 int pxh_constrain(int n, float alpha, float* x, void* stream);
 int pxh_mul(int n, const float* x, float* y, void* stream);          /* y[i] = x[i]*y[i]; x == y allowed */

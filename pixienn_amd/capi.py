@@ -63,6 +63,7 @@ SIGNATURES = {
     "pxh_adam_update": [Z, P, P, P, P, I, I, F, F, F, F, F, I, P],
     "pxh_adam_update_multi": [I, P, P, P, P, P, P, I, I, F, F, F, F, F, P],
     "pxh_rescale_clip_multi": [I, P, P, F, F, P, P, Z, P],
+    "pxh_fill_f32_multi": [I, P, P, F, P],
     "pxh_sgd_update_multi": [I, P, P, P, P, I, F, F, F, P],
 }
 _OTHER_RETURNS = {

@@ -610,6 +610,11 @@ struct SgdMaker {
     }
 };
 
+struct FillMaker {
+    float value;
+    __device__ FillOp operator()(const MultiTable& t, int i) const { return FillOp{ t.stream[0][i], value }; }
+};
+
 template<typename Maker>
 __global__ __launch_bounds__(kBlock) void multi_tensor_kernel(MultiTable t, Maker make)
 {
@@ -640,7 +645,7 @@ __global__ __launch_bounds__(kBlock) void multi_tensor_kernel(MultiTable t, Make
 // Runs `make`'s operation over `count` tensors (host arrays of device pointers and sizes).
 template<int STREAMS, typename Maker>
 int launch_multi(const char* who, int count, float* const* const* buffers, const size_t* n, const int* apply_decay,
-                 int bytes_per_elem, const Maker& make, hipStream_t stream)
+                 int bytes_per_elem, const Maker& make, hipStream_t stream, size_t streaming_from = kStreamingBytes)
 {
     for (int begin = 0; begin < count; begin += kMultiTensors) {
         MultiTable t{};
@@ -660,7 +665,7 @@ int launch_multi(const char* who, int count, float* const* const* buffers, const
             t.n[used] = len;
             t.first_block[used] = static_cast<uint32_t>(blocks);
             if (apply_decay && apply_decay[begin + i]) t.decay_mask |= 1u << used;
-            if (len * static_cast<size_t>(bytes_per_elem) >= kStreamingBytes) t.past_cache_mask |= 1u << used;
+            if (len * static_cast<size_t>(bytes_per_elem) >= streaming_from) t.past_cache_mask |= 1u << used;
             if (aligned) t.vector_mask |= 1u << used;
             blocks += (len + kMultiPerBlock - 1) / kMultiPerBlock;
             ++used;
@@ -1031,6 +1036,15 @@ int pxh_adam_update_multi(int count, float* const* w, float* const* d, float* co
     op.lr = lr; op.eps = eps;
     float* const* const buffers[4] = { w, d, m, v };
     return launch_multi<4>("pxh_adam_update_multi", count, buffers, n, apply_decay, 32, AdamMaker{ op }, as_stream(stream));
+}
+
+int pxh_fill_f32_multi(int count, float* const* x, const size_t* n, float value, void* stream)
+{
+    if (count < 0 || (count && (!x || !n))) return fail_invalid("pxh_fill_f32_multi: bad argument");
+    float* const* const buffers[4] = { x, nullptr, nullptr, nullptr };
+    // a fill streams past the caches from the size on that the single call does
+    return launch_multi<1>("pxh_fill_f32_multi", count, buffers, n, nullptr, 4, FillMaker{ value }, as_stream(stream),
+                           kFillStreamingBytes);
 }
 
 int pxh_sgd_update_multi(int count, float* const* w, float* const* d, const size_t* n, const int* apply_decay, int batch,

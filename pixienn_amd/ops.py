@@ -372,6 +372,12 @@ def sgd_update(w, d, batch, lr, momentum, decay=0.0, apply_decay=False):
          int(bool(apply_decay)), _stream())
 
 
+def fill_multi(xs, value):
+    """pxh_fill_f32 for a list of float tensors in a few launches."""
+    _chk_all(*xs)
+    call("pxh_fill_f32_multi", len(xs), _pointer_table(xs), _size_table(xs), float(value), _stream())
+
+
 def rescale_clip_multi(xs, threshold=0.0, clip=0.0, norms=None):
     """pxh_rescale_clip for a list of tensors in a few launches; `norms`: device float tensor, one per tensor."""
     _chk_all(*xs, norms)

@@ -365,6 +365,19 @@ def test_sgd_update_multi_gives_every_tensor_what_the_single_call_gives(ops):
             assert_bit_exact(host(many[i]), host(one[i]), "sgd multi %s[%d] n=%d" % (name, i, MULTI_SIZES[i]))
 
 
+def test_fill_multi_writes_every_tensor_and_nothing_else(ops):
+    import torch
+    # each tensor sits inside a larger buffer whose other elements must stay untouched
+    bufs = [torch.full((n + 8,), 7.0, device="cuda") for n in MULTI_SIZES]
+    views = [b[4:4 + n] for b, n in zip(bufs, MULTI_SIZES)]
+    views[5] = bufs[5][5:5 + MULTI_SIZES[5]]            # one view off the 16-byte grid
+    ops.fill_multi(views, -0.5)
+    for b, v, n in zip(bufs, views, MULTI_SIZES):
+        assert bool((v == -0.5).all())
+        assert int((b == 7.0).sum()) == 8
+    ops.fill_multi([], 1.0)
+
+
 def test_update_multi_edge_cases(ops):
     import torch
     from pixienn_amd import capi
