@@ -50,6 +50,9 @@ def parse_args():
     ap.add_argument("--no-extras", action="store_true", help="skip the other kernels of the path")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-batch", type=int, default=64, help="images per shape in the CPU sample")
+    ap.add_argument("--plain-step", action="store_true",
+                    help="with --only-model-order: the step as the reference runs it only, none of the optional forms "
+                         "(for a kernel trace whose shares are those of one step)")
     ap.add_argument("--only-model-order", action="store_true",
                     help="run only the YOLOv3 training step in model order (for a kernel trace of that step)")
     return ap.parse_args()
@@ -163,7 +166,7 @@ def run_epilogue_step(ops, shapes, events=None, torch=None, raw=False):
             events.append((act, a, b))
 
 
-def measure_model_order(torch, ops, wl, timer, N=16):
+def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     """One training step of YOLOv3 @608 at batch N with every non-convolution kernel launched in the
     model's own layer order on tensors of their own (21 GB): forward (per layer the delta zero-fill
     of Layer::forward, then the layer), backward in reverse (per layer the gradient rescale + clip
@@ -290,6 +293,10 @@ def measure_model_order(torch, ops, wl, timer, N=16):
     # nothing reads a delta after backward: the pass over them in update() is dead work that a host
     # may drop (Context::helpersTouchDeltaInUpdate of the C++ layer interface)
     out["calls"] = dict(launches)
+    if plain_only:
+        del T, w, g, m, v
+        torch.cuda.empty_cache()
+        return out
     out["update_without_delta_pass_ms"] = round(timer.time(lambda i: update(i, False), 3, warm=1), 3)
     # the 23 shortcuts as first writers of the 46 deltas they reach first: no zero-fill of those,
     # no read of them in the shortcut's backward (an option of the C++ layer interface, "first_writer")
@@ -637,7 +644,8 @@ def main():
     torch.cuda.set_device(0)
     timer = Timer(torch)
     if args.only_model_order:
-        print(json.dumps({"noconv_step_in_model_order_yolov3_608": measure_model_order(torch, ops, wl, timer)}),
+        print(json.dumps({"noconv_step_in_model_order_yolov3_608": measure_model_order(torch, ops, wl, timer,
+                                                                                        plain_only=args.plain_step)}),
               flush=True)
         return
 
