@@ -101,6 +101,22 @@ int pxh_bn_train_act_forward(const float* x, float* y, float* pre_activation, fl
                              int batch, int channels, int spatial, int activation,
                              void* workspace, size_t workspace_bytes, void* stream);
 
+/* pxh_bn_train_act_forward for callers that cannot allocate device memory and have no workspace
+ * to pass (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc): same
+ * arguments without the workspace, same kernels, same results.  The partial sums and per-channel
+ * constants go into a buffer of PXH_BN_STATIC_SCRATCH_BYTES built into the library's device code
+ * (each GPU holds its copy until the process ends); the call allocates and frees nothing.  A shape
+ * for which pxh_bn_workspace_bytes() exceeds that size is rejected with PXH_ERR_WORKSPACE before
+ * anything is launched.  All calls on one GPU share the buffer: two that overlap in time (different
+ * streams or threads) race; order them, or use the workspace form.  The first call on a device looks
+ * up the buffer's address, make it outside a capture.
+ * No counterpart in the reference (its cuDNN calls own their scratch). */
+#define PXH_BN_STATIC_SCRATCH_BYTES ((size_t) 1 << 20)
+int pxh_bn_train_act_forward_static(const float* x, float* y, float* pre_activation, float* x_saved,
+                                    float* x_norm, float* mean, float* var, float* rolling_mean,
+                                    float* rolling_var, const float* scale, const float* bias,
+                                    int batch, int channels, int spatial, int activation, void* stream);
+
 /* Per-channel batch statistics only (first half of the above). */
 int pxh_bn_stats(const float* x, float* mean, float* var, int batch, int channels, int spatial,
                  void* workspace, size_t workspace_bytes, void* stream);

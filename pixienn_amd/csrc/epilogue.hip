@@ -12,10 +12,48 @@
 #include <mutex>
 #include <vector>
 
+// Device memory for pxh_bn_train_act_forward_static, the entry point for callers that must not
+// allocate: the partial sums and per-channel constants its kernels pass from one launch to the next.
+// Every GPU the library runs on holds its own copy until the process ends.  In host code the name is
+// only a handle for hipGetSymbolAddress; kernels are given the address that call returns.
+constexpr size_t kStaticScratchBytes = PXH_BN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace pxh {
 namespace {
 
 constexpr float kEps = .00001f;
+
+// The device address of `scratch` on the current device, looked up once per device.
+int static_scratch(const char* who, void** out)
+{
+    constexpr int kDevices = 64;
+    static std::mutex mutex;
+    static void* address[kDevices] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        set_error("%s: hipGetDevice: %s", who, hipGetErrorString(e));
+        return static_cast<int>(e);
+    }
+    if (dev < 0 || dev >= kDevices) {
+        set_error("%s: device %d is beyond the %d devices the library keeps scratch addresses for", who, dev,
+                  kDevices);
+        return PXH_ERR_UNSUPPORTED;
+    }
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!address[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            set_error("%s: hipGetSymbolAddress(scratch) on device %d: %s", who, dev, hipGetErrorString(e));
+            return e != hipSuccess ? static_cast<int>(e) : PXH_ERR_WORKSPACE;
+        }
+        address[dev] = p;
+    }
+    *out = address[dev];
+    return PXH_OK;
+}
 
 // Folded per-channel constants of the forward pass (32 bytes: two 128-bit loads).
 struct __attribute__((aligned(16))) FoldCoef {
@@ -1020,6 +1058,60 @@ int launch_stats(const float* x, float* mean, float* var, float* rolling_mean, f
     return check_launch("bn_stats_finish");
 }
 
+// BN training forward + activation.  `get_workspace(need, &ws)` is asked for the `need` bytes of the
+// three-launch form only when the shape does not take the one-launch form, which uses none.
+template<typename GetWorkspace>
+int bn_train_forward(const char* who, const float* x, float* y, float* pre_activation, float* x_saved, float* x_norm,
+                     float* mean, float* var, float* rolling_mean, float* rolling_var, const float* scale,
+                     const float* bias, int batch, int channels, int spatial, int activation,
+                     GetWorkspace&& get_workspace, void* stream)
+{
+    if (!x || !y || !mean || !var || !rolling_mean || !rolling_var || !scale || !bias)
+        return fail_invalid("%s: null pointer", who);
+    if (x_saved == x) return fail_invalid("%s: x_saved must not alias x", who);
+    EpilogueArgs a{};
+    int rc = check_shape(who, batch, channels, spatial, &a.total);
+    if (rc) return rc;
+    hipStream_t s = as_stream(stream);
+    {
+        const bool vec = spatial % 4 == 0 && aligned16(x) && aligned16(y) && aligned16(pre_activation) &&
+                         aligned16(x_saved) && aligned16(x_norm);
+        const int per_thread = resident_vectors(batch, channels, spatial, vec);
+        if (per_thread) {
+            const ResidentFwdArgs r{ x, y, pre_activation, x_saved, x_norm, mean, var, rolling_mean, rolling_var,
+                                     scale, bias, resident_geom(batch, channels, spatial) };
+            const dim3 grid(channels), block(kResidentThreads);
+            int large_lds_rc = PXH_OK;
+            const bool known = dispatch_activation(activation, [&]<int ACT>() {
+                if (per_thread > kResidentVectors) {
+                    auto kernel = bn_resident_fwd_kernel<ACT, 4, kResidentLargeRegs, kResidentLargeLds>;
+                    large_lds_rc = allow_large_lds(reinterpret_cast<const void*>(kernel));
+                    if (large_lds_rc == PXH_OK)
+                        hipLaunchKernelGGL(kernel, grid, block, kResidentLargeLdsBytes, s, r);
+                } else if (vec) {
+                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 4, kResidentVectors, 0>), grid, block, 0, s, r);
+                } else {
+                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 1, kResidentVectors, 0>), grid, block, 0, s, r);
+                }
+            });
+            if (!known) return fail_invalid("%s: unknown activation %d", who, activation);
+            if (large_lds_rc) return large_lds_rc;
+            return check_launch(who);
+        }
+    }
+    void* ws;
+    rc = get_workspace(workspace_bytes(batch, channels, spatial), &ws);
+    if (rc) return rc;
+    FoldCoef* table = static_cast<FoldCoef*>(coef_region(ws, batch, channels, spatial));
+    rc = launch_stats(x, mean, var, rolling_mean, rolling_var, scale, bias, table, batch, channels, spatial, a.total,
+                      ws, s);
+    if (rc) return rc;
+    a.x = x; a.y = y; a.pre = pre_activation; a.x_saved = x_saved; a.x_norm = x_norm;
+    a.table = table;
+    a.by_spatial = FastDiv(spatial); a.by_channels = FastDiv(channels);
+    return launch_epilogue_fwd<true>(who, a, activation, s);
+}
+
 }  // namespace
 }  // namespace pxh
 
@@ -1117,50 +1209,31 @@ int pxh_bn_train_act_forward(const float* x, float* y, float* pre_activation, fl
                              const float* bias, int batch, int channels, int spatial, int activation,
                              void* workspace, size_t workspace_bytes_given, void* stream)
 {
-    if (!x || !y || !mean || !var || !rolling_mean || !rolling_var || !scale || !bias)
-        return fail_invalid("pxh_bn_train_act_forward: null pointer");
-    if (x_saved == x) return fail_invalid("pxh_bn_train_act_forward: x_saved must not alias x");
-    EpilogueArgs a{};
-    int rc = check_shape("pxh_bn_train_act_forward", batch, channels, spatial, &a.total);
-    if (rc) return rc;
-    hipStream_t s = as_stream(stream);
-    {
-        const bool vec = spatial % 4 == 0 && aligned16(x) && aligned16(y) && aligned16(pre_activation) &&
-                         aligned16(x_saved) && aligned16(x_norm);
-        const int per_thread = resident_vectors(batch, channels, spatial, vec);
-        if (per_thread) {
-            const ResidentFwdArgs r{ x, y, pre_activation, x_saved, x_norm, mean, var, rolling_mean, rolling_var,
-                                     scale, bias, resident_geom(batch, channels, spatial) };
-            const dim3 grid(channels), block(kResidentThreads);
-            int large_lds_rc = PXH_OK;
-            const bool known = dispatch_activation(activation, [&]<int ACT>() {
-                if (per_thread > kResidentVectors) {
-                    auto kernel = bn_resident_fwd_kernel<ACT, 4, kResidentLargeRegs, kResidentLargeLds>;
-                    large_lds_rc = allow_large_lds(reinterpret_cast<const void*>(kernel));
-                    if (large_lds_rc == PXH_OK)
-                        hipLaunchKernelGGL(kernel, grid, block, kResidentLargeLdsBytes, s, r);
-                } else if (vec) {
-                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 4, kResidentVectors, 0>), grid, block, 0, s, r);
-                } else {
-                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 1, kResidentVectors, 0>), grid, block, 0, s, r);
-                }
-            });
-            if (!known) return fail_invalid("pxh_bn_train_act_forward: unknown activation %d", activation);
-            if (large_lds_rc) return large_lds_rc;
-            return check_launch("pxh_bn_train_act_forward");
-        }
-    }
-    void* ws;
-    rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws);
-    if (rc) return rc;
-    FoldCoef* table = static_cast<FoldCoef*>(coef_region(ws, batch, channels, spatial));
-    rc = launch_stats(x, mean, var, rolling_mean, rolling_var, scale, bias, table, batch, channels, spatial, a.total,
-                      ws, s);
-    if (rc) return rc;
-    a.x = x; a.y = y; a.pre = pre_activation; a.x_saved = x_saved; a.x_norm = x_norm;
-    a.table = table;
-    a.by_spatial = FastDiv(spatial); a.by_channels = FastDiv(channels);
-    return launch_epilogue_fwd<true>("pxh_bn_train_act_forward", a, activation, s);
+    return bn_train_forward(
+        "pxh_bn_train_act_forward", x, y, pre_activation, x_saved, x_norm, mean, var, rolling_mean, rolling_var,
+        scale, bias, batch, channels, spatial, activation,
+        [&](size_t need, void** ws) { return resolve_workspace(workspace, workspace_bytes_given, need, ws); }, stream);
+}
+
+int pxh_bn_train_act_forward_static(const float* x, float* y, float* pre_activation, float* x_saved, float* x_norm,
+                                    float* mean, float* var, float* rolling_mean, float* rolling_var,
+                                    const float* scale, const float* bias, int batch, int channels, int spatial,
+                                    int activation, void* stream)
+{
+    const char* who = "pxh_bn_train_act_forward_static";
+    return bn_train_forward(
+        who, x, y, pre_activation, x_saved, x_norm, mean, var, rolling_mean, rolling_var, scale, bias, batch,
+        channels, spatial, activation,
+        [&](size_t need, void** ws) {
+            if (need > kStaticScratchBytes) {
+                set_error("%s: batch %d x channels %d x spatial %d needs %zu bytes of scratch, the built-in buffer "
+                          "holds %zu; use pxh_bn_train_act_forward with a workspace of pxh_bn_workspace_bytes()",
+                          who, batch, channels, spatial, need, kStaticScratchBytes);
+                return PXH_ERR_WORKSPACE;
+            }
+            return static_scratch(who, ws);
+        },
+        stream);
 }
 
 int pxh_bn_act_backward(float* delta, const float* x, const float* pre_activation, const float* mean,
