@@ -149,7 +149,7 @@ TRAIN_SHAPES = [(4, 8, 52 * 52), (3, 16, 361), (16, 5, 169), (2, 3, 4096 + 512),
                 (8, 192, 4800), (9, 100, 4096 + 8)]
 
 
-@pytest.mark.parametrize("act", ["leaky", "mish", "linear"])
+@pytest.mark.parametrize("act", ["leaky", "mish", "linear", "swish", "logistic"])
 def test_bn_train_forward_matches_oracle(ops, oracle, act):
     for si, (N, C, HW) in enumerate(TRAIN_SHAPES):
         x, scale, bias, rmean, rvar = bn_case(400 + si, N, C, HW, spread=1.5)
@@ -202,7 +202,7 @@ def test_bn_stats_beats_sequential_fp32_at_scale(ops, oracle):
     assert_close(gv, v64, 1e-6, 1e-3, "var vs fp64")
 
 
-@pytest.mark.parametrize("act", ["leaky", "mish", "linear", "logistic"])
+@pytest.mark.parametrize("act", ["leaky", "mish", "linear", "logistic", "swish"])
 @pytest.mark.parametrize("with_pre", [True, False])
 def test_bn_backward_matches_oracle(ops, oracle, act, with_pre):
     for si, (N, C, HW) in enumerate(TRAIN_SHAPES):
@@ -229,6 +229,51 @@ def test_bn_backward_matches_oracle(ops, oracle, act, with_pre):
         assert_close(host(gmd), md_w, RTOL, sum_scale, what + " mean delta")
         assert_close(host(gvd), vd_w, RTOL, sum_scale, what + " var delta")
         assert_close(host(gd), d_w, RTOL, 1e-1, what + " dx")
+
+
+@pytest.mark.parametrize("side", [152, 608])
+def test_bn_distance_from_the_sequential_fp32_reference_at_training_sizes(ops, oracle, side):
+    """At 16 x 152^2 and 16 x 608^2 values per channel (the batch-16, 608 x 608 training shapes) the CPU
+    layer's left-to-right fp32 sums have drifted from the exact statistics by 1e-4 and 7e-3.  The kernel is
+    held to 1e-5 of the checker's double-accumulator variant there; this test records how far it then is
+    from the strict, reference-ordered variant and asserts that the whole of that distance is the strict
+    variant's own drift: d(kernel, strict) <= d(strict, wide) + the 1e-5 the kernel is allowed."""
+    N, C, HW = 16, 4, side * side
+    x = (wl.normal(980 + side, (N, C, HW, 1)) + wl.normal(981 + side, (1, C, 1, 1), std=0.5)).astype(F)
+    scale, bias, rmean, rvar = wl.bn_params(982 + side, C)
+    delta = wl.normal(983 + side, x.shape)
+    res = {}
+    for wide in (False, True):
+        out = x.copy(); pre = np.empty_like(x); xs = np.empty_like(x); xn = np.empty_like(x)
+        mean = np.zeros(C, F); var = np.zeros(C, F)
+        oracle.conv_epilogue_forward(True, True, "linear", N, C, HW, 1, out, pre, mean, var, rmean.copy(),
+                                     rvar.copy(), scale, bias, xs, xn, wide=wide)
+        d = delta.copy(); su = np.zeros(C, F); bu = np.zeros(C, F); md = np.zeros(C, F); vd = np.zeros(C, F)
+        oracle.conv_epilogue_backward(True, "linear", N, C, HW, 1, d, pre, mean, var, md, vd, scale, su, bu, xs, xn,
+                                      wide=wide)
+        res[wide] = dict(mean=mean, var=var, y=out, dx=d)
+        del pre, xs, xn
+    gx = gpu(x); gy = gpu(np.zeros_like(x))
+    gm, gv = gpu(np.zeros(C, F)), gpu(np.zeros(C, F))
+    ops.bn_train_act_forward(gx, gy, gm, gv, gpu(rmean), gpu(rvar), gpu(scale), gpu(bias), "linear")
+    gd = gpu(delta)
+    ops.bn_act_backward(gd, gx, gm, gv, gpu(scale), gpu(bias), gpu(np.zeros(C, F)), gpu(np.zeros(C, F)), "linear")
+    got = dict(mean=host(gm), var=host(gv), y=host(gy), dx=host(gd))
+    sigma = np.sqrt(res[True]["var"].astype(np.float64))
+    y_floor = ((np.abs(res[True]["mean"]) + sigma) / sigma).reshape(1, C, 1, 1)
+    floors = dict(mean=1e-3, var=1e-3, y=y_floor, dx=1e-1)
+    line = []
+    def distance(a, b, k):       # every distance in units of the double-accumulator result
+        return float(np.max(np.abs(a.astype(np.float64) - b) / np.maximum(np.abs(res[True][k]), floors[k])))
+
+    for k in ("mean", "var", "y", "dx"):
+        to_wide = distance(got[k], res[True][k], k)
+        to_strict = distance(got[k], res[False][k], k)
+        drift = distance(res[False][k], res[True][k], k)
+        line.append("%s: kernel-wide %.2e, kernel-strict %.2e, strict-wide %.2e" % (k, to_wide, to_strict, drift))
+        assert to_wide <= RTOL, (k, to_wide)
+        assert to_strict <= drift + RTOL, (k, to_strict, drift)
+    print("\n16 x %d^2 values per channel -- " % side + "; ".join(line))
 
 
 @pytest.mark.parametrize("act", ["linear", "leaky", "logistic"])

@@ -147,7 +147,7 @@ def test_yolo_training_pass_random_heads(ops, oracle):
                                                                            counts.tolist())
         want = oracle_head(oracle, x, truths, counts, W, H, K, mask, anchors, net, **kw)
         got = gpu_head(ops, x, truths, counts, W, H, K, mask, anchors, net, **kw)
-        compare_head(got, want, what, sum_rtol=5e-5)
+        compare_head(got, want, what, masks, kw, sum_rtol=5e-5)
 
 
 def test_yolo_detections_random_heads(ops, oracle):

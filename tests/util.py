@@ -58,9 +58,10 @@ def assert_close(got, want, rtol, floor, what=""):
     bad = err > bound
     if bad.any():
         i = tuple(np.argwhere(bad)[0])
-        raise AssertionError("%s: %d of %d beyond rtol %g (floor %g); first at %s: got %.9g want %.9g; worst rel %.3g"
-                             % (what, int(bad.sum()), bad.size, rtol, floor, i, got[i], want[i],
-                                float(np.max(err / np.maximum(np.abs(want), floor)))))
+        here = float(np.broadcast_to(np.asarray(floor, dtype=np.float64), want.shape)[i])
+        raise AssertionError("%s: %d of %d beyond rtol %g (floor %g there); first at %s: got %.9g want %.9g; "
+                             "worst rel %.3g" % (what, int(bad.sum()), bad.size, rtol, here, i, got[i], want[i],
+                                                 float(np.max(err / np.maximum(np.abs(want), floor)))))
 
 
 def max_rel(got, want, floor):
