@@ -41,9 +41,16 @@ enum pxh_activation {
 const char* pxh_last_error(void);
 /* library version, bumped when a signature changes */
 int pxh_abi_version(void);
-/* Host-only check hook: n / d through the multiply-high division the index maps use
- * (n < 2^31, d >= 1).  No reference counterpart. */
-unsigned pxh_debug_fastdiv(unsigned n, unsigned d);
+
+/* Entry points that take `(workspace, workspace_bytes)` use a per-device buffer owned by the library
+ * when given NULL.  That buffer grows when a call needs more than it holds, which allocates device
+ * memory and is therefore refused (PXH_ERR_WORKSPACE) while the call's stream is being captured into a
+ * graph.  pxh_reserve_workspace makes the current device's buffer hold at least `bytes` (the largest
+ * *_workspace_bytes() of the calls to come) ahead of time; blocks handed out earlier stay allocated, so
+ * addresses that queued work or captured graphs hold remain valid.  The buffer is shared by every
+ * NULL-workspace call on the device: calls that may overlap (several streams or threads) must pass
+ * workspaces of their own.  No counterpart in the reference (cuDNN and cuBLAS own their scratch). */
+int pxh_reserve_workspace(size_t bytes);
 
 /* ------------------------------------------------------------------------
  * Conv-layer epilogue, forward.
@@ -315,9 +322,6 @@ size_t pxh_nms_workspace_bytes(int capacity);
 int pxh_nms(const pxh_detection* records, const int* count, int capacity, int batch, int classes,
             float threshold, pxh_detection* kept, int* kept_count, void* workspace,
             size_t workspace_bytes, void* stream);
-/* Test hook: number (1..6) of whole-array sweeps of the duplicate step before the per-image loop
- * finishes what they left; returns the previous value.  Results do not depend on it. */
-int pxh_debug_nms_sweeps(int sweeps);
 
 size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int width, int height,
                                 int max_truth);

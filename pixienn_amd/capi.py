@@ -59,7 +59,6 @@ SIGNATURES = {
     "pxh_yolo_detections": [P, I, P, I, P, I, I, I, I, I, I, I, I, F, P, I, P, P],
     "pxh_yolo_detections_append": [P, I, P, I, P, I, I, I, I, I, I, I, I, F, U, P, I, P, P],
     "pxh_nms": [P, P, I, I, I, F, P, P, P, Z, P],
-    "pxh_debug_nms_sweeps": [I],
     "pxh_adam": [I, P, P, P, F, F, F, F, I, P],
     "pxh_adam_update": [Z, P, P, P, P, I, I, F, F, F, F, F, I, P],
     "pxh_adam_update_multi": [I, P, P, P, P, P, P, I, I, F, F, F, F, F, P],
@@ -76,7 +75,13 @@ _OTHER_RETURNS = {
     "pxh_rescale_multi_workspace_bytes": (Z, []),
     "pxh_yolo_workspace_bytes": (Z, [I, I, I, I, I, I]),
     "pxh_nms_workspace_bytes": (Z, [I]),
+    "pxh_reserve_workspace": (I, [Z]),
+}
+# test hooks (pixienn_amd/csrc/pixienn_hip_test.h): exported, but not part of the C ABI
+_TEST_HOOKS = {
     "pxh_debug_fastdiv": (ctypes.c_uint, [ctypes.c_uint, ctypes.c_uint]),
+    "pxh_debug_nms_sweeps": (I, [I]),
+    "pxh_debug_library_workspace": (P, [Z]),
 }
 
 
@@ -100,7 +105,7 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = I
-    for name, (res, args) in _OTHER_RETURNS.items():
+    for name, (res, args) in list(_OTHER_RETURNS.items()) + list(_TEST_HOOKS.items()):
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = res
@@ -109,7 +114,12 @@ def load():
 
 
 def declared_symbols():
+    """The C ABI proper (include/pixienn_hip.h)."""
     return sorted(list(SIGNATURES) + list(_OTHER_RETURNS))
+
+
+def test_hook_symbols():
+    return sorted(_TEST_HOOKS)
 
 
 def last_error():

@@ -25,10 +25,9 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---------------------------------------------------------------- workspace
-// Per-device scratch the library owns, grown on demand and kept until exit.
-void* library_workspace(size_t bytes);
-// Picks the caller's workspace when given (checking its size), else the library's.
-int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out);
+// Picks the caller's workspace when given (checking its size), else the per-device buffer the
+// library owns, which grows on demand (never while `stream` is being captured) and is kept until exit.
+int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out, hipStream_t stream);
 
 // ---------------------------------------------------------------- fast division
 // q = n / d for 0 <= n < 2^31 by a multiply-high and a shift (d >= 1).

@@ -911,7 +911,7 @@ int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* nor
     const bool rescale = threshold > 0.0f || norm_out != nullptr;
     if (!rescale && !(clip > 0.0f)) return PXH_OK;
     void* ws = nullptr;
-    int rc = resolve_workspace(workspace, workspace_bytes, pxh_rescale_workspace_bytes(), &ws);
+    int rc = resolve_workspace(workspace, workspace_bytes, pxh_rescale_workspace_bytes(), &ws, as_stream(stream));
     if (rc) return rc;
     double2* partial = static_cast<double2*>(ws);
     hipStream_t s = as_stream(stream);
@@ -951,7 +951,7 @@ int pxh_rescale_clip_multi(int count, float* const* x, const size_t* n, float th
     const bool rescale = threshold > 0.0f || norms != nullptr;
     if (!rescale && !(clip > 0.0f)) return PXH_OK;
     void* ws = nullptr;
-    int rc = resolve_workspace(workspace, workspace_bytes, pxh_rescale_multi_workspace_bytes(), &ws);
+    int rc = resolve_workspace(workspace, workspace_bytes, pxh_rescale_multi_workspace_bytes(), &ws, as_stream(stream));
     if (rc) return rc;
     double2* partial = static_cast<double2*>(ws);
     hipStream_t s = as_stream(stream);

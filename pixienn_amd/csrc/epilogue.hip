@@ -1166,7 +1166,7 @@ int pxh_bn_infer_act_forward(const float* x, float* y, float* pre_activation, co
     int rc = check_shape("pxh_bn_infer_act_forward", batch, channels, spatial, &total);
     if (rc) return rc;
     void* ws;
-    rc = resolve_workspace(workspace, workspace_bytes_given, pxh_bn_folded_bytes(channels), &ws);
+    rc = resolve_workspace(workspace, workspace_bytes_given, pxh_bn_folded_bytes(channels), &ws, as_stream(stream));
     if (rc) return rc;
     rc = pxh_bn_fold(rolling_mean, rolling_var, scale, bias, channels, ws, stream);
     if (rc) return rc;
@@ -1198,7 +1198,7 @@ int pxh_bn_stats(const float* x, float* mean, float* var, int batch, int channel
     int rc = check_shape("pxh_bn_stats", batch, channels, spatial, &total);
     if (rc) return rc;
     void* ws;
-    rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws);
+    rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws, as_stream(stream));
     if (rc) return rc;
     return launch_stats(x, mean, var, nullptr, nullptr, nullptr, nullptr, nullptr, batch, channels, spatial, total,
                         ws, as_stream(stream));
@@ -1212,7 +1212,7 @@ int pxh_bn_train_act_forward(const float* x, float* y, float* pre_activation, fl
     return bn_train_forward(
         "pxh_bn_train_act_forward", x, y, pre_activation, x_saved, x_norm, mean, var, rolling_mean, rolling_var,
         scale, bias, batch, channels, spatial, activation,
-        [&](size_t need, void** ws) { return resolve_workspace(workspace, workspace_bytes_given, need, ws); }, stream);
+        [&](size_t need, void** ws) { return resolve_workspace(workspace, workspace_bytes_given, need, ws, as_stream(stream)); }, stream);
 }
 
 int pxh_bn_train_act_forward_static(const float* x, float* y, float* pre_activation, float* x_saved, float* x_norm,
@@ -1273,7 +1273,7 @@ int pxh_bn_act_backward(float* delta, const float* x, const float* pre_activatio
         }
     }
     void* ws;
-    rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws);
+    rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws, as_stream(stream));
     if (rc) return rc;
     const ReduceGeom g = make_geom(batch, channels, spatial);
     double2* partial = static_cast<double2*>(ws);
@@ -1329,7 +1329,7 @@ int pxh_bias_act_backward(float* delta, const float* pre_activation, float* bias
     int rc = check_shape("pxh_bias_act_backward", batch, channels, spatial, &total);
     if (rc) return rc;
     void* ws;
-    rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws);
+    rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws, as_stream(stream));
     if (rc) return rc;
     hipStream_t s = as_stream(stream);
     const ReduceGeom g = make_geom(batch, channels, spatial);

@@ -13,6 +13,9 @@
 //   4. the greedy pass the same way, one workgroup per group, states in LDS;
 //   5. compaction of the kept records in rank order.
 #include "common.h"
+#include "pixienn_hip_test.h"
+
+#include <atomic>
 
 namespace pxh {
 namespace {
@@ -648,7 +651,7 @@ Workspace carve(void* base, int capacity)
     return w;
 }
 
-int g_sweeps = 6;      // parallel sweeps of the duplicate pass before the per-image loop takes over
+std::atomic<int> g_sweeps{ 6 };      // parallel sweeps of the duplicate pass before the per-image loop takes over
 
 }  // namespace
 }  // namespace pxh
@@ -665,9 +668,8 @@ size_t pxh_nms_workspace_bytes(int capacity)
 
 int pxh_debug_nms_sweeps(int sweeps)
 {
-    const int before = g_sweeps;
-    if (sweeps >= 1 && sweeps <= 6) g_sweeps = sweeps;
-    return before;
+    if (sweeps >= 1 && sweeps <= 6) return g_sweeps.exchange(sweeps);
+    return g_sweeps.load();
 }
 
 int pxh_nms(const pxh_detection* records, const int* count, int capacity, int batch, int classes, float threshold,
@@ -689,7 +691,7 @@ int pxh_nms(const pxh_detection* records, const int* count, int capacity, int ba
         return check_launch("pxh_nms");
     }
     void* ws;
-    int rc = resolve_workspace(workspace, workspace_bytes, carve(nullptr, capacity).bytes, &ws);
+    int rc = resolve_workspace(workspace, workspace_bytes, carve(nullptr, capacity).bytes, &ws, as_stream(stream));
     if (rc) return rc;
     const Workspace w = carve(ws, capacity);
     hipStream_t s = as_stream(stream);
@@ -720,7 +722,7 @@ int pxh_nms(const pxh_detection* records, const int* count, int capacity, int ba
     a.group_key = w.keys[from]; a.rank = w.vals[from];
     a.box = w.box; a.seg = w.seg; a.state = w.state; a.keep = w.keep; a.resume = w.resume; a.counters = w.counters;
     hipLaunchKernelGGL(nms_gather_kernel, per_record, lanes, 0, s, a);
-    const int sweeps = g_sweeps;
+    const int sweeps = g_sweeps.load();      // read once: a call never sees it change
     // one wave per record, at most 64 Ki workgroups (the rest of a longer list comes round again)
     const unsigned sweep_blocks = grid_for(capacity, kBlock / kWave) < 65536u ? grid_for(capacity, kBlock / kWave) : 65536u;
     a.waves = sweep_blocks * (kBlock / kWave);

@@ -1,0 +1,30 @@
+/*
+ * Test hooks of libpixienn_hip.so.  Exported so that the test-suite can reach them through the
+ * shared library, but not part of the C ABI in include/pixienn_hip.h: nothing here is installed,
+ * no host should call these, and none of them has a counterpart in the reference.
+ */
+#ifndef PIXIENN_HIP_TEST_H
+#define PIXIENN_HIP_TEST_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* n / d through the multiply-high division the index maps use (n < 2^31, d >= 1).  Host only. */
+unsigned pxh_debug_fastdiv(unsigned n, unsigned d);
+
+/* Number (1..6) of whole-array sweeps of pxh_nms's duplicate step before the per-image loop finishes
+ * what they left; returns the previous value.  Results do not depend on it.  A call of pxh_nms reads
+ * it once, when it starts. */
+int pxh_debug_nms_sweeps(int sweeps);
+
+/* Address of the current device's library workspace after making it hold at least `bytes`
+ * (NULL when that fails): lets a test see that a block handed out earlier stays where it was. */
+void* pxh_debug_library_workspace(size_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,5 +1,6 @@
 // Error reporting, per-device workspace and small utility entry points.
 #include "common.h"
+#include "pixienn_hip_test.h"
 
 #include <mutex>
 
@@ -44,32 +45,50 @@ int check_launch(const char* what)
     return PXH_OK;
 }
 
-void* library_workspace(size_t bytes)
+// The per-device buffer behind every call that passes no workspace.  A block that has been handed
+// out is never freed: work already queued, and graphs that were captured with its address, may still
+// use it after a later call has asked for more and been given a larger block.  Growing allocates, so
+// it is refused while `stream` is being captured; pxh_reserve_workspace sizes the buffer beforehand.
+int library_workspace(size_t bytes, hipStream_t stream, bool may_grow_in_capture, void** out)
 {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("library workspace: no usable current device (%s)", hipGetErrorString(e));
+        return PXH_ERR_WORKSPACE;
+    }
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     DeviceScratch& s = g_scratch[dev];
-    if (s.bytes >= bytes && s.ptr) return s.ptr;
-    // Grow: work queued on the old buffer must finish before it is released.
-    if (s.ptr) {
-        if (hipDeviceSynchronize() != hipSuccess) return nullptr;
-        (void) hipFree(s.ptr);
-        s.ptr = nullptr;
-        s.bytes = 0;
+    if (s.bytes >= bytes && s.ptr) {
+        *out = s.ptr;
+        return PXH_OK;
     }
-    // 16 MB covers every shape of a YOLOv3-sized network, so the buffer rarely grows after the first
-    // call (growing synchronises the device, which a call inside a graph capture must not do)
-    size_t want = bytes < (16u << 20) ? (16u << 20) : bytes;
-    if (hipMalloc(&s.ptr, want) != hipSuccess) {
-        s.ptr = nullptr;
-        return nullptr;
+    if (!may_grow_in_capture) {
+        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &status) == hipSuccess && status != hipStreamCaptureStatusNone) {
+            set_error("the library's workspace holds %zu bytes and this call needs %zu: it cannot grow while the "
+                      "stream is being captured; call pxh_reserve_workspace(%zu) before the capture, or pass a "
+                      "workspace", s.bytes, bytes, bytes);
+            return PXH_ERR_WORKSPACE;
+        }
+        (void) hipGetLastError();
     }
+    // 16 MB covers every shape of a YOLOv3-sized network, so the buffer rarely grows after the first call
+    const size_t want = bytes < (16u << 20) ? (16u << 20) : bytes;
+    void* fresh = nullptr;
+    e = hipMalloc(&fresh, want);
+    if (e != hipSuccess) {
+        set_error("could not allocate %zu bytes of device workspace: %s", want, hipGetErrorString(e));
+        return PXH_ERR_WORKSPACE;
+    }
+    // the outgrown block stays allocated until the process ends (see above)
+    s.ptr = fresh;
     s.bytes = want;
-    return s.ptr;
+    *out = s.ptr;
+    return PXH_OK;
 }
 
-int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out)
+int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out, hipStream_t stream)
 {
     if (user) {
         if (user_bytes < need) {
@@ -83,13 +102,7 @@ int resolve_workspace(void* user, size_t user_bytes, size_t need, void** out)
         *out = user;
         return PXH_OK;
     }
-    void* p = library_workspace(need);
-    if (!p) {
-        set_error("could not allocate %zu bytes of device workspace", need);
-        return PXH_ERR_WORKSPACE;
-    }
-    *out = p;
-    return PXH_OK;
+    return library_workspace(need, stream, false, out);
 }
 
 }  // namespace pxh
@@ -99,6 +112,19 @@ extern "C" {
 const char* pxh_last_error(void) { return pxh::g_error; }
 
 int pxh_abi_version(void) { return 1; }
+
+int pxh_reserve_workspace(size_t bytes)
+{
+    void* p = nullptr;
+    return pxh::library_workspace(bytes, nullptr, true, &p);
+}
+
+// Test hook: the address of the current device's library workspace once it holds `bytes`.
+void* pxh_debug_library_workspace(size_t bytes)
+{
+    void* p = nullptr;
+    return pxh::library_workspace(bytes, nullptr, true, &p) == PXH_OK ? p : nullptr;
+}
 
 // Host-only check hook for the multiply-high division used by the indexing code.
 unsigned pxh_debug_fastdiv(unsigned n, unsigned d)

@@ -1013,7 +1013,7 @@ int pxh_yolo_forward_train(const float* input, float* output, float* delta, cons
     }
     void* ws;
     rc = resolve_workspace(workspace, workspace_bytes,
-                           yolo_workspace_bytes(batch, mask_count, width, height), &ws);
+                           yolo_workspace_bytes(batch, mask_count, width, height), &ws, as_stream(stream));
     if (rc) return rc;
     return run_training_pass<true>("pxh_yolo_forward_train", input, output, delta, truths, truth_counts, p,
                                    YoloTables{}, stats, cost, 0, ws, as_stream(stream));
@@ -1037,7 +1037,7 @@ int pxh_yolo_loss(const float* output, float* delta, const float* truths, const 
     if (rc) return rc;
     void* ws;
     rc = resolve_workspace(workspace, workspace_bytes,
-                           yolo_workspace_bytes(batch, mask_count, width, height), &ws);
+                           yolo_workspace_bytes(batch, mask_count, width, height), &ws, as_stream(stream));
     if (rc) return rc;
     const YoloTables tb{ assigned_classes, assigned_anchors, assigned_boxes, masks, anchors };
     return run_training_pass<false>("pxh_yolo_loss", output, nullptr, delta, truths, truth_counts, p, tb, stats,

@@ -24,7 +24,16 @@ public:
 
     DeviceVector() = default;
 
-    explicit DeviceVector(size_type n, T value = T()) { allocate(n); fill(value); }
+    // Filled on the null stream and waited for, so that the vector can be used on any stream (also a
+    // non-blocking one, which does not order itself behind the null stream) once the constructor returns.
+    explicit DeviceVector(size_type n, T value = T())
+    {
+        allocate(n);
+        if (n) {
+            fill(value);
+            PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(nullptr));
+        }
+    }
 
     DeviceVector(const T* begin, const T* end)
     {
@@ -71,15 +80,18 @@ public:
         PX_HIP_RUNTIME_CHECK(hipMemcpyAsync(data_, rhs.data_, size_ * sizeof(T), hipMemcpyDeviceToDevice, stream));
     }
 
-    // Blocking host -> device copy of n elements.
-    void copyHost(const T* host, size_type n)
+    // Blocking host -> device copy of n elements.  `stream` is the stream the vector is used on: work
+    // queued there may still read the old contents, so it is waited for first (a non-blocking stream
+    // does not order itself against the copy).
+    void copyHost(const T* host, size_type n, hipStream_t stream = nullptr)
     {
         PX_CHECK(n <= size_, "host source larger than the device vector");
         if (n == 0) return;
+        if (stream) PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(stream));
         PX_HIP_RUNTIME_CHECK(hipMemcpy(data_, host, n * sizeof(T), hipMemcpyHostToDevice));
     }
 
-    void copyHost(const std::vector<T>& host) { copyHost(host.data(), host.size()); }
+    void copyHost(const std::vector<T>& host, hipStream_t stream = nullptr) { copyHost(host.data(), host.size(), stream); }
 
     // Device -> device copy of n elements from a raw device pointer, ordered on `stream`.
     void copyDevice(const T* device, size_type n, hipStream_t stream = nullptr)
@@ -89,11 +101,15 @@ public:
         PX_HIP_RUNTIME_CHECK(hipMemcpyAsync(data_, device, n * sizeof(T), hipMemcpyDeviceToDevice, stream));
     }
 
-    // Blocking device -> host copy (waits for all work queued before it on the null stream).
-    std::vector<T> asVector() const
+    // Blocking device -> host copy.  `stream` is the stream that last wrote the vector: it is waited
+    // for first, since the copy itself only orders behind the null stream and blocking streams.
+    std::vector<T> asVector(hipStream_t stream = nullptr) const
     {
         std::vector<T> host(size_);
-        if (size_) PX_HIP_RUNTIME_CHECK(hipMemcpy(host.data(), data_, size_ * sizeof(T), hipMemcpyDeviceToHost));
+        if (size_) {
+            if (stream) PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(stream));
+            PX_HIP_RUNTIME_CHECK(hipMemcpy(host.data(), data_, size_ * sizeof(T), hipMemcpyDeviceToHost));
+        }
         return host;
     }
 

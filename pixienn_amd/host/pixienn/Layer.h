@@ -125,10 +125,26 @@ public:
         }
         if (truths_.size() != packed.size()) truths_ = FloatVector(packed.size());
         if (truthCounts_.size() != counts.size()) truthCounts_ = IntVector(counts.size());
-        truths_.copyHost(packed);
-        truthCounts_.copyHost(counts);
+        truths_.copyHost(packed, stream);
+        truthCounts_.copyHost(counts, stream);
         maxTruth_ = static_cast<int>(most);
     }
+
+    // One scratch buffer for the layers of this context.  They run one after the other on the
+    // context's stream, so their uses cannot overlap, and another context (another model, another
+    // stream) has a buffer of its own: nothing here goes through the library's shared per-device
+    // workspace.  Layers reserve what their kernels need when they are constructed, so the buffer has
+    // its final size and address before the first forward -- and before any graph capture.  A block
+    // that has been outgrown is kept until the context goes, for graphs captured with its address.
+    void reserveWorkspace(std::size_t bytes)
+    {
+        if (bytes <= workspaceBytes()) return;
+        if (!workspace_.empty()) retiredWorkspaces_.push_back(std::move(workspace_));
+        workspace_ = FloatVector((bytes + sizeof(float) - 1) / sizeof(float));
+    }
+
+    void* workspace() noexcept { return workspace_.empty() ? nullptr : workspace_.data(); }
+    std::size_t workspaceBytes() const noexcept { return workspace_.size() * sizeof(float); }
 
     const FloatVector& truths() const noexcept { return truths_; }
     const IntVector& truthCounts() const noexcept { return truthCounts_; }
@@ -138,6 +154,8 @@ private:
     FloatVector truths_;
     IntVector truthCounts_;
     int maxTruth_ = 0;
+    FloatVector workspace_;
+    std::vector<FloatVector> retiredWorkspaces_;
 };
 
 // ---------------------------------------------------------------- layer
@@ -158,6 +176,7 @@ public:
         index_ = props.get<int>("index", 0);
         inputs_ = props.get<int>("inputs", channels_ * height_ * width_);
         PX_CHECK(batch_ > 0 && channels_ > 0 && height_ >= 0 && width_ >= 0, "layer dimensions must be positive");
+        if (context.training) context.reserveWorkspace(pxh_rescale_workspace_bytes());     // rescaleAndClip()
     }
 
     virtual ~Layer() = default;
@@ -249,8 +268,10 @@ protected:
     void rescaleAndClip(V& tensor)
     {
         if (tensor.empty() || !(gradientRescaling_ || gradientClipping_)) return;
+        context_.reserveWorkspace(pxh_rescale_workspace_bytes());
         PX_HIP_CHECK(pxh_rescale_clip(tensor.data(), tensor.size(), gradientRescaling_ ? gradientThreshold_ : 0.0f,
-                                      gradientClipping_ ? gradientClipValue_ : 0.0f, nullptr, nullptr, 0, stream()));
+                                      gradientClipping_ ? gradientClipValue_ : 0.0f, nullptr, context_.workspace(),
+                                      context_.workspaceBytes(), stream()));
     }
 
     void checkInput(const V& input, const char* who) const

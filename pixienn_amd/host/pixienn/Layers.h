@@ -45,6 +45,7 @@ public:
         const int oh = props.get<int>("out_height", height());
         const int ow = props.get<int>("out_width", width());
         setOutput(filters_, oh, ow);
+        if (training()) context.reserveWorkspace(pxh_bn_workspace_bytes(batch(), filters_, oh * ow));
 
         // The weights live here so that update() and the optimizer sidecar cover the whole layer;
         // their values and gradients are the delegated convolution's business ("weights": count).
@@ -111,7 +112,8 @@ public:
             PX_HIP_CHECK(pxh_bn_train_act_forward(x, output_.data(), nullptr, nullptr, nullptr, mean_.data(),
                                                   var_.data(), rollingMean_.data(), rollingVar_.data(),
                                                   scales_.data(), biases_.data(), batch(), filters_, spatial,
-                                                  activation_, nullptr, 0, stream()));
+                                                  activation_, context().workspace(), context().workspaceBytes(),
+                                                  stream()));
             foldedValid_ = false;       // the rolling statistics moved
         } else {
             if (!foldedValid_) {
@@ -134,14 +136,14 @@ public:
         if (batchNorm_) {
             PX_HIP_CHECK(pxh_bn_act_backward(delta_.data(), x_, nullptr, mean_.data(), var_.data(), scales_.data(),
                                              biases_.data(), scaleUpdates_.data(), biasUpdates_.data(), nullptr,
-                                             nullptr, batch(), filters_, spatial, activation_, nullptr, 0,
-                                             stream()));
+                                             nullptr, batch(), filters_, spatial, activation_, context().workspace(),
+                                             context().workspaceBytes(), stream()));
         } else {
             // pre-activation = x + bias is not kept either; the linear head convs need none
             preActivation(spatial);
             PX_HIP_CHECK(pxh_bias_act_backward(delta_.data(), pre_.empty() ? nullptr : pre_.data(),
                                                biasUpdates_.data(), batch(), filters_, spatial, activation_,
-                                               nullptr, 0, stream()));
+                                               context().workspace(), context().workspaceBytes(), stream()));
         }
         if (convolveBackward_) {
             convolveBackward_(input, delta_, grad);
@@ -207,7 +209,7 @@ public:
             std::vector<float> host(t->size());
             is.read(reinterpret_cast<char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
             PX_CHECK(is.good() || host.empty(), "Could not read weights");
-            t->copyHost(host);
+            t->copyHost(host, stream());
         }
         foldedValid_ = false;
         return is.tellg() - start;
@@ -217,7 +219,7 @@ public:
     {
         const auto start = os.tellp();
         for (const V* t: weightFileOrder()) {
-            const std::vector<float> host = t->asVector();
+            const std::vector<float> host = t->asVector(stream());
             os.write(reinterpret_cast<const char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
         }
         PX_CHECK(os.good(), "Could not write weights");
@@ -229,7 +231,7 @@ public:
     {
         const auto start = os.tellp();
         for (const V* t: { &weightM_, &weightV_, &biasM_, &biasV_, &scaleM_, &scaleV_ }) {
-            const std::vector<float> host = t->asVector();
+            const std::vector<float> host = t->asVector(stream());
             os.write(reinterpret_cast<const char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
         }
         PX_CHECK(os.good(), "Could not write convolution optimizer state");
@@ -243,7 +245,7 @@ public:
             std::vector<float> host(t->size());
             is.read(reinterpret_cast<char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
             PX_CHECK(is.good() || host.empty(), "Could not read convolution optimizer state");
-            t->copyHost(host);
+            t->copyHost(host, stream());
         }
         return is.tellg() - start;
     }
@@ -277,7 +279,7 @@ private:
     void load(V& dst, const std::vector<float>& src)
     {
         PX_CHECK(dst.size() == src.size(), "ConvLayer: parameter vector of the wrong size");
-        dst.copyHost(src);
+        dst.copyHost(src, stream());
     }
 
     // x + bias for a non-linear layer without batch norm (the gradient needs it)
@@ -310,6 +312,7 @@ public:
     BatchNormLayer(Context& context, const Properties& props) : Layer(context, props)
     {
         setOutput(channels(), height(), width());
+        if (training()) context.reserveWorkspace(pxh_bn_workspace_bytes(batch(), channels(), height() * width()));
         const auto c = static_cast<std::size_t>(channels());
         biases_ = V(c, 0.0f);
         scales_ = V(c, 1.0f);
@@ -333,7 +336,8 @@ public:
             PX_HIP_CHECK(pxh_bn_train_act_forward(input.data(), output_.data(), nullptr, nullptr, nullptr, mean_.data(),
                                                   var_.data(), rollingMean_.data(), rollingVar_.data(),
                                                   scales_.data(), biases_.data(), batch(), channels(), spatial,
-                                                  PXH_LINEAR, nullptr, 0, stream()));
+                                                  PXH_LINEAR, context().workspace(), context().workspaceBytes(),
+                                                  stream()));
             foldedValid_ = false;
             return;
         }
@@ -354,7 +358,7 @@ public:
         PX_HIP_CHECK(pxh_bn_act_backward(delta_.data(), input.data(), nullptr, mean_.data(), var_.data(),
                                          scales_.data(), biases_.data(), scaleUpdates_.data(), biasUpdates_.data(),
                                          nullptr, nullptr, batch(), channels(), outHeight() * outWidth(), PXH_LINEAR,
-                                         nullptr, 0, stream()));
+                                         context().workspace(), context().workspaceBytes(), stream()));
         if (grad) PX_HIP_CHECK(pxh_axpy(delta_.size(), 1.0f, delta_.data(), grad->data(), stream()));
     }
 
@@ -392,7 +396,7 @@ public:
             std::vector<float> host(t->size());
             is.read(reinterpret_cast<char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
             PX_CHECK(is.good(), "Could not read batch normalize parameters");
-            t->copyHost(host);
+            t->copyHost(host, stream());
         }
         foldedValid_ = false;
         return is.tellg() - start;
@@ -402,7 +406,7 @@ public:
     {
         const auto start = os.tellp();
         for (const V* t: { &biases_, &scales_, &rollingMean_, &rollingVar_ }) {
-            const std::vector<float> host = t->asVector();
+            const std::vector<float> host = t->asVector(stream());
             os.write(reinterpret_cast<const char*>(host.data()), static_cast<std::streamsize>(host.size() * sizeof(float)));
         }
         PX_CHECK(os.good(), "Could not write batch normalize parameters");
@@ -701,6 +705,7 @@ public:
         spare_ = IntVector(static_cast<std::size_t>(capacity) * 8);
         count_ = IntVector(1, 0);
         spareCount_ = IntVector(1, 0);
+        nmsWorkspace_ = FloatVector((pxh_nms_workspace_bytes(capacity) + sizeof(float) - 1) / sizeof(float));
     }
 
     int capacity() const noexcept { return capacity_; }
@@ -724,7 +729,9 @@ public:
     void nms(int batch, int classes, float threshold, hipStream_t stream = nullptr)
     {
         PX_HIP_CHECK(pxh_nms(records(), count_.data(), capacity_, batch, classes, threshold,
-                             reinterpret_cast<pxh_detection*>(spare_.data()), spareCount_.data(), nullptr, 0, stream));
+                             reinterpret_cast<pxh_detection*>(spare_.data()), spareCount_.data(),
+                             nmsWorkspace_.empty() ? nullptr : nmsWorkspace_.data(),
+                             nmsWorkspace_.size() * sizeof(float), stream));
         std::swap(records_, spare_);
         std::swap(count_, spareCount_);
     }
@@ -756,6 +763,7 @@ public:
 private:
     int capacity_;
     IntVector records_, spare_, count_, spareCount_;
+    FloatVector nmsWorkspace_;      // the list's own: nms of two lists on two streams may overlap
     unsigned nextOrder_ = 0;
 };
 
@@ -788,6 +796,8 @@ public:
         if (training()) {
             stats_ = V(kStats, 0.0f);
             costDevice_ = V(1, 0.0f);
+            context.reserveWorkspace(pxh_yolo_workspace_bytes(batch(), static_cast<int>(mask_.size()), context.classes,
+                                                              width(), height(), 0));
         }
     }
 
@@ -810,7 +820,7 @@ public:
                                             stats_.data(), costDevice_.data(), batch(), masks, numAnchors_,
                                             c.classes, width(), height(), c.width, c.height, ignoreThresh_,
                                             truthThresh_, coordScale_, objectScale_, noObjectScale_, classScale_,
-                                            nullptr, 0, stream()));
+                                            context().workspace(), context().workspaceBytes(), stream()));
         costReady_ = false;
     }
 

@@ -11,8 +11,8 @@ from pixienn_amd import capi
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def header_symbols():
-    text = open(os.path.join(ROOT, "include", "pixienn_hip.h")).read()
+def header_symbols(path=("include", "pixienn_hip.h")):
+    text = open(os.path.join(ROOT, *path)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(pxh_[a-z0-9_]+)\s*\(", text)))
 
@@ -25,6 +25,12 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), "missing export: " + n
     # the Python binding covers the whole header, nothing more, nothing less
     assert sorted(names) == capi.declared_symbols()
+    # the test hooks live in a private header, not in the installed one
+    assert not [n for n in names if "debug" in n]
+    hooks = header_symbols(("pixienn_amd", "csrc", "pixienn_hip_test.h"))
+    assert hooks == capi.test_hook_symbols()
+    for n in hooks:
+        assert hasattr(lib, n), "missing test hook: " + n
 
 
 def test_abi_version():

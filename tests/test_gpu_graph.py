@@ -135,3 +135,58 @@ def test_inference_postprocessing_in_a_graph_matches_eager(capacity):
         assert torch.equal(kept_graph, kept_eager), "replay %d differs from eager" % step
         seen.add(n_graph)
     assert len(seen) > 1, "the replays must have seen different data"
+
+
+def test_library_workspace_keeps_handed_out_blocks_and_refuses_to_grow_under_capture():
+    """The per-device workspace behind NULL-workspace calls: a larger request gives a new block but the
+    earlier one stays allocated (a graph captured with its address replays into live memory); growth
+    inside a capture is refused with PXH_ERR_WORKSPACE, and pxh_reserve_workspace beforehand avoids it."""
+    import torch
+    from pixienn_amd import capi, ops
+    lib = capi.load()
+    small = lib.pxh_debug_library_workspace(1 << 10)
+    assert small, capi.last_error()
+    assert lib.pxh_debug_library_workspace(1 << 12) == small, "a request that fits must not move the buffer"
+
+    # a sequence captured against the current block ...
+    N, C, S = 2, 8, 64
+    x = gpu(wl.normal(9500, (N, C, S, S)))
+    y = torch.empty_like(x); y_eager = torch.empty_like(x)
+    mean, var = torch.zeros(C, device="cuda"), torch.zeros(C, device="cuda")
+    scale, bias, rmean, rvar = (gpu(a) for a in wl.bn_params(9501, C))
+
+    def forward(out):
+        ops.bn_train_act_forward(x, out, mean, var, rmean.clone(), rvar.clone(), scale, bias, "leaky")
+
+    forward(y_eager)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        forward(y)
+
+    # ... then the workspace is outgrown: the graph still replays correctly, on memory that is still there
+    big_bytes = 48 << 20
+    assert lib.pxh_reserve_workspace(big_bytes) == 0, capi.last_error()
+    big = lib.pxh_debug_library_workspace(big_bytes)
+    assert big and big != small
+    scribble = torch.full((8 << 20,), float("nan"), device="cuda")      # would land on a freed block
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_eager)
+    del scribble
+
+    # growth while capturing is refused, and the capture survives it
+    huge_need = lib.pxh_nms_workspace_bytes(1 << 22)
+    assert huge_need > big_bytes
+    cap = 1 << 22
+    rec = torch.zeros((8,), dtype=torch.int32, device="cuda")
+    cnt = torch.zeros(1, dtype=torch.int32, device="cuda")
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2):
+        rc = capi.call_raw("pxh_nms", rec.data_ptr(), cnt.data_ptr(), cap, 1, 1, 0.5, y.data_ptr(), cnt.data_ptr(),
+                           None, 0, torch.cuda.current_stream().cuda_stream)
+        y.add_(1.0)
+    assert rc == -3 and "pxh_reserve_workspace" in capi.last_error(), (rc, capi.last_error())
+    g2.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_eager + 1.0)
