@@ -82,6 +82,7 @@ _TEST_HOOKS = {
     "pxh_debug_fastdiv": (ctypes.c_uint, [ctypes.c_uint, ctypes.c_uint]),
     "pxh_debug_nms_sweeps": (I, [I]),
     "pxh_debug_library_workspace": (P, [Z]),
+    "pxh_debug_yolo_tuning": (I, [I, I, I]),
 }
 
 

@@ -24,6 +24,12 @@ int pxh_debug_nms_sweeps(int sweeps);
  * (NULL when that fails): lets a test see that a block handed out earlier stays where it was. */
 void* pxh_debug_library_workspace(size_t bytes);
 
+/* Forces the shape of the YOLO training pass for the calls that follow: its form (1 = one launch,
+ * 2 = two launches) and, for the one-launch form, lanes per slot (1, 2 or 4) and the number of
+ * persistent head workgroups; 0 = let the library choose.  Results do not depend on any of them beyond
+ * the order of a few fp32 additions.  Returns 0. */
+int pxh_debug_yolo_tuning(int form, int lanes_per_slot, int head_workers);
+
 #ifdef __cplusplus
 }
 #endif

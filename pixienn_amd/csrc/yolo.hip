@@ -9,16 +9,24 @@
 //          Instruction and latency bound: ~1000 vector instructions per wave.
 //   class  the class rows, 94 % of the tensor: logit -> probability -> `out`, and the dense class
 //          delta.  Bandwidth bound, 12 bytes per element.
-// Both run in ONE grid, persistent head workgroups beside the class stream, followed by a small
-// kernel that writes the class delta of the supervised slots and adds up the sums in a fixed order.
+// Both run in ONE grid, persistent head workgroups beside the class stream.  Two forms of the pass,
+// picked by the size of the head (run_training_pass): in ONE launch for small heads, whose time is a
+// head tile's chain of dependent steps -- the head tiles write every delta of their cells, a slot's
+// truth sweep is spread over two lanes, and the workgroup that finishes last adds up the sums; in TWO
+// launches for large heads, whose time is the class stream's -- the stream also writes the zero
+// class deltas, and a small second kernel writes the class deltas of the few supervised slots and
+// adds up the sums.
 // pxh_yolo_forward_train starts from raw logits and assigns the positives on the device;
 // pxh_yolo_loss (the reference's argument list) starts from a decoded head and host-assigned
-// positives, its class stream only writes the zero delta.  pxh_yolo_detections is the
-// inference-side compaction.
+// positives.  pxh_yolo_detections is the inference-side compaction.
 // Box arithmetic follows the CPU layer (include/YoloLayer.h, src/DarkBox.cpp of the reference).
 #include "stream.h"
+#include "pixienn_hip_test.h"
 
+#include <atomic>
 #include <cfloat>
+#include <mutex>
+#include <vector>
 
 namespace pxh {
 namespace {
@@ -142,10 +150,12 @@ struct YoloParams {
     int masks[kMaxMasks];
     float anchors[2 * kMaxAnchors];   // integer pixel sizes held as float
     float anchors_rel[2 * kMaxAnchors];   // anchors[2a] / net_width, anchors[2a+1] / net_height (fp32 division)
-    FastDiv by_tiles;    // workgroups per (image, anchor) in the head sweep
+    FastDiv by_tiles;    // head tiles per (image, anchor)
     FastDiv by_masks;
     FastDiv by_width;
-    uint32_t blocks;     // workgroups of the head sweep
+    FastDiv by_anchors;
+    FastDiv by_area;
+    uint32_t blocks;     // head tiles in all
 };
 
 // Tables of the reference's signature (host-built assignment), all device pointers.
@@ -196,6 +206,776 @@ __device__ __forceinline__ BoxDelta box_delta(const Box& truth, float sx, float 
     d.v[3] = scale * (th - rh);
     return d;
 }
+
+// probability of class row `c` of the slot at `base`, exactly as the class sweep computes it
+template<bool FUSED>
+__device__ __forceinline__ float class_prob(const float* in, size_t base, int c, int area, int classes)
+{
+    if (c < 0 || c >= classes) return 0.0f;      // a label outside the class range reads nothing
+    const float v = in[base + (5 + static_cast<size_t>(c)) * area];
+    if constexpr (FUSED) return sigmoid_fast(v);
+    else return v;
+}
+
+// Sum of 64 lanes, pairwise (butterfly): at most 6 roundings on any path.
+__device__ __forceinline__ float wave_sum_pairwise(float v)
+{
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+constexpr int kWaves = kBlock / kWave;
+
+// ==========================================================================================
+// The training pass in ONE launch: persistent head workgroups that own every delta of their
+// cells, a class stream that only decodes, the final sums inside the same launch.  The form for
+// heads up to a hundred megabytes or so, whose time is one head tile's chain of dependent steps:
+// there it saves the second launch and shortens the chain (several lanes per slot).
+// ==========================================================================================
+namespace one_launch {
+
+// Unpacks one truth; which slot it claims is found afterwards (claim_targets).
+__device__ __forceinline__ TruthSlot make_truth_slot(const float* __restrict__ g)
+{
+    TruthSlot s;
+    const Box box{ g[0], g[1], g[2], g[3] };
+    const bool empty = box.w <= 0.0f || box.h <= 0.0f;
+    s.left = empty ? INFINITY : box.x - box.w / 2.0f;
+    s.top = empty ? INFINITY : box.y - box.h / 2.0f;
+    s.w = box.w; s.h = box.h; s.x = box.x; s.y = box.y;
+    s.cls = static_cast<int>(g[4]);
+    s.target = -1;
+    return s;
+}
+
+// IoU of a truth of size (w, h) with an anchor of size (cw, ch), both centred on the origin, where
+// DarkBox's rectangle intersection reduces to min(w) * min(h) exactly: ordered by left edge the wider
+// box comes first, its overlap bound W - (W/2 - n/2) is never below the narrower width n, and the
+// negative-left test (-W/2 + W < -n/2) is false.  The ratio is then formed as box_iou forms it.
+__device__ __forceinline__ float anchor_iou(float w, float h, float cw, float ch)
+{
+    const bool none = (w <= 0.0f) | (h <= 0.0f) | (cw <= 0.0f) | (ch <= 0.0f);
+    const float inter = none ? 0.0f : fminf(cw, w) * fminf(ch, h);
+    const float aa = cw * ch;
+    const float ab = w * h;
+    float uni = aa + ab;
+    uni = uni - inter;
+    const bool some = (uni > 0.0f) & (inter > 0.0f);
+    const float q = inter / (some ? uni : 1.0f);
+    return some ? q : 0.0f;
+}
+
+// The cell a truth's centre falls into (include/YoloLayer.h:470-476): whichever anchor claims a slot
+// for the truth, it is a slot of this cell.
+__device__ __forceinline__ int truth_cell(float x, float y, const YoloParams& p)
+{
+    int ci = static_cast<int>(x * static_cast<float>(p.width));
+    int cj = static_cast<int>(y * static_cast<float>(p.height));
+    ci = max(0, min(ci, p.width - 1));
+    cj = max(0, min(cj, p.height - 1));
+    return cj * p.width + ci;
+}
+
+// The positive slot staged truth `t` claims, from its IoU with every anchor (row[a]): the best anchor
+// over ALL anchors (strict >, the first wins); a positive only if that anchor belongs to this head, at
+// the cell the truth's centre falls into (include/YoloLayer.h:456-482 ==
+// src/YoloTargetBuilder.cpp:34-56).
+__device__ __forceinline__ void pick_target(TruthSlot* tile, int t, const float* row, const YoloParams& p)
+{
+    float ba = -FLT_MAX;
+    int bi = 0;
+    for (int a = 0; a < p.anchor_count; ++a) {
+        const float iou = row[a];
+        const bool better = iou > ba;
+        ba = better ? iou : ba;
+        bi = better ? a : bi;
+    }
+    int ms = -1;
+    for (int m = 0; m < p.mask_count; ++m)
+        if (p.masks[m] == bi) { ms = m; break; }
+    // the claimed slot lies on mask `ms`, whose anchor is this truth's best anchor
+    if (ms >= 0) tile[t].target = ms * p.area + truth_cell(tile[t].x, tile[t].y, p);
+}
+
+// The same for all `tn` staged truths, however many: one (truth, anchor) pair per lane, so that the
+// divisions of a truth run side by side instead of one after the other; then one lane per truth
+// picks the best.  Called by the whole workgroup, between barriers of its own.
+__device__ __forceinline__ void claim_targets(TruthSlot* tile, int tn, float* pair_iou, const YoloParams& p)
+{
+    const int per = kBlock / p.anchor_count;       // truths per pass (anchor_count <= kMaxAnchors <= kBlock)
+    uint32_t tt, aa;
+    p.by_anchors.divmod(threadIdx.x, tt, aa);
+    for (int c0 = 0; c0 < tn; c0 += per) {
+        const int t = c0 + static_cast<int>(tt);
+        if (static_cast<int>(tt) < per && t < tn)
+            pair_iou[threadIdx.x] = anchor_iou(tile[t].w, tile[t].h, p.anchors_rel[2 * aa], p.anchors_rel[2 * aa + 1]);
+        __syncthreads();
+        const int mine = c0 + static_cast<int>(threadIdx.x);
+        if (static_cast<int>(threadIdx.x) < per && mine < tn) pick_target(tile, mine, pair_iou + threadIdx.x * p.anchor_count, p);
+        __syncthreads();
+    }
+}
+
+// FUSED: raw logits in, decode written to `out`, positives found from the truths on the device
+//        with the CPU layer's rule; statistics as the CPU layer accumulates them.
+// !FUSED: `in` is the already decoded head, positives come from the host-built tables;
+//        statistics as the reference's device path accumulates them.
+struct HeadArgs {
+    const float* in;
+    float* out;
+    float* delta;
+    const float* truths;
+    const int* truth_counts;
+    int wide_delta;      // delta is 16-byte aligned and area % 4 == 0: the class rows are cleared 4 cells at a time
+};
+
+// One head tile: kBlock / L consecutive cells of one (image, anchor), L lanes per slot (image, anchor,
+// cell).  Every lane of a slot decodes the slot's box and objectness; the image's truths, staged in
+// LDS, are dealt round-robin to the L lanes for the overlap sweep and the results are combined with
+// the rules of the sequential sweep (best IoU: strict >, the first truth wins; positive: the last
+// claiming truth wins).  The tile writes the box and objectness deltas and ALL class deltas of its
+// cells (zeros, except at the few supervised slots) and returns its share of the 12 sums.
+// Small heads (19 x 19 at any batch) have far fewer slots than the machine has lanes and are bound by
+// the length of this instruction stream: L > 1 shortens the sweep and gives the machine L times as
+// many waves to run side by side.
+// Returns, in threads 0..kSums-1, the tile's sum of statistic threadIdx.x.
+template<bool FUSED, int L, bool NT>
+__device__ __forceinline__ double head_tile(const uint32_t head_block, const HeadArgs& a, const YoloParams& p,
+                                            const YoloTables& tb, TruthSlot* tile, float* pair_iou,
+                                            double (*wave_sums)[kWaves])
+{
+    static_assert(L == 1 || L == 2 || L == 4, "lanes per slot");
+    constexpr int kCells = kBlock / L;
+    const float* __restrict__ in = a.in;
+    float* __restrict__ out = a.out;
+    float* __restrict__ delta = a.delta;
+    uint32_t bn, tile_id, b, n;
+    p.by_tiles.divmod(head_block, bn, tile_id);
+    p.by_masks.divmod(bn, b, n);
+    const int sub = threadIdx.x & (L - 1);
+    const int cell = tile_id * kCells + threadIdx.x / L;
+    const bool live = cell < p.area;
+    const bool lead = live && sub == 0;        // the lane that stands for its slot in stores and sums
+    const int area = p.area;
+    const int entries = p.classes + 5;
+    const size_t base = (static_cast<size_t>(bn) * entries) * area + (live ? cell : 0);
+
+    // Asked for first, used last: the truth count, this lane's truth of the image and, for the search of
+    // each truth's best anchor, the (truth, anchor) pair this lane evaluates.  None of the addresses
+    // depends on another load, so all of it travels together with the head rows below.
+    // a count beyond the table's rows must not read past them
+    const int count = min(a.truth_counts[b], p.max_truth);
+    const float* image_truths = a.truths + static_cast<size_t>(b) * p.max_truth * 5;
+    float mine[5] = { 0, 0, 0, 0, 0 };
+    if (static_cast<int>(threadIdx.x) < p.max_truth) {
+#pragma unroll
+        for (int k = 0; k < 5; ++k) mine[k] = image_truths[5 * static_cast<size_t>(threadIdx.x) + k];
+    }
+    uint32_t pair_truth = 0, pair_anchor = 0;
+    float pair_w = 0, pair_h = 0, pair_cw = 0, pair_ch = 0;
+    if constexpr (FUSED) {
+        p.by_anchors.divmod(threadIdx.x, pair_truth, pair_anchor);
+        if (static_cast<int>(pair_truth) < p.max_truth) {
+            pair_w = image_truths[5 * static_cast<size_t>(pair_truth) + 2];
+            pair_h = image_truths[5 * static_cast<size_t>(pair_truth) + 3];
+        }
+        pair_cw = p.anchors_rel[2 * pair_anchor];
+        pair_ch = p.anchors_rel[2 * pair_anchor + 1];
+    }
+
+    int mask_anchor;
+    float aw, ah;
+    if constexpr (FUSED) {
+        mask_anchor = p.masks[n];
+        aw = p.anchors[2 * mask_anchor];
+        ah = p.anchors[2 * mask_anchor + 1];
+    } else {
+        mask_anchor = tb.masks[n];
+        aw = tb.anchors[2 * mask_anchor];
+        ah = tb.anchors[2 * mask_anchor + 1];
+    }
+    uint32_t row, col;
+    p.by_width.divmod(live ? cell : 0, row, col);
+    const int i = col, j = row;
+
+    float sx = 0, sy = 0, rw = 0, rh = 0, so = 0;
+    if (live) {
+        const float v0 = in[base], v1 = in[base + area], v2 = in[base + 2 * static_cast<size_t>(area)],
+                    v3 = in[base + 3 * static_cast<size_t>(area)], v4 = in[base + 4 * static_cast<size_t>(area)];
+        if constexpr (FUSED) {
+            // x, y and objectness feed thresholds and box targets: exact division here
+            sx = 1.0f / (1.0f + expf(-v0));
+            sy = 1.0f / (1.0f + expf(-v1));
+            so = 1.0f / (1.0f + expf(-v4));
+            if (lead) {
+                out[base] = sx;
+                out[base + area] = sy;
+                out[base + 2 * static_cast<size_t>(area)] = v2;
+                out[base + 3 * static_cast<size_t>(area)] = v3;
+                out[base + 4 * static_cast<size_t>(area)] = so;
+            }
+        } else {
+            sx = v0; sy = v1; so = v4;
+        }
+        rw = v2; rh = v3;
+    }
+    // The class deltas of the tile are zero except at the few slots something supervises: cleared now
+    // (behind the loads above, which the memory pipeline serves in the order they were asked for), so
+    // that the stores are on their way while the truths are swept.  Every wave clears the rows of its
+    // own cells; where a slot turns out to be supervised, the same wave writes its class deltas later,
+    // after these stores have been acknowledged.
+    {
+        constexpr int kWaveCells = kWave / L;
+        const int lane_ = threadIdx.x & (kWave - 1);
+        const int wave_cell0 = tile_id * kCells + (threadIdx.x / kWave) * kWaveCells;
+        float* rows = delta + (static_cast<size_t>(bn) * entries + 5) * area;
+        if (a.wide_delta && kWaveCells >= 4) {
+            constexpr int kVec = kWaveCells >= 4 ? kWaveCells / 4 : 1;      // vectors per row and wave
+            Pack<4> zero;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) zero.v[k] = 0.0f;
+            for (int v = lane_; v < p.classes * kVec; v += kWave) {
+                const int r = v / kVec, c = wave_cell0 + (v % kVec) * 4;
+                if (c < area) st<4, NT>(rows, static_cast<size_t>(r) * area + c, zero);
+            }
+        } else {
+            for (int v = lane_; v < p.classes * kWaveCells; v += kWave) {
+                const int r = v / kWaveCells, c = wave_cell0 + v % kWaveCells;
+                if (c < area) rows[static_cast<size_t>(r) * area + c] = 0.0f;
+            }
+        }
+    }
+
+    const Box pred = decode_box(sx, sy, rw, rh, i, j, aw, ah, p);
+    const bool pred_empty = pred.w <= 0.0f || pred.h <= 0.0f;
+    // an empty prediction overlaps nothing: park it where every overlap test fails
+    const float pl = pred_empty ? INFINITY : pred.x - pred.w / 2.0f, pt = pred.y - pred.h / 2.0f;
+
+    // Sweep the image's truths through LDS: best IoU (strict >, first wins) and, in the fused
+    // form, the truths that claim this slot as their positive (the last one writes the delta).
+    // IoU is never negative, so "first wins from the lowest float" is: start at truth 0 with 0.
+    float best = 0.0f;
+    int best_k = count > 0 ? 0 : -1;
+    int pos_cls = -1, pos_anchor = mask_anchor, pos_t = -1;
+    Box pos_box{ 0, 0, 0, 0 };
+    float st_iou = 0, st_r50 = 0, st_r75 = 0, st_cat = 0, st_obj = 0, st_count = 0;
+    const int my_slot = live ? static_cast<int>(n) * area + cell : -2;
+    // truths per step and lane: their overlap tests are independent and interleave
+    constexpr int kUnroll = L == 1 ? 4 : 2;
+
+    for (int t0 = 0; t0 < count; t0 += kTruthTile) {
+        const int t = t0 + threadIdx.x;
+        const int tn = min(kTruthTile, count - t0);
+        __syncthreads();       // the previous tile (or the previous head tile of this workgroup) is done with
+        // the first tile of truths comes from the registers filled at the top
+        const bool quick = FUSED && t0 == 0 && tn <= kBlock / p.anchor_count;
+        if (t0 == 0) {
+            if (t < count) tile[threadIdx.x] = make_truth_slot(mine);
+            if (quick && static_cast<int>(pair_truth) < tn)
+                pair_iou[threadIdx.x] = anchor_iou(pair_w, pair_h, pair_cw, pair_ch);
+        } else if (t < count) {
+            tile[threadIdx.x] = make_truth_slot(image_truths + 5 * static_cast<size_t>(t));
+        }
+        __syncthreads();
+        if constexpr (FUSED) {
+            if (quick) {
+                if (static_cast<int>(threadIdx.x) < tn) pick_target(tile, threadIdx.x, pair_iou + threadIdx.x * p.anchor_count, p);
+                __syncthreads();
+            } else {
+                claim_targets(tile, tn, pair_iou, p);
+            }
+        }
+        // The lanes of a slot take the truths in turn (lane `sub`: sub, sub + L, ...), kUnroll per step;
+        // inside a lane the ordered part (best so far, claims) follows in truth order.  Steps past the
+        // last truth re-read it with an empty overlap and no target.
+        for (int k0 = 0; k0 < tn; k0 += kUnroll * L) {
+            float inter[kUnroll], tw[kUnroll], th[kUnroll], iou[kUnroll];
+            int target[kUnroll], at[kUnroll];
+            bool touch = false, claimed = false;
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const int idx = k0 + u * L + sub;
+                const bool real = idx < tn;
+                at[u] = real ? idx : tn - 1;
+                const float4 r = *reinterpret_cast<const float4*>(&tile[at[u]].left);
+                target[u] = real ? tile[at[u]].target : -1;
+                tw[u] = r.z; th[u] = r.w;
+                const float ov = rect_overlap(pl, pt, pred.w, pred.h, r.x, r.y, r.z, r.w);
+                inter[u] = real ? ov : 0.0f;
+                touch = touch | (inter[u] > 0.0f);
+                claimed = claimed | (target[u] == my_slot);
+            }
+            // most steps touch nothing in the whole wave: no divisions then
+            if (__ballot(touch)) {
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) iou[u] = overlap_ratio(inter[u], pred.w, pred.h, tw[u], th[u]);
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    const bool better = iou[u] > best;
+                    best = better ? iou[u] : best;
+                    best_k = better ? t0 + at[u] : best_k;
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) iou[u] = 0.0f;
+            }
+            if constexpr (FUSED) {
+                if (__ballot(claimed)) {
+#pragma unroll
+                    for (int u = 0; u < kUnroll; ++u) {
+                        if (target[u] == my_slot) {
+                            // every claiming truth is counted (include/YoloLayer.h:480-507); the claimed
+                            // slot's anchor is this mask's, so iou[u] is the IoU the CPU layer records
+                            const TruthSlot& ts = tile[at[u]];
+                            pos_t = t0 + at[u];
+                            pos_cls = ts.cls;
+                            pos_box = Box{ ts.x, ts.y, ts.w, ts.h };
+                            st_cat += fminf(1.0f, class_prob<FUSED>(in, base, ts.cls, area, p.classes));
+                            st_iou += iou[u];
+                            if (iou[u] > .5f) st_r50 += 1.0f;
+                            if (iou[u] > .75f) st_r75 += 1.0f;
+                            st_obj += so;
+                            st_count += 1.0f;
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    // What the L lanes of a slot found, combined as the sequential sweep would have it: the larger
+    // IoU, on a tie the earlier truth; the positive of the latest claiming truth; the statistics of
+    // all claiming truths.  Afterwards every lane of the slot holds the slot's values.
+    if constexpr (L > 1) {
+#pragma unroll
+        for (int off = 1; off < L; off <<= 1) {
+            const float o_best = __shfl_xor(best, off, kWave);
+            const int o_k = __shfl_xor(best_k, off, kWave);
+            const bool take = (o_best > best) | ((o_best == best) & (o_k < best_k));
+            best = take ? o_best : best;
+            best_k = take ? o_k : best_k;
+        }
+        if constexpr (FUSED) {
+            if (__ballot(pos_t >= 0)) {
+#pragma unroll
+                for (int off = 1; off < L; off <<= 1) {
+                    const int o_t = __shfl_xor(pos_t, off, kWave);
+                    const int o_cls = __shfl_xor(pos_cls, off, kWave);
+                    const float ox = __shfl_xor(pos_box.x, off, kWave), oy = __shfl_xor(pos_box.y, off, kWave);
+                    const float ow = __shfl_xor(pos_box.w, off, kWave), oh = __shfl_xor(pos_box.h, off, kWave);
+                    const bool take = o_t > pos_t;
+                    pos_t = take ? o_t : pos_t;
+                    pos_cls = take ? o_cls : pos_cls;
+                    pos_box = take ? Box{ ox, oy, ow, oh } : pos_box;
+                    st_cat += __shfl_xor(st_cat, off, kWave);
+                    st_iou += __shfl_xor(st_iou, off, kWave);
+                    st_r50 += __shfl_xor(st_r50, off, kWave);
+                    st_r75 += __shfl_xor(st_r75, off, kWave);
+                    st_obj += __shfl_xor(st_obj, off, kWave);
+                    st_count += __shfl_xor(st_count, off, kWave);
+                }
+            }
+        }
+    }
+
+    if constexpr (!FUSED) {
+        if (live) {
+            const size_t slot = static_cast<size_t>(bn) * area + cell;
+            const int acls = tb.assigned_classes[slot];
+            if (acls >= 0) {
+                pos_cls = acls;
+                pos_anchor = tb.assigned_anchors[slot];
+                const float* bx = tb.assigned_boxes + slot * 4;
+                pos_box = Box{ bx[0], bx[1], bx[2], bx[3] };
+                const float paw = tb.anchors[2 * pos_anchor], pah = tb.anchors[2 * pos_anchor + 1];
+                const float iou = box_iou(decode_box(sx, sy, rw, rh, i, j, paw, pah, p), pos_box);
+                st_iou = iou;
+                st_r50 = iou > .5f ? 1.0f : 0.0f;
+                st_r75 = iou > .75f ? 1.0f : 0.0f;
+                st_obj = so;
+                st_count = 1.0f;
+                st_cat = fminf(1.0f, class_prob<FUSED>(in, base, acls, area, p.classes));
+            }
+        }
+    }
+
+    // region decision (include/YoloLayer.h:531-545), then the positive override (480-497)
+    float d_obj = 0.0f;
+    int cls = -1;            // class the dense class delta is written for, -1: zeros
+    BoxDelta bd{ { 0, 0, 0, 0 } };
+    float c_box = 0, c_obj = 0, c_noobj = 0;
+    if (live) {
+        const bool have_best = best_k >= 0;
+        if (!have_best || best < p.ignore_thresh) d_obj = p.noobject_scale * (0.0f - so);
+        if (have_best && best > p.truth_thresh) {
+            const float* g = image_truths + 5 * static_cast<size_t>(best_k);
+            d_obj = p.object_scale * (1.0f - so);
+            cls = static_cast<int>(g[4]);
+            bd = box_delta(Box{ g[0], g[1], g[2], g[3] }, sx, sy, rw, rh, i, j, aw, ah, p);
+            // deltaYoloClass also feeds the class-probability statistic on this path
+            if constexpr (FUSED) st_cat += fminf(1.0f, class_prob<FUSED>(in, base, cls, area, p.classes));
+        }
+        if (pos_cls >= 0) {
+            float paw = aw, pah = ah;
+            if constexpr (!FUSED) {
+                paw = tb.anchors[2 * pos_anchor];
+                pah = tb.anchors[2 * pos_anchor + 1];
+            }
+            bd = box_delta(pos_box, sx, sy, rw, rh, i, j, paw, pah, p);
+            d_obj = p.object_scale * (1.0f - so);
+            cls = pos_cls;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) c_box += bd.v[k] * bd.v[k];
+        if (d_obj >= 0.0f) c_obj = d_obj * d_obj; else c_noobj = d_obj * d_obj;
+        if (lead) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) delta[base + k * static_cast<size_t>(area)] = bd.v[k];
+            delta[base + 4 * static_cast<size_t>(area)] = d_obj;
+        }
+    }
+
+    // Workgroup sums.  The objectness sum and the no-object cost exist for every slot: pairwise
+    // over the wave.  Everything else is non-zero only at supervised slots, which most waves never
+    // see: their lead lanes are visited one by one, in lane order.  The class deltas of such a slot
+    // are written here, by the whole wave together, one class row per lane, with the probabilities
+    // the class stream writes (the same function of the same logits), and their cost is taken.
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const float dense_obj = wave_sum_pairwise(lead ? so : 0.0f);
+    const float dense_noobj = wave_sum_pairwise(lead ? c_noobj : 0.0f);
+    const float sparse[9] = { st_iou, st_r50, st_r75, st_cat, st_obj, st_count, st_count, c_box, c_obj };
+    constexpr int slot_of[9] = { 0, 1, 2, 3, 4, 6, 7, 8, 9 };
+    double acc[9] = { 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+    double class_cost = 0.0;
+    unsigned long long todo = __ballot(lead && (cls >= 0 || st_count != 0.0f));
+    unsigned long long supervised = __ballot(lead && cls >= 0);
+    while (todo) {
+        const int src_lane = __builtin_ctzll(todo);
+        todo &= todo - 1;
+#pragma unroll
+        for (int k = 0; k < 9; ++k)
+            acc[k] += static_cast<double>(__shfl(sparse[k], src_lane, kWave));
+    }
+    // this wave cleared these class rows at the top of the tile: those stores are through first
+    if (supervised) __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0)
+    // kTogether slots at a time, so that their class rows are fetched in one trip
+    constexpr int kTogether = 4;
+    while (supervised) {
+        int s_cls[kTogether];
+        size_t first[kTogether];
+#pragma unroll
+        for (int q = 0; q < kTogether; ++q) {
+            const bool some = supervised != 0;
+            const int src_lane = some ? __builtin_ctzll(supervised) : 0;
+            supervised &= supervised - 1;      // 0 stays 0
+            s_cls[q] = some ? __shfl(cls, src_lane, kWave) : -1;
+            first[q] = (static_cast<size_t>(bn) * entries + 5) * area + __shfl(cell, src_lane, kWave);
+        }
+        float sq[kTogether];
+#pragma unroll
+        for (int q = 0; q < kTogether; ++q) sq[q] = 0.0f;
+        for (int c = lane; c < p.classes; c += kWave) {
+            float v[kTogether];
+#pragma unroll
+            for (int q = 0; q < kTogether; ++q) v[q] = s_cls[q] >= 0 ? in[first[q] + static_cast<size_t>(c) * area] : 0.0f;
+#pragma unroll
+            for (int q = 0; q < kTogether; ++q) {
+                if (s_cls[q] >= 0) {
+                    const float prob = FUSED ? sigmoid_fast(v[q]) : v[q];
+                    const float t = (c == s_cls[q]) ? 1.0f : 0.0f;
+                    const float d = p.class_scale * (t - prob);
+                    delta[first[q] + static_cast<size_t>(c) * area] = d;
+                    sq[q] += d * d;
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < kTogether; ++q)
+            if (s_cls[q] >= 0) class_cost += static_cast<double>(wave_sum_pairwise(sq[q]));
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int k = 0; k < 9; ++k) wave_sums[slot_of[k]][wave] = acc[k];
+        wave_sums[5][wave] = static_cast<double>(dense_obj);
+        wave_sums[10][wave] = static_cast<double>(dense_noobj);
+        wave_sums[11][wave] = class_cost;
+    }
+    __syncthreads();
+    double total = 0.0;
+    if (threadIdx.x < kSums) {
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) total += wave_sums[threadIdx.x][w];
+    }
+    return total;
+}
+
+// The class rows of one (image, anchor) are one contiguous run of classes * area floats (row after
+// row).  The class stream walks every run in 128-bit vectors at 16-byte aligned addresses, whatever
+// the area: a run that starts `mis` floats past such an address gets one vector slot more, and the
+// slots at its two ends, which reach outside the run, are worked element by element.
+struct ClassRuns {
+    FastDiv by_slots;        // vector slots per run: (run_len + 3 + 3) / 4, enough for any start
+    uint32_t run_len;        // classes * area
+    uint32_t run_stride;     // (classes + 5) * area, from one run to the next
+    uint32_t first;          // 5 * area, the start of the first run
+    uint32_t total_slots;    // runs * slots per run
+    uint32_t elems;          // runs * run_len (for the element-wise form)
+    FastDiv by_run_len;
+};
+
+constexpr int kClassVectors = 4;      // vectors a lane of the class stream has in flight
+
+// Block `block` of the class stream: kClassVectors vector slots per lane, a workgroup-wide stride
+// apart, logit -> probability.
+template<bool NT>
+__device__ __forceinline__ void class_stream_block(const float* __restrict__ in, float* __restrict__ out,
+                                                   const ClassRuns& r, uint32_t block)
+{
+    size_t start[kClassVectors];
+    int lo[kClassVectors];
+    bool live[kClassVectors], whole[kClassVectors];
+    Pack<4> x[kClassVectors];
+#pragma unroll
+    for (int u = 0; u < kClassVectors; ++u) {
+        const uint32_t g = (block * kClassVectors + u) * kBlock + threadIdx.x;
+        live[u] = g < r.total_slots;
+        uint32_t run, slot;
+        r.by_slots.divmod(live[u] ? g : 0u, run, slot);
+        start[u] = static_cast<size_t>(run) * r.run_stride + r.first;
+        lo[u] = static_cast<int>(slot * 4) - static_cast<int>(start[u] & 3);     // first element of the slot, in the run
+        whole[u] = live[u] && lo[u] >= 0 && lo[u] + 3 < static_cast<int>(r.run_len);
+        if (whole[u]) x[u] = ld<4, NT>(in, start[u] + lo[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kClassVectors; ++u) {
+        if (whole[u]) {
+            Pack<4> prob;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) prob.v[k] = sigmoid_fast(x[u].v[k]);
+            st<4, NT>(out, start[u] + lo[u], prob);
+        } else if (live[u]) {
+            for (int k = 0; k < 4; ++k) {
+                const int e = lo[u] + k;
+                if (e >= 0 && e < static_cast<int>(r.run_len)) out[start[u] + e] = sigmoid_fast(in[start[u] + e]);
+            }
+        }
+    }
+}
+
+// ---- adding up the head workers' sums inside the same launch -----------------------------------
+// Every head worker leaves its 12 sums in memory and "arrives" at a counter; the worker that arrives
+// last adds up what all of them left, in a fixed order (worker by worker), so the totals do not depend
+// on which worker that was.  Nothing waits: a worker that is not last simply ends.  Two levels
+// (groups of kGroup workers, then the groups) keep both the number of values one workgroup reads
+// and the number of arrivals at one counter small: device-scope atomic operations on one address
+// take some 15 ns each, one after the other.
+//
+// A counter is a 64-bit word that is 0 whenever no launch is using it: arrivals add 1, the last one
+// puts the 0 back.  The counters live in device memory of the library's own (g_arrival_counters below,
+// zero when the code object is loaded), not in the workspace, whose contents nobody vouches for: a set
+// of counters per workspace address the library has seen, so that launches which may overlap -- they
+// have workspaces of their own -- never share one.  Each counter has a cache line of its own, so
+// that the groups do not queue behind each other at one memory channel.
+constexpr int kGroup = 256;
+constexpr uint32_t kMaxWorkers = 2048;
+constexpr uint32_t kMaxGroups = kMaxWorkers / kGroup;
+constexpr int kCounterStride = 256 / sizeof(unsigned long long);      // words between two counters
+
+constexpr int kCountersPerSet = 1 + kMaxGroups;
+constexpr int kCounterSets = 64;
+__device__ __align__(256) unsigned long long g_arrival_counters[kCounterSets * kCountersPerSet * kCounterStride];
+
+// True for the last of `members` arrivals.
+__device__ __forceinline__ bool arrive(unsigned long long* word, uint32_t members)
+{
+    const unsigned long long before = __hip_atomic_fetch_add(word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return before == members - 1;
+}
+
+struct SumArgs {
+    unsigned long long* counters;   // [1 + kMaxGroups] * kCounterStride: the top counter, then one per group
+    double* partial;                // [kSums][workers]
+    double* group_partial;          // [kSums][groups]
+    float* stats;
+    float* cost;
+    uint32_t workers, groups;
+    int accumulate;
+};
+
+// Everything the workers exchange goes through device-scope atomic accesses, which are performed at
+// the memory side of the caches.  This waits until those the calling wave has issued so far have
+// been acknowledged from there, and keeps the compiler from moving memory accesses across it.  (A
+// release fence of device scope would also do, but it writes back the whole L2 of the XCD, which costs
+// a launch of this size a hundred microseconds; a fence of workgroup scope waits for nothing, since
+// the waves of a workgroup share their first-level cache.)
+__device__ __forceinline__ void performed()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0)
+    asm volatile("" ::: "memory");
+}
+
+__device__ __forceinline__ double coherent_load(const double* p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Sums of `members` (at most 256) consecutive values of three statistics, for the wave that calls it:
+// wave w of the workgroup takes statistics 3w, 3w + 1, 3w + 2 of src[statistic][stride].  Up to four
+// values per lane, all fetched at once (one trip to memory), added lane by lane and then by the
+// wave's butterfly: the same additions in the same order whatever the values, so the sums do not
+// depend on which workgroup forms them.
+__device__ __forceinline__ void add_up(const double* src, uint32_t stride, uint32_t first, uint32_t members,
+                                       double (&sums)[3])
+{
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x / kWave;
+    constexpr int kPerLane = kGroup / kWave;
+    double v[3][kPerLane];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+#pragma unroll
+        for (int q = 0; q < kPerLane; ++q) {
+            const uint32_t j = lane + q * kWave;
+            v[i][q] = j < members ? coherent_load(src + static_cast<size_t>(wave * 3 + i) * stride + first + j) : 0.0;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        double t = v[i][0];
+#pragma unroll
+        for (int q = 1; q < kPerLane; ++q) t += v[i][q];
+        sums[i] = wave_sum(t);
+    }
+}
+
+// Called by every thread of head worker `worker` with its sum of statistic threadIdx.x (threads
+// 0..kSums-1).  `flag` is one int of LDS, `totals` LDS for kSums doubles.
+__device__ __forceinline__ void leave_sums(double total, uint32_t worker, const SumArgs& s, int* flag, double* totals)
+{
+    static_assert(kSums == 3 * kWaves, "three statistics per wave");
+    if (threadIdx.x < kSums)
+        __hip_atomic_store(s.partial + static_cast<size_t>(threadIdx.x) * s.workers + worker, total, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x / kWave;
+    const uint32_t group = worker / kGroup;
+    const uint32_t first = group * kGroup;
+    const uint32_t members = min(static_cast<uint32_t>(kGroup), s.workers - first);
+    unsigned long long* group_counter = s.counters + (1 + group) * kCounterStride;
+    if (threadIdx.x == 0) {
+        performed();           // the workgroup's sums (stored by lanes of this wave) are out before it is counted
+        *flag = arrive(group_counter, members) ? 1 : 0;
+    }
+    __syncthreads();
+    if (!*flag) return;
+    // last of its group: the group's sums
+    double sums[3];
+    add_up(s.partial, s.workers, first, members, sums);
+    if (s.groups > 1) {
+        if (lane == 0) {
+#pragma unroll
+            for (int i = 0; i < 3; ++i)
+                __hip_atomic_store(s.group_partial + static_cast<size_t>(wave * 3 + i) * s.groups + group, sums[i],
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            performed();
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            __hip_atomic_store(group_counter, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *flag = arrive(s.counters, s.groups) ? 1 : 0;
+        }
+        __syncthreads();
+        if (!*flag) return;
+        // last of all: the totals
+        add_up(s.group_partial, s.groups, 0, s.groups, sums);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const int k = wave * 3 + i;
+            totals[k] = sums[i];
+            if (s.stats) {
+                const float v = static_cast<float>(sums[i]);
+                s.stats[k] = (s.accumulate ? s.stats[k] : 0.0f) + v;
+            }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        if (s.cost) {
+            // the cost is the sum of the four squared-delta statistics, added in double
+            const float v = static_cast<float>(((totals[8] + totals[9]) + totals[10]) + totals[11]);
+            *s.cost = (s.accumulate ? *s.cost : 0.0f) + v;
+        }
+        // the counter this workgroup was the last to arrive at is free for the next launch
+        __hip_atomic_store(s.groups > 1 ? s.counters : group_counter, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// ---- training pass: persistent head workgroups + class decode stream in one grid ---------------
+// The head tiles are instruction bound and the class stream is bandwidth bound, so they run side
+// by side: the first `head_workers` workgroups of the grid (dispatched first, a few per compute
+// unit) walk the head tiles with a stride, every other workgroup decodes one vector per lane of the
+// class rows.  Every delta element belongs to exactly one head tile and every class probability to
+// exactly one stream lane, so nothing in the grid waits for anything else in it.
+struct TrainArgs {
+    HeadArgs head;
+    SumArgs sums;
+    ClassRuns runs;
+    uint32_t head_workers;
+};
+
+// FUSED: raw logits in, the class stream decodes them.  !FUSED (the reference's yoloLossGpu
+// argument list): the head is already decoded and the grid consists of head workers only.
+template<bool FUSED, int L, int V, bool NT>
+__global__ __launch_bounds__(kBlock, 4) void yolo_train_kernel(TrainArgs a, YoloParams p, YoloTables tb)
+{
+    __shared__ TruthSlot tile[kTruthTile];
+    __shared__ float pair_iou[kBlock];
+    __shared__ double wave_sums[kSums][kWaves];
+    __shared__ int flag;
+    static_assert(kMaxGroups <= kGroup && kGroup % kWave == 0, "a wave adds up a group");
+    if (!FUSED || blockIdx.x < a.head_workers) {
+        // the head workers are the long pole of the launch: they go first wherever a SIMD has the choice
+        __builtin_amdgcn_s_setprio(3);
+        // one sum per worker and statistic, over its tiles in walking order
+        double total = 0.0;
+        for (uint32_t t = blockIdx.x; t < p.blocks; t += a.head_workers) {
+            total += head_tile<FUSED, L, NT>(t, a.head, p, tb, tile, pair_iou, wave_sums);
+            __syncthreads();      // wave_sums is read by the first lanes until here
+        }
+        // the truth tile is free now: it carries the totals from the waves to the cost
+        leave_sums(total, blockIdx.x, a.sums, &flag, reinterpret_cast<double*>(tile));
+        return;
+    }
+    if constexpr (FUSED) {
+        if constexpr (V == 4) {
+            class_stream_block<NT>(a.head.in, a.head.out, a.runs, blockIdx.x - a.head_workers);
+        } else {
+            // pointers that are not 16-byte aligned: one element per lane
+            const uint32_t e = (blockIdx.x - a.head_workers) * kBlock + threadIdx.x;
+            if (e >= a.runs.elems) return;
+            uint32_t run, at;
+            a.runs.by_run_len.divmod(e, run, at);
+            const size_t where = static_cast<size_t>(run) * a.runs.run_stride + a.runs.first + at;
+            a.head.out[where] = sigmoid_fast(a.head.in[where]);
+        }
+    }
+}
+
+}  // namespace one_launch
+
+// ==========================================================================================
+// The training pass in TWO launches, for large heads, whose time is the class stream's: eight
+// waves per SIMD for the stream (the head tile squeezed into 64 registers beside it), the class
+// stream also writes the zero class deltas, the head tiles leave one int per slot saying what
+// supervises it, and a second, small kernel writes the class deltas of those few slots and adds
+// up the sums.
+// ==========================================================================================
+namespace two_launch {
 
 // Unpacks one truth and, for the fused pass, finds the positive slot it claims (best anchor over
 // ALL anchors against the origin-shifted truth; a positive only if that anchor belongs to this
@@ -249,16 +1029,6 @@ __device__ __forceinline__ TruthSlot make_truth_slot(const float* __restrict__ g
     return s;
 }
 
-// probability of class row `c` of the slot at `base`, exactly as the class sweep computes it
-template<bool FUSED>
-__device__ __forceinline__ float class_prob(const float* in, size_t base, int c, int area, int classes)
-{
-    if (c < 0 || c >= classes) return 0.0f;      // a label outside the class range reads nothing
-    const float v = in[base + (5 + static_cast<size_t>(c)) * area];
-    if constexpr (FUSED) return sigmoid_fast(v);
-    else return v;
-}
-
 // FUSED: raw logits in, decode written to `out`, positives found from the truths on the device
 //        with the CPU layer's rule; statistics as the CPU layer accumulates them.
 // !FUSED: `in` is the already decoded head, positives come from the host-built tables;
@@ -274,15 +1044,6 @@ struct HeadArgs {
     double* partial;
 };
 
-// Sum of 64 lanes, pairwise (butterfly): at most 6 roundings on any path.
-__device__ __forceinline__ float wave_sum_pairwise(float v)
-{
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
-
-constexpr int kWaves = kBlock / kWave;
 constexpr int kTruthUnroll = 4;
 
 // Returns, in threads 0..kSums-1, the tile's sum of statistic threadIdx.x.
@@ -667,6 +1428,8 @@ __global__ __launch_bounds__(kBlock) void yolo_patch_kernel(PatchArgs a)
     if (blockIdx.x < 13) finish_statistic(blockIdx.x, a.cls, slots);
 }
 
+}  // namespace two_launch
+
 // ---------------------------------------------------------------- detections
 // Thresholded compaction of a decoded head (include/YoloLayer.h:601-698): one lane per slot; a slot
 // whose objectness passes walks its class rows, and the lanes of a wave that found a detection in
@@ -799,6 +1562,15 @@ __global__ __launch_bounds__(kBlock) void yolo_detect_kernel(DetectArgs a, YoloP
     }
 }
 
+// Head tiles of kBlock / lanes cells each.
+void set_lanes_per_slot(YoloParams& p, int lanes)
+{
+    const int cells = kBlock / lanes;
+    const int tiles = (p.area + cells - 1) / cells;
+    p.by_tiles = FastDiv(tiles);
+    p.blocks = static_cast<uint32_t>(p.batch) * p.mask_count * tiles;
+}
+
 int fill_params(const char* who, YoloParams& p, int batch, int mask_count, int anchor_count, int classes, int width,
                 int height, int net_width, int net_height, int max_truth, float ignore_thresh, float truth_thresh,
                 float coord_scale, float object_scale, float noobject_scale, float class_scale)
@@ -820,15 +1592,183 @@ int fill_params(const char* who, YoloParams& p, int batch, int mask_count, int a
     p.net_width = net_width; p.net_height = net_height; p.max_truth = max_truth;
     p.ignore_thresh = ignore_thresh; p.truth_thresh = truth_thresh; p.coord_scale = coord_scale;
     p.object_scale = object_scale; p.noobject_scale = noobject_scale; p.class_scale = class_scale;
-    const int tiles = (p.area + kBlock - 1) / kBlock;
-    p.by_tiles = FastDiv(tiles);
     p.by_masks = FastDiv(mask_count);
     p.by_width = FastDiv(width);
-    p.blocks = static_cast<uint32_t>(batch) * mask_count * tiles;
+    p.by_anchors = FastDiv(anchor_count);
+    p.by_area = FastDiv(static_cast<uint32_t>(p.area));
+    set_lanes_per_slot(p, 1);
     return PXH_OK;
 }
 
 size_t align256(size_t b) { return (b + 255) & ~static_cast<size_t>(255); }
+
+namespace one_launch {
+
+// workspace: [12][workers] doubles | [12][groups] doubles
+struct YoloWorkspace {
+    double* partial;
+    double* group_partial;
+};
+
+size_t yolo_workspace_bytes()
+{
+    return align256(static_cast<size_t>(kMaxWorkers) * kSums * sizeof(double)) +
+           align256(static_cast<size_t>(kMaxGroups) * kSums * sizeof(double));
+}
+
+YoloWorkspace carve(void* ws)
+{
+    YoloWorkspace w;
+    char* c = static_cast<char*>(ws);
+    w.partial = reinterpret_cast<double*>(c);
+    c += align256(static_cast<size_t>(kMaxWorkers) * kSums * sizeof(double));
+    w.group_partial = reinterpret_cast<double*>(c);
+    return w;
+}
+
+// The arrival counters of the workspace at `ws` on the current device: a set of g_arrival_counters,
+// handed out the first time the address is seen and kept for it.  Launches that may overlap have
+// workspaces of their own, hence sets of their own.
+int counters_for(const char* who, const void* ws, unsigned long long** out)
+{
+    constexpr int kDevices = 64;
+    struct PerDevice {
+        unsigned long long* base = nullptr;
+        std::vector<const void*> seen;
+    };
+    static std::mutex mutex;
+    static PerDevice devices[kDevices];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kDevices) {
+        set_error("%s: no usable current device (%s)", who, hipGetErrorString(e));
+        return PXH_ERR_WORKSPACE;
+    }
+    std::lock_guard<std::mutex> lock(mutex);
+    PerDevice& d = devices[dev];
+    if (!d.base) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_arrival_counters));
+        if (e != hipSuccess || !p) {
+            set_error("%s: hipGetSymbolAddress(arrival counters): %s", who, hipGetErrorString(e));
+            return e != hipSuccess ? static_cast<int>(e) : PXH_ERR_WORKSPACE;
+        }
+        d.base = static_cast<unsigned long long*>(p);
+    }
+    size_t set = 0;
+    while (set < d.seen.size() && d.seen[set] != ws) ++set;
+    if (set == d.seen.size()) {
+        if (set == static_cast<size_t>(kCounterSets)) {
+            set_error("%s: more than %d different workspace addresses on one device; reuse workspaces", who,
+                      kCounterSets);
+            return PXH_ERR_WORKSPACE;
+        }
+        d.seen.push_back(ws);
+    }
+    *out = d.base + set * kCountersPerSet * kCounterStride;
+    return PXH_OK;
+}
+
+// Test hook state: lanes per slot and head workers forced by pxh_debug_yolo_tuning (0 = chosen here).
+std::atomic<int> g_forced_lanes{ 0 };
+std::atomic<int> g_forced_workers{ 0 };
+// Lanes per slot: a head with few slots is bound by the length of one lane's instruction stream and
+// gains from spreading a slot's truth sweep over two lanes (measured: 64 x 19^2 and 16 x 38^2, 69 k slots,
+// run 12 % faster with two lanes than with one, no faster with four); a head with many slots has
+// enough waves to hide it and is cheapest with one lane per slot.
+int lanes_per_slot(const YoloParams& p)
+{
+    const int forced = g_forced_lanes.load();
+    if (forced == 1 || forced == 2 || forced == 4) return forced;
+    const size_t slots = static_cast<size_t>(p.batch) * p.mask_count * p.area;
+    return slots < 200000 ? 2 : 1;
+}
+
+// Persistent head workgroups of the fused pass.  A head tile takes about kTileMicros however
+// many run side by side, so enough of them are started to be through in the time the class rows
+// take to stream, and no more: every one holds wave slots the stream could use.
+uint32_t head_workers(uint32_t tiles, double stream_us)
+{
+    const int forced = g_forced_workers.load();
+    uint32_t want;
+    if (forced > 0) {
+        want = static_cast<uint32_t>(forced);
+    } else {
+        constexpr double kTileMicros = 22.0;
+        double rounds = stream_us * 0.85 / kTileMicros;
+        if (rounds < 1.0) rounds = 1.0;
+        want = static_cast<uint32_t>(static_cast<double>(tiles) / rounds) + 1;
+    }
+    if (want > kMaxWorkers) want = kMaxWorkers;
+    return want < tiles ? want : tiles;
+}
+
+template<bool FUSED, int L>
+void launch_training(const TrainArgs& ta, const YoloParams& p, const YoloTables& tb, uint32_t grid, bool vec, bool nt,
+                     hipStream_t s)
+{
+    const dim3 g(grid), b(kBlock);
+    if constexpr (!FUSED) {
+        if (nt) hipLaunchKernelGGL((yolo_train_kernel<false, L, 1, true>), g, b, 0, s, ta, p, tb);
+        else hipLaunchKernelGGL((yolo_train_kernel<false, L, 1, false>), g, b, 0, s, ta, p, tb);
+    } else {
+        if (vec && nt) hipLaunchKernelGGL((yolo_train_kernel<true, L, 4, true>), g, b, 0, s, ta, p, tb);
+        else if (vec) hipLaunchKernelGGL((yolo_train_kernel<true, L, 4, false>), g, b, 0, s, ta, p, tb);
+        else hipLaunchKernelGGL((yolo_train_kernel<true, L, 1, false>), g, b, 0, s, ta, p, tb);
+    }
+}
+
+template<bool FUSED>
+int run_training_pass(const char* who, const float* in, float* out, float* delta, const float* truths,
+                      const int* truth_counts, YoloParams p, const YoloTables& tb, float* stats, float* cost,
+                      int accumulate, void* ws, hipStream_t s)
+{
+    const YoloWorkspace w = carve(ws);
+    ClassRuns runs{};
+    runs.run_len = static_cast<uint32_t>(p.classes) * p.area;
+    runs.run_stride = static_cast<uint32_t>(p.classes + 5) * p.area;
+    runs.first = 5u * p.area;
+    const uint32_t slots_per_run = (runs.run_len + 6) / 4;
+    runs.by_slots = FastDiv(slots_per_run);
+    runs.by_run_len = FastDiv(runs.run_len);
+    const uint32_t run_count = static_cast<uint32_t>(p.batch) * p.mask_count;
+    runs.total_slots = run_count * slots_per_run;
+    runs.elems = run_count * runs.run_len;
+    const bool vec = aligned16(in) && aligned16(out);
+    const uint32_t class_blocks = !FUSED ? 0
+                                  : vec ? (runs.total_slots + kBlock * kClassVectors - 1) / (kBlock * kClassVectors)
+                                        : (runs.elems + kBlock - 1) / kBlock;
+
+    const int lanes = lanes_per_slot(p);
+    set_lanes_per_slot(p, lanes);
+    // class rows: read + decode (the deltas are the head workers' business)
+    const double stream_us = static_cast<double>(runs.elems) * 8 / 6.0e6;   // at 6 TB/s
+    TrainArgs ta{};
+    ta.head = HeadArgs{ in, out, delta, truths, truth_counts, (p.area % 4 == 0 && aligned16(delta)) ? 1 : 0 };
+    ta.runs = runs;
+    ta.head_workers = FUSED ? head_workers(p.blocks, stream_us) : (p.blocks < kMaxWorkers ? p.blocks : kMaxWorkers);
+    int rc = counters_for(who, ws, &ta.sums.counters);
+    if (rc) return rc;
+    ta.sums.partial = w.partial;
+    ta.sums.group_partial = w.group_partial;
+    ta.sums.stats = stats;
+    ta.sums.cost = cost;
+    ta.sums.workers = ta.head_workers;
+    ta.sums.groups = (ta.head_workers + kGroup - 1) / kGroup;
+    ta.sums.accumulate = accumulate;
+    const uint32_t grid = ta.head_workers + class_blocks;
+    const bool nt = static_cast<size_t>(runs.elems) * (FUSED ? 12 : 4) >= kStreamingBytes;
+    switch (lanes) {
+    case 1: launch_training<FUSED, 1>(ta, p, tb, grid, vec, nt, s); break;
+    case 2: launch_training<FUSED, 2>(ta, p, tb, grid, vec, nt, s); break;
+    default: launch_training<FUSED, 4>(ta, p, tb, grid, vec, nt, s); break;
+    }
+    return check_launch(who);
+}
+
+}  // namespace one_launch
+
+namespace two_launch {
 
 // workspace: [12][head workgroups] doubles | one int per slot
 struct YoloWorkspace {
@@ -909,6 +1849,37 @@ int run_training_pass(const char* who, const float* in, float* out, float* delta
     return check_launch(who);
 }
 
+}  // namespace two_launch
+
+// Test hook state: the form of the training pass forced by pxh_debug_yolo_tuning (0 = chosen here).
+std::atomic<int> g_forced_form{ 0 };
+
+size_t training_workspace_bytes(int batch, int mask_count, int width, int height)
+{
+    const size_t a = one_launch::yolo_workspace_bytes(), b = two_launch::yolo_workspace_bytes(batch, mask_count, width, height);
+    return a > b ? a : b;
+}
+
+// One launch where the pass is bound by the head tiles' chain of steps, two where it is bound by the
+// class stream (measured on MI355X at 80 classes: below about 150 MB of fused traffic, and below
+// about 40 MB for the form that starts from a decoded head, one launch is the faster).
+template<bool FUSED>
+int run_training_pass(const char* who, const float* in, float* out, float* delta, const float* truths,
+                      const int* truth_counts, const YoloParams& p, const YoloTables& tb, float* stats, float* cost,
+                      int accumulate, void* ws, hipStream_t s)
+{
+    const size_t elems = static_cast<size_t>(p.batch) * p.mask_count * (p.classes + 5) * p.area;
+    const size_t bytes = FUSED ? elems * 12 : elems * 4 + elems * 20 / static_cast<size_t>(p.classes + 5);
+    const int forced = g_forced_form.load();
+    const bool one = forced == 1 || (forced != 2 && bytes < (FUSED ? size_t(150) << 20 : size_t(40) << 20));
+    if (one) return one_launch::run_training_pass<FUSED>(who, in, out, delta, truths, truth_counts, p, tb, stats, cost,
+                                                         accumulate, ws, s);
+    YoloParams q = p;
+    set_lanes_per_slot(q, 1);
+    return two_launch::run_training_pass<FUSED>(who, in, out, delta, truths, truth_counts, q, tb, stats, cost,
+                                                accumulate, ws, s);
+}
+
 }  // namespace
 }  // namespace pxh
 
@@ -978,12 +1949,20 @@ int pxh_yolo_detections(const float* predictions, int batch, const int* host_mas
                                       out, capacity, count, stream);
 }
 
+int pxh_debug_yolo_tuning(int form, int lanes_per_slot, int head_workers)
+{
+    g_forced_form.store(form);
+    one_launch::g_forced_lanes.store(lanes_per_slot);
+    one_launch::g_forced_workers.store(head_workers);
+    return 0;
+}
+
 size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int width, int height, int max_truth)
 {
     (void) classes;
     (void) max_truth;
     if (batch <= 0 || mask_count <= 0 || width <= 0 || height <= 0) return 0;
-    return yolo_workspace_bytes(batch, mask_count, width, height);
+    return training_workspace_bytes(batch, mask_count, width, height);
 }
 
 int pxh_yolo_forward_train(const float* input, float* output, float* delta, const float* truths,
@@ -1012,8 +1991,8 @@ int pxh_yolo_forward_train(const float* input, float* output, float* delta, cons
         p.anchors_rel[a] = p.anchors[a] / static_cast<float>(a % 2 ? net_height : net_width);
     }
     void* ws;
-    rc = resolve_workspace(workspace, workspace_bytes,
-                           yolo_workspace_bytes(batch, mask_count, width, height), &ws, as_stream(stream));
+    rc = resolve_workspace(workspace, workspace_bytes, training_workspace_bytes(batch, mask_count, width, height), &ws,
+                           as_stream(stream));
     if (rc) return rc;
     return run_training_pass<true>("pxh_yolo_forward_train", input, output, delta, truths, truth_counts, p,
                                    YoloTables{}, stats, cost, 0, ws, as_stream(stream));
@@ -1036,8 +2015,8 @@ int pxh_yolo_loss(const float* output, float* delta, const float* truths, const 
                          noobject_scale, class_scale);
     if (rc) return rc;
     void* ws;
-    rc = resolve_workspace(workspace, workspace_bytes,
-                           yolo_workspace_bytes(batch, mask_count, width, height), &ws, as_stream(stream));
+    rc = resolve_workspace(workspace, workspace_bytes, training_workspace_bytes(batch, mask_count, width, height), &ws,
+                           as_stream(stream));
     if (rc) return rc;
     const YoloTables tb{ assigned_classes, assigned_anchors, assigned_boxes, masks, anchors };
     return run_training_pass<false>("pxh_yolo_loss", output, nullptr, delta, truths, truth_counts, p, tb, stats,

@@ -89,8 +89,12 @@ def test_workspace_sizes():
     big = lib.pxh_bn_workspace_bytes(16, 32, 608 * 608)
     assert 0 < small < big < (1 << 24)
     a256 = lambda b: (b + 255) // 256 * 256
-    assert lib.pxh_yolo_workspace_bytes(64, 3, 80, 76, 76, 20) == (a256(64 * 3 * 23 * 12 * 8) +
-                                                                  a256(64 * 3 * 5776 * 4))
+    # the larger of the two forms of the training pass: sums of at most 2048 head workers and their 8 groups,
+    # or the sums of one workgroup per head tile and one int per slot
+    one = a256(2048 * 12 * 8) + a256(8 * 12 * 8)
+    two = a256(64 * 3 * 23 * 12 * 8) + a256(64 * 3 * 5776 * 4)
+    assert lib.pxh_yolo_workspace_bytes(64, 3, 80, 76, 76, 20) == max(one, two)
+    assert lib.pxh_yolo_workspace_bytes(1, 1, 1, 1, 1, 0) == one
     assert lib.pxh_bn_folded_bytes(1024) == 1024 * 32 and lib.pxh_bn_folded_bytes(0) == 0
 
 

@@ -199,6 +199,33 @@ def test_yolo_largest_head(ops, oracle):
     assert again[2] == cost and np.array_equal(again[3], stats), "cost and statistics must not depend on timing"
 
 
+def test_yolo_one_launch_sums_do_not_depend_on_arrival_order(ops, oracle):
+    """64 x 255 x 19^2 in the one-launch form, where whichever head workgroup finishes last adds up the
+    sums of all of them: cost, statistics and every delta are bit-identical from run to run, for each
+    number of lanes per slot, and the runs of different lane counts agree to the checker's tolerance."""
+    from test_gpu_yolo_adam import compare_head, gpu_head, oracle_head
+    from pixienn_amd import capi
+    lib = capi.load()
+    N, K, W = 64, 80, 19
+    x = wl.normal(5019, (N, 3 * (K + 5), W, W), std=2.0)
+    truths, counts = wl.yolo_truths(5101, N)
+    kw = dict(ignore_thresh=0.7, truth_thresh=1.0, coord_scale=1.0, object_scale=2.0, noobject_scale=0.1,
+              class_scale=1.0)
+    mask = wl.YOLOV3_MASKS[W]
+    want = oracle_head(oracle, x, truths, counts, W, W, K, mask, wl.YOLOV3_ANCHORS, 608, **kw)
+    try:
+        for lanes in (1, 2, 4):
+            lib.pxh_debug_yolo_tuning(1, lanes, 0)
+            first = gpu_head(ops, x, truths, counts, W, W, K, mask, wl.YOLOV3_ANCHORS, 608, **kw)
+            compare_head(first, want, "19^2 at batch 64, %d lanes per slot" % lanes, 3, kw, sum_rtol=2e-4)
+            for _ in range(3):
+                again = gpu_head(ops, x, truths, counts, W, W, K, mask, wl.YOLOV3_ANCHORS, 608, **kw)
+                assert_bit_exact(again[1], first[1], "delta of a repeated run")
+                assert again[2] == first[2] and np.array_equal(again[3], first[3]), "sums must not depend on timing"
+    finally:
+        lib.pxh_debug_yolo_tuning(0, 0, 0)
+
+
 def test_adam_full_parameter_buffer(ops, oracle):
     """61.9 M parameters, 10 steps: the first, a middle and the last million against the checker."""
     import torch

@@ -114,7 +114,9 @@ def test_yolo_training_pass_random_heads(ops, oracle):
     """Rectangular heads, 1 to 200 classes, any subset of the anchors as mask, truth tables with
     empty rows, truths outside the image, empty or inverted boxes and labels outside the class
     range: delta support, cost and statistics must follow the CPU layer."""
-    from test_gpu_yolo_adam import compare_head, gpu_head, oracle_head
+    from test_gpu_yolo_adam import YOLO_SHAPES, compare_head, gpu_head, oracle_head
+    from pixienn_amd import capi
+    lib = capi.load()
     r = np.random.default_rng(107)
     for case in range(40):
         W = int(r.integers(1, 30)); H = int(r.integers(1, 30)); K = int(r.choice([1, 2, 3, 7, 20, 64, 80, 129, 200]))
@@ -146,8 +148,14 @@ def test_yolo_training_pass_random_heads(ops, oracle):
         what = "case %d: N%d %dx%d K%d mask %s of %d net %d counts %s" % (case, N, W, H, K, mask, total_anchors, net,
                                                                            counts.tolist())
         want = oracle_head(oracle, x, truths, counts, W, H, K, mask, anchors, net, **kw)
-        got = gpu_head(ops, x, truths, counts, W, H, K, mask, anchors, net, **kw)
-        compare_head(got, want, what, masks, kw, sum_rtol=5e-5)
+        # the library's own choice of form and lanes per slot, and one forced shape per case in turn
+        for form, lanes in ((0, 0), YOLO_SHAPES[1 + case % 4]):
+            lib.pxh_debug_yolo_tuning(form, lanes, 0)
+            try:
+                got = gpu_head(ops, x, truths, counts, W, H, K, mask, anchors, net, **kw)
+            finally:
+                lib.pxh_debug_yolo_tuning(0, 0, 0)
+            compare_head(got, want, what + " form %d lanes %d" % (form, lanes), masks, kw, sum_rtol=5e-5)
 
 
 def test_yolo_detections_random_heads(ops, oracle):

@@ -24,6 +24,21 @@ def ops():
     return o
 
 
+# The training pass has two forms (one launch for small heads, two for large ones) and the one-launch
+# form spreads a slot over 1, 2 or 4 lanes; the library picks by size.  Every head test runs with the
+# library's choice and with each shape forced, so that all of them see every case.
+YOLO_SHAPES = [(0, 0), (1, 1), (1, 2), (1, 4), (2, 0)]
+
+
+@pytest.fixture(params=YOLO_SHAPES, ids=["auto", "one-launch-1", "one-launch-2", "one-launch-4", "two-launches"])
+def yolo_shape(request):
+    from pixienn_amd import capi
+    lib = capi.load()
+    lib.pxh_debug_yolo_tuning(request.param[0], request.param[1], 0)
+    yield request.param
+    lib.pxh_debug_yolo_tuning(0, 0, 0)
+
+
 def oracle_head(oracle, x, truths, counts, W, H, K, mask, anchors, net, **kw):
     N = x.shape[0]
     cfg, keep = oracle.yolo_cfg(N, W, H, K, mask, anchors, net, net, **kw)
@@ -101,7 +116,7 @@ def test_yolo_decode_matches_oracle(ops, oracle, kats):
         assert_bit_exact(host(gx), got, "decode in place")
 
 
-def test_yolo_training_2x2_reference_vector(ops, oracle, kats):
+def test_yolo_training_2x2_reference_vector(ops, oracle, kats, yolo_shape):
     c = kats["yolo_training_2x2"]
     x = np.array([((i % 13) - 6) * np.float32(0.11) for i in range(56)], F).reshape(1, 14, 2, 2)
     truths = np.zeros((1, 3, 5), F); truths[0] = c["truths"]
@@ -117,7 +132,7 @@ def test_yolo_training_2x2_reference_vector(ops, oracle, kats):
 
 
 @pytest.mark.parametrize("W", [13, 19, 38])
-def test_yolo_forward_train_matches_oracle(ops, oracle, W):
+def test_yolo_forward_train_matches_oracle(ops, oracle, W, yolo_shape):
     N, K = 4, 80
     mask = wl.YOLOV3_MASKS[{13: 19, 19: 19, 38: 38}[W]]
     x = wl.normal(2100 + W, (N, 3 * (K + 5), W, W), std=2.0)
@@ -130,7 +145,7 @@ def test_yolo_forward_train_matches_oracle(ops, oracle, W):
     compare_head(got, want, "head %d" % W, 3, kw)
 
 
-def test_yolo_forward_train_edge_cases(ops, oracle):
+def test_yolo_forward_train_edge_cases(ops, oracle, yolo_shape):
     K, W = 6, 5
     anchors = [4, 4, 12, 12, 30, 30]
     x = wl.normal(2200, (3, 2 * (K + 5), W, W), std=1.5)
@@ -152,7 +167,7 @@ def test_yolo_forward_train_edge_cases(ops, oracle):
     assert want[3][6] == 3      # both colliding truths and the border truth are counted
 
 
-def test_yolo_many_truths_tiles(ops, oracle):
+def test_yolo_many_truths_tiles(ops, oracle, yolo_shape):
     """More truths per image than one LDS tile holds."""
     K, W, N = 3, 9, 2
     x = wl.normal(2300, (N, 3 * (K + 5), W, W))
@@ -188,7 +203,7 @@ def run_loss_kat(ops, c, assigned):
     return host(out), host(delta), host(stats), float(host(cost)[0])
 
 
-def test_yolo_loss_reference_kernel_kats(ops, kats):
+def test_yolo_loss_reference_kernel_kats(ops, kats, yolo_shape):
     k = kats["yolo_kernel_kats"]
     s1, sm1 = 1 / (1 + math.exp(-1.0)), 1 / (1 + math.exp(1.0))
     c = k["assigned_target"]
@@ -219,7 +234,7 @@ def test_yolo_loss_reference_kernel_kats(ops, kats):
     assert np.allclose(delta[5:8], c["expected_delta_classes"], atol=1e-7)
 
 
-def test_yolo_loss_with_host_tables_matches_fused(ops, oracle):
+def test_yolo_loss_with_host_tables_matches_fused(ops, oracle, yolo_shape):
     """The reference's split (host target builder + loss kernels) and the fused pass agree."""
     import torch
     N, K, W = 3, 80, 19
