@@ -401,6 +401,39 @@ int pxh_adam_update_multi(int count, float* const* w, float* const* d, float* co
                           float* const* v, const size_t* n, const int* apply_decay, int batch, int t,
                           float lr, float beta1, float beta2, float eps, float decay, void* stream);
 
+/* ------------------------------------------------------------------------
+ * The many-tensor operations over a table kept in device memory: ONE launch for all parameter
+ * tensors of a model (two for rescale + clip), where the host-array forms above take one launch per
+ * 32 tensors.  A model builds its tables once, after its layers exist (the engine's counterpart
+ * would be Model::update, include/Model.h:1772-1792, gathering what ConvLayer::update,
+ * include/cuda/ConvLayer.h:370-413, and Layer::update, include/Layer.h:400-411, step one by one).
+ *
+ * pxh_tensor_table_create: `buffers` is a HOST array of streams * count device pointers, stream after
+ * stream (buffers[k * count + i] = buffer k of tensor i); streams = 1 (fill, rescale + clip: x),
+ * 2 (SGD: w, d) or 4 (Adam: w, d, m, v); n[count] element counts; apply_decay[count] flags or NULL.
+ * Tensors of length 0 are left out; at most 2048 tensors.  Allocates device memory and uploads the
+ * table with a blocking copy: call it at set-up, not under graph capture.  The table belongs to the
+ * device that was current; destroy it with pxh_tensor_table_destroy.  A table with more buffers per
+ * tensor than an operation needs serves it too (an Adam table can be filled or rescaled: buffer 0).
+ * Every tensor ends up exactly as the single-tensor call leaves it.  pxh_rescale_clip_table keeps
+ * its partial sums inside the table, so two calls on one table must not overlap in time; `norms`
+ * (nullable, device) receives one norm per tensor of the table, in table order.
+ * No counterpart in the reference.
+ * ---------------------------------------------------------------------- */
+typedef struct pxh_tensor_table pxh_tensor_table;
+int pxh_tensor_table_create(int count, int streams, float* const* buffers, const size_t* n,
+                            const int* apply_decay, pxh_tensor_table** table);
+void pxh_tensor_table_destroy(pxh_tensor_table* table);
+/* tensors in the table (those of length 0 are not counted) */
+int pxh_tensor_table_count(const pxh_tensor_table* table);
+int pxh_adam_update_table(const pxh_tensor_table* table, int batch, int t, float lr, float beta1,
+                          float beta2, float eps, float decay, void* stream);
+int pxh_sgd_update_table(const pxh_tensor_table* table, int batch, float lr, float momentum, float decay,
+                         void* stream);
+int pxh_fill_f32_table(const pxh_tensor_table* table, float value, void* stream);
+int pxh_rescale_clip_table(const pxh_tensor_table* table, float threshold, float clip, float* norms,
+                           void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -65,6 +65,12 @@ SIGNATURES = {
     "pxh_rescale_clip_multi": [I, P, P, F, F, P, P, Z, P],
     "pxh_fill_f32_multi": [I, P, P, F, P],
     "pxh_sgd_update_multi": [I, P, P, P, P, I, F, F, F, P],
+    "pxh_tensor_table_create": [I, I, P, P, P, P],
+    "pxh_tensor_table_count": [P],
+    "pxh_adam_update_table": [P, I, I, F, F, F, F, F, P],
+    "pxh_sgd_update_table": [P, I, F, F, F, P],
+    "pxh_fill_f32_table": [P, F, P],
+    "pxh_rescale_clip_table": [P, F, F, P, P],
 }
 _OTHER_RETURNS = {
     "pxh_last_error": (ctypes.c_char_p, []),
@@ -76,6 +82,7 @@ _OTHER_RETURNS = {
     "pxh_yolo_workspace_bytes": (Z, [I, I, I, I, I, I]),
     "pxh_nms_workspace_bytes": (Z, [I]),
     "pxh_reserve_workspace": (I, [Z]),
+    "pxh_tensor_table_destroy": (None, [P]),
 }
 # test hooks (pixienn_amd/csrc/pixienn_hip_test.h): exported, but not part of the C ABI
 _TEST_HOOKS = {

@@ -2,6 +2,9 @@
 #include "stream.h"
 
 #include <cmath>
+#include <cstring>
+#include <new>
+#include <vector>
 
 namespace pxh {
 namespace {
@@ -685,6 +688,124 @@ int launch_multi(const char* who, int count, float* const* const* buffers, const
     return PXH_OK;
 }
 
+// ---------------------------------------------------------------- the same over a table kept on the device
+// A by-value table holds 32 tensors, so a model's 222 parameter tensors still take 7 launches per
+// operation.  A table built once and kept in device memory (pxh_tensor_table_create) takes them all in
+// ONE: the launch carries only its address.  Workgroup b copies the list of first workgroups into LDS
+// (one coalesced load), finds its tensor there by bisection and fetches that tensor's record; the
+// per-element work and the order of every sum are those of the single call.
+constexpr int kMaxTableTensors = 2048;
+
+struct __attribute__((aligned(16))) TensorRecord {     // 64 bytes
+    float* stream[4];               // the tensor's buffers, in the operation's own order
+    unsigned long long n;
+    uint32_t decay;                 // the weight decay applies
+    uint32_t vector;                // every buffer is 16-byte aligned: the 128-bit form
+    uint32_t norm_vector;           // stream[0] is 16-byte aligned and n % 4 == 0: the 128-bit form of the norm
+    uint32_t pad[3];
+};
+
+struct TableView {
+    const TensorRecord* records;
+    const uint32_t* first_block;        // [count + 1] workgroups of the streaming operations
+    const uint32_t* first_norm_block;   // [count + 1] workgroups of the norm and rescale passes, = first partials
+    double2* partial;                   // sums of squares and peaks, one per workgroup of the norm pass
+    int count;
+};
+
+// The tensor workgroup `block` works on; `firsts` is LDS for count + 1 entries.
+__device__ __forceinline__ int table_tensor_of_block(const uint32_t* first_block, int count, uint32_t block, uint32_t* firsts)
+{
+    for (int i = threadIdx.x; i <= count; i += kBlock) firsts[i] = first_block[i];
+    __syncthreads();
+    return tensor_of_block(firsts, count, block);
+}
+
+struct AdamFromRecord {
+    AdamUpdateOp base;
+    __device__ AdamUpdateOp operator()(const TensorRecord& r) const
+    {
+        AdamUpdateOp op = base;
+        op.w = r.stream[0]; op.d = r.stream[1]; op.m = r.stream[2]; op.v = r.stream[3];
+        op.apply_decay = static_cast<int>(r.decay);
+        return op;
+    }
+};
+
+struct SgdFromRecord {
+    SgdUpdateOp base;
+    __device__ SgdUpdateOp operator()(const TensorRecord& r) const
+    {
+        SgdUpdateOp op = base;
+        op.w = r.stream[0]; op.d = r.stream[1];
+        op.apply_decay = static_cast<int>(r.decay);
+        return op;
+    }
+};
+
+struct FillFromRecord {
+    float value;
+    __device__ FillOp operator()(const TensorRecord& r) const { return FillOp{ r.stream[0], value }; }
+};
+
+// `streaming_elems`: tensors of at least this many elements go past the caches, as in the single call.
+template<typename Maker>
+__global__ __launch_bounds__(kBlock) void table_stream_kernel(TableView t, Maker make, unsigned long long streaming_elems)
+{
+    __shared__ uint32_t firsts[kMaxTableTensors + 1];
+    const int i = table_tensor_of_block(t.first_block, t.count, blockIdx.x, firsts);
+    const TensorRecord r = t.records[i];
+    const auto op = make(r);
+    const size_t n = r.n;
+    const size_t e = (static_cast<size_t>(blockIdx.x - firsts[i]) * kBlock + threadIdx.x) * 4;
+    if (e >= n) return;
+    using Op = decltype(make(r));
+    if (r.vector && e + 4 <= n) {
+        typename Op::template Regs<4> regs;
+        if (n >= streaming_elems) {
+            op.template load<4, true>(e, regs);
+            op.template finish<4, true>(e, regs);
+        } else {
+            op.template load<4, false>(e, regs);
+            op.template finish<4, false>(e, regs);
+        }
+    } else {
+        for (size_t k = e; k < n && k < e + 4; ++k) {
+            typename Op::template Regs<1> regs;
+            op.template load<1, false>(k, regs);
+            op.template finish<1, false>(k, regs);
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void table_sumsq_kernel(TableView t)
+{
+    __shared__ uint32_t firsts[kMaxTableTensors + 1];
+    const int i = table_tensor_of_block(t.first_norm_block, t.count, blockIdx.x, firsts);
+    const TensorRecord r = t.records[i];
+    const uint32_t block = blockIdx.x - firsts[i], blocks = firsts[i + 1] - firsts[i];
+    double2* out = t.partial + blockIdx.x;
+    if (!r.norm_vector) sumsq_walk<1, false>(r.stream[0], r.n, block, blocks, out);
+    else if (r.n * 4 >= kStreamingBytes) sumsq_walk<4, true>(r.stream[0], r.n, block, blocks, out);
+    else sumsq_walk<4, false>(r.stream[0], r.n, block, blocks, out);
+}
+
+__global__ __launch_bounds__(kBlock) void table_rescale_kernel(TableView t, float threshold, float clip, float* norms)
+{
+    __shared__ uint32_t firsts[kMaxTableTensors + 1];
+    const int i = table_tensor_of_block(t.first_norm_block, t.count, blockIdx.x, firsts);
+    const TensorRecord r = t.records[i];
+    const uint32_t block = blockIdx.x - firsts[i], blocks = firsts[i + 1] - firsts[i];
+    const double2* mine = t.partial + firsts[i];
+    float* norm_out = norms ? norms + i : nullptr;
+    if (!r.norm_vector)
+        rescale_walk<1, false>(r.stream[0], r.n, mine, static_cast<int>(blocks), block, blocks, threshold, clip, norm_out);
+    else if (r.n * 4 >= kStreamingBytes)
+        rescale_walk<4, true>(r.stream[0], r.n, mine, static_cast<int>(blocks), block, blocks, threshold, clip, norm_out);
+    else
+        rescale_walk<4, false>(r.stream[0], r.n, mine, static_cast<int>(blocks), block, blocks, threshold, clip, norm_out);
+}
+
 struct AdamStepOp {
     float* x;
     const float* m;
@@ -1045,6 +1166,174 @@ int pxh_fill_f32_multi(int count, float* const* x, const size_t* n, float value,
     // a fill streams past the caches from the size on that the single call does
     return launch_multi<1>("pxh_fill_f32_multi", count, buffers, n, nullptr, 4, FillMaker{ value }, as_stream(stream),
                            kFillStreamingBytes);
+}
+
+// ---------------------------------------------------------------- tensor tables
+struct pxh_tensor_table {
+    int device;
+    int count, streams;
+    uint32_t blocks, norm_blocks;
+    void* memory;
+    pxh::TableView view;
+};
+
+int pxh_tensor_table_create(int count, int streams, float* const* buffers, const size_t* n, const int* apply_decay,
+                            pxh_tensor_table** table)
+{
+    if (!table) return fail_invalid("pxh_tensor_table_create: null pointer");
+    *table = nullptr;
+    if (count < 0 || (count && (!buffers || !n))) return fail_invalid("pxh_tensor_table_create: bad argument");
+    if (streams != 1 && streams != 2 && streams != 4)
+        return fail_invalid("pxh_tensor_table_create: 1, 2 or 4 buffers per tensor (got %d)", streams);
+    // empty tensors take no part: they are left out of the table
+    std::vector<TensorRecord> records;
+    std::vector<uint32_t> first_block, first_norm_block;
+    unsigned long long blocks = 0, norm_blocks = 0;
+    for (int i = 0; i < count; ++i) {
+        if (n[i] == 0) continue;
+        TensorRecord r{};
+        bool aligned = true;
+        for (int k = 0; k < streams; ++k) {
+            float* ptr = buffers[static_cast<size_t>(k) * count + i];
+            if (!ptr) return fail_invalid("pxh_tensor_table_create: null pointer for tensor %d", i);
+            aligned = aligned && aligned16(ptr);
+            r.stream[k] = ptr;
+        }
+        r.n = n[i];
+        r.decay = apply_decay && apply_decay[i] ? 1u : 0u;
+        r.vector = aligned ? 1u : 0u;
+        r.norm_vector = aligned16(r.stream[0]) && n[i] % 4 == 0 ? 1u : 0u;
+        records.push_back(r);
+        first_block.push_back(static_cast<uint32_t>(blocks));
+        first_norm_block.push_back(static_cast<uint32_t>(norm_blocks));
+        blocks += (n[i] + kMultiPerBlock - 1) / kMultiPerBlock;
+        // the norm pass of the single call: at most kNormBlocks workgroups, each a whole step of loads
+        const size_t per_step = static_cast<size_t>(kBlock) * (r.norm_vector ? 4 : 1) * kNormLoads;
+        const size_t want = (n[i] + per_step - 1) / per_step;
+        norm_blocks += want < static_cast<size_t>(kNormBlocks) ? want : kNormBlocks;
+    }
+    if (records.size() > static_cast<size_t>(kMaxTableTensors)) {
+        set_error("pxh_tensor_table_create: %zu tensors; a table holds %d at most", records.size(), kMaxTableTensors);
+        return PXH_ERR_UNSUPPORTED;
+    }
+    if (blocks > 0x7fffffffull) {
+        set_error("pxh_tensor_table_create: more than 2^31 workgroups in one launch");
+        return PXH_ERR_UNSUPPORTED;
+    }
+    first_block.push_back(static_cast<uint32_t>(blocks));
+    first_norm_block.push_back(static_cast<uint32_t>(norm_blocks));
+
+    auto* t = new (std::nothrow) pxh_tensor_table{};
+    if (!t) return fail_invalid("pxh_tensor_table_create: out of host memory");
+    t->count = static_cast<int>(records.size());
+    t->streams = streams;
+    t->blocks = static_cast<uint32_t>(blocks);
+    t->norm_blocks = static_cast<uint32_t>(norm_blocks);
+    if (hipGetDevice(&t->device) != hipSuccess) t->device = -1;
+    if (t->count == 0) {
+        *table = t;
+        return PXH_OK;
+    }
+    // one allocation: records | first workgroups | first norm workgroups | partial sums of the norm pass
+    const auto align = [](size_t b) { return (b + 255) & ~static_cast<size_t>(255); };
+    const size_t rec_bytes = align(records.size() * sizeof(TensorRecord));
+    const size_t first_bytes = align(first_block.size() * sizeof(uint32_t));
+    const size_t partial_bytes = align(static_cast<size_t>(norm_blocks) * sizeof(double2));
+    const size_t total = rec_bytes + 2 * first_bytes + partial_bytes;
+    hipError_t e = hipMalloc(&t->memory, total);
+    if (e != hipSuccess) {
+        set_error("pxh_tensor_table_create: hipMalloc(%zu): %s", total, hipGetErrorString(e));
+        delete t;
+        return static_cast<int>(e);
+    }
+    char* base = static_cast<char*>(t->memory);
+    std::vector<char> image(rec_bytes + 2 * first_bytes, 0);
+    std::memcpy(image.data(), records.data(), records.size() * sizeof(TensorRecord));
+    std::memcpy(image.data() + rec_bytes, first_block.data(), first_block.size() * sizeof(uint32_t));
+    std::memcpy(image.data() + rec_bytes + first_bytes, first_norm_block.data(), first_norm_block.size() * sizeof(uint32_t));
+    e = hipMemcpy(base, image.data(), image.size(), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        set_error("pxh_tensor_table_create: upload: %s", hipGetErrorString(e));
+        (void) hipFree(t->memory);
+        delete t;
+        return static_cast<int>(e);
+    }
+    t->view.records = reinterpret_cast<const TensorRecord*>(base);
+    t->view.first_block = reinterpret_cast<const uint32_t*>(base + rec_bytes);
+    t->view.first_norm_block = reinterpret_cast<const uint32_t*>(base + rec_bytes + first_bytes);
+    t->view.partial = reinterpret_cast<double2*>(base + rec_bytes + 2 * first_bytes);
+    t->view.count = t->count;
+    *table = t;
+    return PXH_OK;
+}
+
+void pxh_tensor_table_destroy(pxh_tensor_table* table)
+{
+    if (!table) return;
+    if (table->memory) (void) hipFree(table->memory);
+    delete table;
+}
+
+int pxh_tensor_table_count(const pxh_tensor_table* table) { return table ? table->count : 0; }
+
+extern "C++" {
+namespace {
+template<typename Maker>
+int launch_table(const char* who, const pxh_tensor_table* table, int streams_needed, int bytes_per_elem, const Maker& make,
+                 void* stream, size_t streaming_from = kStreamingBytes)
+{
+    if (!table) return fail_invalid("%s: null table", who);
+    if (table->streams < streams_needed)
+        return fail_invalid("%s: the table holds %d buffers per tensor, %d are needed", who, table->streams, streams_needed);
+    if (table->count == 0) return PXH_OK;
+    const unsigned long long streaming_elems = (streaming_from + bytes_per_elem - 1) / bytes_per_elem;
+    hipLaunchKernelGGL((table_stream_kernel<Maker>), dim3(table->blocks), dim3(kBlock), 0, as_stream(stream), table->view,
+                       make, streaming_elems);
+    return check_launch(who);
+}
+}  // namespace
+}  // extern "C++"
+
+int pxh_adam_update_table(const pxh_tensor_table* table, int batch, int t, float lr, float beta1, float beta2, float eps,
+                          float decay, void* stream)
+{
+    if (batch <= 0) return fail_invalid("pxh_adam_update_table: batch must be positive");
+    if (t < 1) return fail_invalid("pxh_adam_update_table: t must be at least 1 (the update count is pre-incremented)");
+    AdamUpdateOp op{};
+    op.inv_batch = 1.0f / static_cast<float>(batch);
+    op.neg_decay = -decay;
+    op.beta1 = beta1; op.beta2 = beta2;
+    op.a1 = 1.0f - beta1; op.a2 = 1.0f - beta2;
+    op.c1 = 1.0f - powf(beta1, static_cast<float>(t));
+    op.c2 = 1.0f - powf(beta2, static_cast<float>(t));
+    op.lr = lr; op.eps = eps;
+    return launch_table("pxh_adam_update_table", table, 4, 32, AdamFromRecord{ op }, stream);
+}
+
+int pxh_sgd_update_table(const pxh_tensor_table* table, int batch, float lr, float momentum, float decay, void* stream)
+{
+    if (batch <= 0) return fail_invalid("pxh_sgd_update_table: batch must be positive");
+    const SgdUpdateOp op{ nullptr, nullptr, -decay * static_cast<float>(batch), lr / static_cast<float>(batch), momentum, 0 };
+    return launch_table("pxh_sgd_update_table", table, 2, 16, SgdFromRecord{ op }, stream);
+}
+
+int pxh_fill_f32_table(const pxh_tensor_table* table, float value, void* stream)
+{
+    return launch_table("pxh_fill_f32_table", table, 1, 4, FillFromRecord{ value }, stream, kFillStreamingBytes);
+}
+
+int pxh_rescale_clip_table(const pxh_tensor_table* table, float threshold, float clip, float* norms, void* stream)
+{
+    if (!table) return fail_invalid("pxh_rescale_clip_table: null table");
+    const bool rescale = threshold > 0.0f || norms != nullptr;
+    if ((!rescale && !(clip > 0.0f)) || table->count == 0) return PXH_OK;
+    hipStream_t s = as_stream(stream);
+    hipLaunchKernelGGL(table_sumsq_kernel, dim3(table->norm_blocks), dim3(kBlock), 0, s, table->view);
+    int rc = check_launch("pxh_rescale_clip_table");
+    if (rc) return rc;
+    hipLaunchKernelGGL(table_rescale_kernel, dim3(table->norm_blocks), dim3(kBlock), 0, s, table->view, threshold, clip,
+                       norms);
+    return check_launch("pxh_rescale_clip_table");
 }
 
 int pxh_sgd_update_multi(int count, float* const* w, float* const* d, const size_t* n, const int* apply_decay, int batch,

@@ -372,6 +372,52 @@ def sgd_update(w, d, batch, lr, momentum, decay=0.0, apply_decay=False):
          int(bool(apply_decay)), _stream())
 
 
+class TensorTable:
+    """A table of tensors kept on the device (pxh_tensor_table): build once, then every operation over all
+    of them is one launch.  `streams` is a list of 1, 2 or 4 lists of tensors (x | w, d | w, d, m, v)."""
+
+    def __init__(self, streams, apply_decay=None):
+        import ctypes
+        count = len(streams[0])
+        for group in streams:
+            assert len(group) == count
+            _chk_all(*group)
+        for tensors in zip(*streams):
+            assert len({x.numel() for x in tensors}) == 1
+        flat = [t for group in streams for t in group]
+        self._keep = flat                      # the tensors must outlive the table
+        handle = ctypes.c_void_p()
+        call("pxh_tensor_table_create", count, len(streams), _pointer_table(flat), _size_table(streams[0]),
+             _flag_table(apply_decay, count), ctypes.byref(handle))
+        self.handle = handle
+        self.count = int(capi.load().pxh_tensor_table_count(handle))
+
+    def close(self):
+        if self.handle:
+            capi.load().pxh_tensor_table_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:      # noqa: BLE001 - interpreter shutdown
+            pass
+
+    def adam_update(self, batch, t, lr, beta1=0.9, beta2=0.999, eps=1e-8, decay=0.0):
+        call("pxh_adam_update_table", self.handle, int(batch), int(t), float(lr), float(beta1), float(beta2),
+             float(eps), float(decay), _stream())
+
+    def sgd_update(self, batch, lr, momentum, decay=0.0):
+        call("pxh_sgd_update_table", self.handle, int(batch), float(lr), float(momentum), float(decay), _stream())
+
+    def fill(self, value):
+        call("pxh_fill_f32_table", self.handle, float(value), _stream())
+
+    def rescale_clip(self, threshold=0.0, clip=0.0, norms=None):
+        _chk(norms)
+        call("pxh_rescale_clip_table", self.handle, float(threshold), float(clip), ptr(norms), _stream())
+
+
 def fill_multi(xs, value):
     """pxh_fill_f32 for a list of float tensors in a few launches."""
     _chk_all(*xs)
