@@ -14,7 +14,10 @@ roofline   the leaky epilogue kernel: algorithmic bytes per launch / its mean la
            from HIP events recorded on the launch stream inside the timed region
 extras     the other kernels of the path (max-pool, upsample, shortcut, YOLO head, BN training
            forward/backward, Adam) at the baseline's shapes, measured after the timed region
-           and reported in the same line, with the non-conv ms/batch of YOLOv3 at 608
+           and reported in the same line; rows under 70 % of the HBM peak carry the time of a plain
+           copy of the same bytes, the largest shape of every family the CPU checker's time
+noconv_ms_per_batch_yolov3_608  one YOLOv3 training step at batch 16, non-conv kernels in model order
+config0_yolov3_tiny_forward_batch1  configs[0]: the tiny network's non-conv forward at batch 1, GPU and CPU
 cpu_baseline  the CPU checker (a port of the reference's single-threaded CPU path) timed on a
            bounded sample of the same workload on this host, one core
 """
@@ -172,7 +175,8 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     of Layer::forward, then the layer), backward in reverse (per layer the gradient rescale + clip
     of Layer::backward with the thresholds of yolov3.yml, 100 and 10, then the layer), update (the
     same helpers once more on every layer's delta and on each of the 222 update buffers, then Adam
-    on the 222 parameter tensors, all through the entry points that take many tensors per launch).
+    on the 222 parameter tensors, all through tables of tensors kept on the device: one or two launches
+    per operation).
     The convolutions' GEMMs are not run: a conv layer reads a resident conv result and its input
     gradient goes nowhere.  Each phase is timed as one HIP graph."""
     dev = torch.device("cuda")
@@ -276,14 +280,18 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
             n += 1
         launches["backward"] = n
 
+    # the tensors of update(), as tables kept on the device (what ParameterSet builds once)
+    delta_table = ops.TensorTable([[t["d"] for i, t in enumerate(T) if not absorbed(i)]])
+    hook_table = ops.TensorTable([pg])
+    adam_table = ops.TensorTable([pw, pg, pm, pv], decayed)
+
     def update(_, touch_delta=True):
         n = 0
         if touch_delta:         # the reference's update() passes every delta through the helpers once more
-            deltas = [t["d"] for i, t in enumerate(T) if not absorbed(i)]
-            ops.rescale_clip_multi(deltas, 100.0, 10.0); n += len(deltas)
-        # the hooks on every update buffer, each with its own norm, then Adam: every tensor in a few launches
-        ops.rescale_clip_multi(pg, 100.0, 10.0)
-        ops.adam_update_multi(pw, pg, pm, pv, N, 1, 1e-3, decay=5e-4, apply_decay=decayed)
+            delta_table.rescale_clip(100.0, 10.0); n += delta_table.count
+        # the hooks on every update buffer, each with its own norm, then Adam: one launch each for all tensors
+        hook_table.rescale_clip(100.0, 10.0)
+        adam_table.adam_update(N, 1, 1e-3, decay=5e-4)
         launches["update"] = n + 2
 
     out = {}
@@ -311,17 +319,42 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     return out
 
 
-def measure_extras(torch, ops, wl, timer, capi):
-    """The other kernels of the path at the baseline's shapes.  Returns (rows, ms_per_batch)."""
+def measure_extras(torch, ops, wl, timer, capi, cpu=None):
+    """The other kernels of the path at the baseline's shapes.  Returns (rows, ms_per_batch).  `cpu`:
+    cpu_rows(), attached to the rows it has a figure for."""
     import numpy as np
     dev = torch.device("cuda:0")
     rows = []
 
-    def add(name, shape, bytes_, ms, note=""):
+    copy_cache = {}
+
+    def copy_same_bytes(bytes_):
+        """A plain copy (half the bytes read, half written, through the route kernel) of the same size,
+        over buffers rotated as the row's are: what one launch of this size costs on this part whatever
+        it computes.  Cached per size rounded to 2 %."""
+        n = max(1024, int(bytes_ // 8) // 256 * 256)
+        key = int(round(np.log(n) / np.log(1.02)))
+        if key not in copy_cache:
+            rot = rotation_for(8 * n)
+            src = [torch.empty((1, n), device=dev).normal_() for _ in range(rot)]
+            dst = [torch.empty((1, n), device=dev) for _ in range(rot)]
+            saved = timer.last_min
+            copy_cache[key] = timer.time(lambda i: ops.route_forward(src[i], dst[i], 0), 20, rotate=rot)
+            timer.last_min = saved
+            del src, dst
+        return copy_cache[key]
+
+    def add(name, shape, bytes_, ms, note="", streaming=True):
         gbs = bytes_ / (ms * 1e-3) / 1e9
-        rows.append(dict(kernel=name, shape=shape, MB=round(bytes_ / 1e6, 1), ms=round(ms, 4),
-                         ms_min=round(timer.last_min, 4), GBps=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 3),
-                         note=note))
+        row = dict(kernel=name, shape=shape, MB=round(bytes_ / 1e6, 1), ms=round(ms, 4),
+                   ms_min=round(timer.last_min, 4), GBps=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 3), note=note)
+        # below the 70 % bar: how long a plain copy of the same bytes takes, i.e. how much of the gap is
+        # the cost of a launch of that size (vs_copy = copy time / this row's time; 1 = as fast as a copy)
+        if streaming and row["frac"] < 0.70 and bytes_ <= (1 << 30):
+            c_ms = copy_same_bytes(bytes_)
+            row["copy_same_bytes_ms"] = round(c_ms, 4)
+            row["vs_copy"] = round(c_ms / ms, 3)
+        rows.append(row)
         return ms
 
     def randn(*shape):
@@ -386,15 +419,14 @@ def measure_extras(torch, ops, wl, timer, capi):
         add("shortcut_bwd", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_b, "20B/elem")
         shortcut_ms[(c, s)] = (ms_f, ms_b, count)
         del a, b, o
-    # ---- YOLO head (config 3): batch 64
-    NB = 64
-    truths_np, counts_np = wl.yolo_truths(5100, NB)
-    truths = torch.from_numpy(truths_np).to(dev)
-    counts = torch.from_numpy(counts_np).to(dev)
+    # ---- YOLO head (config 3): batch 64, and batch 16 for the training step's own heads
     stats = torch.zeros(12, device=dev)
     cost = torch.zeros(1, device=dev)
     head_ms = {}
-    for s in wl.YOLOV3_HEAD_SIZES:
+    for NB, s in [(64, s_) for s_ in wl.YOLOV3_HEAD_SIZES] + [(N, s_) for s_ in wl.YOLOV3_HEAD_SIZES]:
+        truths_np, counts_np = wl.yolo_truths(5100, NB)
+        truths = torch.from_numpy(truths_np).to(dev)
+        counts = torch.from_numpy(counts_np).to(dev)
         e = NB * 255 * s * s
         rot = rotation_for(12 * e)
         xin = [2.0 * randn(NB, 255, s, s) for _ in range(rot)]
@@ -406,7 +438,7 @@ def measure_extras(torch, ops, wl, timer, capi):
             xin[i], out[i], dl[i], truths, counts, truths.shape[1], wl.YOLOV3_MASKS[s], wl.YOLOV3_ANCHORS, stats,
             cost, NB, 80, s, s, 608, 608, 0.7, 1.0, 1.0, 2.0, 0.1, 1.0), 20, rotate=rot)
         add("yolo_decode+delta+cost", "%dx255x%d^2" % (NB, s), 12 * e, ms_t, "fused 12B/elem")
-        head_ms[s] = (ms_d, ms_t)
+        head_ms[(NB, s)] = (ms_d, ms_t)
         # the reference's own split: loss from the decoded head with host-assigned positives
         acls, aanc, abox = wl.yolo_assign_targets(truths_np, counts_np, wl.YOLOV3_MASKS[s], wl.YOLOV3_ANCHORS, s, s,
                                                   608, 608)
@@ -417,7 +449,7 @@ def measure_extras(torch, ops, wl, timer, capi):
                                                   tabs[2], gmasks, ganch, stats, cost, NB, 9, 80, s, s, 608, 608,
                                                   0.7, 1.0, 1.0, 2.0, 0.1, 1.0), 20, rotate=rot)
         add("yolo_delta+cost", "%dx255x%d^2" % (NB, s), (4 + 4 * 5 / 85) * e, ms_l, "decoded input, 4.24B/elem")
-        if s == 76:
+        if s == 76 and NB == 64:
             # detections of the decoded head at a confidence threshold of 0.5: the objectness row of every
             # slot, the box and class rows of the slots that pass (about half of them on these logits)
             cap = 1 << 22
@@ -440,7 +472,7 @@ def measure_extras(torch, ops, wl, timer, capi):
                 passing = float((out[0].view(NB, 3, 85, s * s)[:, :, 4] >= thr).float().mean())
                 add("yolo_detections(thr %s)" % label, "%dx255x%d^2" % (NB, s),
                     4 * slots * (1 + passing * 84) + 32 * min(found, cap), ms_det,
-                    "%d records; %.2g%% of the slots pass" % (found, 100 * passing))
+                    "%d records; %.2g%% of the slots pass" % (found, 100 * passing), streaming=False)
             del rec
         del xin, out, dl
     # ---- non-maximum suppression of device-resident records: an inference-sized list (one image, one
@@ -462,7 +494,7 @@ def measure_extras(torch, ops, wl, timer, capi):
 
         ms = timer.time(suppress, 10)
         add("nms(thr .45)", "%d records, %d image%s" % (n_rec, images, "s" if images > 1 else ""), 64 * n_rec, ms,
-            "%d kept; not bandwidth bound" % int(kept_cnt.item()))
+            "%d kept; not bandwidth bound" % int(kept_cnt.item()), streaming=False)
         del recs, kept, ws
     # ---- BN training forward / backward (config 4): batch 16 @608, 13 shapes
     bn_ms = {}
@@ -544,18 +576,31 @@ def measure_extras(torch, ops, wl, timer, capi):
             ops.adam_update(pw[k], pd[k], pm[k], pv[k], 16, 1, 1e-3, 0.9, 0.999, 1e-8, 5e-4, decayed[k])
 
     ms = timer.time(one_by_one, 3)
-    add("adam_update x222", "%d tensors, %d params" % (len(sizes), P), 32 * P, ms, "one call per tensor, for comparison")
+    add("adam_update x222", "%d tensors, %d params" % (len(sizes), P), 32 * P, ms, "one call per tensor, for comparison",
+        streaming=False)
     ms = timer.time(lambda i: ops.sgd_update_multi(pw, pd, 16, 1e-3, 0.9, 5e-4, decayed), 10)
     add("sgd_update_multi", "%d tensors, %d params" % (len(sizes), P), 16 * P, ms, "7 launches")
     ms = timer.time(lambda i: ops.rescale_clip_multi(pd, 100.0, 10.0), 10)
     add("rescale_clip_multi(no-op)", "%d update buffers" % len(sizes), 4 * P, ms, "14 launches; norm only, 4B/param")
+
+    # ... and through tables kept on the device: one launch per operation (two for the hooks)
+    t_adam = ops.TensorTable([pw, pd, pm, pv], decayed)
+    ms = timer.time(lambda i: t_adam.adam_update(16, 1, 1e-3, 0.9, 0.999, 1e-8, 5e-4), 10)
+    add("adam_update_table", "%d tensors, %d params" % (len(sizes), P), 32 * P, ms, "1 launch")
+    ms = timer.time(lambda i: t_adam.sgd_update(16, 1e-3, 0.9, 5e-4), 10)
+    add("sgd_update_table", "%d tensors, %d params" % (len(sizes), P), 16 * P, ms, "1 launch")
+    t_hooks = ops.TensorTable([pd])
+    ms = timer.time(lambda i: t_hooks.rescale_clip(100.0, 10.0), 10)
+    add("rescale_clip_table(no-op)", "%d update buffers" % len(sizes), 4 * P, ms, "2 launches; norm only, 4B/param")
+    t_adam.close(); t_hooks.close()
 
     def hooks_one_by_one(i):
         for k in range(len(sizes)):
             ops.rescale_clip(pd[k], 100.0, 10.0)
 
     ms = timer.time(hooks_one_by_one, 3)
-    add("rescale_clip x222(no-op)", "%d update buffers" % len(sizes), 4 * P, ms, "one call (two launches) per buffer, for comparison")
+    add("rescale_clip x222(no-op)", "%d update buffers" % len(sizes), 4 * P, ms,
+        "one call (two launches) per buffer, for comparison", streaming=False)
     del w, g, m, v, d, big, pw, pd, pm, pv
     # ---- gradient rescale + clamp of a delta tensor: 4B/elem for the norm, 8B/elem to rewrite
     for c, s_ in [(256, 76), (64, 304)]:
@@ -577,7 +622,7 @@ def measure_extras(torch, ops, wl, timer, capi):
     # ---- non-conv ms per batch, YOLOv3 @608, batch 16, one training step:
     # 72 BN'd conv epilogues fwd+bwd, 3 bias epilogues, 23 shortcuts fwd+bwd, 2 upsamples and 2 route
     # concats fwd+bwd, the four max-pools of the data-movement configuration fwd+bwd, 3 heads (fused
-    # decode+delta) at batch 16 scaled from the batch-64 measurement, Adam
+    # decode+delta) measured at batch 16, Adam
     total = 0.0
     for key, (f, b, count) in bn_ms.items():
         total += (f + b) * count
@@ -586,10 +631,223 @@ def measure_extras(torch, ops, wl, timer, capi):
     for r in rows:
         if r["kernel"] in ("upsample_fwd", "upsample_bwd", "maxpool_fwd", "maxpool_bwd", "route_fwd", "route_bwd"):
             total += r["ms"]
-    for s, (ms_d, ms_t) in head_ms.items():
-        total += ms_t * N / NB
+    for (nb, s), (ms_d, ms_t) in head_ms.items():
+        if nb == N:
+            total += ms_t
     total += ms_adam
+    # the CPU checker beside the largest shape of every family
+    if cpu is not None:
+        for r in rows:
+            r.update(cpu.get((r["kernel"], r["shape"]), {}))
     return rows, total
+
+
+def measure_config0(torch, ops, wl, timer, with_cpu=True):
+    """configs[0]: the non-convolution layers of a YOLOv3-tiny inference forward at batch 1, 3x416x416
+    (the 24 layers of the reference's yolov3-tiny.yml, driven in model order as Model::forward does,
+    include/Model.h:1740-1759).  Every conv result is a resident N(0,1) tensor of the real shape; each
+    conv layer's epilogue (folded BN + leaky, or bias alone for the two head convs), the six max-pools,
+    the upsample, the two routes and the two head decodes run in layer order, once eagerly launched
+    and once as one HIP graph.  Beside it the CPU checker on the same tensors, one core, per layer kind."""
+    import numpy as np
+    dev = torch.device("cuda:0")
+    layers = wl.yolov3_tiny_layers(416)
+    T = []
+    for i, l in enumerate(layers):
+        c, s = l["c"], l["s"]
+        t = {}
+        if l["type"] == "conv":
+            t["x"] = torch.from_numpy(wl.normal(3000 + i, (1, c, s, s))).to(dev)
+            t["y"] = torch.empty_like(t["x"])
+            scale, bias, mean, var = wl.bn_params(2000 + i, c)
+            t["host"] = (scale, bias, mean, var)
+            t["bias"] = torch.from_numpy(bias).to(dev)
+            if l["bn"]:
+                t["folded"] = ops.bn_fold(*(torch.from_numpy(a).to(dev) for a in (mean, var, scale, bias)))
+        elif l["type"] == "maxpool":
+            o = s if l["stride"] == 1 else s // 2
+            t["y"] = torch.empty((1, c, o, o), device=dev)
+            t["idx"] = torch.empty((1, c, o, o), device=dev, dtype=torch.int32)
+        else:
+            t["y"] = torch.empty((1, c, s, s), device=dev)
+        T.append(t)
+
+    def forward(_):
+        for i, (l, t) in enumerate(zip(layers, T)):
+            kind = l["type"]
+            if kind == "conv" and l["bn"]:
+                ops.bn_folded_act_forward(t["x"], t["y"], t["folded"], l["act"])
+            elif kind == "conv":
+                ops.bias_act_forward(t["x"], t["y"], t["bias"], l["act"])
+            elif kind == "maxpool":
+                ops.maxpool_forward(T[i - 1]["y"], t["y"], t["idx"], 2, l["stride"], 1)
+            elif kind == "upsample":
+                ops.upsample_forward(T[i - 1]["y"], t["y"], 2, 1.0)
+            elif kind == "route":
+                offset = 0
+                for src in l["sources"]:
+                    ops.route_forward(T[src]["y"], t["y"], offset)
+                    offset += layers[src]["c"] * l["s"] * l["s"]
+            elif kind == "yolo":
+                ops.yolo_activate(T[i - 1]["y"], t["y"], 1, 3, 80, l["s"] * l["s"])
+
+    out = dict(workload="YOLOv3-tiny inference forward, batch 1, 416x416: non-conv layers in model order "
+                        "(13 conv epilogues, 6 max-pools, 1 upsample, 2 routes, 2 head decodes; 27 launches)")
+    out["gpu_graph_ms"] = round(timer.time(forward, 5, warm=2), 4)
+    timer.use_graphs, saved = False, timer.use_graphs
+    out["gpu_eager_ms"] = round(timer.time(forward, 5, warm=2), 4)
+    timer.use_graphs = saved
+    elems = sum(int(t["y"].numel()) for t in T)
+    out["elements_written"] = elems
+    if with_cpu:
+        import oracle
+        oracle.lib()
+        F = np.float32
+        by_kind = {}
+        H = [None] * len(layers)
+
+        def timed(kind, fn):
+            t0 = time.perf_counter()
+            fn()
+            by_kind[kind] = by_kind.get(kind, 0.0) + (time.perf_counter() - t0) * 1e3
+
+        for i, (l, t) in enumerate(zip(layers, T)):
+            kind, c, s = l["type"], l["c"], l["s"]
+            if kind == "conv":
+                y = t["x"].cpu().numpy().copy()
+                scale, bias, mean, var = t["host"]
+                if l["bn"]:
+                    timed("conv epilogue", lambda: oracle.conv_epilogue_forward(
+                        True, False, l["act"], 1, c, s, s, y, None, np.zeros(c, F), np.zeros(c, F), mean.copy(),
+                        var.copy(), scale, bias, None, None))
+                else:
+                    timed("conv epilogue", lambda: oracle.conv_epilogue_forward(
+                        False, False, l["act"], 1, c, s, s, y, None, None, None, None, None, None, bias, None, None))
+                H[i] = y
+            elif kind == "maxpool":
+                o = s if l["stride"] == 1 else s // 2
+                y = np.empty((1, c, o, o), F); idx = np.empty((1, c, o, o), np.int32)
+                timed("max-pool", lambda: oracle.maxpool_forward(H[i - 1], y, idx, 1, c, s, s, o, o, 2, l["stride"], 1))
+                H[i] = y
+            elif kind == "upsample":
+                y = np.empty((1, c, s, s), F)
+                timed("upsample", lambda: oracle.upsample(H[i - 1], s // 2, s // 2, c, 1, 2, True, 1.0, None, y))
+                H[i] = y
+            elif kind == "route":
+                y = np.empty((1, c * s * s), F)
+
+                def concat():
+                    offset = 0
+                    for src in l["sources"]:
+                        oracle.route_forward(H[src].reshape(1, -1), y, offset)
+                        offset += layers[src]["c"] * s * s
+
+                timed("route", concat)
+                H[i] = y.reshape(1, c, s, s)
+            elif kind == "yolo":
+                cfg, keep = oracle.yolo_cfg(1, s, s, 80, l["mask"], wl.TINY_ANCHORS, 416, 416)
+                y = np.zeros_like(H[i - 1])
+                timed("yolo decode", lambda: oracle.yolo_decode(cfg, H[i - 1], y))
+                H[i] = y
+        out["cpu_ms_by_layer_kind"] = {k: round(v, 3) for k, v in by_kind.items()}
+        out["cpu_ms"] = round(sum(by_kind.values()), 3)
+        out["cpu_cores"] = 1
+        # the chain's last tensors agree: the two runs did the same work
+        last = T[-1]["y"].cpu().numpy()
+        out["gpu_matches_cpu"] = bool(np.allclose(last, H[-1], rtol=1e-5, atol=1e-6))
+    return out
+
+
+def cpu_rows(wl):
+    """The CPU checker (one core) on one image -- or, for the per-channel reductions, on two channels at
+    the full batch -- of the largest shape of each kernel family, scaled to the batch: milliseconds keyed
+    by (kernel, shape) as the extras rows name them."""
+    import numpy as np
+    import oracle
+    oracle.lib()
+    F = np.float32
+    N = 16
+    out = {}
+
+    def ms_of(fn, scale):
+        # the second of two runs: the first also pays for the first touch of freshly allocated pages
+        best = None
+        for _ in range(2):
+            t0 = time.perf_counter()
+            fn()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        return best * 1e3 * scale
+
+    def note(kernel, shape, ms, sample):
+        out[(kernel, shape)] = dict(cpu_ms=round(ms, 2), cpu_sample=sample)
+
+    # max-pool 16x64x304^2
+    c, s = 64, 304
+    x = wl.normal(1, (1, c, s, s)); y = np.empty((1, c, s // 2, s // 2), F); idx = np.empty(y.shape, np.int32)
+    note("maxpool_fwd", "%dx%dx%d^2" % (N, c, s), ms_of(lambda: oracle.maxpool_forward(x, y, idx, 1, c, s, s, s // 2, s // 2, 2, 2, 1), N),
+         "1 image x %d" % N)
+    d = wl.normal(2, y.shape); g = x.copy()
+    note("maxpool_bwd", "%dx%dx%d^2" % (N, c, s), ms_of(lambda: oracle.maxpool_backward(d, idx, g), N), "1 image x %d" % N)
+    # upsample 16x128x38^2 -> 76^2
+    c, s = 128, 38
+    x = wl.normal(3, (1, c, s, s)); y = np.empty((1, c, 2 * s, 2 * s), F)
+    note("upsample_fwd", "%dx%dx%d^2" % (N, c, s), ms_of(lambda: oracle.upsample(x, s, s, c, 1, 2, True, 1.0, None, y), N),
+         "1 image x %d" % N)
+    acc = x.copy()
+    note("upsample_bwd", "%dx%dx%d^2" % (N, c, s), ms_of(lambda: oracle.upsample(x, s, s, c, 1, 2, False, 1.0, acc, y), N),
+         "1 image x %d" % N)
+    # shortcut 16x64x304^2
+    c, s = 64, 304
+    a = wl.normal(4, (1, c, s, s)); b = wl.normal(5, a.shape); o = np.empty_like(a); pre = np.empty_like(a)
+    note("shortcut_fwd", "%dx%dx%d^2" % (N, c, s),
+         ms_of(lambda: oracle.shortcut_forward("linear", 1, s, s, c, a, b, 1.0, 1.0, o, pre), N), "1 image x %d" % N)
+    fd = b.copy(); gr = a.copy()
+    note("shortcut_bwd", "%dx%dx%d^2" % (N, c, s),
+         ms_of(lambda: oracle.shortcut_backward("linear", 1, s, s, c, o, pre, fd, gr, 1.0, 1.0), N), "1 image x %d" % N)
+    # route: the 256-channel source of 16x(128+)256x76^2
+    c1, c2, s = 128, 256, 76
+    src = wl.normal(6, (1, c2 * s * s)); dst = np.empty((1, (c1 + c2) * s * s), F)
+    note("route_fwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), ms_of(lambda: oracle.route_forward(src, dst, c1 * s * s), N),
+         "1 image x %d" % N)
+    note("route_bwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), ms_of(lambda: oracle.route_backward(dst, src, c1 * s * s), N),
+         "1 image x %d" % N)
+    # YOLO head 64x255x76^2: decode, and the training pass with that image's truths
+    NB, s = 64, 76
+    x = wl.normal(7, (1, 255, s, s), std=2.0)
+    truths, counts = wl.yolo_truths(5100, NB)
+    cfg, keep = oracle.yolo_cfg(1, s, s, 80, wl.YOLOV3_MASKS[s], wl.YOLOV3_ANCHORS, 608, 608, ignore_thresh=0.7,
+                                object_scale=2.0, noobject_scale=0.1)
+    y = np.zeros_like(x); dl = np.zeros_like(x)
+    note("yolo_decode", "%dx255x%d^2" % (NB, s), ms_of(lambda: oracle.yolo_decode(cfg, x, y), NB), "1 image x %d" % NB)
+    note("yolo_decode+delta+cost", "%dx255x%d^2" % (NB, s),
+         ms_of(lambda: oracle.yolo_forward(cfg, x, np.ascontiguousarray(truths[:1]), np.ascontiguousarray(counts[:1]),
+                                           truths.shape[1], y, dl), NB), "1 image x %d" % NB)
+    # BN training forward and backward 16x32x608^2: two channels at the full batch
+    c, s, sub = 32, 608, 2
+    x = wl.normal(8, (N, sub, s, s)); scale, bias, rm, rv = wl.bn_params(9, sub)
+    outp = x.copy(); pre = np.empty_like(x); xs = np.empty_like(x); xn = np.empty_like(x)
+    mean = np.zeros(sub, F); var = np.zeros(sub, F)
+    note("bn_train_fwd(leaky)", "%dx%dx%d^2" % (N, c, s),
+         ms_of(lambda: oracle.conv_epilogue_forward(True, True, "leaky", N, sub, s, s, outp, pre, mean, var, rm, rv, scale,
+                                                    bias, xs, xn), c / sub), "%d of %d channels at batch %d, x %d" % (sub, c, N, c // sub))
+    dd = wl.normal(10, x.shape); su = np.zeros(sub, F); bu = np.zeros(sub, F); md = np.zeros(sub, F); vd = np.zeros(sub, F)
+    note("bn_bwd(leaky)", "%dx%dx%d^2" % (N, c, s),
+         ms_of(lambda: oracle.conv_epilogue_backward(True, "leaky", N, sub, s, s, dd, pre, mean, var, md, vd, scale, su, bu,
+                                                     xs, xn), c / sub), "%d of %d channels at batch %d, x %d" % (sub, c, N, c // sub))
+    # Adam, SGD and the gradient helpers on 4 M parameters, scaled to the 61.9 M of the model
+    P, n = wl.YOLOV3_PARAMS, 4 << 20
+    w = wl.normal(11, n, std=0.02); g = wl.normal(12, n, std=1e-3); m = np.zeros(n, F); v = np.zeros(n, F)
+    note("adam_update", "%d params" % P, ms_of(lambda: oracle.adam_update(w, g, m, v, 16, 1, 1e-3, 0.9, 0.999, 1e-8, 5e-4, True), P / n),
+         "%d parameters x %.1f" % (n, P / n))
+    g = wl.normal(12, n, std=1e-3)
+    note("sgd_update", "%d params" % P, ms_of(lambda: oracle.sgd_update(w, g, 16, 1e-3, 0.9, 5e-4, True), P / n),
+         "%d parameters x %.1f" % (n, P / n))
+    e = N * 64 * 304 * 304
+    g = wl.normal(13, n)
+    note("rescale_clip", "%dx%dx%d^2" % (N, 64, 304), ms_of(lambda: oracle.rescale_clip(g, 1e-3, 1e-6), e / n),
+         "%d values x %.1f" % (n, e / n))
+    return out
 
 
 def calibration_copy(torch, ops, timer):
@@ -683,6 +941,9 @@ def main():
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                     frac=round(achieved / HBM_PEAK_GBS, 4),
                     traffic=None if EPILOGUE_TRAFFIC_RATIO is None else round(EPILOGUE_TRAFFIC_RATIO * bytes_per_launch),
+                    traffic_source="profiles/epilogue_sweep_hbm_traffic.txt: FETCH_SIZE + WRITE_SIZE of this kernel in "
+                                   "two rocprofv3 --pmc runs of this script, as a ratio of its algorithmic bytes; not "
+                                   "measured in this run",
                     kernel="epilogue_fwd_kernel<PXH_LEAKY, true, *>",
                     bytes_per_launch=round(bytes_per_launch),
                     mean_launch_ms=round(leaky_ms / launches, 5))
@@ -716,13 +977,23 @@ def main():
     copy_row = calibration_copy(torch, ops, timer)
     log("plain copy of 2 x 512 MiB: %.4f ms %.1f GB/s" % (copy_row["ms"], copy_row["GBps"]))
 
-    extras, ms_batch, model_order = (None, None, None)
+    extras, ms_batch, model_order, config0 = (None, None, None, None)
     if not args.no_extras:
-        extras, ms_batch = measure_extras(torch, ops, wl, timer, capi)
+        config0 = measure_config0(torch, ops, wl, timer, with_cpu=not args.no_cpu)
+        log("configs[0], YOLOv3-tiny inference forward at batch 1, non-conv layers in model order:", config0)
+        cpu_by_row = None
+        if not args.no_cpu:
+            t0 = time.perf_counter()
+            cpu_by_row = cpu_rows(wl)
+            log("CPU checker on the largest shape of every kernel family: %.1f s" % (time.perf_counter() - t0))
+        extras, ms_batch = measure_extras(torch, ops, wl, timer, capi, cpu_by_row)
         for r in extras:
-            log("%-24s %-18s %9.1f MB %8.4f ms %8.1f GB/s  %4.1f%%  %s"
-                % (r["kernel"], r["shape"], r["MB"], r["ms"], r["GBps"], 100 * r["frac"], r["note"]))
-        log("non-conv ms/batch, YOLOv3 @608, batch 16, training step: %.3f" % ms_batch)
+            log("%-26s %-22s %9.1f MB %8.4f ms %8.1f GB/s  %4.1f%%  %s%s%s"
+                % (r["kernel"], r["shape"], r["MB"], r["ms"], r["GBps"], 100 * r["frac"],
+                   ("copy of the same bytes %.4f ms (%.2f)  " % (r["copy_same_bytes_ms"], r["vs_copy"]))
+                   if "vs_copy" in r else "",
+                   ("cpu %.1f ms  " % r["cpu_ms"]) if "cpu_ms" in r else "", r["note"]))
+        log("sum of the layer kernels of one YOLOv3 @608 training step at batch 16: %.3f ms" % ms_batch)
         model_order = measure_model_order(torch, ops, wl, timer)
         log("the same step in model order, with the Layer base's fills and gradient helpers:", model_order)
 
@@ -751,8 +1022,13 @@ def main():
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2)},
         "roofline": roofline,
         "cpu_baseline": cpu,
-        "noconv_ms_per_batch_yolov3_608": None if ms_batch is None else round(ms_batch, 3),
+        # the second half of the metric: one training step of YOLOv3 @608 at batch 16, every non-conv kernel
+        # launched in model order with what the Layer base class adds around each layer (measured, three
+        # HIP graphs); beside it the plain sum of the layer kernels' own rows
+        "noconv_ms_per_batch_yolov3_608": None if model_order is None else model_order["total_ms"],
+        "noconv_layer_kernels_sum_ms_yolov3_608": None if ms_batch is None else round(ms_batch, 3),
         "noconv_step_in_model_order_yolov3_608": model_order,
+        "config0_yolov3_tiny_forward_batch1": config0,
         "value_folding_every_call": round(value_raw, 1),
         "plain_copy": copy_row,
         "per_activation": per_act,

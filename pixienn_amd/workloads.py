@@ -167,6 +167,32 @@ def yolov3_layers(size=608):
     return layers
 
 
+def yolov3_tiny_layers(size=416):
+    """The 24 layers of resources/models/yolov3-tiny.yml of the reference at a size x size input, in
+    model order, as dicts like yolov3_layers': conv (c, s, bn, act), maxpool (c, s = input size, stride),
+    upsample, route (sources), yolo (mask)."""
+    layers = []
+    s = size
+    for c in (16, 32, 64, 128, 256, 512):
+        layers.append(dict(type="conv", c=c, s=s, bn=True, act="leaky"))
+        stride = 1 if c == 512 else 2
+        layers.append(dict(type="maxpool", c=c, s=s, stride=stride))
+        s = s if stride == 1 else s // 2
+    layers.append(dict(type="conv", c=1024, s=s, bn=True, act="leaky"))          # 12
+    layers.append(dict(type="conv", c=256, s=s, bn=True, act="leaky"))           # 13
+    layers.append(dict(type="conv", c=512, s=s, bn=True, act="leaky"))           # 14
+    layers.append(dict(type="conv", c=255, s=s, bn=False, act="linear"))         # 15
+    layers.append(dict(type="yolo", c=255, s=s, mask=TINY_MASKS[0]))             # 16
+    layers.append(dict(type="route", c=256, s=s, sources=[13]))                  # 17
+    layers.append(dict(type="conv", c=128, s=s, bn=True, act="leaky"))           # 18
+    layers.append(dict(type="upsample", c=128, s=2 * s))                         # 19
+    layers.append(dict(type="route", c=384, s=2 * s, sources=[19, 8]))           # 20
+    layers.append(dict(type="conv", c=256, s=2 * s, bn=True, act="leaky"))       # 21
+    layers.append(dict(type="conv", c=255, s=2 * s, bn=False, act="linear"))     # 22
+    layers.append(dict(type="yolo", c=255, s=2 * s, mask=TINY_MASKS[1]))         # 23
+    return layers
+
+
 def yolov3_parameter_tensors(size=608):
     """(elements, takes_weight_decay) of every parameter tensor of YOLOv3 in layer order, as the engine
     holds them: per convolution the weights (filters x input channels x k x k, decayed), the biases and,
