@@ -748,7 +748,12 @@ struct FillFromRecord {
     __device__ FillOp operator()(const TensorRecord& r) const { return FillOp{ r.stream[0], value }; }
 };
 
-// `streaming_elems`: tensors of at least this many elements go past the caches, as in the single call.
+// `streaming_elems`: tensors of at least this many elements go past the caches (0: all of them).
+// A workgroup takes kTableChunks consecutive 1024-element chunks of its tensor, so that the cost of
+// finding the tensor is spread over four times the elements (it is what the single call does not pay).
+constexpr int kTableChunks = 4;
+constexpr uint32_t kTablePerBlock = kMultiPerBlock * kTableChunks;
+
 template<typename Maker>
 __global__ __launch_bounds__(kBlock) void table_stream_kernel(TableView t, Maker make, unsigned long long streaming_elems)
 {
@@ -757,23 +762,37 @@ __global__ __launch_bounds__(kBlock) void table_stream_kernel(TableView t, Maker
     const TensorRecord r = t.records[i];
     const auto op = make(r);
     const size_t n = r.n;
-    const size_t e = (static_cast<size_t>(blockIdx.x - firsts[i]) * kBlock + threadIdx.x) * 4;
-    if (e >= n) return;
     using Op = decltype(make(r));
-    if (r.vector && e + 4 <= n) {
-        typename Op::template Regs<4> regs;
+    const size_t base = static_cast<size_t>(blockIdx.x - firsts[i]) * kTablePerBlock + static_cast<size_t>(threadIdx.x) * 4;
+    if (r.vector && base + (kTableChunks - 1) * kMultiPerBlock + 4 <= n) {
+        // every chunk holds a whole vector for this lane: the loads of all of them go out together
+        typename Op::template Regs<4> regs[kTableChunks];
         if (n >= streaming_elems) {
-            op.template load<4, true>(e, regs);
-            op.template finish<4, true>(e, regs);
+#pragma unroll
+            for (int c = 0; c < kTableChunks; ++c) op.template load<4, true>(base + c * kMultiPerBlock, regs[c]);
+#pragma unroll
+            for (int c = 0; c < kTableChunks; ++c) op.template finish<4, true>(base + c * kMultiPerBlock, regs[c]);
         } else {
+#pragma unroll
+            for (int c = 0; c < kTableChunks; ++c) op.template load<4, false>(base + c * kMultiPerBlock, regs[c]);
+#pragma unroll
+            for (int c = 0; c < kTableChunks; ++c) op.template finish<4, false>(base + c * kMultiPerBlock, regs[c]);
+        }
+        return;
+    }
+    for (int c = 0; c < kTableChunks; ++c) {
+        const size_t e = base + c * kMultiPerBlock;
+        if (e >= n) return;
+        if (r.vector && e + 4 <= n) {
+            typename Op::template Regs<4> regs;
             op.template load<4, false>(e, regs);
             op.template finish<4, false>(e, regs);
-        }
-    } else {
-        for (size_t k = e; k < n && k < e + 4; ++k) {
-            typename Op::template Regs<1> regs;
-            op.template load<1, false>(k, regs);
-            op.template finish<1, false>(k, regs);
+        } else {
+            for (size_t k = e; k < n && k < e + 4; ++k) {
+                typename Op::template Regs<1> regs;
+                op.template load<1, false>(k, regs);
+                op.template finish<1, false>(k, regs);
+            }
         }
     }
 }
@@ -1172,6 +1191,7 @@ int pxh_fill_f32_multi(int count, float* const* x, const size_t* n, float value,
 struct pxh_tensor_table {
     int device;
     int count, streams;
+    unsigned long long total_elems;
     uint32_t blocks, norm_blocks;
     void* memory;
     pxh::TableView view;
@@ -1206,7 +1226,7 @@ int pxh_tensor_table_create(int count, int streams, float* const* buffers, const
         records.push_back(r);
         first_block.push_back(static_cast<uint32_t>(blocks));
         first_norm_block.push_back(static_cast<uint32_t>(norm_blocks));
-        blocks += (n[i] + kMultiPerBlock - 1) / kMultiPerBlock;
+        blocks += (n[i] + kTablePerBlock - 1) / kTablePerBlock;
         // the norm pass of the single call: at most kNormBlocks workgroups, each a whole step of loads
         const size_t per_step = static_cast<size_t>(kBlock) * (r.norm_vector ? 4 : 1) * kNormLoads;
         const size_t want = (n[i] + per_step - 1) / per_step;
@@ -1227,6 +1247,7 @@ int pxh_tensor_table_create(int count, int streams, float* const* buffers, const
     if (!t) return fail_invalid("pxh_tensor_table_create: out of host memory");
     t->count = static_cast<int>(records.size());
     t->streams = streams;
+    for (const TensorRecord& r: records) t->total_elems += r.n;
     t->blocks = static_cast<uint32_t>(blocks);
     t->norm_blocks = static_cast<uint32_t>(norm_blocks);
     if (hipGetDevice(&t->device) != hipSuccess) t->device = -1;
@@ -1286,7 +1307,10 @@ int launch_table(const char* who, const pxh_tensor_table* table, int streams_nee
     if (table->streams < streams_needed)
         return fail_invalid("%s: the table holds %d buffers per tensor, %d are needed", who, table->streams, streams_needed);
     if (table->count == 0) return PXH_OK;
-    const unsigned long long streaming_elems = (streaming_from + bytes_per_elem - 1) / bytes_per_elem;
+    // the tensors of a table are walked in one sweep: whether that sweep outgrows the last-level cache is a
+    // matter of all of them together, not of each one's size
+    const bool past_cache = table->total_elems * static_cast<unsigned long long>(bytes_per_elem) >= streaming_from;
+    const unsigned long long streaming_elems = past_cache ? 0ull : ~0ull;
     hipLaunchKernelGGL((table_stream_kernel<Maker>), dim3(table->blocks), dim3(kBlock), 0, as_stream(stream), table->view,
                        make, streaming_elems);
     return check_launch(who);
