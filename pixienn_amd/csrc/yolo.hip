@@ -1432,9 +1432,11 @@ __global__ __launch_bounds__(kBlock) void yolo_patch_kernel(PatchArgs a)
 
 // ---------------------------------------------------------------- detections
 // Thresholded compaction of a decoded head (include/YoloLayer.h:601-698): one lane per slot; a slot
-// whose objectness passes walks its class rows, and the lanes of a wave that found a detection in
-// the same class step reserve their output places with one atomic between them.  The records
-// carry their position in the reference's emission order, so sorting by it restores that order.
+// whose objectness passes walks its class rows, and all lanes of a workgroup that found detections
+// in the same class step reserve their output places with one atomic between them: the counter is
+// one address for the whole grid, takes about 15 ns per atomic, and at one atomic per wave that
+// was most of the kernel's time when half the slots pass.  The records carry their position in the
+// reference's emission order, so sorting by it restores that order.
 struct DetectArgs {
     const float* pred;
     pxh_detection* out;
@@ -1447,9 +1449,13 @@ struct DetectArgs {
     FastDiv by_area;
 };
 
-__global__ __launch_bounds__(kBlock) void yolo_detect_kernel(DetectArgs a, YoloParams p)
+constexpr int kDetectBlock = 512;
+
+__global__ __launch_bounds__(kDetectBlock) void yolo_detect_kernel(DetectArgs a, YoloParams p)
 {
-    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    __shared__ int wave_first[kDetectBlock / kWave];
+    __shared__ int group_first;
+    const uint32_t t = blockIdx.x * kDetectBlock + threadIdx.x;
     const bool live = t < a.slots;
     const uint32_t slot = live ? t : 0;
     uint32_t bn, cell, b, n;
@@ -1503,13 +1509,17 @@ __global__ __launch_bounds__(kBlock) void yolo_detect_kernel(DetectArgs a, YoloP
             by = bh > 0.0f ? y - bh / 2.0f : y;
         }
     }
-    if (!__ballot(pass)) return;
+    if (!__syncthreads_or(pass)) return;
     const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
     const uint32_t order0 = ((b * static_cast<uint32_t>(area) + cell) * p.mask_count + n) * p.classes;
     const float* rows = a.pred + base + 5 * static_cast<size_t>(area);
-    // 128 classes at a time: each lane notes its hits in a bit mask, the wave reserves the places
-    // of all of them with ONE atomic (a counter shared by the whole grid cannot take one per hit),
-    // then every lane writes its records one after the other.
+    // 128 classes at a time: each lane notes its hits in a bit mask, the workgroup reserves the
+    // places of all of them with ONE atomic, then every lane writes its records one after the other.
+    // The class rows are read 32 at a time with their loads in flight together (one after the other
+    // they cost a memory latency each, the larger part of the kernel's time when many slots pass),
+    // and read again, from the cache, for the words that hold a hit.  Keeping 64 of them in registers
+    // over the reservation instead was slower: 171 registers, two waves per SIMD.
     constexpr int kWords = 4;
     for (int j0 = 0; j0 < p.classes; j0 += 32 * kWords) {
         uint32_t hits[kWords];
@@ -1518,12 +1528,15 @@ __global__ __launch_bounds__(kBlock) void yolo_detect_kernel(DetectArgs a, YoloP
         for (int w = 0; w < kWords; ++w) {
             hits[w] = 0u;
             const int first = j0 + 32 * w;
-            const int last = min(first + 32, p.classes);
-            if (pass) {
-                for (int j = first; j < last; ++j) {
-                    const float prob = objectness * rows[static_cast<size_t>(j) * area];
-                    if (prob >= a.threshold) {
-                        hits[w] |= 1u << (j - first);
+            const int rows_here = min(32, p.classes - first);
+            if (pass && rows_here > 0) {
+                float v[32];
+#pragma unroll
+                for (int k = 0; k < 32; ++k) v[k] = rows[static_cast<size_t>(first + min(k, rows_here - 1)) * area];
+#pragma unroll
+                for (int k = 0; k < 32; ++k) {
+                    if (k < rows_here && objectness * v[k] >= a.threshold) {
+                        hits[w] |= 1u << k;
                         ++mine;
                     }
                 }
@@ -1532,28 +1545,46 @@ __global__ __launch_bounds__(kBlock) void yolo_detect_kernel(DetectArgs a, YoloP
         int upto = mine;      // inclusive prefix sum over the lanes
 #pragma unroll
         for (int off = 1; off < kWave; off <<= 1) {
-            const int v = __shfl_up(upto, off, kWave);
-            if (lane >= off) upto += v;
+            const int up = __shfl_up(upto, off, kWave);
+            if (lane >= off) upto += up;
         }
-        const int total = __shfl(upto, kWave - 1, kWave);
-        if (total == 0) continue;
-        int first_place = 0;
-        if (lane == kWave - 1) first_place = atomicAdd(a.count, total);
-        first_place = __shfl(first_place, kWave - 1, kWave);
-        int at = first_place + upto - mine;
+        if (j0 > 0) __syncthreads();      // the previous step's places have been read
+        if (lane == kWave - 1) wave_first[wave] = upto;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int sum = 0;
+#pragma unroll
+            for (int w = 0; w < kDetectBlock / kWave; ++w) {
+                const int n_w = wave_first[w];
+                wave_first[w] = sum;
+                sum += n_w;
+            }
+            group_first = sum ? atomicAdd(a.count, sum) : 0;
+        }
+        __syncthreads();
+        int at = group_first + wave_first[wave] + upto - mine;
 #pragma unroll
         for (int w = 0; w < kWords; ++w) {
-            uint32_t bits = hits[w];
-            while (bits) {
-                const int j = j0 + 32 * w + __builtin_ctz(bits);
-                bits &= bits - 1;
+            if (!hits[w]) continue;
+            if (at >= a.capacity) {
+                at += __builtin_popcount(hits[w]);
+                continue;
+            }
+            const int first = j0 + 32 * w;
+            const int rows_here = min(32, p.classes - first);
+            float v[32];
+#pragma unroll
+            for (int k = 0; k < 32; ++k) v[k] = rows[static_cast<size_t>(first + min(k, rows_here - 1)) * area];
+#pragma unroll
+            for (int k = 0; k < 32; ++k) {
+                if (!((hits[w] >> k) & 1u)) continue;
                 if (at < a.capacity) {
                     pxh_detection d;
                     d.x = bx; d.y = by; d.w = bw; d.h = bh;
-                    d.prob = objectness * rows[static_cast<size_t>(j) * area];
+                    d.prob = objectness * v[k];
                     d.batch = static_cast<int>(b);
-                    d.class_index = j;
-                    d.order = a.order_base + order0 + j;
+                    d.class_index = first + k;
+                    d.order = a.order_base + order0 + first + k;
                     a.out[at] = d;
                 }
                 ++at;
@@ -1932,7 +1963,7 @@ int pxh_yolo_detections_append(const float* predictions, int batch, const int* h
     a.slots = static_cast<uint32_t>(batch) * mask_count * p.area;
     a.order_base = order_base;
     a.by_area = FastDiv(p.area);
-    hipLaunchKernelGGL(yolo_detect_kernel, dim3(grid_for(a.slots, kBlock)), dim3(kBlock), 0, s, a, p);
+    hipLaunchKernelGGL(yolo_detect_kernel, dim3(grid_for(a.slots, kDetectBlock)), dim3(kDetectBlock), 0, s, a, p);
     return check_launch("pxh_yolo_detections");
 }
 
