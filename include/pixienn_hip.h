@@ -378,6 +378,35 @@ size_t pxh_rescale_multi_workspace_bytes(void);
 int pxh_rescale_clip_multi(int count, float* const* x, const size_t* n, float threshold, float clip,
                            float* norms, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Norm and largest magnitude from the kernel that writes the delta.  Layer::backward opens with the
+ * two helpers above on the layer's own delta (include/Layer.h:385-397), which costs a read of the
+ * tensor just for the norm.  Where one of this library's kernels is the LAST to write that delta
+ * before its layer's backward -- the convolution in front of a shortcut receives its whole delta
+ * from the shortcut's backward (include/ShortcutLayer.h:98-111), the layer in front of a YOLO head
+ * from the head's `grad += delta` (include/YoloLayer.h:741-750) -- that kernel can leave behind, per
+ * group of 256 values, the sum of squares and the largest magnitude of what it wrote (8 bytes per
+ * KiB of tensor), and pxh_rescale_clip_from_groups starts from those instead of reading the tensor.
+ * The sums are added in the order pxh_rescale_clip itself adds them: norm, verdict and rewritten
+ * tensor are the same to the bit.
+ *   groups: device buffer of pxh_norm_groups_bytes(n) bytes, 8-byte aligned, owned by the caller;
+ *           it describes the tensor only until the tensor is written again.
+ * A tensor that is not 16-byte aligned, or whose length is not a multiple of 4, has no group sums:
+ * the producers then leave the buffer alone and pxh_rescale_clip_from_groups reads the tensor, so the
+ * pair can be used without looking at the pointer.
+ *   pxh_norm_groups               the group sums of a tensor as it is (one read)
+ *   pxh_axpy_norm                 pxh_axpy, + the group sums of y
+ *   pxh_shortcut_backward_norm    pxh_shortcut_backward (first == 0) or pxh_shortcut_backward_first
+ *                                 (first != 0), + the group sums of grad, which is required */
+size_t pxh_norm_groups_bytes(size_t n);
+int pxh_norm_groups(const float* x, size_t n, void* groups, void* stream);
+int pxh_axpy_norm(size_t n, float alpha, const float* x, float* y, void* y_groups, void* stream);
+int pxh_shortcut_backward_norm(float* delta, const float* pre_activation, float* from_delta,
+                               float* grad, size_t n, float alpha, float beta, int activation,
+                               int first, void* grad_groups, void* stream);
+int pxh_rescale_clip_from_groups(float* x, size_t n, float threshold, float clip, float* norm_out,
+                                 const void* groups, void* workspace, size_t workspace_bytes,
+                                 void* stream);
+
 /* ------------------------------------------------------------------------
  * Adam.  include/Adam.cuh:21, include/cuda/Adam.h:49-90.
  * ---------------------------------------------------------------------- */

@@ -56,6 +56,10 @@ SIGNATURES = {
     "pxh_yolo_forward_train": [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, F, F, F, F, P, Z, P],
     "pxh_sgd_update": [Z, P, P, I, F, F, F, I, P],
     "pxh_rescale_clip": [P, Z, F, F, P, P, Z, P],
+    "pxh_norm_groups": [P, Z, P, P],
+    "pxh_axpy_norm": [Z, F, P, P, P, P],
+    "pxh_shortcut_backward_norm": [P, P, P, P, Z, F, F, I, I, P, P],
+    "pxh_rescale_clip_from_groups": [P, Z, F, F, P, P, P, Z, P],
     "pxh_yolo_detections": [P, I, P, I, P, I, I, I, I, I, I, I, I, F, P, I, P, P],
     "pxh_yolo_detections_append": [P, I, P, I, P, I, I, I, I, I, I, I, I, F, U, P, I, P, P],
     "pxh_nms": [P, P, I, I, I, F, P, P, P, Z, P],
@@ -78,6 +82,7 @@ _OTHER_RETURNS = {
     "pxh_bn_workspace_bytes": (Z, [I, I, I]),
     "pxh_bn_folded_bytes": (Z, [I]),
     "pxh_rescale_workspace_bytes": (Z, []),
+    "pxh_norm_groups_bytes": (Z, [Z]),
     "pxh_rescale_multi_workspace_bytes": (Z, []),
     "pxh_yolo_workspace_bytes": (Z, [I, I, I, I, I, I]),
     "pxh_nms_workspace_bytes": (Z, [I]),

@@ -269,6 +269,51 @@ __device__ __forceinline__ float wave_sum(float v)
     return v;
 }
 
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// The value of another lane of the same row of 16 (a data-parallel-primitive operand: no trip through
+// the LDS crossbar, unlike __shfl).  CTRL: 0xB1 = lane ^ 1, 0x4E = lane ^ 2, 0x141 = 7 - lane within each
+// half row, 0x140 = 15 - lane within the row.  All lanes of the wave must be active.
+template<int CTRL>
+__device__ __forceinline__ float lane_in_row(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+__device__ __forceinline__ float from_lane(float v, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// Sum over the 64 lanes in one fixed tree -- pairs, quads, eights, rows of 16, then
+// (row0 + row1) + (row2 + row3) -- with the same total in every lane.  Four full-rate
+// instructions and four lane reads: the form for a sum that is taken once per vector loaded.
+// All lanes of the wave must be active.
+__device__ __forceinline__ float wave_sum_by_rows(float v)
+{
+    v += lane_in_row<0xB1>(v);
+    v += lane_in_row<0x4E>(v);
+    v += lane_in_row<0x141>(v);
+    v += lane_in_row<0x140>(v);
+    const float r0 = from_lane(v, 0), r1 = from_lane(v, 16), r2 = from_lane(v, 32), r3 = from_lane(v, 48);
+    return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ float wave_max_by_rows(float v)
+{
+    v = fmaxf(v, lane_in_row<0xB1>(v));
+    v = fmaxf(v, lane_in_row<0x4E>(v));
+    v = fmaxf(v, lane_in_row<0x141>(v));
+    v = fmaxf(v, lane_in_row<0x140>(v));
+    const float r0 = from_lane(v, 0), r1 = from_lane(v, 16), r2 = from_lane(v, 32), r3 = from_lane(v, 48);
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
 // Sum over a kBlock-thread workgroup through LDS; result valid in thread 0.
 // `slots` is LDS of at least kBlock / kWave doubles per concurrently reduced value.
 __device__ __forceinline__ double block_sum(double v, double* slots)

@@ -105,7 +105,9 @@ struct AxpyOp {
         r.x = ld<V, NT>(x, e);
         r.y = ld<V, NT>(y, e);
     }
-    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const { finish_value<V, NT>(e, r); }
+    // ... and returns what it left in y
+    template<int V, bool NT> __device__ Pack<V> finish_value(size_t e, const Regs<V>& r) const
     {
         Pack<V> o;
 #pragma unroll
@@ -114,6 +116,7 @@ struct AxpyOp {
             o.v[k] = r.y.v[k] + p;
         }
         st<V, NT>(y, e, o);
+        return o;
     }
 };
 
@@ -224,7 +227,9 @@ struct ShortcutBackwardOp {
             if (grad) r.g = ld<V, NT>(grad, e);
         }
     }
-    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const { finish_value<V, NT>(e, r); }
+    // ... and returns what it left in grad (which must be there)
+    template<int V, bool NT> __device__ Pack<V> finish_value(size_t e, const Regs<V>& r) const
     {
         Pack<V> d = r.d, f, g;
 #pragma unroll
@@ -244,6 +249,7 @@ struct ShortcutBackwardOp {
         if constexpr (ACT != PXH_LINEAR) st<V, NT>(delta, e, d);
         st<V, NT>(from_delta, e, f);
         if (grad) st<V, NT>(grad, e, g);
+        return g;
     }
 };
 
@@ -311,58 +317,138 @@ constexpr int kNormLoads = 8;         // 128-bit loads in flight per lane
 
 // Per workgroup: the sum of squares and the largest magnitude (NaN-free; a NaN shows in the sum).
 // (workgroup `block` of `blocks` that share the tensor; the result goes to *out)
+//
+// The 128-bit walk adds in an order that a flat kernel with one vector per lane can reproduce, so
+// that a kernel which writes the tensor can leave these sums behind and spare the tensor a read:
+//   group g    = the 256 values [256 g, 256 g + 256), one vector per lane of a wave; its sum is
+//                q_g = wave_sum_by_rows over the lanes of ((x0^2 + x1^2) + x2^2) + x3^2
+//                in fp32, values past the end counting as zero;
+//   chain      = for workgroup b of B, vector u of kNormLoads, wave w:  T = sum over the steps i, in
+//                order, of (double) q_g with g = ((i B + b) kNormLoads + u) 4 + w;
+//   partial[b] = butterfly (offsets 16 .. 1) in fp64 over the workgroup's 32 chains, chain u*4 + w
+//                in lane u*4 + w.
+// norm_chains_kernel forms the same partials from stored group sums.
+constexpr int kChains = kNormLoads * (kBlock / kWave);     // per workgroup
+static_assert(kChains == 32, "the chains of a workgroup fill half a wave");
+
+// The 32 chains of a workgroup, one per lane of the first half-wave (other lanes: anything), to the
+// workgroup's partial; valid in lane 0.
+__device__ __forceinline__ double chains_to_partial(double chain)
+{
+#pragma unroll
+    for (int off = kChains / 2; off > 0; off >>= 1) chain += __shfl_xor(chain, off, kWave);
+    return chain;
+}
+
 template<int V, bool NT>
 __device__ __forceinline__ void sumsq_walk(const float* x, size_t n_vec, uint32_t block, uint32_t blocks, double2* out)
 {
-    __shared__ double slots[kBlock / kWave];
-    __shared__ float peaks[kBlock / kWave];
     const size_t per_step = static_cast<size_t>(kBlock) * V * kNormLoads;
-    double s = 0.0;
-    float peak = 0.0f;
-    for (size_t base = static_cast<size_t>(block) * per_step; base < n_vec;
-         base += static_cast<size_t>(blocks) * per_step) {
-        Pack<V> v[kNormLoads];
-        float a = 0.0f;
-        // a whole step has no branch between its loads (behind one each load is waited for before the
-        // next goes out); only the last step of the tensor tests every vector
-        if (base + per_step <= n_vec) {
+    if constexpr (V == 4) {
+        __shared__ double chains[kChains];
+        __shared__ float peaks[kBlock / kWave];
+        double chain[kNormLoads];
 #pragma unroll
-            for (int u = 0; u < kNormLoads; ++u)
-                v[u] = ld<V, NT>(x, base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V);
+        for (int u = 0; u < kNormLoads; ++u) chain[u] = 0.0;
+        float peak = 0.0f;
+        for (size_t base = static_cast<size_t>(block) * per_step; base < n_vec;
+             base += static_cast<size_t>(blocks) * per_step) {
+            Pack<V> v[kNormLoads];
+            // a whole step has no branch between its loads (behind one each load is waited for before
+            // the next goes out); only the last step of the tensor tests every vector
+            if (base + per_step <= n_vec) {
 #pragma unroll
-            for (int u = 0; u < kNormLoads; ++u) {
+                for (int u = 0; u < kNormLoads; ++u)
+                    v[u] = ld<V, NT>(x, base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V);
+            } else {
 #pragma unroll
-                for (int k = 0; k < V; ++k) {
-                    a += v[u].v[k] * v[u].v[k];
-                    peak = fmaxf(peak, fabsf(v[u].v[k]));
+                for (int u = 0; u < kNormLoads; ++u) {
+                    const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
+#pragma unroll
+                    for (int k = 0; k < V; ++k) v[u].v[k] = 0.0f;
+                    if (e < n_vec) v[u] = ld<V, NT>(x, e);
                 }
             }
-        } else {
+#pragma unroll
+            for (int u = 0; u < kNormLoads; ++u) {
+                peak = fmaxf(peak, peak_of(v[u]));
+                chain[u] += static_cast<double>(wave_sum_by_rows(square_sum(v[u])));
+            }
+        }
+        peak = wave_max(peak);
+        const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+        if (lane == 0) {
+            peaks[wave] = peak;
+#pragma unroll
+            for (int u = 0; u < kNormLoads; ++u) chains[u * (kBlock / kWave) + wave] = chain[u];
+        }
+        __syncthreads();
+        if (wave == 0) {
+            const double total = chains_to_partial(chains[lane & (kChains - 1)]);
+            if (lane == 0) {
+                float top = peaks[0];
+#pragma unroll
+                for (int w = 1; w < kBlock / kWave; ++w) top = fmaxf(top, peaks[w]);
+                *out = make_double2(total, static_cast<double>(top));
+            }
+        }
+    } else {
+        // one value per lane (a tensor that is not 16-byte aligned or not a multiple of 4 long):
+        // fp32 over a step, fp64 over the steps and the workgroup
+        __shared__ double slots[kBlock / kWave];
+        __shared__ float peaks[kBlock / kWave];
+        double s = 0.0;
+        float peak = 0.0f;
+        for (size_t base = static_cast<size_t>(block) * per_step; base < n_vec;
+             base += static_cast<size_t>(blocks) * per_step) {
+            float a = 0.0f;
 #pragma unroll
             for (int u = 0; u < kNormLoads; ++u) {
                 const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
                 if (e < n_vec) {
-                    v[u] = ld<V, NT>(x, e);
+                    const Pack<V> v = ld<V, NT>(x, e);
 #pragma unroll
                     for (int k = 0; k < V; ++k) {
-                        a += v[u].v[k] * v[u].v[k];
-                        peak = fmaxf(peak, fabsf(v[u].v[k]));
+                        a += v.v[k] * v.v[k];
+                        peak = fmaxf(peak, fabsf(v.v[k]));
                     }
                 }
             }
+            s += static_cast<double>(a);
         }
-        s += static_cast<double>(a);
-    }
+        peak = wave_max(peak);
+        if ((threadIdx.x & (kWave - 1)) == 0) peaks[threadIdx.x / kWave] = peak;
+        const double total = block_sum(s, slots);       // synchronises the workgroup twice
+        if (threadIdx.x == 0) {
+            float top = peaks[0];
 #pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) peak = fmaxf(peak, __shfl_xor(peak, off, kWave));
-    if ((threadIdx.x & (kWave - 1)) == 0) peaks[threadIdx.x / kWave] = peak;
-    const double total = block_sum(s, slots);       // synchronises the workgroup twice
-    if (threadIdx.x == 0) {
-        float top = peaks[0];
-#pragma unroll
-        for (int w = 1; w < kBlock / kWave; ++w) top = fmaxf(top, peaks[w]);
-        *out = make_double2(total, static_cast<double>(top));
+            for (int w = 1; w < kBlock / kWave; ++w) top = fmaxf(top, peaks[w]);
+            *out = make_double2(total, static_cast<double>(top));
+        }
     }
+}
+
+// Group sums that a kernel left while writing the tensor (float2: sum of squares, largest
+// magnitude), to the partials of the walk above: one lane per chain.
+__global__ __launch_bounds__(kBlock) void norm_chains_kernel(const float2* groups, size_t n_groups, uint32_t blocks,
+                                                            double2* partial)
+{
+    const uint32_t chain = blockIdx.x * kBlock + threadIdx.x;      // = b * kChains + u * 4 + w
+    const size_t per_step = static_cast<size_t>(blocks) * kChains;
+    double total = 0.0;
+    float peak = 0.0f;
+    if (chain < per_step) {
+        for (size_t g = chain; g < n_groups; g += per_step) {
+            const float2 q = groups[g];
+            total += static_cast<double>(q.x);
+            peak = fmaxf(peak, q.y);
+        }
+    }
+    total = chains_to_partial(total);
+#pragma unroll
+    for (int off = kChains / 2; off > 0; off >>= 1) peak = fmaxf(peak, __shfl_xor(peak, off, kWave));
+    if ((threadIdx.x & (kChains - 1)) == 0 && chain < per_step)
+        partial[chain / kChains] = make_double2(total, static_cast<double>(peak));
 }
 
 template<int V, bool NT>
@@ -856,6 +942,24 @@ struct AdamStepOp {
 
 using namespace pxh;
 
+namespace pxh {
+namespace {
+// The tensor as it is: what a kernel of this file that cannot leave group sums itself is followed by.
+struct GroupsOnlyOp {
+    const float* x;
+    template<int V> struct Regs { Pack<V> x; };
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const { r.x = ld<V, NT>(x, e); }
+    template<int V, bool NT> __device__ void finish(size_t, const Regs<V>&) const {}
+    template<int V, bool NT> __device__ Pack<V> finish_value(size_t, const Regs<V>& r) const { return r.x; }
+};
+
+// The norm pass reads a tensor 128 bits at a time under this condition, and only then do group sums
+// describe it; otherwise nothing is written to, or read from, a group buffer.
+inline bool has_groups(const float* x, size_t n) { return aligned16(x) && n % 4 == 0; }
+
+}  // namespace
+}  // namespace pxh
+
 extern "C" {
 
 int pxh_activate(int activation, float* x, size_t n, void* stream)
@@ -1038,15 +1142,74 @@ int pxh_sgd_update(size_t n, float* w, float* d, int batch, float lr, float mome
     return launch_stream("pxh_sgd_update", n, aligned16(w) && aligned16(d), 16, op, as_stream(stream));
 }
 
+// ---------------------------------------------------------------- norm + peak from the writing kernel
+size_t pxh_norm_groups_bytes(size_t n)
+{
+    return (n + kGroupValues - 1) / kGroupValues * sizeof(float2);
+}
+
+int pxh_norm_groups(const float* x, size_t n, void* groups, void* stream)
+{
+    if ((!x || !groups) && n) return fail_invalid("pxh_norm_groups: null pointer");
+    if (!has_groups(x, n)) return PXH_OK;
+    return launch_stream_groups("pxh_norm_groups", n, 4, GroupsOnlyOp{ x }, static_cast<float2*>(groups),
+                                as_stream(stream));
+}
+
+int pxh_axpy_norm(size_t n, float alpha, const float* x, float* y, void* y_groups, void* stream)
+{
+    if ((!x || !y || !y_groups) && n) return fail_invalid("pxh_axpy_norm: null pointer");
+    if (has_groups(y, n) && aligned16(x))
+        return launch_stream_groups("pxh_axpy_norm", n, 12, AxpyOp{ x, y, alpha }, static_cast<float2*>(y_groups),
+                                    as_stream(stream));
+    const int rc = pxh_axpy(n, alpha, x, y, stream);
+    return rc ? rc : pxh_norm_groups(y, n, y_groups, stream);
+}
+
+int pxh_shortcut_backward_norm(float* delta, const float* pre_activation, float* from_delta, float* grad, size_t n,
+                               float alpha, float beta, int activation, int first, void* grad_groups, void* stream)
+{
+    if ((!grad || !grad_groups) && n) return fail_invalid("pxh_shortcut_backward_norm: grad and its group buffer are required");
+    const bool flat = has_groups(grad, n) && aligned16(delta) && aligned16(pre_activation) && aligned16(from_delta);
+    if (!flat) {
+        const int rc = first ? pxh_shortcut_backward_first(delta, pre_activation, from_delta, grad, n, alpha, beta,
+                                                           activation, stream)
+                             : pxh_shortcut_backward(delta, pre_activation, from_delta, grad, n, alpha, beta,
+                                                     activation, stream);
+        return rc ? rc : pxh_norm_groups(grad, n, grad_groups, stream);
+    }
+    if ((!delta || !from_delta) && n) return fail_invalid("pxh_shortcut_backward_norm: null pointer");
+    if (activation != PXH_LINEAR && !pre_activation && n)
+        return fail_invalid("pxh_shortcut_backward_norm: pre_activation is required for a non-linear activation");
+    if (first && from_delta == grad && n)
+        return fail_invalid("pxh_shortcut_backward_norm: from_delta and grad must be distinct when both are overwritten");
+    int rc = PXH_OK;
+    float2* groups = static_cast<float2*>(grad_groups);
+    const bool known = dispatch_activation(activation, [&]<int ACT>() {
+        if (first)
+            rc = launch_stream_groups("pxh_shortcut_backward_norm", n, 12,
+                                      ShortcutBackwardOp<ACT, true>{ delta, pre_activation, from_delta, grad, alpha, beta },
+                                      groups, as_stream(stream));
+        else
+            rc = launch_stream_groups("pxh_shortcut_backward_norm", n, 20,
+                                      ShortcutBackwardOp<ACT>{ delta, pre_activation, from_delta, grad, alpha, beta },
+                                      groups, as_stream(stream));
+    });
+    if (!known) return fail_invalid("pxh_shortcut_backward_norm: unknown activation %d", activation);
+    return rc;
+}
+
 size_t pxh_rescale_workspace_bytes(void)
 {
     return kNormBlocks * sizeof(double2);      // partial sums and peaks
 }
 
-int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* norm_out, void* workspace,
-                     size_t workspace_bytes, void* stream)
+namespace {
+// `groups`: the group sums a kernel left when it wrote x, or null to read x for them.
+int rescale_clip(const char* who, float* x, size_t n, float threshold, float clip, float* norm_out,
+                 const float2* groups, void* workspace, size_t workspace_bytes, void* stream)
 {
-    if (!x && n) return fail_invalid("pxh_rescale_clip: null pointer");
+    if (!x && n) return fail_invalid("%s: null pointer", who);
     if (n == 0) return PXH_OK;
     const bool rescale = threshold > 0.0f || norm_out != nullptr;
     if (!rescale && !(clip > 0.0f)) return PXH_OK;
@@ -1055,7 +1218,7 @@ int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* nor
     if (rc) return rc;
     double2* partial = static_cast<double2*>(ws);
     hipStream_t s = as_stream(stream);
-    const bool vec = aligned16(x) && n % 4 == 0;
+    const bool vec = has_groups(x, n);
     const int v = vec ? 4 : 1;
     // a tensor past the last-level cache gains nothing from being kept for the next pass
     const bool nt = vec && n * 4 >= kStreamingBytes;
@@ -1063,10 +1226,15 @@ int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* nor
     const size_t per_step = static_cast<size_t>(kBlock) * v * kNormLoads;
     const size_t want = (n + per_step - 1) / per_step;
     const int blocks = static_cast<int>(want < static_cast<size_t>(kNormBlocks) ? want : kNormBlocks);
-    if (nt) hipLaunchKernelGGL((sumsq_partial_kernel<4, true>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
+    if (vec && groups) {
+        const size_t n_groups = (n + kGroupValues - 1) / kGroupValues;
+        hipLaunchKernelGGL(norm_chains_kernel, dim3(grid_for(static_cast<size_t>(blocks) * kChains, kBlock)),
+                           dim3(kBlock), 0, s, groups, n_groups, static_cast<uint32_t>(blocks), partial);
+    }
+    else if (nt) hipLaunchKernelGGL((sumsq_partial_kernel<4, true>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
     else if (vec) hipLaunchKernelGGL((sumsq_partial_kernel<4, false>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
     else hipLaunchKernelGGL((sumsq_partial_kernel<1, false>), dim3(blocks), dim3(kBlock), 0, s, x, n, partial);
-    rc = check_launch("pxh_rescale_clip");
+    rc = check_launch(who);
     if (rc) return rc;
     // only the norm asked for: one workgroup adds up the partials and writes it
     const dim3 grid(threshold > 0.0f || clip > 0.0f ? static_cast<unsigned>(blocks) : 1u);
@@ -1076,7 +1244,22 @@ int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* nor
                                      threshold, clip, norm_out);
     else hipLaunchKernelGGL((rescale_clip_kernel<1, false>), grid, dim3(kBlock), 0, s, x, n, partial, blocks,
                             threshold, clip, norm_out);
-    return check_launch("pxh_rescale_clip");
+    return check_launch(who);
+}
+}  // namespace
+
+int pxh_rescale_clip(float* x, size_t n, float threshold, float clip, float* norm_out, void* workspace,
+                     size_t workspace_bytes, void* stream)
+{
+    return rescale_clip("pxh_rescale_clip", x, n, threshold, clip, norm_out, nullptr, workspace, workspace_bytes, stream);
+}
+
+int pxh_rescale_clip_from_groups(float* x, size_t n, float threshold, float clip, float* norm_out, const void* groups,
+                                 void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!groups && n) return fail_invalid("pxh_rescale_clip_from_groups: null group buffer");
+    return rescale_clip("pxh_rescale_clip_from_groups", x, n, threshold, clip, norm_out,
+                        static_cast<const float2*>(groups), workspace, workspace_bytes, stream);
 }
 
 size_t pxh_rescale_multi_workspace_bytes(void)

@@ -120,6 +120,59 @@ __global__ __launch_bounds__(kWave) void stream_tail_kernel(size_t begin, size_t
     }
 }
 
+// ---------------------------------------------------------------- group sums of a written tensor
+// Layer::backward opens with the L2 norm and the largest magnitude of the layer's delta
+// (include/Layer.h:385-397, 479-499).  A flat kernel that is the last to write that delta can leave
+// them behind per group of 256 values -- one wave's vectors -- and spare the tensor a read: the sum
+// of squares of a group is wave_sum_by_rows over the lanes of ((x0^2 + x1^2) + x2^2) + x3^2, the order
+// in which the norm pass itself adds, so the norm comes out the same to the bit either way.
+__device__ __forceinline__ float square_sum(const Pack<4>& v)
+{
+    return ((v.v[0] * v.v[0] + v.v[1] * v.v[1]) + v.v[2] * v.v[2]) + v.v[3] * v.v[3];
+}
+
+__device__ __forceinline__ float peak_of(const Pack<4>& v)      // NaN-free unless all four are NaN
+{
+    return fmaxf(fmaxf(fabsf(v.v[0]), fabsf(v.v[1])), fmaxf(fabsf(v.v[2]), fabsf(v.v[3])));
+}
+
+constexpr int kGroupValues = kWave * 4;
+
+// The op also supplies
+//     template<int V, bool NT> __device__ Pack<V> finish_value(size_t e, const Regs<V>&) const;
+// which does what finish does and returns the values it left in the tensor the groups describe.
+// groups[g] = (sum of squares, largest magnitude) of values [256 g, 256 g + 256); n_vec % 4 == 0.
+template<bool NT, typename Op>
+__global__ __launch_bounds__(kBlock) void stream_groups_kernel(size_t n_vec, Op op, float2* groups)
+{
+    const size_t e = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
+    float a = 0.0f, peak = 0.0f;
+    if (e < n_vec) {
+        typename Op::template Regs<4> r;
+        op.template load<4, NT>(e, r);
+        const Pack<4> v = op.template finish_value<4, NT>(e, r);
+        a = square_sum(v);
+        peak = peak_of(v);
+    }
+    a = wave_sum_by_rows(a);
+    peak = wave_max_by_rows(peak);
+    const size_t first = (static_cast<size_t>(blockIdx.x) * kBlock + (threadIdx.x & ~(kWave - 1))) * 4;
+    if ((threadIdx.x & (kWave - 1)) == 0 && first < n_vec) groups[first / kGroupValues] = make_float2(a, peak);
+}
+
+// Launches op over n elements (n % 4 == 0, every pointer 16-byte aligned) and leaves the group sums.
+template<typename Op>
+int launch_stream_groups(const char* name, size_t n, int bytes_per_elem, const Op& op, float2* groups,
+                         hipStream_t stream)
+{
+    if (n == 0) return PXH_OK;
+    const bool nt = n * static_cast<size_t>(bytes_per_elem) >= kStreamingBytes;
+    const dim3 grid(grid_for(n, static_cast<size_t>(kBlock) * 4));
+    if (nt) hipLaunchKernelGGL((stream_groups_kernel<true, Op>), grid, dim3(kBlock), 0, stream, n, op, groups);
+    else hipLaunchKernelGGL((stream_groups_kernel<false, Op>), grid, dim3(kBlock), 0, stream, n, op, groups);
+    return check_launch(name);
+}
+
 // Launches op over n elements.  `vector_ok`: every pointer the op touches is 16-byte aligned.
 // `bytes_per_elem`: bytes the op moves per element, which picks the non-temporal variant from
 // `streaming_from` bytes per launch on.

@@ -18,6 +18,7 @@
 #include <memory>
 #include <string>
 #include <variant>
+#include <unordered_map>
 #include <vector>
 
 #include "DeviceVector.h"
@@ -146,6 +147,22 @@ public:
     void* workspace() noexcept { return workspace_.empty() ? nullptr : workspace_.data(); }
     std::size_t workspaceBytes() const noexcept { return workspace_.size() * sizeof(float); }
 
+    // Norm + peak from the kernel that wrote a delta (pxh_shortcut_backward_norm, pxh_axpy_norm): the
+    // writer notes where it left the tensor's group sums, and the rescaleAndClip() that opens the
+    // backward of the tensor's layer takes the note and starts from them instead of reading the
+    // tensor.  A note is good for one use, and only if nothing writes the tensor in between: the
+    // layers that leave one do so on request ("leaves_norm"), and whoever asks vouches for that.
+    void noteNormGroups(const float* tensor, const float* groups) { normGroups_[tensor] = groups; }
+
+    const float* takeNormGroups(const float* tensor)
+    {
+        const auto it = normGroups_.find(tensor);
+        if (it == normGroups_.end()) return nullptr;
+        const float* groups = it->second;
+        normGroups_.erase(it);
+        return groups;
+    }
+
     const FloatVector& truths() const noexcept { return truths_; }
     const IntVector& truthCounts() const noexcept { return truthCounts_; }
     int maxTruth() const noexcept { return maxTruth_; }
@@ -156,6 +173,7 @@ private:
     int maxTruth_ = 0;
     FloatVector workspace_;
     std::vector<FloatVector> retiredWorkspaces_;
+    std::unordered_map<const float*, const float*> normGroups_;
 };
 
 // ---------------------------------------------------------------- layer
@@ -265,14 +283,27 @@ protected:
 
     // scaleTensor then constrain on one tensor, when the layer's flags ask for them; one fused call
     // that reads the tensor once and rewrites it only if some value has to change.
+    // Where the kernel that wrote the tensor left its norm and peak behind (Context::noteNormGroups),
+    // the tensor is not read at all unless it has to change; the result is the same to the bit.
     void rescaleAndClip(V& tensor)
     {
-        if (tensor.empty() || !(gradientRescaling_ || gradientClipping_)) return;
+        if (tensor.empty()) return;
+        const float* groups = context_.takeNormGroups(tensor.data());
+        if (!(gradientRescaling_ || gradientClipping_)) return;
         context_.reserveWorkspace(pxh_rescale_workspace_bytes());
-        PX_HIP_CHECK(pxh_rescale_clip(tensor.data(), tensor.size(), gradientRescaling_ ? gradientThreshold_ : 0.0f,
-                                      gradientClipping_ ? gradientClipValue_ : 0.0f, nullptr, context_.workspace(),
-                                      context_.workspaceBytes(), stream()));
+        const float threshold = gradientRescaling_ ? gradientThreshold_ : 0.0f;
+        const float clip = gradientClipping_ ? gradientClipValue_ : 0.0f;
+        if (groups)
+            PX_HIP_CHECK(pxh_rescale_clip_from_groups(tensor.data(), tensor.size(), threshold, clip, nullptr, groups,
+                                                      context_.workspace(), context_.workspaceBytes(), stream()));
+        else
+            PX_HIP_CHECK(pxh_rescale_clip(tensor.data(), tensor.size(), threshold, clip, nullptr, context_.workspace(),
+                                          context_.workspaceBytes(), stream()));
     }
+
+    // For a layer that leaves the norm of the delta in front of it behind ("leaves_norm"): the buffer
+    // of group sums for a tensor of n values, allocated when the layer is built.
+    static V normGroupsFor(std::size_t n) { return V((pxh_norm_groups_bytes(n) + sizeof(float) - 1) / sizeof(float)); }
 
     void checkInput(const V& input, const char* who) const
     {

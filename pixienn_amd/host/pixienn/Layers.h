@@ -560,6 +560,12 @@ public:
         // layer in front by whoever builds the network (setFirstConsumerOverwrites).
         firstWriter_ = training() && sameShape_ && props.get<bool>("first_writer", false);
         if (firstWriter_) from_->setFirstConsumerOverwrites(true);
+        // "leaves_norm": this shortcut is the LAST to write the delta of the layer in front of it before
+        // that layer's backward (true when nothing else reads that layer's output, as in a residual
+        // block).  Its backward then leaves the norm and peak of that delta behind, and the gradient
+        // rescale + clip that opens that layer's backward does not read the tensor for them.
+        leavesNorm_ = training() && sameShape_ && props.get<bool>("leaves_norm", false);
+        if (leavesNorm_) normGroups_ = normGroupsFor(output_.size());
     }
 
     void forward(const V& input) override
@@ -585,6 +591,13 @@ public:
     {
         Layer::backward(input, grad);
         const float* pre = preActivation_.empty() ? nullptr : preActivation_.data();
+        if (leavesNorm_ && grad) {
+            PX_HIP_CHECK(pxh_shortcut_backward_norm(delta_.data(), pre, from_->delta().data(), grad->data(),
+                                                    delta_.size(), alpha_, beta_, activation_, firstWriter_ ? 1 : 0,
+                                                    normGroups_.data(), stream()));
+            context().noteNormGroups(grad->data(), normGroups_.data());
+            return;
+        }
         if (firstWriter_) {
             PX_CHECK(grad != nullptr, "a first-writer shortcut needs the delta of the layer in front of it");
             PX_HIP_CHECK(pxh_shortcut_backward_first(delta_.data(), pre, from_->delta().data(), grad->data(),
@@ -609,8 +622,8 @@ private:
     Layer::Ptr from_;
     int activation_ = PXH_LINEAR;
     float alpha_ = 1.0f, beta_ = 1.0f;
-    bool sameShape_ = true, firstWriter_ = false;
-    V preActivation_;
+    bool sameShape_ = true, firstWriter_ = false, leavesNorm_ = false;
+    V preActivation_, normGroups_;
 };
 
 // ---------------------------------------------------------------- route
@@ -798,6 +811,10 @@ public:
             costDevice_ = V(1, 0.0f);
             context.reserveWorkspace(pxh_yolo_workspace_bytes(batch(), static_cast<int>(mask_.size()), context.classes,
                                                               width(), height(), 0));
+            // "leaves_norm": nothing but this head reads the layer in front of it (true of every head of
+            // the shipped networks), so `grad += delta` below is the last write of that layer's delta
+            // and leaves its norm and peak behind for the rescale + clip that opens its backward.
+            if (props.get<bool>("leaves_norm", false)) normGroups_ = normGroupsFor(output_.size());
         }
     }
 
@@ -828,6 +845,11 @@ public:
     {
         Layer::backward(input, grad);
         if (grad == nullptr) return;
+        if (!normGroups_.empty()) {
+            PX_HIP_CHECK(pxh_axpy_norm(delta_.size(), 1.0f, delta_.data(), grad->data(), normGroups_.data(), stream()));
+            context().noteNormGroups(grad->data(), normGroups_.data());
+            return;
+        }
         PX_HIP_CHECK(pxh_axpy(delta_.size(), 1.0f, delta_.data(), grad->data(), stream()));
     }
 
@@ -914,6 +936,7 @@ private:
     float ignoreThresh_, truthThresh_, coordScale_, objectScale_, noObjectScale_, classScale_;
     V stats_, costDevice_;
     bool costReady_ = false;
+    V normGroups_;
     IntVector detectRecords_, detectCount_;
     int detectCapacity_ = 0;
 };

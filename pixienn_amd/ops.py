@@ -439,6 +439,40 @@ def rescale_clip(x, threshold=0.0, clip=0.0, norm_out=None):
     call("pxh_rescale_clip", ptr(x), x.numel(), float(threshold), float(clip), ptr(norm_out), None, 0, _stream())
 
 
+def norm_groups_like(x):
+    """A group-sum buffer for a tensor of x's size (8 bytes per 256 values), on x's device."""
+    import torch
+    n = capi.load().pxh_norm_groups_bytes(x.numel()) // 4
+    return torch.empty(max(n, 2), dtype=torch.float32, device=x.device)
+
+
+def norm_groups(x, groups):
+    """The group sums of x as it is."""
+    _chk_all(x, groups)
+    call("pxh_norm_groups", ptr(x), x.numel(), ptr(groups), _stream())
+
+
+def axpy_norm(alpha, x, y, y_groups):
+    """axpy that also leaves the group sums of y."""
+    _chk_all(x, y, y_groups)
+    call("pxh_axpy_norm", x.numel(), float(alpha), ptr(x), ptr(y), ptr(y_groups), _stream())
+
+
+def shortcut_backward_norm(delta, from_delta, grad, grad_groups, activation="linear", alpha=1.0, beta=1.0,
+                           pre_activation=None, first=False):
+    """shortcut_backward / shortcut_backward_first that also leaves the group sums of grad."""
+    _chk_all(delta, from_delta, grad, pre_activation, grad_groups)
+    call("pxh_shortcut_backward_norm", ptr(delta), ptr(pre_activation), ptr(from_delta), ptr(grad), delta.numel(),
+         float(alpha), float(beta), act_id(activation), int(bool(first)), ptr(grad_groups), _stream())
+
+
+def rescale_clip_from_groups(x, groups, threshold=0.0, clip=0.0, norm_out=None):
+    """rescale_clip that starts from the group sums the writer of x left instead of reading x for them."""
+    _chk_all(x, groups, norm_out)
+    call("pxh_rescale_clip_from_groups", ptr(x), x.numel(), float(threshold), float(clip), ptr(norm_out), ptr(groups),
+         None, 0, _stream())
+
+
 DETECTION_DTYPE = workloads.DETECTION_DTYPE
 
 

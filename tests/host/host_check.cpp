@@ -163,7 +163,7 @@ struct Net {
         return { conv0.get(), pool1.get(), conv2.get(), short3.get(), up4.get(), route5.get(), conv6.get(), yolo7.get() };
     }
 
-    explicit Net(bool training)
+    explicit Net(bool training, bool leavesNorm = false)
     {
         ctx.training = training;
         ctx.width = ctx.height = 128;
@@ -182,7 +182,8 @@ struct Net {
                                                              { "activation", std::string("mish") } });
         short3 = std::make_shared<ShortcutLayer>(ctx, Properties{ { "batch", N }, { "channels", C },
                                                                   { "height", S / 2 }, { "width", S / 2 },
-                                                                  { "alpha", 1.0f }, { "beta", 0.5f } }, pool1);
+                                                                  { "alpha", 1.0f }, { "beta", 0.5f },
+                                                                  { "leaves_norm", leavesNorm } }, pool1);
         up4 = std::make_shared<UpsampleLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S / 2 },
                                                                { "width", S / 2 }, { "stride", 2 } });
         route5 = std::make_shared<RouteLayer>(ctx, Properties{ { "batch", N }, { "channels", 2 * C },
@@ -194,7 +195,8 @@ struct Net {
         yolo7 = std::make_shared<YoloLayer>(ctx, Properties{ { "batch", N }, { "channels", 2 * C }, { "height", S },
                                                              { "width", S }, { "num", 3 }, { "mask", mask },
                                                              { "anchors", anchors }, { "ignore_thresh", 0.5f },
-                                                             { "object_scale", 2.0f }, { "noobject_scale", 0.5f } });
+                                                             { "object_scale", 2.0f }, { "noobject_scale", 0.5f },
+                                                             { "leaves_norm", leavesNorm } });
         scale0 = uniforms(11, C, 0.5f, 1.5f); bias0 = normals(12, C, 0.1f);
         scale2 = uniforms(13, C, 0.5f, 1.5f); bias2 = normals(14, C, 0.1f);
         bias6 = normals(15, 2 * C, 0.1f);
@@ -899,6 +901,122 @@ void firstWriterShortcutChecks()
     }
 }
 
+// A residual block whose shortcut leaves the norm and peak of the delta it writes last: the rescale +
+// clip that opens the backward of the layer in front starts from them instead of reading the tensor,
+// and every gradient behind it is the same to the bit -- below the threshold, above it, and clamped.
+void leavesNormShortcutChecks()
+{
+    struct Block {
+        Context ctx;
+        std::shared_ptr<ConvLayer> a, b, c;
+        std::shared_ptr<ShortcutLayer> add;
+        Block(bool leavesNorm, bool firstWriter, float threshold, float clip)
+        {
+            ctx.training = true;
+            const Properties conv{ { "batch", N }, { "channels", C }, { "height", S }, { "width", S }, { "filters", C },
+                                   { "batch_normalize", true }, { "activation", std::string("leaky") } };
+            a = std::make_shared<ConvLayer>(ctx, conv);
+            b = std::make_shared<ConvLayer>(ctx, conv);
+            c = std::make_shared<ConvLayer>(ctx, conv);
+            add = std::make_shared<ShortcutLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S },
+                                                                   { "width", S }, { "first_writer", firstWriter },
+                                                                   { "leaves_norm", leavesNorm } }, a);
+            if (firstWriter) c->setFirstConsumerOverwrites(true);
+            for (auto* l: { a.get(), b.get(), c.get() }) {
+                l->setGradientRescaling(threshold > 0.0f, threshold);
+                l->setGradientClipping(clip > 0.0f, clip);
+            }
+        }
+        void step(const FloatVector& input, const Host& outDelta)
+        {
+            a->forward(input);
+            b->forward(a->output());
+            c->forward(b->output());
+            add->forward(c->output());
+            add->delta().copyHost(outDelta);
+            add->backward(c->output(), &c->delta());
+            c->backward(b->output(), &b->delta());
+            b->backward(a->output(), &a->delta());
+            a->backward(input, nullptr);
+        }
+    };
+    const FloatVector input(normals(711, size_t(N) * C * S * S));
+    const Host outDelta = normals(712, size_t(N) * C * S * S);
+    double norm = 0.0;
+    for (float v: outDelta) norm += double(v) * v;
+    norm = std::sqrt(norm);
+    struct Case { const char* name; float threshold, clip; };
+    const Case cases[] = { { "below the threshold", float(4.0 * norm), 0.0f }, { "rescaled", float(0.5 * norm), 0.0f },
+                           { "rescaled and clamped", float(0.5 * norm), 0.25f }, { "helpers off", 0.0f, 0.0f } };
+    for (const bool firstWriter: { false, true }) {
+        for (const Case& k: cases) {
+            Block plain(false, firstWriter, k.threshold, k.clip), fused(true, firstWriter, k.threshold, k.clip);
+            for (int round = 0; round < 2; ++round) {
+                plain.step(input, outDelta);
+                fused.step(input, outDelta);
+                const std::string tag = std::string(" (") + k.name + (firstWriter ? ", first writer" : "") + ", step " +
+                                        std::to_string(round + 1) + ")";
+                report("norm from the shortcut: delta behind the layer in front" + tag,
+                       fused.b->delta().asVector() == plain.b->delta().asVector());
+                report("norm from the shortcut: scale updates of the layer in front" + tag,
+                       fused.c->scaleUpdates().asVector() == plain.c->scaleUpdates().asVector());
+                report("norm from the shortcut: delta of the from layer" + tag,
+                       fused.a->delta().asVector() == plain.a->delta().asVector());
+            }
+            report(std::string("norm from the shortcut: the note is taken (") + k.name + ")",
+                   fused.ctx.takeNormGroups(fused.c->delta().data()) == nullptr);
+        }
+    }
+}
+
+// The small network with the shortcut and the head leaving the norms of the deltas they write last
+// (conv2's and conv6's): every delta and every update buffer as without, bit for bit.
+void leavesNormNetChecks()
+{
+    Net plain(true), fused(true, true);
+    const auto truth = makeTruth();
+    FloatVector input(size_t(N) * C * S * S);
+    input.copyHost(normals(910, input.size()));
+    Net* nets[2] = { &plain, &fused };
+    for (int step = 1; step <= 2; ++step) {
+        for (Net* n: nets) {
+            n->ctx.setGroundTruth(truth);
+            for (Layer* l: n->all()) {
+                l->setGradientRescaling(true, step == 1 ? 0.05f : 1e6f);      // bites on the first step only
+                l->setGradientClipping(true, 0.01f);
+            }
+            n->conv0->forward(input);
+            n->pool1->forward(n->conv0->output());
+            n->conv2->forward(n->pool1->output());
+            n->short3->forward(n->conv2->output());
+            n->up4->forward(n->short3->output());
+            n->route5->forward(n->up4->output());
+            n->conv6->forward(n->route5->output());
+            n->yolo7->forward(n->conv6->output());
+            n->yolo7->backward(n->conv6->output(), &n->conv6->delta());
+            n->conv6->backward(n->route5->output(), &n->route5->delta());
+            n->route5->backward(n->up4->output(), &n->up4->delta());
+            n->up4->backward(n->short3->output(), &n->short3->delta());
+            n->short3->backward(n->conv2->output(), &n->conv2->delta());
+            n->conv2->backward(n->pool1->output(), &n->pool1->delta());
+            n->pool1->backward(n->conv0->output(), &n->conv0->delta());
+            n->conv0->backward(input, nullptr);
+        }
+        const bool same = fused.conv6->delta().asVector() == plain.conv6->delta().asVector() &&
+                          fused.conv6->biasUpdates().asVector() == plain.conv6->biasUpdates().asVector() &&
+                          fused.conv2->delta().asVector() == plain.conv2->delta().asVector() &&
+                          fused.conv2->scaleUpdates().asVector() == plain.conv2->scaleUpdates().asVector() &&
+                          fused.pool1->delta().asVector() == plain.pool1->delta().asVector() &&
+                          fused.conv0->delta().asVector() == plain.conv0->delta().asVector() &&
+                          fused.conv0->scaleUpdates().asVector() == plain.conv0->scaleUpdates().asVector();
+        report("norms from the shortcut and the head: every gradient as without, step " + std::to_string(step), same);
+    }
+    const Host moved = fused.conv0->scaleUpdates().asVector();
+    bool any = false;
+    for (float v: moved) any = any || v != 0.0f;
+    report("norms from the shortcut and the head: gradients reached the first layer", any);
+}
+
 // A model's weights file: header of either seen-width, every layer's section in network order, exact length.
 void weightsFileChecks()
 {
@@ -1017,6 +1135,8 @@ int main(int argc, char** argv)
             batchNormLayerChecks();
             weightsFileChecks();
             firstWriterShortcutChecks();
+            leavesNormShortcutChecks();
+            leavesNormNetChecks();
             capturedSequenceChecks();
             parameterSetChecks();
         }
