@@ -169,6 +169,29 @@ def run_epilogue_step(ops, shapes, events=None, torch=None, raw=False):
             events.append((act, a, b))
 
 
+def same_bytes_copier(torch, ops, timer):
+    """Returns copy_same_bytes(bytes, cap=None): the time of a plain copy (half the bytes read, half
+    written, through the route kernel) of the same size, over buffers rotated as the row's are: what
+    one launch of this size costs on this part whatever it computes.  Cached per size rounded to 2 %."""
+    cache = {}
+    dev = torch.device("cuda")
+
+    def copy_same_bytes(bytes_, cap=None):
+        n = max(1024, int(bytes_ // 8) // 256 * 256)
+        key = (int(round(np.log(n) / np.log(1.02))), cap)
+        if key not in cache:
+            rot = rotation_for(8 * n) if cap is None else rotation_for(8 * n, cap=cap)
+            src = [torch.empty((1, n), device=dev).normal_() for _ in range(rot)]
+            dst = [torch.empty((1, n), device=dev) for _ in range(rot)]
+            saved = timer.last_min
+            cache[key] = timer.time(lambda i: ops.route_forward(src[i], dst[i], 0), 20, rotate=rot)
+            timer.last_min = saved
+            del src, dst
+        return cache[key]
+
+    return copy_same_bytes
+
+
 def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     """One training step of YOLOv3 @608 at batch N with every non-convolution kernel launched in the
     model's own layer order on tensors of their own (21 GB): forward (per layer the delta zero-fill
@@ -346,23 +369,7 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None):
     dev = torch.device("cuda:0")
     rows = []
 
-    copy_cache = {}
-
-    def copy_same_bytes(bytes_):
-        """A plain copy (half the bytes read, half written, through the route kernel) of the same size,
-        over buffers rotated as the row's are: what one launch of this size costs on this part whatever
-        it computes.  Cached per size rounded to 2 %."""
-        n = max(1024, int(bytes_ // 8) // 256 * 256)
-        key = int(round(np.log(n) / np.log(1.02)))
-        if key not in copy_cache:
-            rot = rotation_for(8 * n)
-            src = [torch.empty((1, n), device=dev).normal_() for _ in range(rot)]
-            dst = [torch.empty((1, n), device=dev) for _ in range(rot)]
-            saved = timer.last_min
-            copy_cache[key] = timer.time(lambda i: ops.route_forward(src[i], dst[i], 0), 20, rotate=rot)
-            timer.last_min = saved
-            del src, dst
-        return copy_cache[key]
+    copy_same_bytes = same_bytes_copier(torch, ops, timer)
 
     def add(name, shape, bytes_, ms, note="", streaming=True):
         gbs = bytes_ / (ms * 1e-3) / 1e9
@@ -982,6 +989,7 @@ def main():
     # per shape, each measured alone over rotating buffers (HIP events around 20 launches)
     per_shape = []
     if not args.no_extras:
+        copy_of_size = same_bytes_copier(torch, ops, timer)
         for sh in shapes:
             rot = rotation_for(8 * sh["elems"], cap=3)
             xs = [sh["x"]] + [torch.randn_like(sh["x"]) for _ in range(rot - 1)]
@@ -990,8 +998,14 @@ def main():
                 ms = timer.time(lambda i: ops.bn_folded_act_forward(xs[i], ys[i], sh["folded"], act), 20, rotate=rot)
                 r = dict(act=act, shape="%dx%dx%d^2" % (EPILOGUE_BATCH, sh["c"], sh["s"]), ms=round(ms, 4),
                          ms_min=round(timer.last_min, 4), GBps=round(8.0 * sh["elems"] / (ms * 1e-3) / 1e9, 1))
+                if r["GBps"] < 0.70 * HBM_PEAK_GBS:      # as for the other kernels' rows under the bar
+                    c_ms = copy_of_size(8 * sh["elems"], cap=3)
+                    r["copy_same_bytes_ms"] = round(c_ms, 4)
+                    r["vs_copy"] = round(c_ms / ms, 3)
                 per_shape.append(r)
-                log("epilogue %-9s %-16s %8.4f ms %8.1f GB/s" % (r["act"], r["shape"], r["ms"], r["GBps"]))
+                log("epilogue %-9s %-16s %8.4f ms %8.1f GB/s%s" % (r["act"], r["shape"], r["ms"], r["GBps"],
+                    ("  copy of the same bytes %.4f ms (%.2f)" % (r["copy_same_bytes_ms"], r["vs_copy"]))
+                    if "vs_copy" in r else ""))
             del xs, ys
 
     copy_row = calibration_copy(torch, ops, timer)
