@@ -173,6 +173,7 @@ def same_bytes_copier(torch, ops, timer):
     """Returns copy_same_bytes(bytes, cap=None): the time of a plain copy (half the bytes read, half
     written, through the route kernel) of the same size, over buffers rotated as the row's are: what
     one launch of this size costs on this part whatever it computes.  Cached per size rounded to 2 %."""
+    import numpy as np
     cache = {}
     dev = torch.device("cuda")
 
@@ -644,7 +645,20 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None):
         add("rescale_clip", "%dx%dx%d^2" % (N, c, s_), 12 * e, ms, "norm 4B + rewrite 8B per elem")
         ms = timer.time(lambda i: ops.rescale_clip(xs[i], 1e30, 0.0), 10, rotate=rot)
         add("rescale_clip(no-op)", "%dx%dx%d^2" % (N, c, s_), 4 * e, ms, "below the threshold: norm only, 4B/elem")
-        del xs
+        # the same verdict from the group sums that the kernel which wrote the tensor left behind
+        # (pxh_shortcut_backward_norm, pxh_axpy_norm): the tensor is not read; and that writer beside the plain one
+        groups = [ops.norm_groups_like(xs[0]) for _ in range(rot)]
+        for x, g in zip(xs, groups):
+            ops.norm_groups(x, g)
+        ms = timer.time(lambda i: ops.rescale_clip_from_groups(xs[i], groups[i], 1e30, 0.0), 10, rotate=rot)
+        add("rescale_clip_from_groups(no-op)", "%dx%dx%d^2" % (N, c, s_), 8 * (e // 256), ms,
+            "two launches, 8 B per 256 values read; against the row above", streaming=False)
+        ds = [torch.randn_like(xs[0]) for _ in range(rot)]
+        fs = [torch.randn_like(xs[0]) for _ in range(rot)]
+        ms = timer.time(lambda i: ops.shortcut_backward_norm(ds[i], fs[i], xs[i], groups[i], "linear"), 10, rotate=rot)
+        add("shortcut_bwd+norm", "%dx%dx%d^2" % (N, c, s_), 20 * e, ms,
+            "20B/elem + the group sums of grad; shortcut_bwd of this shape: %.4f ms" % shortcut_ms[(c, s_)][1])
+        del xs, groups, ds, fs
 
     # ---- non-conv ms per batch, YOLOv3 @608, batch 16, one training step:
     # 72 BN'd conv epilogues fwd+bwd, 3 bias epilogues, 23 shortcuts fwd+bwd, 2 upsamples and 2 route

@@ -39,7 +39,9 @@ enum pxh_activation {
 };
 
 const char* pxh_last_error(void);
-/* library version, bumped when a signature changes */
+/* library version, bumped when a signature changes or a declaration leaves this header
+ * (2: the test hooks moved to a private header; the tensor tables, the norm-from-the-writer entry
+ * points, pxh_reserve_workspace and pxh_bn_train_act_forward_static were added) */
 int pxh_abi_version(void);
 
 /* Entry points that take `(workspace, workspace_bytes)` use a per-device buffer owned by the library

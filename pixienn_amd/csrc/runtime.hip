@@ -111,7 +111,7 @@ extern "C" {
 
 const char* pxh_last_error(void) { return pxh::g_error; }
 
-int pxh_abi_version(void) { return 1; }
+int pxh_abi_version(void) { return 2; }
 
 int pxh_reserve_workspace(size_t bytes)
 {

@@ -784,7 +784,7 @@ constexpr uint32_t kMaxGroups = kMaxWorkers / kGroup;
 constexpr int kCounterStride = 256 / sizeof(unsigned long long);      // words between two counters
 
 constexpr int kCountersPerSet = 1 + kMaxGroups;
-constexpr int kCounterSets = 64;
+constexpr int kCounterSets = 256;
 __device__ __align__(256) unsigned long long g_arrival_counters[kCounterSets * kCountersPerSet * kCounterStride];
 
 // True for the last of `members` arrivals.
@@ -1659,13 +1659,25 @@ YoloWorkspace carve(void* ws)
 
 // The arrival counters of the workspace at `ws` on the current device: a set of g_arrival_counters,
 // handed out the first time the address is seen and kept for it.  Launches that may overlap have
-// workspaces of their own, hence sets of their own.
-int counters_for(const char* who, const void* ws, unsigned long long** out)
+// workspaces of their own, hence sets of their own.  When every set is taken, the address that has
+// gone unused longest among those last used on `stream` gives up its set: the launch that used it
+// is ordered before this one, and its counters are back at zero when it has run.  (A graph captured
+// with a workspace bakes its set in: workspaces of captured calls should be long-lived ones.)
+// kNoCounterSet: every set belongs to an address last used on another stream.
+constexpr int kNoCounterSet = -1000;      // internal, never returned to a caller of the library
+
+int counters_for(const char* who, const void* ws, hipStream_t stream, unsigned long long** out)
 {
     constexpr int kDevices = 64;
+    struct Owner {
+        const void* ws;
+        hipStream_t stream;
+        unsigned long long last_use;
+    };
     struct PerDevice {
         unsigned long long* base = nullptr;
-        std::vector<const void*> seen;
+        unsigned long long uses = 0;
+        std::vector<Owner> owners;      // owners[i] holds set i
     };
     static std::mutex mutex;
     static PerDevice devices[kDevices];
@@ -1687,15 +1699,22 @@ int counters_for(const char* who, const void* ws, unsigned long long** out)
         d.base = static_cast<unsigned long long*>(p);
     }
     size_t set = 0;
-    while (set < d.seen.size() && d.seen[set] != ws) ++set;
-    if (set == d.seen.size()) {
-        if (set == static_cast<size_t>(kCounterSets)) {
-            set_error("%s: more than %d different workspace addresses on one device; reuse workspaces", who,
-                      kCounterSets);
-            return PXH_ERR_WORKSPACE;
+    while (set < d.owners.size() && d.owners[set].ws != ws) ++set;
+    if (set == d.owners.size()) {
+        if (set < static_cast<size_t>(kCounterSets)) {
+            d.owners.push_back(Owner{ ws, stream, 0 });
+        } else {
+            size_t oldest = d.owners.size();
+            for (size_t i = 0; i < d.owners.size(); ++i)
+                if (d.owners[i].stream == stream && (oldest == d.owners.size() || d.owners[i].last_use < d.owners[oldest].last_use))
+                    oldest = i;
+            if (oldest == d.owners.size()) return kNoCounterSet;     // the caller takes the form without counters
+            set = oldest;
+            d.owners[set].ws = ws;
         }
-        d.seen.push_back(ws);
     }
+    d.owners[set].stream = stream;
+    d.owners[set].last_use = ++d.uses;
     *out = d.base + set * kCountersPerSet * kCounterStride;
     return PXH_OK;
 }
@@ -1778,7 +1797,7 @@ int run_training_pass(const char* who, const float* in, float* out, float* delta
     ta.head = HeadArgs{ in, out, delta, truths, truth_counts, (p.area % 4 == 0 && aligned16(delta)) ? 1 : 0 };
     ta.runs = runs;
     ta.head_workers = FUSED ? head_workers(p.blocks, stream_us) : (p.blocks < kMaxWorkers ? p.blocks : kMaxWorkers);
-    int rc = counters_for(who, ws, &ta.sums.counters);
+    int rc = counters_for(who, ws, s, &ta.sums.counters);
     if (rc) return rc;
     ta.sums.partial = w.partial;
     ta.sums.group_partial = w.group_partial;
@@ -1903,8 +1922,13 @@ int run_training_pass(const char* who, const float* in, float* out, float* delta
     const size_t bytes = FUSED ? elems * 12 : elems * 4 + elems * 20 / static_cast<size_t>(p.classes + 5);
     const int forced = g_forced_form.load();
     const bool one = forced == 1 || (forced != 2 && bytes < (FUSED ? size_t(150) << 20 : size_t(40) << 20));
-    if (one) return one_launch::run_training_pass<FUSED>(who, in, out, delta, truths, truth_counts, p, tb, stats, cost,
-                                                         accumulate, ws, s);
+    if (one) {
+        const int rc = one_launch::run_training_pass<FUSED>(who, in, out, delta, truths, truth_counts, p, tb, stats, cost,
+                                                            accumulate, ws, s);
+        // no arrival counters to be had for this workspace address (see counters_for): nothing was
+        // launched, and the form that needs none does the same work
+        if (rc != one_launch::kNoCounterSet) return rc;
+    }
     YoloParams q = p;
     set_lanes_per_slot(q, 1);
     return two_launch::run_training_pass<FUSED>(who, in, out, delta, truths, truth_counts, q, tb, stats, cost,

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_abi_version():
-    assert capi.load().pxh_abi_version() == 1
+    assert capi.load().pxh_abi_version() == 2
 
 
 def test_fastdiv_matches_integer_division():

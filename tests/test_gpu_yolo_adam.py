@@ -562,3 +562,49 @@ def test_yolo_detections_capacity_and_empty(ops, oracle):
     assert set(got["order"]) <= set(want["order"])
     got, found_g = ops.yolo_detections(gpu(decoded), N, mask, anchors, K, W, W, 416, 416, 1.5, 10)
     assert found_g == 0 and len(got) == 0
+
+
+def test_yolo_training_pass_with_more_workspaces_than_counter_sets(ops):
+    """The one-launch form keeps its arrival counters in device memory of the library, one set per
+    workspace address.  A caller whose allocator hands out a new address every time must go on
+    working: on one stream, the address unused longest gives up its set.  300 workspaces in turn
+    (256 sets exist), twice round, every result equal to the first; then an address on ANOTHER stream
+    with every set taken by this one: the call takes the two-launch form, which needs no counters, and
+    gives the same result to the tolerance between the two forms."""
+    import torch
+    from pixienn_amd import capi
+    N, K, W = 2, 3, 13
+    mask, anchors = [0, 1, 2], [10, 13, 16, 30, 33, 23]
+    x = gpu(wl.normal(5200, (N, 3 * (K + 5), W, W), std=2.0))
+    truths_np, counts_np = wl.yolo_truths(5201, N)
+    truths, counts = gpu(truths_np), gpu(counts_np)
+    need = capi.load().pxh_yolo_workspace_bytes(N, 3, K, W, W, truths_np.shape[1])
+    pool = torch.empty((300, (need + 255) // 256 * 64), dtype=torch.float32, device="cuda")     # 256-byte aligned rows
+    out = torch.empty_like(x); delta = torch.empty_like(x)
+    stats = torch.zeros(12, device="cuda"); cost = torch.zeros(1, device="cuda")
+
+    def run(ws):
+        ops.yolo_forward_train(x, out, delta, truths, counts, truths_np.shape[1], mask, anchors, stats, cost, N, K, W, W,
+                               416, 416, 0.7, 1.0, workspace=ws)
+        return host(delta).copy(), float(host(cost)[0]), host(stats).copy()
+
+    capi.load().pxh_debug_yolo_tuning(1, 0, 0)
+    try:
+        first = run(pool[0])
+        assert first[1] > 0.0
+        for turn in range(2):
+            for i in range(300):
+                got = run(pool[i])
+                assert got[1] == first[1] and np.array_equal(got[2], first[2]), "workspace %d, turn %d" % (i, turn)
+                assert_bit_exact(got[0], first[0], "delta with workspace %d, turn %d" % (i, turn))
+        other = torch.cuda.Stream()
+        fresh = torch.empty((need + 3) // 4, dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        with torch.cuda.stream(other):
+            elsewhere = run(fresh)
+        assert abs(elsewhere[1] - first[1]) <= 2e-5 * first[1]
+        assert_close(elsewhere[0], first[0], 1e-5, 1.0, "delta through the form without counters")
+        torch.cuda.synchronize()
+        assert run(pool[7])[1] == first[1]
+    finally:
+        capi.load().pxh_debug_yolo_tuning(0, 0, 0)
