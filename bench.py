@@ -552,6 +552,12 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None):
         add("bn_bwd(leaky)", "%dx%dx%d^2" % (N, c, s), (16 if one_launch else 20) * e, ms_b,
             "one launch: delta once, x twice, 16B per elem (three launches move 20)" if one_launch
             else "sums 8B + dx 12B per elem; pre recomputed")
+        if one_launch:
+            # both conventions in the row: the bytes this launch moves (frac above) and the 12 / 20 B per
+            # element that the three-launch form moves, which is the figure the per-kernel bar was written for
+            for row, per_elem, ms in ((rows[-2], 12, ms_f), (rows[-1], 20, ms_b)):
+                row["three_launch_bytes_MB"] = round(per_elem * e / 1e6, 1)
+                row["frac_of_peak_at_three_launch_bytes"] = round(per_elem * e / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 3)
         bn_ms[(c, s)] = (ms_f, ms_b, count)
         del x, y, d
     # ---- linear bias epilogue of the three head convs at batch 16
