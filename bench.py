@@ -447,6 +447,14 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None):
         add("shortcut_bwd", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_b, "20B/elem")
         shortcut_ms[(c, s)] = (ms_f, ms_b, count)
         del a, b, o
+    # ---- the delta zero-fill of Layer::forward (include/Layer.h:377-383): write-only, 4 B per element
+    for c, s in [(32, 608), (256, 76), (1024, 19)]:
+        e = N * c * s * s
+        rot = rotation_for(4 * e)
+        ds_ = [torch.empty((N, c, s, s), device=dev) for _ in range(rot)]
+        ms = timer.time(lambda i: ops.fill(ds_[i], 0.0), 20, rotate=rot)
+        add("fill(delta = 0)", "%dx%dx%d^2" % (N, c, s), 4 * e, ms, "4B/elem written")
+        del ds_
     # ---- YOLO head (config 3): batch 64, and batch 16 for the training step's own heads
     stats = torch.zeros(12, device=dev)
     cost = torch.zeros(1, device=dev)
