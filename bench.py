@@ -1014,6 +1014,12 @@ def main():
     value_raw = bytes_step / ((time.perf_counter() - t0) / args.steps) / 1e9
     log("whole sweep: %.1f GB/s with folded constants, %.1f GB/s folding on every call" % (value, value_raw))
 
+    # the same step with its 21 launches recorded in a HIP graph (what a host that captures its layer
+    # sequence runs): no gaps between the launches, nothing else changes
+    graph_ms = timer.time(lambda i: run_epilogue_step(ops, shapes), 10, warm=1)
+    value_graph = bytes_step / (graph_ms * 1e-3) / 1e9
+    log("whole sweep as one HIP graph: %.4f ms per step, %.1f GB/s" % (graph_ms, value_graph))
+
     # per shape, each measured alone over rotating buffers (HIP events around 20 launches)
     per_shape = []
     if not args.no_extras:
@@ -1092,6 +1098,7 @@ def main():
         "noconv_step_in_model_order_yolov3_608": model_order,
         "config0_yolov3_tiny_forward_batch1": config0,
         "value_folding_every_call": round(value_raw, 1),
+        "value_as_one_hip_graph": round(value_graph, 1),
         "plain_copy": copy_row,
         "per_activation": per_act,
         "per_shape": per_shape,
