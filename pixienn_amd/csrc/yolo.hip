@@ -400,6 +400,12 @@ __device__ __forceinline__ double head_tile(const uint32_t head_block, const Hea
     const int i = col, j = row;
 
     float sx = 0, sy = 0, rw = 0, rh = 0, so = 0;
+    // the host-built table says whether something supervises this slot: asked for with the head rows
+    // (it is needed after the sweep, where it would be a trip to memory of its own)
+    int table_cls = -1;
+    if constexpr (!FUSED) {
+        if (live) table_cls = tb.assigned_classes[static_cast<size_t>(bn) * area + cell];
+    }
     if (live) {
         const float v0 = in[base], v1 = in[base + area], v2 = in[base + 2 * static_cast<size_t>(area)],
                     v3 = in[base + 3 * static_cast<size_t>(area)], v4 = in[base + 4 * static_cast<size_t>(area)];
@@ -582,7 +588,7 @@ __device__ __forceinline__ double head_tile(const uint32_t head_block, const Hea
     if constexpr (!FUSED) {
         if (live) {
             const size_t slot = static_cast<size_t>(bn) * area + cell;
-            const int acls = tb.assigned_classes[slot];
+            const int acls = table_cls;
             if (acls >= 0) {
                 pos_cls = acls;
                 pos_anchor = tb.assigned_anchors[slot];
@@ -1084,6 +1090,12 @@ __device__ __forceinline__ double head_tile(const uint32_t head_block, const Hea
     const int i = col, j = row;
 
     float sx = 0, sy = 0, rw = 0, rh = 0, so = 0;
+    // the host-built table says whether something supervises this slot: asked for with the head rows
+    // (it is needed after the sweep, where it would be a trip to memory of its own)
+    int table_cls = -1;
+    if constexpr (!FUSED) {
+        if (live) table_cls = tb.assigned_classes[static_cast<size_t>(bn) * area + cell];
+    }
     if (live) {
         const float v0 = in[base], v1 = in[base + area], v2 = in[base + 2 * static_cast<size_t>(area)],
                     v3 = in[base + 3 * static_cast<size_t>(area)], v4 = in[base + 4 * static_cast<size_t>(area)];
@@ -1182,7 +1194,7 @@ __device__ __forceinline__ double head_tile(const uint32_t head_block, const Hea
     if constexpr (!FUSED) {
         if (live) {
             const size_t slot = static_cast<size_t>(bn) * area + cell;
-            const int acls = tb.assigned_classes[slot];
+            const int acls = table_cls;
             if (acls >= 0) {
                 pos_cls = acls;
                 pos_anchor = tb.assigned_anchors[slot];
