@@ -1868,6 +1868,17 @@ uint32_t head_workers(uint32_t tiles, double stream_us)
     return want < tiles ? want : tiles;
 }
 
+// The same for the form that starts from a decoded head, whose stream only writes zeros.  A head
+// worker holds a workgroup slot for the whole pass, and such a stream is done in a few tens of
+// microseconds: beyond about 3.5 workers per compute unit it is starved of slots until the workers
+// leave, and the two run one after the other (measured at 64 x 255 x 76^2, 4332 tiles: 900 workers
+// 60 us, 1500 workers 77 us, 1900 workers 83 us; at 32 x 255 x 76^2: 39 us against 46 us).  Up to
+// 1200 tiles every tile gets its worker: one round of tiles is the shortest the pass can be.
+uint32_t head_workers_beside_fill(uint32_t tiles)
+{
+    return tiles <= 1200u ? tiles : 900u;
+}
+
 template<bool FUSED>
 int run_training_pass(const char* who, const float* in, float* out, float* delta, const float* truths,
                       const int* truth_counts, const YoloParams& p, const YoloTables& tb, float* stats, float* cost,
@@ -1896,7 +1907,9 @@ int run_training_pass(const char* who, const float* in, float* out, float* delta
 
     const int stream_bytes = FUSED ? 12 : 4;      // per class element: read + decode + zero delta, or the zero delta alone
     const double stream_us = static_cast<double>(space.elems) * stream_bytes / 6.0e6;   // at 6 TB/s
-    FusedArgs fa{ ha, space, head_workers(p.blocks, stream_us) };
+    FusedArgs fa{ ha, space, FUSED ? head_workers(p.blocks, stream_us) : head_workers_beside_fill(p.blocks) };
+    if (const int forced = one_launch::g_forced_workers.load(); forced > 0)
+        fa.head_workers = static_cast<uint32_t>(forced) < p.blocks ? static_cast<uint32_t>(forced) : p.blocks;
     ca.head_blocks = fa.head_workers;      // one partial sum per worker
     const uint32_t grid = fa.head_workers + class_blocks;
     const bool nt = static_cast<size_t>(space.elems) * stream_bytes >= kStreamingBytes;
@@ -1923,7 +1936,7 @@ size_t training_workspace_bytes(int batch, int mask_count, int width, int height
 }
 
 // One launch where the pass is bound by the head tiles' chain of steps, two where it is bound by the
-// class stream (measured on MI355X at 80 classes: below about 150 MB of fused traffic, and below
+// class stream (measured on MI355X at 80 classes: below about 110 MB of fused traffic, and below
 // about 40 MB for the form that starts from a decoded head, one launch is the faster).
 template<bool FUSED>
 int run_training_pass(const char* who, const float* in, float* out, float* delta, const float* truths,
@@ -1933,7 +1946,7 @@ int run_training_pass(const char* who, const float* in, float* out, float* delta
     const size_t elems = static_cast<size_t>(p.batch) * p.mask_count * (p.classes + 5) * p.area;
     const size_t bytes = FUSED ? elems * 12 : elems * 4 + elems * 20 / static_cast<size_t>(p.classes + 5);
     const int forced = g_forced_form.load();
-    const bool one = forced == 1 || (forced != 2 && bytes < (FUSED ? size_t(150) << 20 : size_t(40) << 20));
+    const bool one = forced == 1 || (forced != 2 && bytes < (FUSED ? size_t(110) << 20 : size_t(40) << 20));
     if (one) {
         const int rc = one_launch::run_training_pass<FUSED>(who, in, out, delta, truths, truth_counts, p, tb, stats, cost,
                                                             accumulate, ws, s);
