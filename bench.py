@@ -56,6 +56,9 @@ def parse_args():
     ap.add_argument("--plain-step", action="store_true",
                     help="with --only-model-order: the step as the reference runs it only, none of the optional forms "
                          "(for a kernel trace whose shares are those of one step)")
+    ap.add_argument("--only-heads", action="store_true",
+                    help="run only the YOLO head rows: decode, training pass, loss form, detections (for a kernel "
+                         "trace of those kernels)")
     ap.add_argument("--only-model-order", action="store_true",
                     help="run only the YOLOv3 training step in model order (for a kernel trace of that step)")
     return ap.parse_args()
@@ -363,7 +366,7 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     return out
 
 
-def measure_extras(torch, ops, wl, timer, capi, cpu=None):
+def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
     """The other kernels of the path at the baseline's shapes.  Returns (rows, ms_per_batch).  `cpu`:
     cpu_rows(), attached to the rows it has a figure for."""
     import numpy as np
@@ -389,72 +392,78 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None):
         return torch.randn(shape, device=dev)
 
     N = 16
-    # ---- route concat of YOLOv3 @608: 256x38^2 (upsampled) ++ 512x38^2, and 128x76^2 ++ 256x76^2.
-    # The upsample in front writes its channels straight into the concat buffer (timed below, same
-    # bytes as the dense form), so the route moves the other source only.
-    for (c1, c2, s) in [(256, 512, 38), (128, 256, 76)]:
-        e = N * c2 * s * s
-        e_up = N * c1 * s * s
-        rot = rotation_for(5 * e_up)      # the smallest of the three launches sets the number of buffer sets
-        bs = [randn(N, c2, s, s) for _ in range(rot)]
-        rs = [torch.empty((N, c1 + c2, s, s), device=dev) for _ in range(rot)]
-        ms = timer.time(lambda i: ops.route_forward(bs[i], rs[i], c1 * s * s), 20, rotate=rot)
-        add("route_fwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), 8 * e, ms, "the %d-channel source, 8B/elem" % c2)
-        ms = timer.time(lambda i: ops.route_backward(rs[i], bs[i], c1 * s * s), 20, rotate=rot)
-        add("route_bwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), 12 * e, ms, "the %d-channel source, 12B/elem" % c2)
-        xs = [randn(N, c1, s // 2, s // 2) for _ in range(rot)]
-        ms = timer.time(lambda i: ops.upsample_forward_into(xs[i], rs[i], 0, 2, 1.0), 20, rotate=rot)
-        add("upsample_fwd(into route)", "%dx%dx%d^2" % (N, c1, s // 2), 5 * e_up, ms, "same bytes as upsample_fwd; "
-            "not in ms/batch twice")
-        del bs, rs, xs
-    # ---- max-pool 2x2 s2 forward + backward (config 2)
-    for c, s in wl.YOLOV3_MAXPOOL_SHAPES:
-        e_in = N * c * s * s
-        e_out = e_in // 4
-        rot = rotation_for(4 * e_in + 8 * e_out)
-        xs = [randn(N, c, s, s) for _ in range(rot)]
-        outs = [torch.empty((N, c, s // 2, s // 2), device=dev) for _ in range(rot)]
-        idxs = [torch.empty((N, c, s // 2, s // 2), device=dev, dtype=torch.int32) for _ in range(rot)]
-        ms = timer.time(lambda i: ops.maxpool_forward(xs[i], outs[i], idxs[i], 2, 2, 1), 20, rotate=rot)
-        add("maxpool_fwd", "%dx%dx%d^2" % (N, c, s), 4 * e_in + 8 * e_out, ms, "4B/in + 8B/out")
-        deltas = [randn(N, c, s // 2, s // 2) for _ in range(rot)]
-        ms = timer.time(lambda i: ops.maxpool_backward(deltas[i], idxs[i], xs[i], 2, 2, 1), 20, rotate=rot)
-        add("maxpool_bwd", "%dx%dx%d^2" % (N, c, s), 8 * e_out + 8 * e_in, ms, "full-grad RMW: 8B/out + 8B/in")
-        del xs, outs, idxs, deltas
-    # ---- upsample x2 forward + backward
-    for c, s in wl.YOLOV3_UPSAMPLE_SHAPES:
-        e_in = N * c * s * s
-        e_out = 4 * e_in
-        rot = rotation_for(4 * e_in + 4 * e_out)
-        xs = [randn(N, c, s, s) for _ in range(rot)]
-        outs = [torch.empty((N, c, 2 * s, 2 * s), device=dev) for _ in range(rot)]
-        ms_f = timer.time(lambda i: ops.upsample_forward(xs[i], outs[i], 2, 1.0), 50, rotate=rot)
-        add("upsample_fwd", "%dx%dx%d^2" % (N, c, s), 4 * e_in + 4 * e_out, ms_f, "4B/in + 4B/out")
-        ms_b = timer.time(lambda i: ops.upsample_backward(outs[i], xs[i], 2, 1.0), 50, rotate=rot)
-        add("upsample_bwd", "%dx%dx%d^2" % (N, c, s), 4 * e_out + 8 * e_in, ms_b, "4B/out + 8B/in")
-        del xs, outs
-    # ---- shortcut forward + backward
-    shortcut_ms = {}
-    for c, s, count in wl.YOLOV3_SHORTCUT_SHAPES:
-        e = N * c * s * s
-        rot = rotation_for(12 * e)
-        a = [randn(N, c, s, s) for _ in range(rot)]
-        b = [randn(N, c, s, s) for _ in range(rot)]
-        o = [torch.empty((N, c, s, s), device=dev) for _ in range(rot)]
-        ms_f = timer.time(lambda i: ops.shortcut_forward(a[i], b[i], o[i], "linear"), 20, rotate=rot)
-        add("shortcut_fwd", "%dx%dx%d^2" % (N, c, s), 12 * e, ms_f, "12B/elem")
-        ms_b = timer.time(lambda i: ops.shortcut_backward(o[i], a[i], b[i], "linear"), 20, rotate=rot)
-        add("shortcut_bwd", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_b, "20B/elem")
-        shortcut_ms[(c, s)] = (ms_f, ms_b, count)
-        del a, b, o
-    # ---- the delta zero-fill of Layer::forward (include/Layer.h:377-383): write-only, 4 B per element
-    for c, s in [(32, 608), (256, 76), (1024, 19)]:
-        e = N * c * s * s
-        rot = rotation_for(4 * e)
-        ds_ = [torch.empty((N, c, s, s), device=dev) for _ in range(rot)]
-        ms = timer.time(lambda i: ops.fill(ds_[i], 0.0), 20, rotate=rot)
-        add("fill(delta = 0)", "%dx%dx%d^2" % (N, c, s), 4 * e, ms, "4B/elem written")
-        del ds_
+    if not only_heads:      # (the sections in front of the heads)
+        # ---- route concat of YOLOv3 @608: 256x38^2 (upsampled) ++ 512x38^2, and 128x76^2 ++ 256x76^2.
+        # The upsample in front writes its channels straight into the concat buffer (timed below, same
+        # bytes as the dense form), so the route moves the other source only.
+        for (c1, c2, s) in [(256, 512, 38), (128, 256, 76)]:
+            e = N * c2 * s * s
+            e_up = N * c1 * s * s
+            rot = rotation_for(5 * e_up)      # the smallest of the three launches sets the number of buffer sets
+            bs = [randn(N, c2, s, s) for _ in range(rot)]
+            rs = [torch.empty((N, c1 + c2, s, s), device=dev) for _ in range(rot)]
+            ms = timer.time(lambda i: ops.route_forward(bs[i], rs[i], c1 * s * s), 20, rotate=rot)
+            add("route_fwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), 8 * e, ms, "the %d-channel source, 8B/elem" % c2)
+            ms = timer.time(lambda i: ops.route_backward(rs[i], bs[i], c1 * s * s), 20, rotate=rot)
+            add("route_bwd", "%dx(%d+)%dx%d^2" % (N, c1, c2, s), 12 * e, ms, "the %d-channel source, 12B/elem" % c2)
+            xs = [randn(N, c1, s // 2, s // 2) for _ in range(rot)]
+            ms = timer.time(lambda i: ops.upsample_forward_into(xs[i], rs[i], 0, 2, 1.0), 20, rotate=rot)
+            add("upsample_fwd(into route)", "%dx%dx%d^2" % (N, c1, s // 2), 5 * e_up, ms, "same bytes as upsample_fwd; "
+                "not in ms/batch twice")
+            del bs, rs, xs
+        # ---- max-pool 2x2 s2 forward + backward (config 2)
+        for c, s in wl.YOLOV3_MAXPOOL_SHAPES:
+            e_in = N * c * s * s
+            e_out = e_in // 4
+            rot = rotation_for(4 * e_in + 8 * e_out)
+            xs = [randn(N, c, s, s) for _ in range(rot)]
+            outs = [torch.empty((N, c, s // 2, s // 2), device=dev) for _ in range(rot)]
+            idxs = [torch.empty((N, c, s // 2, s // 2), device=dev, dtype=torch.int32) for _ in range(rot)]
+            ms = timer.time(lambda i: ops.maxpool_forward(xs[i], outs[i], idxs[i], 2, 2, 1), 20, rotate=rot)
+            add("maxpool_fwd", "%dx%dx%d^2" % (N, c, s), 4 * e_in + 8 * e_out, ms, "4B/in + 8B/out")
+            deltas = [randn(N, c, s // 2, s // 2) for _ in range(rot)]
+            ms = timer.time(lambda i: ops.maxpool_backward(deltas[i], idxs[i], xs[i], 2, 2, 1), 20, rotate=rot)
+            add("maxpool_bwd", "%dx%dx%d^2" % (N, c, s), 8 * e_out + 8 * e_in, ms, "full-grad RMW: 8B/out + 8B/in")
+            del xs, outs, idxs, deltas
+        # ---- upsample x2 forward + backward
+        for c, s in wl.YOLOV3_UPSAMPLE_SHAPES:
+            e_in = N * c * s * s
+            e_out = 4 * e_in
+            rot = rotation_for(4 * e_in + 4 * e_out)
+            xs = [randn(N, c, s, s) for _ in range(rot)]
+            outs = [torch.empty((N, c, 2 * s, 2 * s), device=dev) for _ in range(rot)]
+            ms_f = timer.time(lambda i: ops.upsample_forward(xs[i], outs[i], 2, 1.0), 50, rotate=rot)
+            add("upsample_fwd", "%dx%dx%d^2" % (N, c, s), 4 * e_in + 4 * e_out, ms_f, "4B/in + 4B/out")
+            ms_b = timer.time(lambda i: ops.upsample_backward(outs[i], xs[i], 2, 1.0), 50, rotate=rot)
+            add("upsample_bwd", "%dx%dx%d^2" % (N, c, s), 4 * e_out + 8 * e_in, ms_b, "4B/out + 8B/in")
+            del xs, outs
+        # ---- shortcut forward + backward
+        shortcut_ms = {}
+        for c, s, count in wl.YOLOV3_SHORTCUT_SHAPES:
+            e = N * c * s * s
+            rot = rotation_for(12 * e)
+            a = [randn(N, c, s, s) for _ in range(rot)]
+            b = [randn(N, c, s, s) for _ in range(rot)]
+            o = [torch.empty((N, c, s, s), device=dev) for _ in range(rot)]
+            ms_f = timer.time(lambda i: ops.shortcut_forward(a[i], b[i], o[i], "linear"), 20, rotate=rot)
+            add("shortcut_fwd", "%dx%dx%d^2" % (N, c, s), 12 * e, ms_f, "12B/elem")
+            ms_b = timer.time(lambda i: ops.shortcut_backward(o[i], a[i], b[i], "linear"), 20, rotate=rot)
+            add("shortcut_bwd", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_b, "20B/elem")
+            # the same on the same buffers, also leaving the norm and peak of what it wrote to grad
+            groups = [ops.norm_groups_like(b[0]) for _ in range(rot)]
+            ms_n = timer.time(lambda i: ops.shortcut_backward_norm(o[i], a[i], b[i], groups[i], "linear"), 20, rotate=rot)
+            add("shortcut_bwd+norm", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_n, "20B/elem + 8B per 256 values of grad")
+            del groups
+            shortcut_ms[(c, s)] = (ms_f, ms_b, count)
+            del a, b, o
+        # ---- the delta zero-fill of Layer::forward (include/Layer.h:377-383): write-only, 4 B per element
+        for c, s in [(32, 608), (256, 76), (1024, 19)]:
+            e = N * c * s * s
+            rot = rotation_for(4 * e)
+            ds_ = [torch.empty((N, c, s, s), device=dev) for _ in range(rot)]
+            ms = timer.time(lambda i: ops.fill(ds_[i], 0.0), 20, rotate=rot)
+            add("fill(delta = 0)", "%dx%dx%d^2" % (N, c, s), 4 * e, ms, "4B/elem written")
+            del ds_
     # ---- YOLO head (config 3): batch 64, and batch 16 for the training step's own heads
     stats = torch.zeros(12, device=dev)
     cost = torch.zeros(1, device=dev)
@@ -511,6 +520,8 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None):
                     "%d records; %.2g%% of the slots pass" % (found, 100 * passing), streaming=False)
             del rec
         del xin, out, dl
+    if only_heads:
+        return rows, 0.0
     # ---- non-maximum suppression of device-resident records: an inference-sized list (one image, one
     # launch) and a validation-sized one (64 images, low confidence threshold).  Not a streaming kernel:
     # the time is comparisons between records, the bytes column is just the records read and written.
@@ -660,19 +671,14 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None):
         ms = timer.time(lambda i: ops.rescale_clip(xs[i], 1e30, 0.0), 10, rotate=rot)
         add("rescale_clip(no-op)", "%dx%dx%d^2" % (N, c, s_), 4 * e, ms, "below the threshold: norm only, 4B/elem")
         # the same verdict from the group sums that the kernel which wrote the tensor left behind
-        # (pxh_shortcut_backward_norm, pxh_axpy_norm): the tensor is not read; and that writer beside the plain one
+        # (pxh_shortcut_backward_norm, pxh_axpy_norm): the tensor is not read
         groups = [ops.norm_groups_like(xs[0]) for _ in range(rot)]
         for x, g in zip(xs, groups):
             ops.norm_groups(x, g)
         ms = timer.time(lambda i: ops.rescale_clip_from_groups(xs[i], groups[i], 1e30, 0.0), 10, rotate=rot)
         add("rescale_clip_from_groups(no-op)", "%dx%dx%d^2" % (N, c, s_), 8 * (e // 256), ms,
             "two launches, 8 B per 256 values read; against the row above", streaming=False)
-        ds = [torch.randn_like(xs[0]) for _ in range(rot)]
-        fs = [torch.randn_like(xs[0]) for _ in range(rot)]
-        ms = timer.time(lambda i: ops.shortcut_backward_norm(ds[i], fs[i], xs[i], groups[i], "linear"), 10, rotate=rot)
-        add("shortcut_bwd+norm", "%dx%dx%d^2" % (N, c, s_), 20 * e, ms,
-            "20B/elem + the group sums of grad; shortcut_bwd of this shape: %.4f ms" % shortcut_ms[(c, s_)][1])
-        del xs, groups, ds, fs
+        del xs, groups
 
     # ---- non-conv ms per batch, YOLOv3 @608, batch 16, one training step:
     # 72 BN'd conv epilogues fwd+bwd, 3 bias epilogues, 23 shortcuts fwd+bwd, 2 upsamples and 2 route
@@ -960,6 +966,14 @@ def main():
         print(json.dumps({"noconv_step_in_model_order_yolov3_608": measure_model_order(torch, ops, wl, timer,
                                                                                         plain_only=args.plain_step)}),
               flush=True)
+        return
+
+    if args.only_heads:
+        rows, _ = measure_extras(torch, ops, wl, timer, capi, only_heads=True)
+        for r in rows:
+            log("%-26s %-22s %9.1f MB %8.4f ms %8.1f GB/s  %4.1f%%  %s" % (r["kernel"], r["shape"], r["MB"], r["ms"],
+                                                                          r["GBps"], 100 * r["frac"], r["note"]))
+        print(json.dumps({"yolo_heads": rows}), flush=True)
         return
 
     shapes = epilogue_workload(torch, wl)
