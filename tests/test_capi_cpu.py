@@ -116,3 +116,27 @@ def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
     assert "not built" in str(e.value) and "pixienn_amd.build" in str(e.value)
     with pytest.raises(capi.PxError):
         capi.call("pxh_abi_version")
+
+
+def test_size_functions_and_argument_checks_need_no_device():
+    """The pure size functions, and the argument checks that reject a call before anything is
+    launched, work without a GPU (include/pixienn_hip.h: negative status = rejected before launch)."""
+    import ctypes
+    lib = capi.load()
+    for n, want in ((0, 0), (1, 8), (256, 8), (257, 16), (8192, 256), (94_633_984, 94_633_984 // 256 * 8)):
+        assert lib.pxh_norm_groups_bytes(n) == want
+    assert lib.pxh_rescale_workspace_bytes() == 1024 * 16
+    assert lib.pxh_bn_workspace_bytes(16, 256, 76 * 76) > 0
+    # null pointers and impossible table shapes
+    assert capi.call_raw("pxh_norm_groups", None, 1024, None, None) < 0
+    assert "null" in capi.last_error()
+    assert capi.call_raw("pxh_rescale_clip_from_groups", None, 1024, 1.0, 0.0, None, None, None, 0, None) < 0
+    assert capi.call_raw("pxh_rescale_clip_from_groups", None, 0, 1.0, 0.0, None, None, None, 0, None) == 0      # empty: nothing to do
+    assert capi.call_raw("pxh_shortcut_backward_norm", None, None, None, None, 16, 1.0, 1.0, 1, 0, None, None) < 0
+    handle = ctypes.c_void_p()
+    assert capi.call_raw("pxh_tensor_table_create", 3, 3, None, None, None, ctypes.byref(handle)) < 0
+    assert capi.call_raw("pxh_tensor_table_create", 0, 4, None, None, None, ctypes.byref(handle)) == 0
+    assert handle.value and lib.pxh_tensor_table_count(handle) == 0
+    assert capi.call_raw("pxh_adam_update_table", handle, 16, 1, 1e-3, 0.9, 0.999, 1e-8, 5e-4, None) == 0      # nothing to do
+    lib.pxh_tensor_table_destroy(handle)
+    assert capi.call_raw("pxh_adam_update_table", None, 16, 1, 1e-3, 0.9, 0.999, 1e-8, 5e-4, None) < 0
