@@ -945,6 +945,79 @@ def cpu_baseline(wl, batch):
                 host_cpus=os.cpu_count())
 
 
+MAX_LINE_BYTES = 4096      # whoever keeps only the tail of stdout must still find the whole record in it
+
+
+def clean(obj):
+    """The same structure with non-finite floats replaced by None, so that the line is strict JSON."""
+    if isinstance(obj, float):
+        return obj if obj == obj and abs(obj) != float("inf") else None
+    if isinstance(obj, dict):
+        return {k: clean(v) for k, v in obj.items()}
+    if isinstance(obj, (list, tuple)):
+        return [clean(v) for v in obj]
+    return obj
+
+
+def write_details(details, folder=None):
+    """Writes the per-shape and per-kernel rows to a file beside the script (they are also on stderr as
+    they are measured) and returns its path relative to the script, or None if it cannot be written."""
+    folder = folder or os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(folder, exist_ok=True)
+        path = os.path.join(folder, "bench_details.json")
+        with open(path, "w") as f:
+            json.dump(clean(details), f, indent=1, allow_nan=False)
+        return os.path.relpath(path, ROOT)
+    except OSError as e:
+        log("details not written: %s" % e)
+        return None
+
+
+def final_line(steps, warmup, value, ms_per_step, bytes_step, launches_per_step, roofline, cpu, model_order,
+               layer_kernels_sum_ms, value_raw, value_graph, config0, details_file=None):
+    """The ONE line of stdout: the record of the run, a few kB of strict JSON.  Everything that is a
+    table (rows per shape, per kernel, the phases of the model-order step) goes to stderr and to the
+    details file; from them this line keeps scalars only."""
+    mo = model_order or {}
+    c0 = config0 or {}
+    line = {
+        "metric": "fused BN+act epilogue GB/s (% of HBM peak); non-conv ms/batch YOLOv3 608",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: fused BN-inference+bias+activation epilogue sweep, NCHW fp32, N=64, "
+                               "7 YOLOv3-tiny conv-output shapes x {leaky, mish, logistic}; per-channel constants "
+                               "folded once before the timed region",
+                   "bytes_per_step": int(bytes_step), "launches_per_step": launches_per_step,
+                   "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        # the second half of the metric: one training step of YOLOv3 @608 at batch 16, every non-conv kernel
+        # launched in model order with what the Layer base class adds around each layer (three HIP graphs);
+        # beside it the leanest form of the same step and the plain sum of the layer kernels' own rows
+        "noconv_ms_per_batch_yolov3_608": mo.get("total_ms"),
+        "noconv_ms_per_batch_yolov3_608_leanest": mo.get("leanest_total_ms"),
+        "noconv_layer_kernels_sum_ms_yolov3_608": None if layer_kernels_sum_ms is None else round(layer_kernels_sum_ms, 3),
+        "config0_gpu_ms": c0.get("gpu_graph_ms"),
+        "config0_cpu_ms": c0.get("cpu_ms"),
+        "value_folding_every_call": round(value_raw, 1),
+        "value_as_one_hip_graph": round(value_graph, 1),
+        "details": details_file,
+    }
+    text = json.dumps(clean(line), allow_nan=False, separators=(",", ":"))
+    assert len(text) < MAX_LINE_BYTES, "the final line grew to %d bytes" % len(text)
+    return text
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -1008,9 +1081,8 @@ def main():
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                     frac=round(achieved / HBM_PEAK_GBS, 4),
                     traffic=None if EPILOGUE_TRAFFIC_RATIO is None else round(EPILOGUE_TRAFFIC_RATIO * bytes_per_launch),
-                    traffic_source="profiles/epilogue_sweep_hbm_traffic.txt: FETCH_SIZE + WRITE_SIZE of this kernel in "
-                                   "two rocprofv3 --pmc runs of this script, as a ratio of its algorithmic bytes; not "
-                                   "measured in this run",
+                    traffic_source="profiles/epilogue_sweep_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of "
+                                   "this script; not measured in this run)",
                     kernel="epilogue_fwd_kernel<PXH_LEAKY, true, *>",
                     bytes_per_launch=round(bytes_per_launch),
                     mean_launch_ms=round(leaky_ms / launches, 5))
@@ -1082,41 +1154,18 @@ def main():
         cpu = cpu_baseline(wl, args.cpu_batch)
         log("cpu baseline:", cpu)
 
-    line = {
-        "metric": "fused BN+act epilogue GB/s (% of HBM peak); non-conv ms/batch YOLOv3 608",
-        "value": round(value, 1),
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": "configs[1]: fused BN-inference+bias+activation epilogue sweep, NCHW fp32, N=64, "
-                               "7 YOLOv3-tiny conv-output shapes x {leaky, mish, logistic}; per-channel constants "
-                               "folded once before the timed region, as a layer does after loading its weights",
-                   "bytes_per_step": int(bytes_step), "launches_per_step": len(shapes) * len(EPILOGUE_ACTS),
-                   "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2)},
-        "roofline": roofline,
-        "cpu_baseline": cpu,
-        # the second half of the metric: one training step of YOLOv3 @608 at batch 16, every non-conv kernel
-        # launched in model order with what the Layer base class adds around each layer (measured, three
-        # HIP graphs); beside it the plain sum of the layer kernels' own rows
-        "noconv_ms_per_batch_yolov3_608": None if model_order is None else model_order["total_ms"],
-        "noconv_layer_kernels_sum_ms_yolov3_608": None if ms_batch is None else round(ms_batch, 3),
+    details = {
         "noconv_step_in_model_order_yolov3_608": model_order,
         "config0_yolov3_tiny_forward_batch1": config0,
-        "value_folding_every_call": round(value_raw, 1),
-        "value_as_one_hip_graph": round(value_graph, 1),
         "plain_copy": copy_row,
         "per_activation": per_act,
         "per_shape": per_shape,
         "extras": extras,
     }
-    print(json.dumps(line), flush=True)
+    line = final_line(args.steps, args.warmup, value, ms_per_step, bytes_step, len(shapes) * len(EPILOGUE_ACTS),
+                      roofline, cpu, model_order, ms_batch, value_raw, value_graph, config0,
+                      details_file=write_details(details))
+    print(line, flush=True)
 
 
 if __name__ == "__main__":
