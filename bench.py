@@ -84,6 +84,8 @@ class Timer:
         prepare() runs untimed before every trial (for a kernel that changes what it will do next
         time on the same data)."""
         t = self.torch
+        if rotate > 1:      # every buffer set in every replay, each as often as the others
+            reps = -(-reps // rotate) * rotate
         if prepare:
             prepare()
         for i in range(max(warm, rotate)):
@@ -125,9 +127,10 @@ class Timer:
         return samples[len(samples) // 2]
 
 
-def rotation_for(bytes_per_set, llc_bytes=256 << 20, cap=8):
+def rotation_for(bytes_per_set, llc_bytes=256 << 20, cap=96):
     """Distinct buffer sets needed so that a set has left the 256 MB last-level cache before
-    it is touched again."""
+    it is touched again: more than twice the cache of distinct bytes between two uses of a set.  (The
+    cap only bounds the number of allocations for sets under 6 MB; no row here is that small.)"""
     n = int(llc_bytes * 2 // max(1, bytes_per_set)) + 1
     return max(1, min(cap, n))
 
@@ -285,12 +288,15 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     groups = {i - 1: ops.norm_groups_like(T[i - 1]["d"]) for i, l in enumerate(layers)
               if l["type"] in ("shortcut", "yolo")}
 
-    def backward(_, first_writer=False, norm_from_writer=False):
+    def backward(_, first_writer=False, norm_from_writer=False, two_calls=False):
         n = 0
         for i in reversed(range(len(layers))):
             l, t = layers[i], T[i]
             kind = l["type"]
-            if not absorbed(i):
+            # a convolution's rescale + clip rides on its epilogue's backward (pxh_*_backward_clipped) unless
+            # the kernel that wrote its delta last left the norm behind; `two_calls`: as two calls, for comparison
+            fused = kind == "conv" and not two_calls and not (norm_from_writer and i in groups)
+            if not absorbed(i) and not fused:
                 if norm_from_writer and i in groups:
                     ops.rescale_clip_from_groups(t["d"], groups[i], 100.0, 10.0)
                 else:
@@ -303,9 +309,14 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
                                            first=first_writer)
             elif kind == "yolo":
                 ops.axpy(1.0, t["d"], T[i - 1]["d"])
+            elif kind == "conv" and l["bn"] and fused:
+                ops.bn_act_backward_clipped(t["d"], t["x"], t["mean"], t["var"], t["scale"], t["bias"], t["su"],
+                                            t["bu"], "leaky", 100.0, 10.0)
             elif kind == "conv" and l["bn"]:
                 ops.bn_act_backward(t["d"], t["x"], t["mean"], t["var"], t["scale"], t["bias"], t["su"], t["bu"],
                                     "leaky")
+            elif kind == "conv" and fused:
+                ops.bias_act_backward_clipped(t["d"], None, t["bu"], "linear", 100.0, 10.0)
             elif kind == "conv":
                 ops.bias_act_backward(t["d"], None, t["bu"], "linear")
             elif kind == "shortcut" and first_writer:
@@ -347,6 +358,9 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
         del T, w, g, m, v
         torch.cuda.empty_cache()
         return out
+    # the same backward with every convolution's rescale + clip as a call of its own in front of the
+    # epilogue's backward (pxh_rescale_clip, then pxh_bn_act_backward): what the fused call saves
+    out["backward_rescale_clip_as_its_own_call_ms"] = round(timer.time(lambda i: backward(i, two_calls=True), 3, warm=1), 3)
     out["update_without_delta_pass_ms"] = round(timer.time(lambda i: update(i, False), 3, warm=1), 3)
     # the 23 shortcuts as first writers of the 46 deltas they reach first: no zero-fill of those,
     # no read of them in the shortcut's backward (an option of the C++ layer interface, "first_writer")
@@ -375,10 +389,12 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
 
     copy_same_bytes = same_bytes_copier(torch, ops, timer)
 
-    def add(name, shape, bytes_, ms, note="", streaming=True):
+    def add(name, shape, bytes_, ms, note="", streaming=True, cache_warm=False):
         gbs = bytes_ / (ms * 1e-3) / 1e9
         row = dict(kernel=name, shape=shape, MB=round(bytes_ / 1e6, 1), ms=round(ms, 4),
                    ms_min=round(timer.last_min, 4), GBps=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 3), note=note)
+        if cache_warm:      # timed on one buffer that stays in the last-level cache: not an HBM figure
+            row["cache_warm"] = True
         # below the 70 % bar: how long a plain copy of the same bytes takes, i.e. how much of the gap is
         # the cost of a launch of that size (vs_copy = copy time / this row's time; 1 = as fast as a copy)
         if streaming and row["frac"] < 0.70 and bytes_ <= (1 << 30):
@@ -473,7 +489,7 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
         truths = torch.from_numpy(truths_np).to(dev)
         counts = torch.from_numpy(counts_np).to(dev)
         e = NB * 255 * s * s
-        rot = rotation_for(12 * e)
+        rot = rotation_for(4 * e)        # the loss form touches little more than one of a set's three tensors
         xin = [2.0 * randn(NB, 255, s, s) for _ in range(rot)]
         out = [torch.empty((NB, 255, s, s), device=dev) for _ in range(rot)]
         dl = [torch.empty((NB, 255, s, s), device=dev) for _ in range(rot)]
@@ -547,7 +563,7 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
     bn_ms = {}
     for (c, s), count in zip(wl.YOLOV3_BN_SHAPES, wl.YOLOV3_BN_COUNTS):
         e = N * c * s * s
-        rot = rotation_for(12 * e, cap=4)
+        rot = rotation_for(8 * e)        # the forward touches 8 of a set's 12 bytes per element
         x = [randn(N, c, s, s) for _ in range(rot)]
         y = [torch.empty((N, c, s, s), device=dev) for _ in range(rot)]
         d = [randn(N, c, s, s) for _ in range(rot)]
@@ -571,10 +587,16 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
         add("bn_bwd(leaky)", "%dx%dx%d^2" % (N, c, s), (16 if one_launch else 20) * e, ms_b,
             "one launch: delta once, x twice, 16B per elem (three launches move 20)" if one_launch
             else "sums 8B + dx 12B per elem; pre recomputed")
+        # the same with Layer::backward's rescale + clip riding on it (thresholds far away: nothing changes,
+        # as in the model-order step); same bytes as the plain backward, against backward + a 4 B/elem norm read
+        ms_c = timer.time(lambda i: ops.bn_act_backward_clipped(d[i], x[i], mean, var, scale, bias, su, bu, "leaky",
+                                                                1e30, 1e30), 10, rotate=rot)
+        add("bn_bwd_clipped(leaky)", "%dx%dx%d^2" % (N, c, s), (16 if one_launch else 20) * e, ms_c,
+            "rescale + clip decided in the backward's own first pass; plain backward %.4f ms" % ms_b)
         if one_launch:
             # both conventions in the row: the bytes this launch moves (frac above) and the 12 / 20 B per
             # element that the three-launch form moves, which is the figure the per-kernel bar was written for
-            for row, per_elem, ms in ((rows[-2], 12, ms_f), (rows[-1], 20, ms_b)):
+            for row, per_elem, ms in ((rows[-3], 12, ms_f), (rows[-2], 20, ms_b)):
                 row["three_launch_bytes_MB"] = round(per_elem * e / 1e6, 1)
                 row["frac_of_peak_at_three_launch_bytes"] = round(per_elem * e / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 3)
         bn_ms[(c, s)] = (ms_f, ms_b, count)
@@ -582,10 +604,12 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
     # ---- linear bias epilogue of the three head convs at batch 16
     for c, s in wl.YOLOV3_HEAD_CONV_SHAPES:
         e = N * c * s * s
-        x = randn(N, c, s, s)
+        rot = rotation_for(4 * e)
+        xs = [randn(N, c, s, s) for _ in range(rot)]
         bias = randn(c)
-        ms = timer.time(lambda i: ops.bias_act_forward(x, x, bias, "linear"), 20)
-        add("bias_fwd(linear)", "%dx%dx%d^2" % (N, c, s), 8 * e, ms, "in place, cache resident")
+        ms = timer.time(lambda i: ops.bias_act_forward(xs[i], xs[i], bias, "linear"), 20, rotate=rot)
+        add("bias_fwd(linear)", "%dx%dx%d^2" % (N, c, s), 8 * e, ms, "in place")
+        del xs
         bn_ms[("head", s)] = (ms, 0.0, 1)
     # ---- Adam (config 4): 61.9M parameters, 10 steps
     P = wl.YOLOV3_PARAMS
@@ -1109,7 +1133,7 @@ def main():
     if not args.no_extras:
         copy_of_size = same_bytes_copier(torch, ops, timer)
         for sh in shapes:
-            rot = rotation_for(8 * sh["elems"], cap=3)
+            rot = rotation_for(8 * sh["elems"])
             xs = [sh["x"]] + [torch.randn_like(sh["x"]) for _ in range(rot - 1)]
             ys = [sh["y"]] + [torch.empty_like(sh["y"]) for _ in range(rot - 1)]
             for act in EPILOGUE_ACTS:
@@ -1117,7 +1141,7 @@ def main():
                 r = dict(act=act, shape="%dx%dx%d^2" % (EPILOGUE_BATCH, sh["c"], sh["s"]), ms=round(ms, 4),
                          ms_min=round(timer.last_min, 4), GBps=round(8.0 * sh["elems"] / (ms * 1e-3) / 1e9, 1))
                 if r["GBps"] < 0.70 * HBM_PEAK_GBS:      # as for the other kernels' rows under the bar
-                    c_ms = copy_of_size(8 * sh["elems"], cap=3)
+                    c_ms = copy_of_size(8 * sh["elems"])
                     r["copy_same_bytes_ms"] = round(c_ms, 4)
                     r["vs_copy"] = round(c_ms / ms, 3)
                 per_shape.append(r)

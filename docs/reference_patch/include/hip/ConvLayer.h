@@ -68,18 +68,24 @@ inline void ConvLayer<Device::HIP>::forward(const V& input)
 template<>
 inline void ConvLayer<Device::HIP>::backward(const V& input, V* grad)
 {
-    Layer<Device::HIP>::backward(input, grad);
+    // Layer<D>::backward (include/Layer.h:385-397) is scaleTensor(delta_) and clipDelta(): a read of delta_
+    // for its norm, a rewrite when the norm is beyond the threshold, a clamp.  The clipped entry points take
+    // the two thresholds and fold all of it into the backward's own first pass over delta_, so the base
+    // class's method is not called here.
+    const float threshold = this->gradientRescaling_ ? this->gradientThreshold_ : 0.0f;
+    const float clip = this->gradientClipping_ ? this->gradientClipValue_ : 0.0f;
     const int spatial = this->outHeight() * this->outWidth();
     const int act = activation_->type();
     if (batchNorm_) {
         // activation gradient, batch-norm backward and `delta_.copy(xNorm_)` in one call, in place on delta_
-        PX_HIP_CHECK(pxh_bn_act_backward(this->delta_.data(), x_.data(), nullptr, mean_.data(), var_.data(),
-                                         scales_.data(), biases_.data(), scaleUpdates_.data(), biasUpdates_.data(),
-                                         nullptr, nullptr, this->batch(), filters_, spatial, act, nullptr, 0, nullptr));
+        PX_HIP_CHECK(pxh_bn_act_backward_clipped(this->delta_.data(), x_.data(), nullptr, mean_.data(), var_.data(),
+                                                 scales_.data(), biases_.data(), scaleUpdates_.data(),
+                                                 biasUpdates_.data(), nullptr, nullptr, this->batch(), filters_, spatial,
+                                                 act, threshold, clip, nullptr, nullptr, 0, nullptr));
     } else {
         const float* pre = act != LINEAR ? this->preActivation_.data() : nullptr;
-        PX_HIP_CHECK(pxh_bias_act_backward(this->delta_.data(), pre, biasUpdates_.data(), this->batch(), filters_,
-                                           spatial, act, nullptr, 0, nullptr));
+        PX_HIP_CHECK(pxh_bias_act_backward_clipped(this->delta_.data(), pre, biasUpdates_.data(), this->batch(), filters_,
+                                                   spatial, act, threshold, clip, nullptr, nullptr, 0, nullptr));
     }
     convolveBackward(input, weights_, this->delta_, weightUpdates_, grad);
 }

@@ -156,6 +156,34 @@ int pxh_bias_act_backward(float* delta, const float* pre_activation, float* bias
                           int batch, int channels, int spatial, int activation,
                           void* workspace, size_t workspace_bytes, void* stream);
 
+/* Layer::backward's gradient rescale + clip (include/Layer.h:385-397: scaleTensor when the norm of
+ * the delta is beyond `threshold`, then clipDelta at +-`clip`; either is off when its figure is <= 0)
+ * and the ConvLayer::backward epilogue that follows it (include/ConvLayer.h:238-252) in one call:
+ * the same results as pxh_rescale_clip(delta, ...) followed by pxh_bn_act_backward(delta, ...), but the
+ * delta is not read once just for its norm -- the first pass of the backward carries the sum of
+ * squares and the largest magnitude, the decision is taken on the device, and when nothing has to
+ * change (the usual case with the shipped thresholds) the call costs what pxh_bn_act_backward
+ * costs plus launches that leave at once.  *norm_out (nullable, device) receives the norm of the
+ * delta as it came.  A shape that takes the one-launch backward rescales a channel that was not
+ * clamped by linearity (dx and the updates times the factor) instead of rounding factor * delta
+ * first: within rounding of the two-call sequence, not bit-identical to it.
+ * workspace: pxh_bn_clipped_workspace_bytes(), or NULL for the library's. */
+size_t pxh_bn_clipped_workspace_bytes(int batch, int channels, int spatial);
+int pxh_bn_act_backward_clipped(float* delta, const float* x, const float* pre_activation,
+                                const float* mean, const float* var, const float* scale, const float* bias,
+                                float* scale_updates, float* bias_updates, float* mean_delta, float* var_delta,
+                                int batch, int channels, int spatial, int activation,
+                                float threshold, float clip, float* norm_out,
+                                void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same in front of pxh_bias_act_backward (a ConvLayer without batch_normalize): delta is left
+ * rescaled, clamped and multiplied by act'(pre), as the two calls leave it; with a linear activation
+ * and nothing to change it is only read.  workspace: pxh_bn_clipped_workspace_bytes(). */
+int pxh_bias_act_backward_clipped(float* delta, const float* pre_activation, float* bias_updates,
+                                  int batch, int channels, int spatial, int activation,
+                                  float threshold, float clip, float* norm_out,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------
  * Stand-alone pieces with the reference's own signatures.
  * ---------------------------------------------------------------------- */

@@ -31,6 +31,8 @@ SIGNATURES = {
     "pxh_bn_stats": [P, P, P, I, I, I, P, Z, P],
     "pxh_bn_act_backward": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, P, Z, P],
     "pxh_bias_act_backward": [P, P, P, I, I, I, I, P, Z, P],
+    "pxh_bn_act_backward_clipped": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, F, F, P, P, Z, P],
+    "pxh_bias_act_backward_clipped": [P, P, P, I, I, I, I, F, F, P, P, Z, P],
     "pxh_activate": [I, P, Z, P],
     "pxh_gradient": [I, P, Z, P, P],
     "pxh_add_bias": [P, P, I, I, I, P],
@@ -81,6 +83,7 @@ _OTHER_RETURNS = {
     "pxh_abi_version": (I, []),
     "pxh_bn_workspace_bytes": (Z, [I, I, I]),
     "pxh_bn_folded_bytes": (Z, [I]),
+    "pxh_bn_clipped_workspace_bytes": (Z, [I, I, I]),
     "pxh_rescale_workspace_bytes": (Z, []),
     "pxh_norm_groups_bytes": (Z, [Z]),
     "pxh_rescale_multi_workspace_bytes": (Z, []),

@@ -178,12 +178,14 @@ __device__ __forceinline__ float act_apply(float x)
     if constexpr (ACT == PXH_LEAKY) return x > 0.0f ? x : 0.1f * x;
     else if constexpr (ACT == PXH_LINEAR) return x;
     else if constexpr (ACT == PXH_LOGGY) return 2.0f / (1.0f + expf(-x)) - 1.0f;
-    // logistic and swish: the accurate exp, then a hardware reciprocal (1 ulp) in place of the division
-    else if constexpr (ACT == PXH_LOGISTIC) return __builtin_amdgcn_rcpf(1.0f + expf(-x));
+    // logistic and swish: the short exp (a unit in the last place, as for mish) and a hardware reciprocal
+    // (1 ulp) in place of the division: the sum 1 + e absorbs e's last place wherever the result is not
+    // already proportional to 1 / e
+    else if constexpr (ACT == PXH_LOGISTIC) return __builtin_amdgcn_rcpf(1.0f + exp_by_exp2(-x));
     else if constexpr (ACT == PXH_MISH) return mish_apply<false>(x);
     else if constexpr (ACT == PXH_RELU) return x > 0.0f ? x : 0.0f;
     else if constexpr (ACT == PXH_SOFTPLUS) return softplus_apply(x);
-    else if constexpr (ACT == PXH_SWISH) return x * __builtin_amdgcn_rcpf(1.0f + expf(-1.0f * x));
+    else if constexpr (ACT == PXH_SWISH) return x * __builtin_amdgcn_rcpf(1.0f + exp_by_exp2(-1.0f * x));
     else return tanhf(x);
 }
 
@@ -330,6 +332,38 @@ __device__ __forceinline__ double block_sum(double v, double* slots)
         for (int w = 0; w < kBlock / kWave; ++w) total += slots[w];
     }
     return total;
+}
+
+// ---------------------------------------------------------------- gradient rescale + clip: the decision
+// Layer::backward's two helpers on a delta (include/Layer.h:385-397, 479-499 of the reference):
+//   norm = |x|_2;  if (norm > 0 && norm > threshold) x *= threshold / norm;  then clamp to +-clip.
+// From the sum of squares and the largest magnitude: the norm, the factor, and whether anything can
+// change -- a factor other than 1, or a value that the clamp would move.  The scaled magnitudes are at
+// most fl(factor * peak) (rounding is monotonic), so a peak within the clamp after scaling means no
+// element changes; a NaN anywhere (it shows in the sum) or an infinite peak keeps the rewrite, which
+// treats them as the CPU loop does.
+struct RescalePlan {
+    float norm, factor;
+    bool work;
+};
+
+__device__ __forceinline__ RescalePlan plan_from_totals(double total, float peak, float threshold, float clip)
+{
+    RescalePlan plan;
+    plan.norm = static_cast<float>(sqrt(total));
+    plan.factor = 1.0f;
+    if (threshold > 0.0f && plan.norm > 0.0f && plan.norm > threshold) plan.factor = threshold / plan.norm;
+    const bool clamps = clip > 0.0f && (!(plan.factor * peak <= clip) || total != total);
+    plan.work = plan.factor != 1.0f || clamps;
+    return plan;
+}
+
+// One value through the two helpers.
+__device__ __forceinline__ float rescaled_clipped(float x, float factor, float clip)
+{
+    float t = factor == 1.0f ? x : factor * x;
+    if (clip > 0.0f) t = fminf(clip, fmaxf(-clip, t));
+    return t;
 }
 
 inline unsigned grid_for(size_t items, size_t per_block)

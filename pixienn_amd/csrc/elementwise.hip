@@ -457,17 +457,8 @@ __global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(const float* x, s
     sumsq_walk<V, NT>(x, n_vec, blockIdx.x, gridDim.x, partial + blockIdx.x);
 }
 
-// The plan of the rewrite, formed by every workgroup for itself from the same partials in the same
-// order (so all arrive at the same one): the norm, the factor, and whether anything can change -- a
-// factor other than 1, or a value that the clamp would move.  The scaled magnitudes are at most
-// fl(factor * peak) (rounding is monotonic), so a peak within the clamp after scaling means no
-// element changes; a NaN anywhere (it shows in the sum) or an infinite peak keeps the rewrite, which
-// treats them as the CPU loop does.
-struct RescalePlan {
-    float norm, factor;
-    bool work;
-};
-
+// The plan of the rewrite (plan_from_totals), formed by every workgroup for itself from the same
+// partials in the same order, so all arrive at the same one.
 __device__ __forceinline__ RescalePlan rescale_plan(const double2* partial, int partials, float threshold, float clip)
 {
     __shared__ double sums[kBlock / kWave];
@@ -495,13 +486,7 @@ __device__ __forceinline__ RescalePlan rescale_plan(const double2* partial, int 
         total += sums[w];
         peak = fmaxf(peak, static_cast<float>(tops[w]));
     }
-    RescalePlan plan;
-    plan.norm = static_cast<float>(sqrt(total));
-    plan.factor = 1.0f;
-    if (threshold > 0.0f && plan.norm > 0.0f && plan.norm > threshold) plan.factor = threshold / plan.norm;
-    const bool clamps = clip > 0.0f && (!(plan.factor * peak <= clip) || total != total);
-    plan.work = plan.factor != 1.0f || clamps;
-    return plan;
+    return plan_from_totals(total, peak, threshold, clip);
 }
 
 // x = clamp(factor * x); leaves without touching the tensor when there is nothing to do.  The grid
@@ -521,11 +506,7 @@ __device__ __forceinline__ void rescale_walk(float* x, size_t n_vec, const doubl
         Pack<V> v[kNormLoads];
         const auto rewrite = [&](Pack<V>& p) {
 #pragma unroll
-            for (int k = 0; k < V; ++k) {
-                float t = factor == 1.0f ? p.v[k] : factor * p.v[k];
-                if (clip > 0.0f) t = fminf(clip, fmaxf(-clip, t));
-                p.v[k] = t;
-            }
+            for (int k = 0; k < V; ++k) p.v[k] = rescaled_clipped(p.v[k], factor, clip);
         };
         if (base + per_step <= n_vec) {      // a whole step: no branch between its loads
 #pragma unroll

@@ -418,6 +418,65 @@ __global__ __launch_bounds__(kBlock) void bn_stats_finish_kernel(const float* x,
     }
 }
 
+// ---- Layer::backward's gradient rescale + clip in front of the backward sums ----
+// The layer's backward opens with the norm of its delta, a rescale when the norm is beyond a threshold
+// and a clamp (include/Layer.h:385-397, 479-499), and only then runs the activation gradient and the
+// batch-norm backward (include/ConvLayer.h:238-252).  The first pass over the delta can carry the sum
+// of squares and the largest magnitude along with its own sums, which saves the read that the norm
+// alone would cost; the decision is formed on the device (ClipPlan) and the later kernels follow it.
+struct __attribute__((aligned(16))) ClipPlan {
+    float norm, factor, clip;
+    int work;       // 0: no value of the delta changes
+};
+
+// The plan from `count` partial (sum of squares, largest magnitude) pairs, added in an order that
+// depends on THREADS alone: every workgroup that forms it arrives at the same one.  All THREADS
+// threads of the workgroup call it; every one returns the plan.
+template<int THREADS>
+__device__ __forceinline__ ClipPlan clip_plan_from(const double2* part, int count, float threshold, float clip)
+{
+    __shared__ double plan_sums[THREADS / kWave];
+    __shared__ float plan_tops[THREADS / kWave];
+    double s = 0.0;
+    float top = 0.0f;
+    for (int j = threadIdx.x; j < count; j += THREADS) {
+        const double2 p = part[j];
+        s += p.x;
+        top = fmaxf(top, static_cast<float>(p.y));
+    }
+    s = wave_sum(s);
+    top = wave_max(top);
+    __syncthreads();       // the arrays may still be read from an earlier call
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        plan_sums[threadIdx.x / kWave] = s;
+        plan_tops[threadIdx.x / kWave] = top;
+    }
+    __syncthreads();
+    double total = 0.0;
+    float peak = 0.0f;
+#pragma unroll
+    for (int w = 0; w < THREADS / kWave; ++w) {
+        total += plan_sums[w];
+        peak = fmaxf(peak, plan_tops[w]);
+    }
+    const RescalePlan r = plan_from_totals(total, peak, threshold, clip);
+    return ClipPlan{ r.norm, r.factor, clip, r.work ? 1 : 0 };
+}
+
+// What the clipped forms add to a launch: where the first pass leaves its norm partials, and the
+// plan that the finish kernel of the first pass writes and everything after it reads.
+struct ClipArgs {
+    double2* norm_partial;     // [workgroups of the first pass]
+    ClipPlan* plan;
+    float threshold, clip;
+    float* norm_out;           // nullable
+};
+
+// The passes of a backward:  kPlain -- no rescale + clip in front;  kFirst -- the sums as if nothing
+// had to change, plus the norm partials;  kRedo -- after the plan: leaves at once when nothing has to
+// change, else forms the sums again from the rescaled and clamped delta.
+enum { kPlain = 0, kFirst = 1, kRedo = 2 };
+
 // ---- backward sums: A = sum d', B = sum d' * (x - mean), d' = delta * act'(pre) ----
 struct BackwardArgs {
     float* delta;
@@ -429,16 +488,32 @@ struct BackwardArgs {
     const float* bias;
 };
 
-template<int ACT, bool BN, bool WRITE, int V, bool NT>
-__global__ __launch_bounds__(kBlock) void bwd_partial_kernel(BackwardArgs a, ReduceGeom g, double2* partial)
+// WRITE (the bias-only layer, which has no dx pass): d' goes back into delta.  With kFirst nothing is
+// written (the delta is still needed as it came); with kRedo the pass also runs, writing, when nothing
+// has to change but the activation has a gradient to apply.
+template<int ACT, bool BN, bool WRITE, int V, bool NT, int MODE = kPlain>
+__global__ __launch_bounds__(kBlock) void bwd_partial_kernel(BackwardArgs a, ReduceGeom g, double2* partial,
+                                                             ClipArgs clip = ClipArgs{})
 {
+    static_assert(!(WRITE && MODE == kFirst), "the first pass of a clipped backward leaves the delta alone");
     __shared__ double slots[2][kBlock / kWave];
+    [[maybe_unused]] float factor = 1.0f, limit = 0.0f;
+    [[maybe_unused]] bool changes = false;
+    if constexpr (MODE == kRedo) {
+        const ClipPlan plan = *clip.plan;
+        changes = plan.work != 0;
+        if (!changes && !(WRITE && ACT != PXH_LINEAR)) return;
+        factor = changes ? plan.factor : 1.0f;
+        limit = changes ? plan.clip : 0.0f;
+    }
     uint32_t c, j;
     g.by_blocks.divmod(blockIdx.x, c, j);
     FoldCoef k;
     if constexpr (BN) k = make_coef(a.mean[c], a.var[c], a.scale[c], a.bias[c]);
     const bool recompute = BN && a.pre == nullptr;
     double sa = 0.0, sb = 0.0;
+    [[maybe_unused]] double sq = 0.0;
+    [[maybe_unused]] float peak = 0.0f;
     for_each_item(g, c, j, [&](size_t base, int seg0, int seg1, int lane) {
         constexpr int kLoads = kSeg / (kWave * V);
         Pack<V> d[kLoads], xv[kLoads], pv[kLoads];
@@ -454,6 +529,7 @@ __global__ __launch_bounds__(kBlock) void bwd_partial_kernel(BackwardArgs a, Red
             }
         }
         float fa = 0.0f, fb = 0.0f;
+        [[maybe_unused]] float fq = 0.0f;
 #pragma unroll
         for (int u = 0; u < kLoads; ++u) {
             const int off = seg0 + (u * kWave + lane) * V;
@@ -461,6 +537,14 @@ __global__ __launch_bounds__(kBlock) void bwd_partial_kernel(BackwardArgs a, Red
 #pragma unroll
                 for (int q = 0; q < V; ++q) {
                     float dv = d[u].v[q];
+                    if constexpr (MODE == kFirst) {
+                        fq += dv * dv;
+                        peak = fmaxf(peak, fabsf(dv));
+                    }
+                    if constexpr (MODE == kRedo) {
+                        dv = rescaled_clipped(dv, factor, limit);
+                        d[u].v[q] = dv;
+                    }
                     if constexpr (ACT != PXH_LINEAR) {
                         float pre;
                         if (recompute) pre = affine(normalize(xv[u].v[q], k), k);
@@ -471,15 +555,31 @@ __global__ __launch_bounds__(kBlock) void bwd_partial_kernel(BackwardArgs a, Red
                     fa += dv;
                     if constexpr (BN) fb += dv * (xv[u].v[q] - k.mean);
                 }
-                if constexpr (WRITE && ACT != PXH_LINEAR) st<V, NT>(a.delta, base + off, d[u]);
+                if constexpr (WRITE && (ACT != PXH_LINEAR || MODE == kRedo)) {
+                    if (ACT != PXH_LINEAR || changes) st<V, NT>(a.delta, base + off, d[u]);
+                }
             }
         }
         sa += static_cast<double>(fa);
         sb += static_cast<double>(fb);
+        if constexpr (MODE == kFirst) sq += static_cast<double>(fq);
     });
     const double ta = block_sum(sa, slots[0]);
     const double tb = block_sum(sb, slots[1]);
     if (threadIdx.x == 0) partial[blockIdx.x] = make_double2(ta, tb);
+    if constexpr (MODE == kFirst) {
+        __shared__ float peaks[kBlock / kWave];
+        const double tq = block_sum(sq, slots[0]);      // synchronises before it reuses the slots
+        peak = wave_max(peak);
+        if ((threadIdx.x & (kWave - 1)) == 0) peaks[threadIdx.x / kWave] = peak;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float top = peaks[0];
+#pragma unroll
+            for (int w = 1; w < kBlock / kWave; ++w) top = fmaxf(top, peaks[w]);
+            clip.norm_partial[blockIdx.x] = make_double2(tq, static_cast<double>(top));
+        }
+    }
 }
 
 // Per-channel constants of the dx pass, produced by the finish kernel (64 bytes).
@@ -524,13 +624,27 @@ __device__ __forceinline__ DxCoef finish_backward(double sa, double sb, int c, i
     return k;
 }
 
-template<bool BN>
+// kFirst: every workgroup forms the plan from all norm partials of the first pass (the same additions
+// in the same order everywhere), the first one records it, and the channels are finished only when
+// nothing has to change; kRedo: finishes them from the second pass's sums when something had to.
+template<bool BN, int MODE = kPlain>
 __global__ __launch_bounds__(kBlock) void bwd_finish_kernel(const double2* partial, int channels, int blocks, int count,
                                                             const float* mean, const float* var, const float* scale,
                                                             const float* bias, float* scale_updates,
                                                             float* bias_updates, float* mean_delta, float* var_delta,
-                                                            DxCoef* coef)
+                                                            DxCoef* coef, ClipArgs clip = ClipArgs{})
 {
+    if constexpr (MODE == kFirst) {
+        const ClipPlan plan = clip_plan_from<kBlock>(clip.norm_partial, channels * blocks, clip.threshold, clip.clip);
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            *clip.plan = plan;
+            if (clip.norm_out) *clip.norm_out = plan.norm;
+        }
+        if (plan.work) return;
+    }
+    if constexpr (MODE == kRedo) {
+        if (!clip.plan->work) return;
+    }
     const int lane = threadIdx.x & (kWave - 1);
     const int c = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
     if (c >= channels) return;
@@ -557,7 +671,21 @@ struct DxArgs {
     FastDiv by_spatial;
     FastDiv by_channels;
     uint32_t total;
+    const ClipPlan* plan;     // the clipped form: the delta goes through the plan's rescale + clamp first
 };
+
+// The delta as the sums saw it: through the plan when there is one and it changes anything.
+template<bool CLIPPED, int V>
+__device__ __forceinline__ void apply_plan(const DxArgs& a, Pack<V>& d)
+{
+    if constexpr (CLIPPED) {
+        const ClipPlan plan = *a.plan;
+        if (plan.work) {
+#pragma unroll
+            for (int k = 0; k < V; ++k) d.v[k] = rescaled_clipped(d.v[k], plan.factor, plan.clip);
+        }
+    }
+}
 
 template<int ACT>
 __device__ __forceinline__ float dx_value(float d, float x, float pre_in, bool recompute, const DxCoef& k)
@@ -574,7 +702,7 @@ __device__ __forceinline__ float dx_value(float d, float x, float pre_in, bool r
     return static_cast<float>(v);
 }
 
-template<int ACT, bool NT>
+template<int ACT, bool NT, bool CLIPPED = false>
 __global__ __launch_bounds__(kBlock) void bn_dx_kernel(DxArgs a)
 {
     const uint32_t e = (blockIdx.x * static_cast<uint32_t>(kBlock) + threadIdx.x) * 4;
@@ -595,6 +723,7 @@ __global__ __launch_bounds__(kBlock) void bn_dx_kernel(DxArgs a)
             pin.v[k] = (ok && ACT != PXH_LINEAR && !recompute) ? a.pre[e + k] : 0.0f;
         }
     }
+    apply_plan<CLIPPED, 4>(a, din);
     const uint32_t hw = a.by_spatial.d;
     uint32_t plane, r, q, c;
     a.by_spatial.divmod(e, plane, r);
@@ -644,7 +773,7 @@ __global__ __launch_bounds__(kBlock) void bn_dx_kernel(DxArgs a)
     }
 }
 
-template<int ACT>
+template<int ACT, bool CLIPPED = false>
 __global__ __launch_bounds__(kBlock) void bn_dx_scalar_kernel(DxArgs a)
 {
     const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
@@ -654,7 +783,10 @@ __global__ __launch_bounds__(kBlock) void bn_dx_scalar_kernel(DxArgs a)
     a.by_channels.divmod(plane, q, c);
     const bool recompute = a.pre == nullptr;
     const float pre = (ACT != PXH_LINEAR && !recompute) ? a.pre[e] : 0.0f;
-    a.delta[e] = dx_value<ACT>(a.delta[e], a.x[e], pre, recompute, a.coef[c]);
+    Pack<1> d;
+    d.v[0] = a.delta[e];
+    apply_plan<CLIPPED, 1>(a, d);
+    a.delta[e] = dx_value<ACT>(d.v[0], a.x[e], pre, recompute, a.coef[c]);
 }
 
 // ---------------------------------------------------------------- channel-resident training passes
@@ -686,6 +818,39 @@ __device__ __forceinline__ void resident_sum2(double& a, double& b, double (*slo
     }
     a = ta;
     b = tb;
+}
+
+// The same for three sums and a maximum (the first pass of a clipped backward).
+__device__ __forceinline__ void resident_sum3_max(double& a, double& b, double& q, float& top,
+                                                  double (*slots)[kResidentWaves], float* tops)
+{
+    a = wave_sum(a);
+    b = wave_sum(b);
+    q = wave_sum(q);
+    top = wave_max(top);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) {
+        slots[0][wave] = a;
+        slots[1][wave] = b;
+        slots[2][wave] = q;
+        tops[wave] = top;
+    }
+    __syncthreads();
+    double ta = 0.0, tb = 0.0, tq = 0.0;
+    float tt = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kResidentWaves; ++w) {
+        ta += slots[0][w];
+        tb += slots[1][w];
+        tq += slots[2][w];
+        tt = fmaxf(tt, tops[w]);
+    }
+    a = ta;
+    b = tb;
+    q = tq;
+    top = tt;
 }
 
 struct ResidentGeom {
@@ -815,21 +980,89 @@ struct ResidentBwdArgs {
     float* mean_delta;   // nullable
     float* var_delta;    // nullable
     ResidentGeom g;
+    // the clipped form (else null): per channel the (sum of squares, largest magnitude) of its delta,
+    // the two sums it was finished with, and whether it was finished at all
+    double2* channel_norm;
+    double2* channel_sums;
+    int* channel_done;
+    ClipArgs clip;
 };
+
+// A channel that was finished with the sums (sa, sb) of its unscaled delta, after the plan turned out
+// to rescale by `factor` (and its clamp to move nothing in this channel): everything the backward left
+// is linear in the delta, so the accumulated updates get the difference and the two per-channel deltas
+// are formed again.  The dx values are scaled by the caller.
+__device__ __forceinline__ void rescale_finished_channel(double sa, double sb, double factor, int c, const float* var,
+                                                         const float* scale, float* scale_updates,
+                                                         float* bias_updates, float* mean_delta, float* var_delta)
+{
+    bias_updates[c] += static_cast<float>((factor - 1.0) * sa);
+    const float v = var[c];
+    const float s = scale[c];
+    const double denom = sqrt(static_cast<double>(v)) + static_cast<double>(kEps);
+    scale_updates[c] += static_cast<float>((factor - 1.0) * sb / denom);
+    const float sum_dd = static_cast<float>(factor * sa * static_cast<double>(s));
+    const float sum_ddx = static_cast<float>(factor * sb * static_cast<double>(s));
+    const float ve = v + kEps;
+    if (mean_delta) mean_delta[c] = static_cast<float>(static_cast<double>(sum_dd) * (-1. / static_cast<double>(sqrtf(ve))));
+    if (var_delta) var_delta[c] = sum_ddx * (-.5f * powf(ve, -3.0f / 2.0f));
+}
 
 // The workgroup keeps d' = delta * act'(pre) (registers + LDS); x is read again for the dx phase
 // (it is still in the cache: one channel's slice is a few hundred KB).
-template<int ACT, int V, int R, int L>
+//
+// With Layer::backward's rescale + clip in front (kFirst, then a kRedo launch of the same shape): the
+// first launch also adds up the channel's squares and finds its largest magnitude.  The norm that
+// decides the rescale is the whole tensor's and is not known inside the launch; but the factor is at
+// most 1, so a channel whose own largest magnitude is within the clamp cannot be clamped whatever the
+// factor turns out to be, and all it leaves is linear in its delta: it is finished as if nothing had
+// to change.  A channel above the clamp is left untouched.  The second launch forms the plan from the
+// per-channel figures and leaves at once in the usual case (nothing to change); else a finished
+// channel is scaled by the factor, and an untouched one runs the whole pass on the rescaled and
+// clamped delta.
+template<int ACT, int V, int R, int L, int MODE = kPlain>
 __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(ResidentBwdArgs a)
 {
     extern __shared__ __align__(16) float resident_lds[];
-    __shared__ double slots[2][kResidentWaves];
+    __shared__ double slots[MODE == kFirst ? 3 : 2][kResidentWaves];
     __shared__ DxCoef shared_coef;
     const uint32_t c = blockIdx.x;
+    [[maybe_unused]] float factor = 1.0f, limit = 0.0f;
+    if constexpr (MODE == kRedo) {
+        const ClipPlan plan = clip_plan_from<kResidentThreads>(a.channel_norm, a.g.channels, a.clip.threshold,
+                                                               a.clip.clip);
+        if (c == 0 && threadIdx.x == 0) {
+            *a.clip.plan = plan;
+            if (a.clip.norm_out) *a.clip.norm_out = plan.norm;
+        }
+        if (a.channel_done[c]) {
+            if (plan.factor == 1.0f) return;
+#pragma unroll 1
+            for (int r = 0; r < R + L; ++r) {
+                const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+                if (e < a.g.per_channel) {
+                    const size_t where = a.g.at(c, e);
+                    Pack<V> t = ld<V, true>(a.b.delta, where);
+#pragma unroll
+                    for (int q = 0; q < V; ++q) t.v[q] = plan.factor * t.v[q];
+                    st<V, true>(a.b.delta, where, t);
+                }
+            }
+            if (threadIdx.x == 0) {
+                const double2 sums = a.channel_sums[c];
+                rescale_finished_channel(sums.x, sums.y, static_cast<double>(plan.factor), c, a.b.var, a.b.scale,
+                                         a.scale_updates, a.bias_updates, a.mean_delta, a.var_delta);
+            }
+            return;
+        }
+        factor = plan.factor;
+        limit = plan.clip;
+    }
     const FoldCoef k = make_coef(a.b.mean[c], a.b.var[c], a.b.scale[c], a.b.bias[c]);
     const bool recompute = a.b.pre == nullptr;
     Pack<V> d[R];
     float fa = 0.0f, fb = 0.0f;
+    [[maybe_unused]] float fq = 0.0f, peak = 0.0f;
     // Two shapes of the same two passes.  The large form (part of the slice in LDS) is bound by its
     // loads and takes them in groups with no branch in between; the small form does more arithmetic
     // per byte than it waits, and is fastest when a step past the end of the slice is skipped outright.
@@ -845,17 +1078,25 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
         const uint32_t e = element(r);
         return a.g.at(c, e < a.g.per_channel ? e : 0u);
     };
+    // one value of the delta on its way to d': the norm's share of it first (kFirst), or the plan's
+    // rescale + clamp (kRedo), then the activation's gradient
+    const auto prepared = [&](float t, float pre, bool valid) {
+        if constexpr (MODE == kFirst) {
+            fq += valid ? t * t : 0.0f;
+            peak = fmaxf(peak, valid ? fabsf(t) : 0.0f);
+        }
+        if constexpr (MODE == kRedo) t = rescaled_clipped(t, factor, limit);
+        if constexpr (ACT != PXH_LINEAR) t = t * act_grad<ACT>(pre);
+        return t;
+    };
     if constexpr (L > 0) {
-        // delta * f'(pre) in dv, and the step's share of the two sums
+        // delta * f'(pre) in dv, and the step's share of the sums
         const auto take = [&](int r, Pack<V>& dv, const Pack<V>& xv, const Pack<V>& pv) {
             const bool valid = element(r) < a.g.per_channel;
 #pragma unroll
             for (int q = 0; q < V; ++q) {
-                float t = dv.v[q];
-                if constexpr (ACT != PXH_LINEAR) {
-                    t = t * act_grad<ACT>(pv.v[q]);
-                    dv.v[q] = t;
-                }
+                const float t = prepared(dv.v[q], ACT != PXH_LINEAR ? pv.v[q] : 0.0f, valid);
+                dv.v[q] = t;
                 fa += valid ? t : 0.0f;
                 fb += valid ? t * (xv.v[q] - k.mean) : 0.0f;
             }
@@ -894,7 +1135,8 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
             // puts the additions off to the end of the pass and keeps every group's values until then),
             // and the next group's loads stay behind this one's arithmetic -- either would need more
             // registers than a lane has.
-            asm volatile("" : "+v"(fa), "+v"(fb));
+            if constexpr (MODE == kFirst) asm volatile("" : "+v"(fa), "+v"(fb), "+v"(fq), "+v"(peak));
+            else asm volatile("" : "+v"(fa), "+v"(fb));
             __builtin_amdgcn_sched_barrier(0);
         }
     } else {
@@ -911,14 +1153,13 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
                 }
 #pragma unroll
                 for (int q = 0; q < V; ++q) {
-                    float t = dv.v[q];
+                    float pre = 0.0f;
                     if constexpr (ACT != PXH_LINEAR) {
-                        float pre;
                         if (recompute) pre = affine(normalize(xv.v[q], k), k);
                         else pre = pv.v[q];
-                        t = t * act_grad<ACT>(pre);
-                        dv.v[q] = t;
                     }
+                    const float t = prepared(dv.v[q], pre, true);
+                    dv.v[q] = t;
                     fa += t;
                     fb += t * (xv.v[q] - k.mean);
                 }
@@ -928,11 +1169,33 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
         }
     }
     double sa = static_cast<double>(fa), sb = static_cast<double>(fb);
-    resident_sum2(sa, sb, slots);
-    if (threadIdx.x == 0)
-        shared_coef = finish_backward<true>(sa, sb, c, static_cast<int>(a.g.per_channel), a.b.mean, a.b.var, a.b.scale,
-                                            a.b.bias, a.scale_updates, a.bias_updates, a.mean_delta, a.var_delta);
-    __syncthreads();
+    if constexpr (MODE == kFirst) {
+        __shared__ float tops[kResidentWaves];
+        __shared__ int finished;
+        double sq = static_cast<double>(fq);
+        resident_sum3_max(sa, sb, sq, peak, slots, tops);
+        if (threadIdx.x == 0) {
+            const float lim = a.clip.clip;
+            const bool within = !(lim > 0.0f) || (peak <= lim && sq == sq);
+            a.channel_norm[c] = make_double2(sq, static_cast<double>(peak));
+            a.channel_sums[c] = make_double2(sa, sb);
+            a.channel_done[c] = within ? 1 : 0;
+            finished = within ? 1 : 0;
+            if (within)
+                shared_coef = finish_backward<true>(sa, sb, c, static_cast<int>(a.g.per_channel), a.b.mean, a.b.var,
+                                                    a.b.scale, a.b.bias, a.scale_updates, a.bias_updates,
+                                                    a.mean_delta, a.var_delta);
+        }
+        __syncthreads();
+        if (!finished) return;
+    } else {
+        resident_sum2(sa, sb, slots);
+        if (threadIdx.x == 0)
+            shared_coef = finish_backward<true>(sa, sb, c, static_cast<int>(a.g.per_channel), a.b.mean, a.b.var,
+                                                a.b.scale, a.b.bias, a.scale_updates, a.bias_updates, a.mean_delta,
+                                                a.var_delta);
+        __syncthreads();
+    }
     const DxCoef kd = shared_coef;
     if constexpr (L > 0) {
         asm volatile("" : "+v"(lane));
@@ -1028,6 +1291,43 @@ size_t workspace_bytes(int batch, int channels, int spatial)
 void* coef_region(void* ws, int batch, int channels, int spatial)
 {
     return static_cast<char*>(ws) + partial_bytes(batch, channels, spatial);
+}
+
+// The clipped backward: [partial sums][per-channel constants][norm partials][plan] for the three
+// launches, [per-channel norm figures][per-channel sums][per-channel flags][plan] for the one-launch form.
+constexpr size_t align256(size_t b) { return (b + 255) & ~static_cast<size_t>(255); }
+
+struct ClippedRegions {
+    double2* partial;
+    DxCoef* coef;
+    double2* norm_partial;
+    double2* channel_norm;
+    double2* channel_sums;
+    int* channel_done;
+    ClipPlan* plan;
+};
+
+size_t clipped_workspace_bytes(int batch, int channels, int spatial)
+{
+    const size_t c = static_cast<size_t>(channels);
+    const size_t three = 2 * partial_bytes(batch, channels, spatial) + align256(c * sizeof(DxCoef)) + 256;
+    const size_t one = 2 * align256(c * sizeof(double2)) + align256(c * sizeof(int)) + 256;
+    return three > one ? three : one;
+}
+
+ClippedRegions clipped_regions(void* ws, int batch, int channels, int spatial)
+{
+    const size_t c = static_cast<size_t>(channels);
+    char* base = static_cast<char*>(ws);
+    ClippedRegions r;
+    r.partial = reinterpret_cast<double2*>(base);
+    r.coef = reinterpret_cast<DxCoef*>(base + partial_bytes(batch, channels, spatial));
+    r.norm_partial = reinterpret_cast<double2*>(reinterpret_cast<char*>(r.coef) + align256(c * sizeof(DxCoef)));
+    r.channel_norm = reinterpret_cast<double2*>(base);
+    r.channel_sums = reinterpret_cast<double2*>(base + align256(c * sizeof(double2)));
+    r.channel_done = reinterpret_cast<int*>(base + 2 * align256(c * sizeof(double2)));
+    r.plan = reinterpret_cast<ClipPlan*>(base + clipped_workspace_bytes(batch, channels, spatial) - 256);
+    return r;
 }
 
 // A tensor this large cannot stay in the last-level cache between two passes over it.
@@ -1236,121 +1536,235 @@ int pxh_bn_train_act_forward_static(const float* x, float* y, float* pre_activat
         stream);
 }
 
-int pxh_bn_act_backward(float* delta, const float* x, const float* pre_activation, const float* mean,
-                        const float* var, const float* scale, const float* bias, float* scale_updates,
-                        float* bias_updates, float* mean_delta, float* var_delta, int batch, int channels,
-                        int spatial, int activation, void* workspace, size_t workspace_bytes_given, void* stream)
+// The rescale + clip in front of a backward, or none.
+struct ClipSpec {
+    bool on;
+    float threshold, clip;
+    float* norm_out;
+};
+
+static int bn_backward(const char* who, float* delta, const float* x, const float* pre_activation, const float* mean,
+                       const float* var, const float* scale, const float* bias, float* scale_updates,
+                       float* bias_updates, float* mean_delta, float* var_delta, int batch, int channels, int spatial,
+                       int activation, const ClipSpec& cs, void* workspace, size_t workspace_bytes_given, void* stream)
 {
     if (!delta || !x || !mean || !var || !scale || !bias || !scale_updates || !bias_updates)
-        return fail_invalid("pxh_bn_act_backward: null pointer");
+        return fail_invalid("%s: null pointer", who);
     uint32_t total;
-    int rc = check_shape("pxh_bn_act_backward", batch, channels, spatial, &total);
+    int rc = check_shape(who, batch, channels, spatial, &total);
     if (rc) return rc;
     hipStream_t s = as_stream(stream);
-    {
-        const bool rvec = spatial % 4 == 0 && aligned16(delta) && aligned16(x) && aligned16(pre_activation);
-        const int per_thread = resident_vectors(batch, channels, spatial, rvec);
-        if (per_thread) {
-            const ResidentBwdArgs r{ BackwardArgs{ delta, x, pre_activation, mean, var, scale, bias }, scale_updates,
-                                     bias_updates, mean_delta, var_delta, resident_geom(batch, channels, spatial) };
-            const dim3 grid(channels), block(kResidentThreads);
-            int large_lds_rc = PXH_OK;
-            const bool known = dispatch_activation(activation, [&]<int ACT>() {
-                if (per_thread > kResidentVectors) {
-                    auto kernel = bn_resident_bwd_kernel<ACT, 4, kResidentLargeRegs, kResidentLargeLds>;
-                    large_lds_rc = allow_large_lds(reinterpret_cast<const void*>(kernel));
-                    if (large_lds_rc == PXH_OK)
-                        hipLaunchKernelGGL(kernel, grid, block, kResidentLargeLdsBytes, s, r);
-                } else if (rvec) {
-                    hipLaunchKernelGGL((bn_resident_bwd_kernel<ACT, 4, kResidentVectors, 0>), grid, block, 0, s, r);
-                } else {
-                    hipLaunchKernelGGL((bn_resident_bwd_kernel<ACT, 1, kResidentVectors, 0>), grid, block, 0, s, r);
-                }
-            });
-            if (!known) return fail_invalid("pxh_bn_act_backward: unknown activation %d", activation);
-            if (large_lds_rc) return large_lds_rc;
-            return check_launch("pxh_bn_act_backward");
-        }
+    const bool rvec = spatial % 4 == 0 && aligned16(delta) && aligned16(x) && aligned16(pre_activation);
+    const int per_thread = resident_vectors(batch, channels, spatial, rvec);
+    void* ws = nullptr;
+    ClippedRegions region{};
+    ClipArgs clip{};
+    if (cs.on) {
+        rc = resolve_workspace(workspace, workspace_bytes_given, clipped_workspace_bytes(batch, channels, spatial), &ws, s);
+        if (rc) return rc;
+        region = clipped_regions(ws, batch, channels, spatial);
+        clip = ClipArgs{ region.norm_partial, region.plan, cs.threshold, cs.clip, cs.norm_out };
     }
-    void* ws;
-    rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws, as_stream(stream));
-    if (rc) return rc;
+    if (per_thread) {
+        const ResidentBwdArgs r{ BackwardArgs{ delta, x, pre_activation, mean, var, scale, bias }, scale_updates,
+                                 bias_updates, mean_delta, var_delta, resident_geom(batch, channels, spatial),
+                                 region.channel_norm, region.channel_sums, region.channel_done, clip };
+        const dim3 grid(channels), block(kResidentThreads);
+        int large_lds_rc = PXH_OK;
+        const auto launch = [&]<int ACT, int MODE>() {
+            if (per_thread > kResidentVectors) {
+                auto kernel = bn_resident_bwd_kernel<ACT, 4, kResidentLargeRegs, kResidentLargeLds, MODE>;
+                large_lds_rc = allow_large_lds(reinterpret_cast<const void*>(kernel));
+                if (large_lds_rc == PXH_OK) hipLaunchKernelGGL(kernel, grid, block, kResidentLargeLdsBytes, s, r);
+            } else if (rvec) {
+                hipLaunchKernelGGL((bn_resident_bwd_kernel<ACT, 4, kResidentVectors, 0, MODE>), grid, block, 0, s, r);
+            } else {
+                hipLaunchKernelGGL((bn_resident_bwd_kernel<ACT, 1, kResidentVectors, 0, MODE>), grid, block, 0, s, r);
+            }
+        };
+        const bool known = dispatch_activation(activation, [&]<int ACT>() {
+            if (!cs.on) {
+                launch.template operator()<ACT, kPlain>();
+            } else {
+                launch.template operator()<ACT, kFirst>();
+                if (large_lds_rc == PXH_OK) launch.template operator()<ACT, kRedo>();
+            }
+        });
+        if (!known) return fail_invalid("%s: unknown activation %d", who, activation);
+        if (large_lds_rc) return large_lds_rc;
+        return check_launch(who);
+    }
+    if (!cs.on) {
+        rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws, s);
+        if (rc) return rc;
+    }
     const ReduceGeom g = make_geom(batch, channels, spatial);
     double2* partial = static_cast<double2*>(ws);
     DxCoef* coef = static_cast<DxCoef*>(coef_region(ws, batch, channels, spatial));
 
     BackwardArgs b{ delta, x, pre_activation, mean, var, scale, bias };
-    const bool vec = spatial % 4 == 0 && aligned16(delta) && aligned16(x) && aligned16(pre_activation);
+    const bool vec = rvec;
     const int tensors = pre_activation ? 3 : 2;
     const bool nt = vec && streams_past_cache(total, tensors);
     const dim3 grid(static_cast<unsigned>(channels) * g.blocks);
-    const bool known = dispatch_activation(activation, [&]<int ACT>() {
+    const dim3 finish_grid(grid_for(channels, kBlock / kWave));
+    const auto sums = [&]<int ACT, int MODE>() {
         if (nt) {
-            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 4, true>), grid, dim3(kBlock), 0, s, b, g, partial);
+            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 4, true, MODE>), grid, dim3(kBlock), 0, s, b, g,
+                               partial, clip);
         } else if (vec) {
-            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 4, false>), grid, dim3(kBlock), 0, s, b, g, partial);
+            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 4, false, MODE>), grid, dim3(kBlock), 0, s, b, g,
+                               partial, clip);
         } else {
-            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 1, false>), grid, dim3(kBlock), 0, s, b, g, partial);
+            hipLaunchKernelGGL((bwd_partial_kernel<ACT, true, false, 1, false, MODE>), grid, dim3(kBlock), 0, s, b, g,
+                               partial, clip);
+        }
+    };
+    const auto finish = [&]<int MODE>() {
+        hipLaunchKernelGGL((bwd_finish_kernel<true, MODE>), finish_grid, dim3(kBlock), 0, s, partial, channels, g.blocks,
+                           batch * spatial, mean, var, scale, bias, scale_updates, bias_updates, mean_delta, var_delta,
+                           coef, clip);
+    };
+    const bool known = dispatch_activation(activation, [&]<int ACT>() {
+        if (!cs.on) {
+            sums.template operator()<ACT, kPlain>();
+        } else {
+            sums.template operator()<ACT, kFirst>();
+            finish.template operator()<kFirst>();
+            sums.template operator()<ACT, kRedo>();
         }
     });
-    if (!known) return fail_invalid("pxh_bn_act_backward: unknown activation %d", activation);
+    if (!known) return fail_invalid("%s: unknown activation %d", who, activation);
     rc = check_launch("bn_backward_partial");
     if (rc) return rc;
-    hipLaunchKernelGGL((bwd_finish_kernel<true>), dim3(grid_for(channels, kBlock / kWave)), dim3(kBlock), 0, s, partial,
-                       channels, g.blocks, batch * spatial, mean, var, scale, bias, scale_updates, bias_updates,
-                       mean_delta, var_delta, coef);
+    if (cs.on) finish.template operator()<kRedo>();
+    else finish.template operator()<kPlain>();
     rc = check_launch("bn_backward_finish");
     if (rc) return rc;
 
     DxArgs d{};
     d.delta = delta; d.x = x; d.pre = pre_activation; d.coef = coef;
     d.by_spatial = FastDiv(spatial); d.by_channels = FastDiv(channels); d.total = total;
+    d.plan = cs.on ? region.plan : nullptr;
     const bool dx_vec = aligned16(delta) && aligned16(x) && aligned16(pre_activation);
     const bool dx_nt = streams_past_cache(total, tensors + 1);
-    dispatch_activation(activation, [&]<int ACT>() {
+    const auto dx = [&]<int ACT, bool CLIPPED>() {
         if (dx_vec) {
             const dim3 dx_grid(grid_for(total, static_cast<size_t>(kBlock) * 4));
-            if (dx_nt) hipLaunchKernelGGL((bn_dx_kernel<ACT, true>), dx_grid, dim3(kBlock), 0, s, d);
-            else hipLaunchKernelGGL((bn_dx_kernel<ACT, false>), dx_grid, dim3(kBlock), 0, s, d);
+            if (dx_nt) hipLaunchKernelGGL((bn_dx_kernel<ACT, true, CLIPPED>), dx_grid, dim3(kBlock), 0, s, d);
+            else hipLaunchKernelGGL((bn_dx_kernel<ACT, false, CLIPPED>), dx_grid, dim3(kBlock), 0, s, d);
         } else {
-            hipLaunchKernelGGL((bn_dx_scalar_kernel<ACT>), dim3(grid_for(total, kBlock)), dim3(kBlock), 0, s, d);
+            hipLaunchKernelGGL((bn_dx_scalar_kernel<ACT, CLIPPED>), dim3(grid_for(total, kBlock)), dim3(kBlock), 0, s, d);
         }
+    };
+    dispatch_activation(activation, [&]<int ACT>() {
+        if (cs.on) dx.template operator()<ACT, true>();
+        else dx.template operator()<ACT, false>();
     });
     return check_launch("bn_backward_dx");
+}
+
+int pxh_bn_act_backward(float* delta, const float* x, const float* pre_activation, const float* mean,
+                        const float* var, const float* scale, const float* bias, float* scale_updates,
+                        float* bias_updates, float* mean_delta, float* var_delta, int batch, int channels,
+                        int spatial, int activation, void* workspace, size_t workspace_bytes_given, void* stream)
+{
+    return bn_backward("pxh_bn_act_backward", delta, x, pre_activation, mean, var, scale, bias, scale_updates,
+                       bias_updates, mean_delta, var_delta, batch, channels, spatial, activation,
+                       ClipSpec{ false, 0.0f, 0.0f, nullptr }, workspace, workspace_bytes_given, stream);
+}
+
+size_t pxh_bn_clipped_workspace_bytes(int batch, int channels, int spatial)
+{
+    if (batch <= 0 || channels <= 0 || spatial <= 0) return 0;
+    return clipped_workspace_bytes(batch, channels, spatial);
+}
+
+int pxh_bn_act_backward_clipped(float* delta, const float* x, const float* pre_activation, const float* mean,
+                                const float* var, const float* scale, const float* bias, float* scale_updates,
+                                float* bias_updates, float* mean_delta, float* var_delta, int batch, int channels,
+                                int spatial, int activation, float threshold, float clip, float* norm_out,
+                                void* workspace, size_t workspace_bytes_given, void* stream)
+{
+    return bn_backward("pxh_bn_act_backward_clipped", delta, x, pre_activation, mean, var, scale, bias, scale_updates,
+                       bias_updates, mean_delta, var_delta, batch, channels, spatial, activation,
+                       ClipSpec{ true, threshold, clip, norm_out }, workspace, workspace_bytes_given, stream);
+}
+
+static int bias_backward(const char* who, float* delta, const float* pre_activation, float* bias_updates, int batch,
+                         int channels, int spatial, int activation, const ClipSpec& cs, void* workspace,
+                         size_t workspace_bytes_given, void* stream)
+{
+    if (!delta || !bias_updates) return fail_invalid("%s: null pointer", who);
+    if (activation != PXH_LINEAR && !pre_activation)
+        return fail_invalid("%s: pre_activation is required for a non-linear activation", who);
+    uint32_t total;
+    int rc = check_shape(who, batch, channels, spatial, &total);
+    if (rc) return rc;
+    hipStream_t s = as_stream(stream);
+    void* ws;
+    rc = resolve_workspace(workspace, workspace_bytes_given,
+                           cs.on ? clipped_workspace_bytes(batch, channels, spatial)
+                                 : workspace_bytes(batch, channels, spatial), &ws, s);
+    if (rc) return rc;
+    const ReduceGeom g = make_geom(batch, channels, spatial);
+    double2* partial = static_cast<double2*>(ws);
+    ClipArgs clip{};
+    if (cs.on) {
+        const ClippedRegions region = clipped_regions(ws, batch, channels, spatial);
+        clip = ClipArgs{ region.norm_partial, region.plan, cs.threshold, cs.clip, cs.norm_out };
+    }
+    BackwardArgs b{ delta, nullptr, pre_activation, nullptr, nullptr, nullptr, nullptr };
+    const bool vec = spatial % 4 == 0 && aligned16(delta) && aligned16(pre_activation);
+    const dim3 grid(static_cast<unsigned>(channels) * g.blocks);
+    const dim3 finish_grid(grid_for(channels, kBlock / kWave));
+    const auto sums = [&]<int ACT, bool WRITE, int MODE>() {
+        if (vec) {
+            hipLaunchKernelGGL((bwd_partial_kernel<ACT, false, WRITE, 4, false, MODE>), grid, dim3(kBlock), 0, s, b, g,
+                               partial, clip);
+        } else {
+            hipLaunchKernelGGL((bwd_partial_kernel<ACT, false, WRITE, 1, false, MODE>), grid, dim3(kBlock), 0, s, b, g,
+                               partial, clip);
+        }
+    };
+    const auto finish = [&]<int MODE>() {
+        hipLaunchKernelGGL((bwd_finish_kernel<false, MODE>), finish_grid, dim3(kBlock), 0, s, partial, channels,
+                           g.blocks, batch * spatial, nullptr, nullptr, nullptr, nullptr, nullptr, bias_updates, nullptr,
+                           nullptr, nullptr, clip);
+    };
+    const bool known = dispatch_activation(activation, [&]<int ACT>() {
+        if (!cs.on) {
+            sums.template operator()<ACT, true, kPlain>();
+        } else {
+            // the sums of the delta as it came (nothing written), the plan, then the pass that writes:
+            // it leaves at once when nothing changes and the activation is linear
+            sums.template operator()<ACT, false, kFirst>();
+            finish.template operator()<kFirst>();
+            sums.template operator()<ACT, true, kRedo>();
+        }
+    });
+    if (!known) return fail_invalid("%s: unknown activation %d", who, activation);
+    rc = check_launch("bias_backward_partial");
+    if (rc) return rc;
+    if (cs.on) finish.template operator()<kRedo>();
+    else finish.template operator()<kPlain>();
+    return check_launch("bias_backward_finish");
 }
 
 int pxh_bias_act_backward(float* delta, const float* pre_activation, float* bias_updates, int batch, int channels,
                           int spatial, int activation, void* workspace, size_t workspace_bytes_given, void* stream)
 {
-    if (!delta || !bias_updates) return fail_invalid("pxh_bias_act_backward: null pointer");
-    if (activation != PXH_LINEAR && !pre_activation)
-        return fail_invalid("pxh_bias_act_backward: pre_activation is required for a non-linear activation");
-    uint32_t total;
-    int rc = check_shape("pxh_bias_act_backward", batch, channels, spatial, &total);
-    if (rc) return rc;
-    void* ws;
-    rc = resolve_workspace(workspace, workspace_bytes_given, workspace_bytes(batch, channels, spatial), &ws, as_stream(stream));
-    if (rc) return rc;
-    hipStream_t s = as_stream(stream);
-    const ReduceGeom g = make_geom(batch, channels, spatial);
-    double2* partial = static_cast<double2*>(ws);
-    BackwardArgs b{ delta, nullptr, pre_activation, nullptr, nullptr, nullptr, nullptr };
-    const bool vec = spatial % 4 == 0 && aligned16(delta) && aligned16(pre_activation);
-    const dim3 grid(static_cast<unsigned>(channels) * g.blocks);
-    const bool known = dispatch_activation(activation, [&]<int ACT>() {
-        if (vec) {
-            hipLaunchKernelGGL((bwd_partial_kernel<ACT, false, true, 4, false>), grid, dim3(kBlock), 0, s, b, g, partial);
-        } else {
-            hipLaunchKernelGGL((bwd_partial_kernel<ACT, false, true, 1, false>), grid, dim3(kBlock), 0, s, b, g, partial);
-        }
-    });
-    if (!known) return fail_invalid("pxh_bias_act_backward: unknown activation %d", activation);
-    rc = check_launch("bias_backward_partial");
-    if (rc) return rc;
-    hipLaunchKernelGGL((bwd_finish_kernel<false>), dim3(grid_for(channels, kBlock / kWave)), dim3(kBlock), 0, s,
-                       partial, channels, g.blocks, batch * spatial, nullptr, nullptr, nullptr, nullptr, nullptr,
-                       bias_updates, nullptr, nullptr, nullptr);
-    return check_launch("bias_backward_finish");
+    return bias_backward("pxh_bias_act_backward", delta, pre_activation, bias_updates, batch, channels, spatial,
+                         activation, ClipSpec{ false, 0.0f, 0.0f, nullptr }, workspace, workspace_bytes_given, stream);
+}
+
+int pxh_bias_act_backward_clipped(float* delta, const float* pre_activation, float* bias_updates, int batch,
+                                  int channels, int spatial, int activation, float threshold, float clip,
+                                  float* norm_out, void* workspace, size_t workspace_bytes_given, void* stream)
+{
+    return bias_backward("pxh_bias_act_backward_clipped", delta, pre_activation, bias_updates, batch, channels,
+                         spatial, activation, ClipSpec{ true, threshold, clip, norm_out }, workspace,
+                         workspace_bytes_given, stream);
 }
 
 int pxh_backward_bias(float* bias_updates, const float* delta, int batch, int n, int size, void* workspace,

@@ -154,6 +154,8 @@ public:
     // layers that leave one do so on request ("leaves_norm"), and whoever asks vouches for that.
     void noteNormGroups(const float* tensor, const float* groups) { normGroups_[tensor] = groups; }
 
+    bool hasNormGroups(const float* tensor) const { return normGroups_.count(tensor) != 0; }
+
     const float* takeNormGroups(const float* tensor)
     {
         const auto it = normGroups_.find(tensor);

@@ -45,7 +45,10 @@ public:
         const int oh = props.get<int>("out_height", height());
         const int ow = props.get<int>("out_width", width());
         setOutput(filters_, oh, ow);
-        if (training()) context.reserveWorkspace(pxh_bn_workspace_bytes(batch(), filters_, oh * ow));
+        if (training()) {
+            context.reserveWorkspace(pxh_bn_workspace_bytes(batch(), filters_, oh * ow));
+            context.reserveWorkspace(pxh_bn_clipped_workspace_bytes(batch(), filters_, oh * ow));
+        }
 
         // The weights live here so that update() and the optimizer sidecar cover the whole layer;
         // their values and gradients are the delegated convolution's business ("weights": count).
@@ -128,22 +131,43 @@ public:
 
     // Needs the conv result of the matching forward to be unchanged (it is re-read instead of
     // keeping saved copies of it, of x_hat and of the pre-activation).
+    //
+    // Layer::backward's rescale + clip of delta_ rides on the first pass of the epilogue's backward (one
+    // call, the delta is not read for its norm alone) -- unless the kernel that wrote delta_ last left its
+    // norm behind, in which case the helpers need no read of it anyway and run as in every other layer.
     void backward(const V& input, V* grad) override
     {
-        Layer::backward(input, grad);
         PX_CHECK(training() && x_ != nullptr, "ConvLayer: backward without a training forward");
+        const float threshold = rescaleThreshold(), clip = clipValue();
+        const bool fused = (threshold > 0.0f || clip > 0.0f) && !context().hasNormGroups(delta_.data());
+        if (!fused) Layer::backward(input, grad);
         const int spatial = outHeight() * outWidth();
         if (batchNorm_) {
-            PX_HIP_CHECK(pxh_bn_act_backward(delta_.data(), x_, nullptr, mean_.data(), var_.data(), scales_.data(),
-                                             biases_.data(), scaleUpdates_.data(), biasUpdates_.data(), nullptr,
-                                             nullptr, batch(), filters_, spatial, activation_, context().workspace(),
-                                             context().workspaceBytes(), stream()));
+            if (fused)
+                PX_HIP_CHECK(pxh_bn_act_backward_clipped(delta_.data(), x_, nullptr, mean_.data(), var_.data(),
+                                                         scales_.data(), biases_.data(), scaleUpdates_.data(),
+                                                         biasUpdates_.data(), nullptr, nullptr, batch(), filters_,
+                                                         spatial, activation_, threshold, clip, nullptr,
+                                                         context().workspace(), context().workspaceBytes(), stream()));
+            else
+                PX_HIP_CHECK(pxh_bn_act_backward(delta_.data(), x_, nullptr, mean_.data(), var_.data(),
+                                                 scales_.data(), biases_.data(), scaleUpdates_.data(),
+                                                 biasUpdates_.data(), nullptr, nullptr, batch(), filters_, spatial,
+                                                 activation_, context().workspace(), context().workspaceBytes(),
+                                                 stream()));
         } else {
             // pre-activation = x + bias is not kept either; the linear head convs need none
             preActivation(spatial);
-            PX_HIP_CHECK(pxh_bias_act_backward(delta_.data(), pre_.empty() ? nullptr : pre_.data(),
-                                               biasUpdates_.data(), batch(), filters_, spatial, activation_,
-                                               context().workspace(), context().workspaceBytes(), stream()));
+            const float* pre = pre_.empty() ? nullptr : pre_.data();
+            if (fused)
+                PX_HIP_CHECK(pxh_bias_act_backward_clipped(delta_.data(), pre, biasUpdates_.data(), batch(), filters_,
+                                                           spatial, activation_, threshold, clip, nullptr,
+                                                           context().workspace(), context().workspaceBytes(),
+                                                           stream()));
+            else
+                PX_HIP_CHECK(pxh_bias_act_backward(delta_.data(), pre, biasUpdates_.data(), batch(), filters_, spatial,
+                                                   activation_, context().workspace(), context().workspaceBytes(),
+                                                   stream()));
         }
         if (convolveBackward_) {
             convolveBackward_(input, delta_, grad);

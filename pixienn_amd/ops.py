@@ -121,6 +121,30 @@ def bias_act_backward(delta, pre_activation, bias_updates, activation, workspace
     return delta
 
 
+def bn_act_backward_clipped(delta, x, mean, var, scale, bias, scale_updates, bias_updates, activation, threshold,
+                            clip, norm_out=None, pre_activation=None, mean_delta=None, var_delta=None, workspace=None):
+    """rescale_clip(delta, threshold, clip) then bn_act_backward, without the read of delta for its norm."""
+    _chk_all(delta, x, mean, var, scale, bias, scale_updates, bias_updates, pre_activation, mean_delta, var_delta,
+             norm_out)
+    n, c, s = _nchw(delta)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("pxh_bn_act_backward_clipped", ptr(delta), ptr(x), ptr(pre_activation), ptr(mean), ptr(var), ptr(scale),
+         ptr(bias), ptr(scale_updates), ptr(bias_updates), ptr(mean_delta), ptr(var_delta), n, c, s,
+         act_id(activation), float(threshold), float(clip), ptr(norm_out), ptr(workspace), wb, _stream())
+    return delta
+
+
+def bias_act_backward_clipped(delta, pre_activation, bias_updates, activation, threshold, clip, norm_out=None,
+                              workspace=None):
+    """rescale_clip(delta, threshold, clip) then bias_act_backward, without the read of delta for its norm."""
+    _chk_all(delta, pre_activation, bias_updates, norm_out)
+    n, c, s = _nchw(delta)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("pxh_bias_act_backward_clipped", ptr(delta), ptr(pre_activation), ptr(bias_updates), n, c, s,
+         act_id(activation), float(threshold), float(clip), ptr(norm_out), ptr(workspace), wb, _stream())
+    return delta
+
+
 # ---------------------------------------------------------------- stand-alone pieces
 def activate(activation, x):
     _chk(x)

@@ -338,6 +338,33 @@ def test_shortcut_closed_form(oracle):
     assert oracle.shortcut(1, 4, 4, 1, a, 2, 4, 1, 1.0, 1.0, out) != 0
 
 
+def test_route_is_channel_concat_and_slice_add(oracle):
+    """Route has no reference test: forward is np.concatenate over channels (include/RouteLayer.h:91-113),
+    backward adds each source's channel slice of the route's delta to that source's delta (115-137)."""
+    rng = np.random.default_rng(33)
+    N, H, W = 3, 4, 5
+    a = rng.standard_normal((N, 2, H, W)).astype(F)
+    b = rng.standard_normal((N, 5, H, W)).astype(F)
+    c = rng.standard_normal((N, 1, H, W)).astype(F)
+    out = np.full((N, 8, H, W), np.nan, F)
+    at = 0
+    for src in (a, b, c):
+        oracle.route_forward(src, out, at)
+        at += src[0].size
+    assert np.array_equal(out, np.concatenate([a, b, c], axis=1))
+    d = rng.standard_normal(out.shape).astype(F)
+    da0, db0, dc0 = (rng.standard_normal(t.shape).astype(F) for t in (a, b, c))
+    da, db, dc = da0.copy(), db0.copy(), dc0.copy()
+    at = 0
+    for dst in (da, db, dc):
+        oracle.route_backward(d, dst, at)
+        at += dst[0].size
+    assert np.array_equal(da, da0 + d[:, 0:2]) and np.array_equal(db, db0 + d[:, 2:7])
+    assert np.array_equal(dc, dc0 + d[:, 7:8])
+    # a transposed or batch-strided mistake would show with N > 1 and unequal source sizes; so would "=" for "+="
+    assert not np.array_equal(db, d[:, 2:7])
+
+
 # ---------------------------------------------------------------- boxes
 def test_darkbox_kats(oracle, kats):
     c = kats["darkbox"]
