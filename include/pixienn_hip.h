@@ -164,9 +164,11 @@ int pxh_bias_act_backward(float* delta, const float* pre_activation, float* bias
  * squares and the largest magnitude, the decision is taken on the device, and when nothing has to
  * change (the usual case with the shipped thresholds) the call costs what pxh_bn_act_backward
  * costs plus launches that leave at once.  *norm_out (nullable, device) receives the norm of the
- * delta as it came.  A shape that takes the one-launch backward rescales a channel that was not
- * clamped by linearity (dx and the updates times the factor) instead of rounding factor * delta
- * first: within rounding of the two-call sequence, not bit-identical to it.
+ * delta as it came.  When the delta is rescaled and the clamp moves nothing (in the one-launch
+ * backward: nothing in a channel), the sums are not formed again from the rounded factor * delta: they
+ * are linear in the delta and are multiplied by the factor instead -- within rounding of the two-call
+ * sequence, not bit-identical to it.  When nothing changes the results are those of
+ * pxh_bn_act_backward to the bit.
  * workspace: pxh_bn_clipped_workspace_bytes(), or NULL for the library's. */
 size_t pxh_bn_clipped_workspace_bytes(int batch, int channels, int spatial);
 int pxh_bn_act_backward_clipped(float* delta, const float* x, const float* pre_activation,

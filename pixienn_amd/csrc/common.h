@@ -344,7 +344,8 @@ __device__ __forceinline__ double block_sum(double v, double* slots)
 // treats them as the CPU loop does.
 struct RescalePlan {
     float norm, factor;
-    bool work;
+    bool work;      // some value changes
+    bool clamps;    // ... and not by the factor alone: the clamp may move one
 };
 
 __device__ __forceinline__ RescalePlan plan_from_totals(double total, float peak, float threshold, float clip)
@@ -353,8 +354,8 @@ __device__ __forceinline__ RescalePlan plan_from_totals(double total, float peak
     plan.norm = static_cast<float>(sqrt(total));
     plan.factor = 1.0f;
     if (threshold > 0.0f && plan.norm > 0.0f && plan.norm > threshold) plan.factor = threshold / plan.norm;
-    const bool clamps = clip > 0.0f && (!(plan.factor * peak <= clip) || total != total);
-    plan.work = plan.factor != 1.0f || clamps;
+    plan.clamps = clip > 0.0f && (!(plan.factor * peak <= clip) || total != total);
+    plan.work = plan.factor != 1.0f || plan.clamps;
     return plan;
 }
 

@@ -426,8 +426,9 @@ __global__ __launch_bounds__(kBlock) void bn_stats_finish_kernel(const float* x,
 // alone would cost; the decision is formed on the device (ClipPlan) and the later kernels follow it.
 struct __attribute__((aligned(16))) ClipPlan {
     float norm, factor, clip;
-    int work;       // 0: no value of the delta changes
+    int work;       // 0: no value of the delta changes; kChanges: some do; | kClamps: and the clamp may move one
 };
+enum { kChanges = 1, kClamps = 2 };
 
 // The plan from `count` partial (sum of squares, largest magnitude) pairs, added in an order that
 // depends on THREADS alone: every workgroup that forms it arrives at the same one.  All THREADS
@@ -439,10 +440,22 @@ __device__ __forceinline__ ClipPlan clip_plan_from(const double2* part, int coun
     __shared__ float plan_tops[THREADS / kWave];
     double s = 0.0;
     float top = 0.0f;
-    for (int j = threadIdx.x; j < count; j += THREADS) {
-        const double2 p = part[j];
-        s += p.x;
-        top = fmaxf(top, static_cast<float>(p.y));
+    // kPlanLoads partials per thread and round, their loads in flight together (one after the other each
+    // costs a trip to memory: 45 of them per thread at 16 x 32 x 608^2 with 256 threads)
+    constexpr int kPlanLoads = 8;
+    for (int base = 0; base < count; base += THREADS * kPlanLoads) {
+        double2 p[kPlanLoads];
+#pragma unroll
+        for (int u = 0; u < kPlanLoads; ++u) {
+            const int j = base + u * THREADS + static_cast<int>(threadIdx.x);
+            p[u] = part[j < count ? j : 0];
+        }
+#pragma unroll
+        for (int u = 0; u < kPlanLoads; ++u) {
+            const bool valid = base + u * THREADS + static_cast<int>(threadIdx.x) < count;
+            s += valid ? p[u].x : 0.0;
+            top = fmaxf(top, valid ? static_cast<float>(p[u].y) : 0.0f);
+        }
     }
     s = wave_sum(s);
     top = wave_max(top);
@@ -460,7 +473,7 @@ __device__ __forceinline__ ClipPlan clip_plan_from(const double2* part, int coun
         peak = fmaxf(peak, plan_tops[w]);
     }
     const RescalePlan r = plan_from_totals(total, peak, threshold, clip);
-    return ClipPlan{ r.norm, r.factor, clip, r.work ? 1 : 0 };
+    return ClipPlan{ r.norm, r.factor, clip, (r.work ? kChanges : 0) | (r.clamps ? kClamps : 0) };
 }
 
 // What the clipped forms add to a launch: where the first pass leaves its norm partials, and the
@@ -472,9 +485,15 @@ struct ClipArgs {
     float* norm_out;           // nullable
 };
 
+constexpr int kPlanThreads = 1024;
+constexpr int kRedoWorkgroups = 256;      // of the one-launch form's second launch
+
 // The passes of a backward:  kPlain -- no rescale + clip in front;  kFirst -- the sums as if nothing
-// had to change, plus the norm partials;  kRedo -- after the plan: leaves at once when nothing has to
-// change, else forms the sums again from the rescaled and clamped delta.
+// had to change, plus the norm partials;  kRedo -- after the plan: leaves at once when the sums of the
+// first pass still serve, else forms them again from the rescaled and clamped delta.
+// The sums of the first pass serve when nothing changes, and for the batch-norm backward also when the
+// delta is only rescaled (the clamp moves no value): they are linear in the delta, so the finish
+// kernel multiplies them by the factor and the dx pass applies the factor to the delta it reads.
 enum { kPlain = 0, kFirst = 1, kRedo = 2 };
 
 // ---- backward sums: A = sum d', B = sum d' * (x - mean), d' = delta * act'(pre) ----
@@ -502,7 +521,10 @@ __global__ __launch_bounds__(kBlock) void bwd_partial_kernel(BackwardArgs a, Red
     if constexpr (MODE == kRedo) {
         const ClipPlan plan = *clip.plan;
         changes = plan.work != 0;
-        if (!changes && !(WRITE && ACT != PXH_LINEAR)) return;
+        // the writing form has the delta to rewrite whenever a value changes; the other only its sums to
+        // form again, and only when the clamp takes part
+        const bool again = WRITE ? changes : (plan.work & kClamps) != 0;
+        if (!again && !(WRITE && ACT != PXH_LINEAR)) return;
         factor = changes ? plan.factor : 1.0f;
         limit = changes ? plan.clip : 0.0f;
     }
@@ -624,29 +646,35 @@ __device__ __forceinline__ DxCoef finish_backward(double sa, double sb, int c, i
     return k;
 }
 
-// kFirst: every workgroup forms the plan from all norm partials of the first pass (the same additions
-// in the same order everywhere), the first one records it, and the channels are finished only when
-// nothing has to change; kRedo: finishes them from the second pass's sums when something had to.
-template<bool BN, int MODE = kPlain>
-__global__ __launch_bounds__(kBlock) void bwd_finish_kernel(const double2* partial, int channels, int blocks, int count,
-                                                            const float* mean, const float* var, const float* scale,
-                                                            const float* bias, float* scale_updates,
-                                                            float* bias_updates, float* mean_delta, float* var_delta,
-                                                            DxCoef* coef, ClipArgs clip = ClipArgs{})
+// kFirst (workgroups of kPlanThreads): every workgroup forms the plan from all norm partials of the first
+// pass (the same additions in the same order everywhere), the first one records it, and the channels
+// are finished only when nothing has to change; kRedo: finishes them from the second pass's sums when
+// something had to.
+template<bool BN, int MODE = kPlain, int THREADS = kBlock>
+__global__ __launch_bounds__(THREADS) void bwd_finish_kernel(const double2* partial, int channels, int blocks, int count,
+                                                             const float* mean, const float* var, const float* scale,
+                                                             const float* bias, float* scale_updates,
+                                                             float* bias_updates, float* mean_delta, float* var_delta,
+                                                             DxCoef* coef, ClipArgs clip = ClipArgs{})
 {
+    [[maybe_unused]] double sums_factor = 1.0;
     if constexpr (MODE == kFirst) {
-        const ClipPlan plan = clip_plan_from<kBlock>(clip.norm_partial, channels * blocks, clip.threshold, clip.clip);
+        const ClipPlan plan = clip_plan_from<THREADS>(clip.norm_partial, channels * blocks, clip.threshold, clip.clip);
         if (blockIdx.x == 0 && threadIdx.x == 0) {
             *clip.plan = plan;
             if (clip.norm_out) *clip.norm_out = plan.norm;
         }
-        if (plan.work) return;
+        // with batch-norm the sums serve unless the clamp takes part; a bias-only layer's delta is
+        // rewritten by the second pass whenever a value changes, and that pass leaves exact sums
+        if (BN ? (plan.work & kClamps) != 0 : plan.work != 0) return;
+        sums_factor = static_cast<double>(plan.factor);
     }
     if constexpr (MODE == kRedo) {
-        if (!clip.plan->work) return;
+        const int work = clip.plan->work;
+        if (BN ? (work & kClamps) == 0 : work == 0) return;
     }
     const int lane = threadIdx.x & (kWave - 1);
-    const int c = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+    const int c = blockIdx.x * (THREADS / kWave) + threadIdx.x / kWave;
     if (c >= channels) return;
     double sa = 0.0, sb = 0.0;
     for (int j = lane; j < blocks; j += kWave) {
@@ -656,6 +684,12 @@ __global__ __launch_bounds__(kBlock) void bwd_finish_kernel(const double2* parti
     }
     sa = wave_sum(sa);
     sb = wave_sum(sb);
+    if constexpr (MODE == kFirst) {
+        if (sums_factor != 1.0) {
+            sa *= sums_factor;
+            sb *= sums_factor;
+        }
+    }
     if (lane == 0) {
         const DxCoef k = finish_backward<BN>(sa, sb, c, count, mean, var, scale, bias, scale_updates, bias_updates,
                                              mean_delta, var_delta);
@@ -840,7 +874,8 @@ __device__ __forceinline__ void resident_sum3_max(double& a, double& b, double& 
     __syncthreads();
     double ta = 0.0, tb = 0.0, tq = 0.0;
     float tt = 0.0f;
-#pragma unroll
+    // four waves' figures at a time: all sixteen at once are 100 registers of LDS loads in flight
+#pragma unroll 4
     for (int w = 0; w < kResidentWaves; ++w) {
         ta += slots[0][w];
         tb += slots[1][w];
@@ -1016,48 +1051,42 @@ __device__ __forceinline__ void rescale_finished_channel(double sa, double sb, d
 // decides the rescale is the whole tensor's and is not known inside the launch; but the factor is at
 // most 1, so a channel whose own largest magnitude is within the clamp cannot be clamped whatever the
 // factor turns out to be, and all it leaves is linear in its delta: it is finished as if nothing had
-// to change.  A channel above the clamp is left untouched.  The second launch forms the plan from the
+// to change.  A channel above the clamp is left untouched.  The kRedo launch forms the plan from the
 // per-channel figures and leaves at once in the usual case (nothing to change); else a finished
 // channel is scaled by the factor, and an untouched one runs the whole pass on the rescaled and
 // clamped delta.
-template<int ACT, int V, int R, int L, int MODE = kPlain>
-__global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(ResidentBwdArgs a)
+// Channel c of a backward whose first launch finished it with the sums of its unscaled delta, scaled
+// by the factor the plan arrived at.
+template<int V, int R, int L>
+__device__ __forceinline__ void resident_rescale_channel(const ResidentBwdArgs& a, uint32_t c, float factor)
+{
+#pragma unroll 1
+    for (int r = 0; r < R + L; ++r) {
+        const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+        if (e < a.g.per_channel) {
+            const size_t where = a.g.at(c, e);
+            Pack<V> t = ld<V, true>(a.b.delta, where);
+#pragma unroll
+            for (int q = 0; q < V; ++q) t.v[q] = factor * t.v[q];
+            st<V, true>(a.b.delta, where, t);
+        }
+    }
+    if (threadIdx.x == 0) {
+        const double2 sums = a.channel_sums[c];
+        rescale_finished_channel(sums.x, sums.y, static_cast<double>(factor), c, a.b.var, a.b.scale, a.scale_updates,
+                                 a.bias_updates, a.mean_delta, a.var_delta);
+    }
+}
+
+// Channel c by the whole workgroup; `factor` and `limit` are the plan's (kRedo only).
+template<int ACT, int V, int R, int L, int MODE>
+__device__ __forceinline__ void resident_bwd_channel(const ResidentBwdArgs& a, const uint32_t c,
+                                                     [[maybe_unused]] const float factor,
+                                                     [[maybe_unused]] const float limit)
 {
     extern __shared__ __align__(16) float resident_lds[];
     __shared__ double slots[MODE == kFirst ? 3 : 2][kResidentWaves];
     __shared__ DxCoef shared_coef;
-    const uint32_t c = blockIdx.x;
-    [[maybe_unused]] float factor = 1.0f, limit = 0.0f;
-    if constexpr (MODE == kRedo) {
-        const ClipPlan plan = clip_plan_from<kResidentThreads>(a.channel_norm, a.g.channels, a.clip.threshold,
-                                                               a.clip.clip);
-        if (c == 0 && threadIdx.x == 0) {
-            *a.clip.plan = plan;
-            if (a.clip.norm_out) *a.clip.norm_out = plan.norm;
-        }
-        if (a.channel_done[c]) {
-            if (plan.factor == 1.0f) return;
-#pragma unroll 1
-            for (int r = 0; r < R + L; ++r) {
-                const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
-                if (e < a.g.per_channel) {
-                    const size_t where = a.g.at(c, e);
-                    Pack<V> t = ld<V, true>(a.b.delta, where);
-#pragma unroll
-                    for (int q = 0; q < V; ++q) t.v[q] = plan.factor * t.v[q];
-                    st<V, true>(a.b.delta, where, t);
-                }
-            }
-            if (threadIdx.x == 0) {
-                const double2 sums = a.channel_sums[c];
-                rescale_finished_channel(sums.x, sums.y, static_cast<double>(plan.factor), c, a.b.var, a.b.scale,
-                                         a.scale_updates, a.bias_updates, a.mean_delta, a.var_delta);
-            }
-            return;
-        }
-        factor = plan.factor;
-        limit = plan.clip;
-    }
     const FoldCoef k = make_coef(a.b.mean[c], a.b.var[c], a.b.scale[c], a.b.bias[c]);
     const bool recompute = a.b.pre == nullptr;
     Pack<V> d[R];
@@ -1142,7 +1171,7 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
     } else {
 #pragma unroll
         for (int r = R + L - 1; r >= 0; --r) {
-            const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+            const uint32_t e = (r * kResidentThreads + lane) * V;
             if (e < a.g.per_channel) {
                 const size_t where = a.g.at(c, e);
                 Pack<V> dv = ld<V, true>(a.b.delta, where);
@@ -1165,6 +1194,14 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
                 }
                 if (r < R) d[r < R ? r : 0] = dv;
                 else *resident_lds_slot<V, R>(resident_lds, r) = dv;
+            }
+            // the scalar form with the norm's two extra sums: the steps in two halves, so that half of
+            // their loads are in flight at a time and the lane stays within its 64 registers
+            if constexpr (MODE == kFirst && V == 1) {
+                if (r == (R + L) / 2) {
+                    asm volatile("" : "+v"(fa), "+v"(fb), "+v"(fq), "+v"(peak));
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
     }
@@ -1216,9 +1253,10 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
             __builtin_amdgcn_sched_barrier(0);
         }
     } else {
+        asm volatile("" : "+v"(lane));      // addresses formed again, not kept from the first pass
 #pragma unroll
         for (int r = 0; r < R + L; ++r) {
-            const uint32_t e = (r * kResidentThreads + threadIdx.x) * V;
+            const uint32_t e = (r * kResidentThreads + lane) * V;
             if (e < a.g.per_channel) {
                 const size_t where = a.g.at(c, e);
                 const Pack<V> xv = ld<V, false>(a.b.x, where);
@@ -1229,6 +1267,38 @@ __global__ __launch_bounds__(kResidentThreads) void bn_resident_bwd_kernel(Resid
                 st<V, true>(a.b.delta, where, out);
             }
         }
+    }
+}
+// One workgroup per channel.  (The forms without an LDS part are held to 64 registers, two workgroups
+// per compute unit: they run the 19 x 19 and 38 x 38 layers, whose launches are too short to fill the
+// machine with one.)  The workgroups of the kRedo launch form the plan from the per-channel figures of
+// the first launch and leave at once when nothing has to change; the forms without an LDS part run it
+// as a capped grid that walks the channels otherwise.
+template<int ACT, int V, int R, int L, int MODE = kPlain>
+__global__ __launch_bounds__(kResidentThreads, L == 0 && MODE != kRedo ? 8 : 4) void bn_resident_bwd_kernel(ResidentBwdArgs a)
+{
+    if constexpr (MODE == kRedo) {
+        const ClipPlan plan = clip_plan_from<kResidentThreads>(a.channel_norm, a.g.channels, a.clip.threshold,
+                                                               a.clip.clip);
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            *a.clip.plan = plan;
+            if (a.clip.norm_out) *a.clip.norm_out = plan.norm;
+        }
+        if (!plan.work) return;
+        if constexpr (L > 0) {
+            // (one workgroup per channel: walking several costs the large form 450 bytes of spills per lane)
+            const uint32_t c = blockIdx.x;
+            if (!a.channel_done[c]) resident_bwd_channel<ACT, V, R, L, kRedo>(a, c, plan.factor, plan.clip);
+            else if (plan.factor != 1.0f) resident_rescale_channel<V, R, L>(a, c, plan.factor);
+        } else {
+            for (uint32_t c = blockIdx.x; c < static_cast<uint32_t>(a.g.channels); c += gridDim.x) {
+                if (!a.channel_done[c]) resident_bwd_channel<ACT, V, R, L, kRedo>(a, c, plan.factor, plan.clip);
+                else if (plan.factor != 1.0f) resident_rescale_channel<V, R, L>(a, c, plan.factor);
+                __syncthreads();       // the next channel reuses the workgroup's LDS
+            }
+        }
+    } else {
+        resident_bwd_channel<ACT, V, R, L, MODE>(a, blockIdx.x, 1.0f, 0.0f);
     }
 }
 // Vectors per thread the resident kernels are built for, and whether a shape takes that path:
@@ -1569,9 +1639,12 @@ static int bn_backward(const char* who, float* delta, const float* x, const floa
         const ResidentBwdArgs r{ BackwardArgs{ delta, x, pre_activation, mean, var, scale, bias }, scale_updates,
                                  bias_updates, mean_delta, var_delta, resident_geom(batch, channels, spatial),
                                  region.channel_norm, region.channel_sums, region.channel_done, clip };
-        const dim3 grid(channels), block(kResidentThreads);
+        const dim3 block(kResidentThreads);
         int large_lds_rc = PXH_OK;
         const auto launch = [&]<int ACT, int MODE>() {
+            // the launch that follows the plan: one workgroup per compute unit at most, each walks channels
+            const bool walks = MODE == kRedo && per_thread <= kResidentVectors && channels > kRedoWorkgroups;
+            const dim3 grid(walks ? kRedoWorkgroups : channels);
             if (per_thread > kResidentVectors) {
                 auto kernel = bn_resident_bwd_kernel<ACT, 4, kResidentLargeRegs, kResidentLargeLds, MODE>;
                 large_lds_rc = allow_large_lds(reinterpret_cast<const void*>(kernel));
@@ -1621,9 +1694,14 @@ static int bn_backward(const char* who, float* delta, const float* x, const floa
         }
     };
     const auto finish = [&]<int MODE>() {
-        hipLaunchKernelGGL((bwd_finish_kernel<true, MODE>), finish_grid, dim3(kBlock), 0, s, partial, channels, g.blocks,
-                           batch * spatial, mean, var, scale, bias, scale_updates, bias_updates, mean_delta, var_delta,
-                           coef, clip);
+        if constexpr (MODE == kFirst)
+            hipLaunchKernelGGL((bwd_finish_kernel<true, MODE, kPlanThreads>), dim3(grid_for(channels, kPlanThreads / kWave)),
+                               dim3(kPlanThreads), 0, s, partial, channels, g.blocks, batch * spatial, mean, var, scale,
+                               bias, scale_updates, bias_updates, mean_delta, var_delta, coef, clip);
+        else
+            hipLaunchKernelGGL((bwd_finish_kernel<true, MODE>), finish_grid, dim3(kBlock), 0, s, partial, channels,
+                               g.blocks, batch * spatial, mean, var, scale, bias, scale_updates, bias_updates,
+                               mean_delta, var_delta, coef, clip);
     };
     const bool known = dispatch_activation(activation, [&]<int ACT>() {
         if (!cs.on) {
@@ -1728,9 +1806,14 @@ static int bias_backward(const char* who, float* delta, const float* pre_activat
         }
     };
     const auto finish = [&]<int MODE>() {
-        hipLaunchKernelGGL((bwd_finish_kernel<false, MODE>), finish_grid, dim3(kBlock), 0, s, partial, channels,
-                           g.blocks, batch * spatial, nullptr, nullptr, nullptr, nullptr, nullptr, bias_updates, nullptr,
-                           nullptr, nullptr, clip);
+        if constexpr (MODE == kFirst)
+            hipLaunchKernelGGL((bwd_finish_kernel<false, MODE, kPlanThreads>), dim3(grid_for(channels, kPlanThreads / kWave)),
+                               dim3(kPlanThreads), 0, s, partial, channels, g.blocks, batch * spatial, nullptr, nullptr,
+                               nullptr, nullptr, nullptr, bias_updates, nullptr, nullptr, nullptr, clip);
+        else
+            hipLaunchKernelGGL((bwd_finish_kernel<false, MODE>), finish_grid, dim3(kBlock), 0, s, partial, channels,
+                               g.blocks, batch * spatial, nullptr, nullptr, nullptr, nullptr, nullptr, bias_updates,
+                               nullptr, nullptr, nullptr, clip);
     };
     const bool known = dispatch_activation(activation, [&]<int ACT>() {
         if (!cs.on) {
