@@ -199,6 +199,29 @@ def same_bytes_copier(torch, ops, timer):
     return copy_same_bytes
 
 
+def stream_mix_ms(torch, capi, timer, reads, writes, n):
+    """A kernel with no arithmetic that reads `reads` and writes `writes` streams of n floats, launched as the
+    library launches its streaming kernels, over buffers rotated past the cache: what that mix of reads
+    and writes costs on this part whatever is computed (pxh_debug_stream_mix, a test hook)."""
+    import ctypes
+    n = n // 4 * 4
+    rot = rotation_for(4 * n * (reads + writes))
+    dev = torch.device("cuda")
+    sets = []
+    for _ in range(rot):
+        ins = [torch.empty(n, device=dev).normal_() for _ in range(reads)]
+        outs = [torch.empty(n, device=dev) for _ in range(writes)]
+        pin = (ctypes.c_void_p * reads)(*[t.data_ptr() for t in ins])
+        pout = (ctypes.c_void_p * writes)(*[t.data_ptr() for t in outs])
+        sets.append((ins, outs, pin, pout))
+    saved = timer.last_min
+    ms = timer.time(lambda i: capi.call("pxh_debug_stream_mix", reads, writes, n, ctypes.addressof(sets[i][2]),
+                                        ctypes.addressof(sets[i][3]), torch.cuda.current_stream().cuda_stream),
+                    10, rotate=rot)
+    timer.last_min = saved
+    return ms
+
+
 def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     """One training step of YOLOv3 @608 at batch N with every non-convolution kernel launched in the
     model's own layer order on tensors of their own (21 GB): forward (per layer the delta zero-fill
@@ -251,7 +274,12 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
         if l["type"] == "shortcut":
             overwritten.update((i - 1, l["frm"]))
 
-    def forward(_, first_writer=False, fills_together=False):
+    head_table = ops.yolo_head_table([dict(input=T[i - 1]["y"], output=T[i]["y"], delta=T[i]["d"], masks=l["mask"],
+                                           width=l["s"], height=l["s"], stats=T[i]["stats"], cost=T[i]["cost"],
+                                           ignore_thresh=0.7, truth_thresh=1.0)
+                                      for i, l in enumerate(layers) if l["type"] == "yolo"])
+
+    def forward(_, first_writer=False, fills_together=False, heads_apart=False):
         n = 0
         cleared = [t["d"] for i, t in enumerate(T) if not absorbed(i) and not (first_writer and i in overwritten)]
         if fills_together:      # the deltas of all layers cleared at the start of the pass, in a few launches
@@ -275,11 +303,17 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
             elif kind == "route":
                 up, other = l["sources"]
                 ops.route_forward(T[other]["y"], t["y"], layers[up]["c"] * l["s"] * l["s"])
-            elif kind == "yolo":
+            elif kind == "yolo" and heads_apart:
                 ops.yolo_forward_train(T[i - 1]["y"], t["y"], t["d"], truths, counts, truths.shape[1], l["mask"],
                                        wl.YOLOV3_ANCHORS, t["stats"], t["cost"], N, 80, l["s"], l["s"], 608, 608,
                                        0.7, 1.0, 1.0, 1.0, 1.0, 1.0)
             n += 1
+        if not heads_apart:
+            # nothing reads a head's delta or cost before backward: the heads wait for the last one and
+            # run as one pass (pxh_yolo_forward_train_heads)
+            ops.yolo_forward_train_heads(None, truths, counts, truths.shape[1], wl.YOLOV3_ANCHORS, N, 80, 608, 608,
+                                         table=head_table[0])
+            n -= len(head_table[0]) - 1
         launches["forward"] = n
 
     # deltas whose last writer before their layer's backward is a shortcut or a YOLO head (the layer in
@@ -364,6 +398,8 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     out["update_without_delta_pass_ms"] = round(timer.time(lambda i: update(i, False), 3, warm=1), 3)
     # the 23 shortcuts as first writers of the 46 deltas they reach first: no zero-fill of those,
     # no read of them in the shortcut's backward (an option of the C++ layer interface, "first_writer")
+    # every head where it sits in the graph, one call each: what the single pass over all heads saves
+    out["forward_heads_one_call_each_ms"] = round(timer.time(lambda i: forward(i, heads_apart=True), 3, warm=1), 3)
     out["forward_fills_together_ms"] = round(timer.time(lambda i: forward(i, False, True), 3, warm=1), 3)
     out["forward_first_writer_ms"] = round(timer.time(lambda i: forward(i, True, True), 3, warm=1), 3)
     out["backward_first_writer_ms"] = round(timer.time(lambda i: backward(i, True), 3, warm=1), 3)
@@ -536,6 +572,33 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
                     "%d records; %.2g%% of the slots pass" % (found, 100 * passing), streaming=False)
             del rec
         del xin, out, dl
+    # ---- the three heads of the model in one pass (pxh_yolo_forward_train_heads): the small heads' chains of
+    # dependent steps run under the class rows of the large one
+    for NB in (64, N):
+        truths_np, counts_np = wl.yolo_truths(5100, NB)
+        truths = torch.from_numpy(truths_np).to(dev)
+        counts = torch.from_numpy(counts_np).to(dev)
+        e_all = sum(NB * 255 * s * s for s in wl.YOLOV3_HEAD_SIZES)
+        rot = rotation_for(12 * e_all)
+        sets = []
+        for _ in range(rot):
+            heads = [dict(input=2.0 * randn(NB, 255, s, s), output=torch.empty((NB, 255, s, s), device=dev),
+                          delta=torch.empty((NB, 255, s, s), device=dev), masks=wl.YOLOV3_MASKS[s], width=s, height=s,
+                          stats=torch.zeros(12, device=dev), cost=torch.zeros(1, device=dev), ignore_thresh=0.7,
+                          truth_thresh=1.0, coord_scale=1.0, object_scale=2.0, noobject_scale=0.1, class_scale=1.0)
+                     for s in wl.YOLOV3_HEAD_SIZES]
+            sets.append((heads, ops.yolo_head_table(heads)))
+        ms_h = timer.time(lambda i: ops.yolo_forward_train_heads(None, truths, counts, truths.shape[1], wl.YOLOV3_ANCHORS,
+                                                                 NB, 80, 608, 608, table=sets[i][1][0]), 20, rotate=rot)
+        separately = sum(head_ms[(NB, s)][1] for s in wl.YOLOV3_HEAD_SIZES)
+        add("yolo_decode+delta+cost x3", "%dx255x{19,38,76}^2" % NB, 12 * e_all, ms_h,
+            "the three heads in one pass, 12B/elem; one call per head: %.4f ms" % separately)
+        # the pass reads one stream and writes two: the same mix without any arithmetic, same bytes
+        mix_ms = stream_mix_ms(torch, capi, timer, 1, 2, e_all)
+        rows[-1]["copy_same_mix_ms"] = round(mix_ms, 4)
+        rows[-1]["vs_same_mix"] = round(mix_ms / ms_h, 3)
+        head_ms[(NB, "all")] = (0.0, ms_h)
+        del sets
     if only_heads:
         return rows, 0.0
     # ---- non-maximum suppression of device-resident records: an inference-sized list (one image, one
@@ -628,6 +691,12 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
     d.copy_(g)
     ms_adam = timer.time(adam_step, 10)
     add("adam_update", "%d params" % P, 32 * P, ms_adam, "32B/param, L2 folded into the update; gradients zero after the first repetition")
+    # four streams read and four written, no arithmetic: what the update's mix of reads and writes costs
+    mix_ms = stream_mix_ms(torch, capi, timer, 4, 4, P)
+    rows[-1]["copy_same_mix_ms"] = round(mix_ms, 4)
+    rows[-1]["vs_same_mix"] = round(mix_ms / ms_adam, 3)
+    add("copy_same_mix(4 read + 4 written)", "%d floats per stream" % P, 32 * P, mix_ms,
+        "no arithmetic: the ceiling of Adam's traffic mix; a 1+1 copy of these bytes runs at 6.5 TB/s")
 
     # ---- SGD with momentum over the same buffer (the optimiser of the shipped presets)
     ms_sgd = timer.time(lambda i: ops.sgd_update(w, d, 16, 1e-3, 0.9, 5e-4, True), 10)
@@ -714,9 +783,7 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
     for r in rows:
         if r["kernel"] in ("upsample_fwd", "upsample_bwd", "maxpool_fwd", "maxpool_bwd", "route_fwd", "route_bwd"):
             total += r["ms"]
-    for (nb, s), (ms_d, ms_t) in head_ms.items():
-        if nb == N:
-            total += ms_t
+    total += head_ms[(N, "all")][1]      # the three heads as one pass
     total += ms_adam
     # the CPU checker beside the largest shape of every family
     if cpu is not None:
@@ -1066,8 +1133,10 @@ def main():
     if args.only_heads:
         rows, _ = measure_extras(torch, ops, wl, timer, capi, only_heads=True)
         for r in rows:
-            log("%-26s %-22s %9.1f MB %8.4f ms %8.1f GB/s  %4.1f%%  %s" % (r["kernel"], r["shape"], r["MB"], r["ms"],
-                                                                          r["GBps"], 100 * r["frac"], r["note"]))
+            log("%-26s %-22s %9.1f MB %8.4f ms %8.1f GB/s  %4.1f%%  %s%s" % (
+                r["kernel"], r["shape"], r["MB"], r["ms"], r["GBps"], 100 * r["frac"],
+                ("same mix of streams, no arithmetic %.4f ms (%.2f)  " % (r["copy_same_mix_ms"], r["vs_same_mix"]))
+                if "vs_same_mix" in r else "", r["note"]))
         print(json.dumps({"yolo_heads": rows}), flush=True)
         return
 
@@ -1166,8 +1235,10 @@ def main():
         for r in extras:
             log("%-26s %-22s %9.1f MB %8.4f ms %8.1f GB/s  %4.1f%%  %s%s%s"
                 % (r["kernel"], r["shape"], r["MB"], r["ms"], r["GBps"], 100 * r["frac"],
-                   ("copy of the same bytes %.4f ms (%.2f)  " % (r["copy_same_bytes_ms"], r["vs_copy"]))
-                   if "vs_copy" in r else "",
+                   (("copy of the same bytes %.4f ms (%.2f)  " % (r["copy_same_bytes_ms"], r["vs_copy"]))
+                    if "vs_copy" in r else "") +
+                   (("same mix of streams, no arithmetic %.4f ms (%.2f)  " % (r["copy_same_mix_ms"], r["vs_same_mix"]))
+                    if "vs_same_mix" in r else ""),
                    ("cpu %.1f ms  " % r["cpu_ms"]) if "cpu_ms" in r else "", r["note"]))
         log("sum of the layer kernels of one YOLOv3 @608 training step at batch 16: %.3f ms" % ms_batch)
         model_order = measure_model_order(torch, ops, wl, timer)

@@ -311,6 +311,33 @@ int pxh_yolo_loss(const float* output, float* delta, const float* truths, const 
                   float noobject_scale, float class_scale, void* workspace, size_t workspace_bytes,
                   void* stream);
 
+/* All heads of a model in one pass.  The engine runs each YoloLayer where it sits in the graph
+ * (include/Model.h:1740-1759, include/YoloLayer.h:164-239), but nothing reads a head's output delta,
+ * cost or statistics before the backward pass: a host that defers its heads to the end of forward
+ * hands them over together, and the small heads -- each of which alone is one long chain of dependent
+ * steps on a mostly idle machine -- run under the class rows of the large one: two launches for all
+ * heads.  Per head the results are those of pxh_yolo_forward_train on that head (output and delta to
+ * the bit; the sums are added in another grouping).  Heads share the batch, the truths, the anchor
+ * list, the class count and the network size, as the YoloLayers of one model do.
+ * masks: host memory; stats[12] / cost[1]: device, nullable.  At most 4 heads per call.
+ * workspace: pxh_yolo_heads_workspace_bytes(), or NULL for the library's. */
+typedef struct pxh_yolo_head {
+    const float* input;
+    float* output;
+    float* delta;
+    const int* masks;
+    int mask_count;
+    int width, height;
+    float ignore_thresh, truth_thresh, coord_scale, object_scale, noobject_scale, class_scale;
+    float* stats;
+    float* cost;
+} pxh_yolo_head;
+size_t pxh_yolo_heads_workspace_bytes(int count, const pxh_yolo_head* heads, int batch);
+int pxh_yolo_forward_train_heads(int count, const pxh_yolo_head* heads, const float* truths,
+                                 const int* truth_counts, int max_truth, const int* host_anchors,
+                                 int anchor_count, int batch, int classes, int net_width, int net_height,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+
 /* Detections of a decoded head without copying the head to the host: YoloLayer::addDetects
  * (include/YoloLayer.h:601-698) as a thresholded compaction on the device.  A slot passes when its
  * objectness is not below `threshold`; each of its classes with objectness * probability >=

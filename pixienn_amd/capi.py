@@ -56,6 +56,7 @@ SIGNATURES = {
     "pxh_yolo_activate": [P, P, I, I, I, I, P],
     "pxh_yolo_loss": [P, P, P, P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, F, F, F, F, F, P, Z, P],
     "pxh_yolo_forward_train": [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, F, F, F, F, P, Z, P],
+    "pxh_yolo_forward_train_heads": [I, P, P, P, I, P, I, I, I, I, I, P, Z, P],
     "pxh_sgd_update": [Z, P, P, I, F, F, F, I, P],
     "pxh_rescale_clip": [P, Z, F, F, P, P, Z, P],
     "pxh_norm_groups": [P, Z, P, P],
@@ -88,6 +89,7 @@ _OTHER_RETURNS = {
     "pxh_norm_groups_bytes": (Z, [Z]),
     "pxh_rescale_multi_workspace_bytes": (Z, []),
     "pxh_yolo_workspace_bytes": (Z, [I, I, I, I, I, I]),
+    "pxh_yolo_heads_workspace_bytes": (Z, [I, P, I]),
     "pxh_nms_workspace_bytes": (Z, [I]),
     "pxh_reserve_workspace": (I, [Z]),
     "pxh_tensor_table_destroy": (None, [P]),
@@ -98,7 +100,15 @@ _TEST_HOOKS = {
     "pxh_debug_nms_sweeps": (I, [I]),
     "pxh_debug_library_workspace": (P, [Z]),
     "pxh_debug_yolo_tuning": (I, [I, I, I]),
+    "pxh_debug_stream_mix": (I, [I, I, Z, P, P, P]),
 }
+
+
+class YoloHead(ctypes.Structure):
+    """pxh_yolo_head of include/pixienn_hip.h."""
+    _fields_ = [("input", P), ("output", P), ("delta", P), ("masks", P), ("mask_count", I), ("width", I), ("height", I),
+                ("ignore_thresh", F), ("truth_thresh", F), ("coord_scale", F), ("object_scale", F),
+                ("noobject_scale", F), ("class_scale", F), ("stats", P), ("cost", P)]
 
 
 class PxError(RuntimeError):

@@ -1,5 +1,6 @@
 // Flat fp32 streaming kernels: activation, fill/clip/multiply/axpy helpers, shortcut, Adam.
 #include "stream.h"
+#include "pixienn_hip_test.h"
 
 #include <cmath>
 #include <cstring>
@@ -918,6 +919,40 @@ struct AdamStepOp {
     }
 };
 
+// ---------------------------------------------------------------- a mix of streams, nothing else
+// R streams read, their sum written to W streams: the cost of a read/write mix itself (test hook).
+template<int R, int W>
+struct MixOp {
+    const float* in[4];
+    float* out[4];
+    template<int V> struct Regs { Pack<V> x[R]; };
+    template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
+    {
+#pragma unroll
+        for (int i = 0; i < R; ++i) r.x[i] = ld<V, NT>(in[i], e);
+    }
+    template<int V, bool NT> __device__ void finish(size_t e, const Regs<V>& r) const
+    {
+        Pack<V> sum = r.x[0];
+#pragma unroll
+        for (int i = 1; i < R; ++i) {
+#pragma unroll
+            for (int k = 0; k < V; ++k) sum.v[k] += r.x[i].v[k];
+        }
+#pragma unroll
+        for (int i = 0; i < W; ++i) st<V, NT>(out[i], e, sum);
+    }
+};
+
+template<int R, int W>
+int launch_mix(size_t n, const float* const* in, float* const* out, hipStream_t s)
+{
+    MixOp<R, W> op{};
+    for (int i = 0; i < R; ++i) op.in[i] = in[i];
+    for (int i = 0; i < W; ++i) op.out[i] = out[i];
+    return launch_stream("pxh_debug_stream_mix", n, true, 4 * (R + W), op, s);
+}
+
 }  // namespace
 }  // namespace pxh
 
@@ -1532,6 +1567,35 @@ int pxh_sgd_update_multi(int count, float* const* w, float* const* d, const size
     const SgdUpdateOp op{ nullptr, nullptr, -decay * static_cast<float>(batch), lr / static_cast<float>(batch), momentum, 0 };
     float* const* const buffers[4] = { w, d, nullptr, nullptr };
     return launch_multi<2>("pxh_sgd_update_multi", count, buffers, n, apply_decay, 16, SgdMaker{ op }, as_stream(stream));
+}
+
+int pxh_debug_stream_mix(int reads, int writes, size_t n, const float* const* in, float* const* out, void* stream)
+{
+    if (reads < 1 || reads > 4 || writes < 1 || writes > 4 || !in || !out || n % 4)
+        return fail_invalid("pxh_debug_stream_mix: 1..4 streams each way, n a multiple of 4");
+    for (int i = 0; i < reads; ++i)
+        if (!in[i] || !aligned16(in[i])) return fail_invalid("pxh_debug_stream_mix: bad input pointer %d", i);
+    for (int i = 0; i < writes; ++i)
+        if (!out[i] || !aligned16(out[i])) return fail_invalid("pxh_debug_stream_mix: bad output pointer %d", i);
+    hipStream_t s = as_stream(stream);
+    switch (reads * 10 + writes) {
+    case 11: return launch_mix<1, 1>(n, in, out, s);
+    case 12: return launch_mix<1, 2>(n, in, out, s);
+    case 13: return launch_mix<1, 3>(n, in, out, s);
+    case 14: return launch_mix<1, 4>(n, in, out, s);
+    case 21: return launch_mix<2, 1>(n, in, out, s);
+    case 22: return launch_mix<2, 2>(n, in, out, s);
+    case 23: return launch_mix<2, 3>(n, in, out, s);
+    case 24: return launch_mix<2, 4>(n, in, out, s);
+    case 31: return launch_mix<3, 1>(n, in, out, s);
+    case 32: return launch_mix<3, 2>(n, in, out, s);
+    case 33: return launch_mix<3, 3>(n, in, out, s);
+    case 34: return launch_mix<3, 4>(n, in, out, s);
+    case 41: return launch_mix<4, 1>(n, in, out, s);
+    case 42: return launch_mix<4, 2>(n, in, out, s);
+    case 43: return launch_mix<4, 3>(n, in, out, s);
+    default: return launch_mix<4, 4>(n, in, out, s);
+    }
 }
 
 }

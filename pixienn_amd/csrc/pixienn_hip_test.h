@@ -30,6 +30,12 @@ void* pxh_debug_library_workspace(size_t bytes);
  * the order of a few fp32 additions.  Returns 0. */
 int pxh_debug_yolo_tuning(int form, int lanes_per_slot, int head_workers);
 
+/* A kernel with no arithmetic to speak of that reads `reads` and writes `writes` streams of n floats each
+ * (1 <= reads, writes <= 4; every pointer 16-byte aligned; n % 4 == 0), launched as the library launches
+ * its streaming kernels: what that mix of reads and writes costs on the device whatever is computed.
+ * in / out: host arrays of device pointers. */
+int pxh_debug_stream_mix(int reads, int writes, size_t n, const float* const* in, float* const* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1442,6 +1442,145 @@ __global__ __launch_bounds__(kBlock) void yolo_patch_kernel(PatchArgs a)
 
 }  // namespace two_launch
 
+// ==========================================================================================
+// All heads of a model in one pass.  A model runs each of its heads where it sits in the graph
+// (include/Model.h:1740-1759, include/YoloLayer.h:164-239 of the reference), but nothing reads a
+// head's delta or cost before the backward pass, so the heads can all wait for the last one: one grid
+// whose head workers walk the tiles of every head and whose class stream covers every head's class
+// rows, then one small kernel for the supervised slots' class deltas and the sums of every head.  A
+// small head alone is bound by the chain of steps of one head tile, with most of the machine idle;
+// here that chain runs under the class stream of the large head.  The two-launch form's kernels, per
+// head: the results per head are those of pxh_yolo_forward_train on that head.
+// ==========================================================================================
+namespace all_heads {
+
+constexpr int kMaxHeads = 4;
+
+struct HeadPart {
+    two_launch::HeadArgs head;
+    two_launch::ClassSpace space;
+    uint32_t head_workers;      // persistent workgroups that walk this head's tiles
+    uint32_t first_worker;      // ... and the first of them in the grid
+    uint32_t class_blocks;      // workgroups of the class stream on this head
+    uint32_t first_class_block; // ... counted from the end of the head workers
+    int vec;                    // 128-bit accesses on this head's class rows
+    int nt;
+};
+
+struct HeadsArgs {
+    int count;
+    uint32_t workers;           // head workers of all heads
+    HeadPart part[kMaxHeads];
+    YoloParams p[kMaxHeads];
+};
+
+// The head that workgroup `index` of a run of workgroups belongs to: the last one whose first
+// workgroup is not beyond it (`firsts` ascend).
+template<typename First>
+__device__ __forceinline__ int head_of(int count, uint32_t index, First&& first)
+{
+    int h = 0;
+#pragma unroll
+    for (int k = 1; k < kMaxHeads; ++k)
+        if (k < count && index >= first(k)) h = k;
+    return h;
+}
+
+// Block `block` of a head's class stream, one vector per lane: logit -> probability -> `out`, and the
+// zero class delta.  (One read and two written streams: a plain kernel of that mix moves 5.9 TB/s on
+// this part against 6.6 for a copy; two or four vectors per lane were slower, here and there.)
+template<int V, bool NT>
+__device__ __forceinline__ void class_block(const HeadPart& part, uint32_t block)
+{
+    const uint32_t e = (block * kBlock + threadIdx.x) * V;
+    if (e >= part.space.elems) return;
+    uint32_t bn, c, cell;
+    part.space.locate(e, bn, c, cell);
+    const size_t at = part.space.offset(bn, c, cell);
+    Pack<V> zero;
+#pragma unroll
+    for (int k = 0; k < V; ++k) zero.v[k] = 0.0f;
+    const Pack<V> x = ld<V, NT>(part.head.in, at);
+    Pack<V> prob;
+#pragma unroll
+    for (int k = 0; k < V; ++k) prob.v[k] = sigmoid_fast(x.v[k]);
+    st<V, NT>(part.head.out, at, prob);
+    st<V, NT>(part.head.delta, at, zero);
+}
+
+__global__ __launch_bounds__(kBlock, 8) void yolo_heads_kernel(HeadsArgs a)
+{
+    __shared__ TruthSlot tile[kTruthTile];
+    __shared__ double wave_sums[kSums][kWaves];
+    if (blockIdx.x < a.workers) {
+        const int h = head_of(a.count, blockIdx.x, [&](int k) { return a.part[k].first_worker; });
+        const HeadPart& part = a.part[h];
+        const YoloParams& p = a.p[h];
+        const uint32_t worker = blockIdx.x - part.first_worker;
+        // one sum per worker and statistic, over its tiles in walking order
+        double total = 0.0;
+        for (uint32_t t = worker; t < p.blocks; t += part.head_workers) {
+            total += two_launch::head_tile<true>(t, part.head, p, YoloTables{}, tile, wave_sums);
+            __syncthreads();      // wave_sums is read by the first lanes until here
+        }
+        if (threadIdx.x < kSums) part.head.partial[static_cast<size_t>(threadIdx.x) * part.head_workers + worker] = total;
+        return;
+    }
+    const uint32_t block = blockIdx.x - a.workers;
+    const int h = head_of(a.count, block, [&](int k) { return a.part[k].first_class_block; });
+    const HeadPart& part = a.part[h];
+    const uint32_t local = block - part.first_class_block;
+    if (part.vec) {
+        if (part.nt) class_block<4, true>(part, local);
+        else class_block<4, false>(part, local);
+    } else {
+        class_block<1, false>(part, local);
+    }
+}
+
+struct PatchPart {
+    two_launch::ClassArgs cls;      // in = the decoded head
+    uint32_t slots;                 // batch * masks * area
+    uint32_t first_block;           // of this head's slots in the grid
+    int classes;
+};
+
+struct PatchHeadsArgs {
+    int count;
+    PatchPart part[kMaxHeads];
+};
+
+// The supervised slots' class deltas of every head (one lane per slot finds them, a wave writes each
+// slot's class rows together); the first 13 workgroups per head also add up that head's sums.
+__global__ __launch_bounds__(kBlock) void yolo_heads_patch_kernel(PatchHeadsArgs a)
+{
+    __shared__ double slots[kBlock / kWave];
+    {
+        const int h = head_of(a.count, blockIdx.x, [&](int k) { return a.part[k].first_block; });
+        const PatchPart& part = a.part[h];
+        const uint32_t slot = (blockIdx.x - part.first_block) * kBlock + threadIdx.x;
+        const int cls = slot < part.slots ? part.cls.decision[slot] : -1;
+        const int lane = threadIdx.x & (kWave - 1);
+        unsigned long long todo = __ballot(cls >= 0);
+        while (todo) {
+            const int src = __builtin_ctzll(todo);
+            todo &= todo - 1;
+            const uint32_t s_slot = __shfl(slot, src, kWave);
+            const int s_cls = __shfl(cls, src, kWave);
+            uint32_t bn, cell;
+            part.cls.space.by_area.divmod(s_slot, bn, cell);
+            for (int c = lane; c < part.classes; c += kWave) {
+                const size_t at = part.cls.space.offset(bn, c, cell);
+                const float t = (c == s_cls) ? 1.0f : 0.0f;
+                part.cls.delta[at] = part.cls.class_scale * (t - part.cls.in[at]);
+            }
+        }
+    }
+    if (blockIdx.x < 13u * a.count) two_launch::finish_statistic(blockIdx.x % 13, a.part[blockIdx.x / 13].cls, slots);
+}
+
+}  // namespace all_heads
+
 // ---------------------------------------------------------------- detections
 // Thresholded compaction of a decoded head (include/YoloLayer.h:601-698): one lane per slot; a slot
 // whose objectness passes walks its class rows, and all lanes of a workgroup that found detections
@@ -1960,6 +2099,93 @@ int run_training_pass(const char* who, const float* in, float* out, float* delta
                                                 accumulate, ws, s);
 }
 
+namespace all_heads {
+
+// workspace: per head the two-launch form's [12][head workers] doubles and one int per slot
+size_t workspace_bytes(int count, const pxh_yolo_head* heads, int batch)
+{
+    size_t total = 0;
+    for (int h = 0; h < count; ++h)
+        total += two_launch::yolo_workspace_bytes(batch, heads[h].mask_count, heads[h].width, heads[h].height);
+    return total;
+}
+
+int run(const char* who, int count, const pxh_yolo_head* heads, const YoloParams* params, const float* truths,
+        const int* truth_counts, void* ws, hipStream_t s)
+{
+    HeadsArgs a{};
+    PatchHeadsArgs pa{};
+    a.count = pa.count = count;
+    // the class stream of all heads together sets the time the head workers have
+    double stream_us = 0.0;
+    for (int h = 0; h < count; ++h) {
+        const YoloParams& p = params[h];
+        stream_us += static_cast<double>(p.batch) * p.mask_count * p.classes * p.area * 12 / 6.0e6;   // at 6 TB/s
+    }
+    uint64_t tiles_total = 0;
+    for (int h = 0; h < count; ++h) tiles_total += params[h].blocks;
+    char* at = static_cast<char*>(ws);
+    uint32_t workers = 0, class_blocks = 0, patch_blocks = 0;
+    for (int h = 0; h < count; ++h) {
+        const YoloParams& p = params[h];
+        a.p[h] = p;
+        const two_launch::YoloWorkspace w = two_launch::carve(at, p);
+        at += two_launch::yolo_workspace_bytes(p.batch, p.mask_count, p.width, p.height);
+        const two_launch::ClassSpace space{ FastDiv(p.area), FastDiv(p.classes), static_cast<uint32_t>(p.area),
+                                            static_cast<uint32_t>(p.classes + 5),
+                                            static_cast<uint32_t>(static_cast<size_t>(p.batch) * p.mask_count *
+                                                                  p.classes * p.area) };
+        HeadPart& part = a.part[h];
+        part.head = two_launch::HeadArgs{ heads[h].input, heads[h].output, heads[h].delta, truths, truth_counts,
+                                          w.decision, w.partial };
+        part.space = space;
+        part.head_workers = two_launch::head_workers(p.blocks, stream_us);
+        if (const int forced = one_launch::g_forced_workers.load(); forced > 0) {
+            // the test hook's figure is for the call: every head gets its share by tiles, one at least
+            const uint64_t share = static_cast<uint64_t>(forced) * p.blocks / tiles_total;
+            part.head_workers = share < 1 ? 1u : share < p.blocks ? static_cast<uint32_t>(share) : p.blocks;
+        }
+        part.first_worker = workers;
+        workers += part.head_workers;
+        part.vec = p.area % 4 == 0 && aligned16(heads[h].input) && aligned16(heads[h].output) && aligned16(heads[h].delta);
+        const uint32_t per_block = kBlock * (part.vec ? 4 : 1);
+        part.class_blocks = (space.elems + per_block - 1) / per_block;
+        part.first_class_block = class_blocks;
+        class_blocks += part.class_blocks;
+        part.nt = stream_us * 6.0e6 >= static_cast<double>(kStreamingBytes);
+
+        PatchPart& pp = pa.part[h];
+        pp.cls.in = heads[h].output;
+        pp.cls.delta = heads[h].delta;
+        pp.cls.decision = w.decision;
+        pp.cls.partial = w.partial;
+        pp.cls.stats = heads[h].stats;
+        pp.cls.cost = heads[h].cost;
+        pp.cls.space = space;
+        pp.cls.head_blocks = part.head_workers;
+        pp.cls.class_scale = p.class_scale;
+        pp.cls.accumulate = 0;
+        pp.slots = static_cast<uint32_t>(p.batch) * p.mask_count * p.area;
+        pp.classes = p.classes;
+        pp.first_block = patch_blocks;
+        patch_blocks += grid_for(pp.slots, kBlock);
+    }
+    a.workers = workers;
+    const unsigned long long grid = 1ull * workers + class_blocks;
+    if (grid >= (1ull << 31)) {
+        set_error("%s: more than 2^31 workgroups in one launch", who);
+        return PXH_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(yolo_heads_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, s, a);
+    int rc = check_launch(who);
+    if (rc) return rc;
+    const uint32_t least = 13u * count;
+    hipLaunchKernelGGL(yolo_heads_patch_kernel, dim3(patch_blocks < least ? least : patch_blocks), dim3(kBlock), 0, s, pa);
+    return check_launch(who);
+}
+
+}  // namespace all_heads
+
 }  // namespace
 }  // namespace pxh
 
@@ -2076,6 +2302,64 @@ int pxh_yolo_forward_train(const float* input, float* output, float* delta, cons
     if (rc) return rc;
     return run_training_pass<true>("pxh_yolo_forward_train", input, output, delta, truths, truth_counts, p,
                                    YoloTables{}, stats, cost, 0, ws, as_stream(stream));
+}
+
+static int heads_params(const char* who, int count, const pxh_yolo_head* heads, const int* host_anchors,
+                        int anchor_count, int batch, int classes, int net_width, int net_height, int max_truth,
+                        YoloParams* params)
+{
+    if (count <= 0 || count > all_heads::kMaxHeads) {
+        set_error("%s: between 1 and %d heads per call, not %d", who, all_heads::kMaxHeads, count);
+        return count <= 0 ? PXH_ERR_INVALID_ARGUMENT : PXH_ERR_UNSUPPORTED;
+    }
+    if (!heads || !host_anchors) return fail_invalid("%s: null pointer", who);
+    for (int h = 0; h < count; ++h) {
+        const pxh_yolo_head& hd = heads[h];
+        if (!hd.input || !hd.output || !hd.delta || !hd.masks) return fail_invalid("%s: null pointer in head %d", who, h);
+        if (hd.input == hd.output || hd.input == hd.delta || hd.output == hd.delta)
+            return fail_invalid("%s: input, output and delta of head %d must be distinct buffers", who, h);
+        YoloParams& p = params[h];
+        p = YoloParams{};
+        int rc = fill_params(who, p, batch, hd.mask_count, anchor_count, classes, hd.width, hd.height, net_width,
+                             net_height, max_truth, hd.ignore_thresh, hd.truth_thresh, hd.coord_scale, hd.object_scale,
+                             hd.noobject_scale, hd.class_scale);
+        if (rc) return rc;
+        for (int m = 0; m < hd.mask_count; ++m) {
+            if (hd.masks[m] < 0 || hd.masks[m] >= anchor_count)
+                return fail_invalid("%s: mask %d of head %d names anchor %d of %d", who, m, h, hd.masks[m], anchor_count);
+            p.masks[m] = hd.masks[m];
+        }
+        for (int a = 0; a < 2 * anchor_count; ++a) {
+            p.anchors[a] = static_cast<float>(host_anchors[a]);
+            p.anchors_rel[a] = p.anchors[a] / static_cast<float>(a % 2 ? net_height : net_width);
+        }
+    }
+    return PXH_OK;
+}
+
+size_t pxh_yolo_heads_workspace_bytes(int count, const pxh_yolo_head* heads, int batch)
+{
+    if (count <= 0 || count > all_heads::kMaxHeads || !heads || batch <= 0) return 0;
+    for (int h = 0; h < count; ++h)
+        if (heads[h].mask_count <= 0 || heads[h].width <= 0 || heads[h].height <= 0) return 0;
+    return all_heads::workspace_bytes(count, heads, batch);
+}
+
+int pxh_yolo_forward_train_heads(int count, const pxh_yolo_head* heads, const float* truths, const int* truth_counts,
+                                 int max_truth, const int* host_anchors, int anchor_count, int batch, int classes,
+                                 int net_width, int net_height, void* workspace, size_t workspace_bytes, void* stream)
+{
+    const char* who = "pxh_yolo_forward_train_heads";
+    if (!truth_counts || (!truths && max_truth > 0)) return fail_invalid("%s: null pointer", who);
+    YoloParams params[all_heads::kMaxHeads];
+    int rc = heads_params(who, count, heads, host_anchors, anchor_count, batch, classes, net_width, net_height,
+                          max_truth, params);
+    if (rc) return rc;
+    void* ws;
+    rc = resolve_workspace(workspace, workspace_bytes, all_heads::workspace_bytes(count, heads, batch), &ws,
+                           as_stream(stream));
+    if (rc) return rc;
+    return all_heads::run(who, count, heads, params, truths, truth_counts, ws, as_stream(stream));
 }
 
 int pxh_yolo_loss(const float* output, float* delta, const float* truths, const int* truth_counts, int max_truth,

@@ -87,6 +87,8 @@ using GroundTruthVec = std::vector<GroundTruth>;
 
 // ---------------------------------------------------------------- context
 // The part of the owning model the layers read.
+class Layer;
+
 class Context
 {
 public:
@@ -164,6 +166,13 @@ public:
         normGroups_.erase(it);
         return groups;
     }
+
+    // YOLO heads that put their training forward off until the model's forward pass is over ("deferred"),
+    // in the order they were reached: nothing reads a head's delta, cost or statistics before backward,
+    // so all of them run as ONE pass then (YoloLayer::forwardDeferred), the small ones under the class
+    // rows of the large one.  What they need of the context's workspace adds up, head by head.
+    std::vector<Layer*> deferredHeads;
+    std::size_t deferredHeadsWorkspace = 0;
 
     const FloatVector& truths() const noexcept { return truths_; }
     const IntVector& truthCounts() const noexcept { return truthCounts_; }

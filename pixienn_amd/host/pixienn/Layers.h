@@ -839,10 +839,48 @@ public:
             // the shipped networks), so `grad += delta` below is the last write of that layer's delta
             // and leaves its norm and peak behind for the rescale + clip that opens its backward.
             if (props.get<bool>("leaves_norm", false)) normGroups_ = normGroupsFor(output_.size());
+            // "deferred": the training forward of this head waits for forwardDeferred(), which the model
+            // calls once after its last layer's forward and which runs all waiting heads as one pass
+            deferred_ = props.get<bool>("deferred", false);
+            if (deferred_) {
+                context.deferredHeadsWorkspace += pxh_yolo_workspace_bytes(batch(), static_cast<int>(mask_.size()),
+                                                                           context.classes, width(), height(), 0);
+                context.reserveWorkspace(context.deferredHeadsWorkspace);
+            }
         }
     }
 
     bool hasCost() const noexcept override { return true; }
+
+    // Runs the training forward of every head of `context` that is waiting for it (reference: each
+    // YoloLayer's own forward, include/YoloLayer.h:164-239, in one device pass).  To be called after the
+    // forward of the model's last layer, before anything reads a head's delta, cost or statistics.
+    static void forwardDeferred(Context& context)
+    {
+        auto& waiting = context.deferredHeads;
+        if (waiting.empty()) return;
+        constexpr std::size_t kPerCall = 4;      // heads per call of the library
+        for (std::size_t first = 0; first < waiting.size(); first += kPerCall) {
+            const std::size_t count = std::min(kPerCall, waiting.size() - first);
+            pxh_yolo_head heads[kPerCall];
+            const YoloLayer* lead = static_cast<const YoloLayer*>(waiting[first]);
+            for (std::size_t h = 0; h < count; ++h) {
+                auto* y = static_cast<YoloLayer*>(waiting[first + h]);
+                PX_CHECK(y->batch() == lead->batch() && y->anchors_ == lead->anchors_,
+                         "yolo: deferred heads must share the batch and the anchor list");
+                heads[h] = pxh_yolo_head{ y->pendingInput_, y->output_.data(), y->delta_.data(), y->mask_.data(),
+                                          static_cast<int>(y->mask_.size()), y->width(), y->height(), y->ignoreThresh_,
+                                          y->truthThresh_, y->coordScale_, y->objectScale_, y->noObjectScale_,
+                                          y->classScale_, y->stats_.data(), y->costDevice_.data() };
+            }
+            PX_HIP_CHECK(pxh_yolo_forward_train_heads(static_cast<int>(count), heads, context.truths().data(),
+                                                      context.truthCounts().data(), context.maxTruth(),
+                                                      lead->anchors_.data(), lead->numAnchors_, lead->batch(),
+                                                      context.classes, context.width, context.height,
+                                                      context.workspace(), context.workspaceBytes(), context.stream));
+        }
+        waiting.clear();
+    }
 
     void forward(const V& input) override
     {
@@ -856,6 +894,12 @@ public:
             return;
         }
         PX_CHECK(static_cast<int>(c.truthCounts().size()) == batch(), "yolo: ground truth of another batch size");
+        costReady_ = false;
+        if (deferred_) {
+            pendingInput_ = input.data();
+            context().deferredHeads.push_back(this);
+            return;
+        }
         PX_HIP_CHECK(pxh_yolo_forward_train(input.data(), output_.data(), delta_.data(), c.truths().data(),
                                             c.truthCounts().data(), c.maxTruth(), mask_.data(), anchors_.data(),
                                             stats_.data(), costDevice_.data(), batch(), masks, numAnchors_,
@@ -960,6 +1004,8 @@ private:
     float ignoreThresh_, truthThresh_, coordScale_, objectScale_, noObjectScale_, classScale_;
     V stats_, costDevice_;
     bool costReady_ = false;
+    bool deferred_ = false;
+    const float* pendingInput_ = nullptr;
     V normGroups_;
     IntVector detectRecords_, detectCount_;
     int detectCapacity_ = 0;

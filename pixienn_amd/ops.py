@@ -3,6 +3,8 @@
 Every function launches on torch's current HIP stream and returns without synchronising.
 Tensors must be fp32 (int32 for indices), contiguous and on a HIP device.
 """
+import ctypes
+
 import numpy as np
 import torch
 
@@ -321,6 +323,42 @@ def yolo_forward_train(inp, out, delta, truths, truth_counts, max_truth, masks, 
          m.ctypes.data, a.ctypes.data, ptr(stats), ptr(cost), batch, len(m), len(a) // 2, classes, width, height,
          net_width, net_height, float(ignore_thresh), float(truth_thresh), float(coord_scale), float(object_scale),
          float(noobject_scale), float(class_scale), ptr(workspace), wb, _stream())
+
+
+def yolo_head_table(heads):
+    """An array of pxh_yolo_head from dicts with keys input, output, delta, masks, width, height and, optionally,
+    stats, cost, ignore_thresh (0.7), truth_thresh (1), coord_scale, object_scale, noobject_scale, class_scale (1).
+    Returns (array, keep-alive list)."""
+    table = (capi.YoloHead * len(heads))()
+    keep = []
+    for t, h in zip(table, heads):
+        _chk_all(h["input"], h["output"], h["delta"], h.get("stats"), h.get("cost"))
+        m = np.ascontiguousarray(h["masks"], dtype=np.int32)
+        keep.append(m)
+        t.input, t.output, t.delta = ptr(h["input"]), ptr(h["output"]), ptr(h["delta"])
+        t.masks, t.mask_count = m.ctypes.data, len(m)
+        t.width, t.height = int(h["width"]), int(h["height"])
+        t.ignore_thresh = float(h.get("ignore_thresh", 0.7)); t.truth_thresh = float(h.get("truth_thresh", 1.0))
+        t.coord_scale = float(h.get("coord_scale", 1.0)); t.object_scale = float(h.get("object_scale", 1.0))
+        t.noobject_scale = float(h.get("noobject_scale", 1.0)); t.class_scale = float(h.get("class_scale", 1.0))
+        t.stats, t.cost = ptr(h.get("stats")), ptr(h.get("cost"))
+    return table, keep
+
+
+def yolo_forward_train_heads(heads, truths, truth_counts, max_truth, anchors, batch, classes, net_width, net_height,
+                             workspace=None, table=None):
+    """All heads of a model in one pass (pxh_yolo_forward_train_heads); `heads` as for yolo_head_table, or a
+    table built by it beforehand."""
+    _chk_all(truths)
+    _chk(truth_counts, torch.int32, "truth_counts")
+    keep = None
+    if table is None:
+        table, keep = yolo_head_table(heads)
+    a = np.ascontiguousarray(anchors, dtype=np.int32)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("pxh_yolo_forward_train_heads", len(table), ctypes.addressof(table), ptr(truths), ptr(truth_counts),
+         int(max_truth), a.ctypes.data, len(a) // 2, batch, classes, net_width, net_height, ptr(workspace), wb, _stream())
+    del keep
 
 
 def yolo_loss(output, delta, truths, truth_counts, max_truth, assigned_classes, assigned_anchors, assigned_boxes,

@@ -462,11 +462,17 @@ void trainingChecks()
         Host d = net.conv6->delta().asVector();
         Host biasUpd(2 * C, 0.0f);
         const Host pre = net.conv6->output().asVector();      // linear: the output is the pre-activation
+        // Layer::backward's helpers ride on the bias backward: the rescale bites, the clamp is far away
+        Host probe = d;
+        const float norm = pxo_rescale_clip(probe.data(), probe.size(), 0.0f, 0.0f);
+        pxo_rescale_clip(d.data(), d.size(), 0.5f * norm, 1e3f);
+        net.conv6->setGradientRescaling(true, 0.5f * norm);
+        net.conv6->setGradientClipping(true, 1e3f);
         pxo_conv_epilogue_backward(0, PXO_LINEAR, N, 2 * C, S, S, d.data(), pre.data(), nullptr, nullptr, nullptr,
                                    nullptr, nullptr, nullptr, biasUpd.data(), nullptr, nullptr, 0);
         net.conv6->backward(net.route5->output(), &net.route5->delta());
-        expectClose("conv6 bias updates", net.conv6->biasUpdates().asVector(), biasUpd, 1e-5, 1.0);
-        expectExact("conv6 backward into route5 delta", net.route5->delta().asVector(), d);
+        expectClose("conv6 bias updates (delta rescaled)", net.conv6->biasUpdates().asVector(), biasUpd, 1e-5, 1.0);
+        expectExact("conv6 backward into route5 delta (rescaled)", net.route5->delta().asVector(), d);
     }
     {   // route5 -> up4.delta and conv0.delta
         const Host rd = net.route5->delta().asVector();
@@ -506,6 +512,13 @@ void trainingChecks()
             const float scaled = xn[i] * net.scale2[c];
             pre[i] = scaled + net.bias2[c];
         }
+        // Layer::backward's helpers ride on the epilogue's backward: rescale and clamp both bite here
+        Host probe = d;
+        const float norm = pxo_rescale_clip(probe.data(), probe.size(), 0.0f, 0.0f);
+        const float rms = norm / std::sqrt(static_cast<float>(d.size()));
+        pxo_rescale_clip(d.data(), d.size(), 0.6f * norm, 0.9f * rms);
+        net.conv2->setGradientRescaling(true, 0.6f * norm);
+        net.conv2->setGradientClipping(true, 0.9f * rms);
         Host md(C), vd(C), su(C, 0.0f), bu(C, 0.0f);
         pxo_conv_epilogue_backward(1, PXO_MISH, N, C, S / 2, S / 2, d.data(), pre.data(), mean.data(), var.data(),
                                    md.data(), vd.data(), net.scale2.data(), su.data(), bu.data(), x.data(), xn.data(),
@@ -513,9 +526,9 @@ void trainingChecks()
         Host want = net.pool1->delta().asVector();
         for (size_t i = 0; i < want.size(); ++i) want[i] += d[i];
         net.conv2->backward(net.pool1->output(), &net.pool1->delta());
-        expectClose("conv2 scale updates", net.conv2->scaleUpdates().asVector(), su, 1e-5, 1.0);
-        expectClose("conv2 bias updates", net.conv2->biasUpdates().asVector(), bu, 1e-5, 1.0);
-        expectClose("conv2 backward into pool1 delta", net.pool1->delta().asVector(), want, 1e-5, 1.0);
+        expectClose("conv2 scale updates (delta rescaled, clamped)", net.conv2->scaleUpdates().asVector(), su, 1e-5, 1.0);
+        expectClose("conv2 bias updates (delta rescaled, clamped)", net.conv2->biasUpdates().asVector(), bu, 1e-5, 1.0);
+        expectClose("conv2 backward into pool1 delta (rescaled, clamped)", net.pool1->delta().asVector(), want, 1e-5, 1.0);
     }
     {   // pool1 -> conv0.delta
         const Host d = net.pool1->delta().asVector();
@@ -1018,6 +1031,58 @@ void leavesNormNetChecks()
 }
 
 // A model's weights file: header of either seen-width, every layer's section in network order, exact length.
+// Two heads that wait for the end of the forward pass and run as one pass give what each gives alone.
+void deferredHeadsChecks()
+{
+    const std::vector<int> anchors{ 10, 14, 23, 27, 37, 58, 81, 82 };
+    struct Pair {
+        Context ctx;
+        std::shared_ptr<YoloLayer> small, large;
+    };
+    const auto build = [&](Pair& p, bool deferred) {
+        p.ctx.training = true;
+        p.ctx.width = p.ctx.height = 128;
+        p.ctx.classes = CLASSES;
+        p.small = std::make_shared<YoloLayer>(p.ctx, Properties{ { "batch", N }, { "channels", 2 * (CLASSES + 5) },
+                                                                 { "height", 5 }, { "width", 5 }, { "num", 4 },
+                                                                 { "mask", std::vector<int>{ 2, 3 } },
+                                                                 { "anchors", anchors }, { "ignore_thresh", 0.5f },
+                                                                 { "object_scale", 2.0f }, { "deferred", deferred } });
+        p.large = std::make_shared<YoloLayer>(p.ctx, Properties{ { "batch", N }, { "channels", 2 * (CLASSES + 5) },
+                                                                 { "height", 12 }, { "width", 12 }, { "num", 4 },
+                                                                 { "mask", std::vector<int>{ 0, 1 } },
+                                                                 { "anchors", anchors }, { "ignore_thresh", 0.7f },
+                                                                 { "noobject_scale", 0.5f }, { "deferred", deferred } });
+        std::vector<GroundTruthVec> truth(N);
+        Rng r(77);
+        for (int b = 0; b < N; ++b)
+            for (int t = 0; t < 1 + b % 3; ++t)
+                truth[b].push_back(GroundTruth{ r.uniform(), r.uniform(), 0.05f + 0.5f * r.uniform(),
+                                                0.05f + 0.5f * r.uniform(), static_cast<int>(r.next() % CLASSES) });
+        p.ctx.setGroundTruth(truth);
+    };
+    Pair apart, together;
+    build(apart, false);
+    build(together, true);
+    Layer::V inSmall(static_cast<size_t>(N) * 2 * (CLASSES + 5) * 25), inLarge(static_cast<size_t>(N) * 2 * (CLASSES + 5) * 144);
+    inSmall.copyHost(normals(78, inSmall.size(), 1.5f));
+    inLarge.copyHost(normals(79, inLarge.size(), 1.5f));
+    apart.small->forward(inSmall);
+    apart.large->forward(inLarge);
+    together.small->forward(inSmall);
+    together.large->forward(inLarge);
+    report("deferred heads wait for the end of the pass", together.ctx.deferredHeads.size() == 2);
+    YoloLayer::forwardDeferred(together.ctx);
+    report("... and are gone from the list once run", together.ctx.deferredHeads.empty());
+    expectExact("deferred small head: output", together.small->output().asVector(), apart.small->output().asVector());
+    expectExact("deferred small head: delta", together.small->delta().asVector(), apart.small->delta().asVector());
+    expectExact("deferred large head: output", together.large->output().asVector(), apart.large->output().asVector());
+    expectExact("deferred large head: delta", together.large->delta().asVector(), apart.large->delta().asVector());
+    expectClose("deferred small head: cost", Host{ together.small->fetchCost() }, Host{ apart.small->fetchCost() }, 1e-6, 1e-3);
+    expectClose("deferred large head: cost", Host{ together.large->fetchCost() }, Host{ apart.large->fetchCost() }, 1e-6, 1e-3);
+    expectClose("deferred large head: statistics", together.large->fetchStats(), apart.large->fetchStats(), 1e-5, 1.0);
+}
+
 void weightsFileChecks()
 {
     auto build = [](Context& ctx) {
@@ -1137,6 +1202,7 @@ int main(int argc, char** argv)
             firstWriterShortcutChecks();
             leavesNormShortcutChecks();
             leavesNormNetChecks();
+            deferredHeadsChecks();
             capturedSequenceChecks();
             parameterSetChecks();
         }
