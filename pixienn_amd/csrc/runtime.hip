@@ -65,7 +65,11 @@ int library_workspace(size_t bytes, hipStream_t stream, bool may_grow_in_capture
     }
     if (!may_grow_in_capture) {
         hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(stream, &status) == hipSuccess && status != hipStreamCaptureStatusNone) {
+        // (asking about the null stream while another stream of the thread captures is itself an error of the
+        // capture kind: that, too, means no allocation now)
+        const hipError_t asked = hipStreamIsCapturing(stream, &status);
+        if (asked == hipErrorStreamCaptureImplicit || (asked == hipSuccess && status != hipStreamCaptureStatusNone)) {
+            (void) hipGetLastError();
             set_error("the library's workspace holds %zu bytes and this call needs %zu: it cannot grow while the "
                       "stream is being captured; call pxh_reserve_workspace(%zu) before the capture, or pass a "
                       "workspace", s.bytes, bytes, bytes);
@@ -73,8 +77,11 @@ int library_workspace(size_t bytes, hipStream_t stream, bool may_grow_in_capture
         }
         (void) hipGetLastError();
     }
-    // 16 MB covers every shape of a YOLOv3-sized network, so the buffer rarely grows after the first call
-    const size_t want = bytes < (16u << 20) ? (16u << 20) : bytes;
+    // 16 MB covers every shape of a YOLOv3-sized network, so the buffer rarely grows after the first call;
+    // when it does it at least doubles, so that the blocks left behind (they are never freed, see above) add up
+    // to less than the live one however slowly the requests rise
+    size_t want = bytes < (16u << 20) ? (16u << 20) : bytes;
+    if (want < 2 * s.bytes) want = 2 * s.bytes;
     void* fresh = nullptr;
     e = hipMalloc(&fresh, want);
     if (e != hipSuccess) {
@@ -115,8 +122,9 @@ int pxh_abi_version(void) { return 2; }
 
 int pxh_reserve_workspace(size_t bytes)
 {
+    // growing allocates: refused (PXH_ERR_WORKSPACE) while the calling thread is capturing
     void* p = nullptr;
-    return pxh::library_workspace(bytes, nullptr, true, &p);
+    return pxh::library_workspace(bytes, nullptr, false, &p);
 }
 
 // Test hook: the address of the current device's library workspace once it holds `bytes`.

@@ -24,14 +24,15 @@ public:
 
     DeviceVector() = default;
 
-    // Filled on the null stream and waited for, so that the vector can be used on any stream (also a
-    // non-blocking one, which does not order itself behind the null stream) once the constructor returns.
-    explicit DeviceVector(size_type n, T value = T())
+    // Filled on `stream` and waited for, so that the vector can be used on any stream (also a non-blocking
+    // one, which does not order itself behind the null stream) once the constructor returns.  Pass the stream
+    // the vector will live on: waiting for the null stream drains every blocking stream of the device.
+    explicit DeviceVector(size_type n, T value = T(), hipStream_t stream = nullptr)
     {
         allocate(n);
         if (n) {
-            fill(value);
-            PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(nullptr));
+            fill(value, stream);
+            PX_HIP_RUNTIME_CHECK(hipStreamSynchronize(stream));
         }
     }
 

@@ -139,11 +139,21 @@ public:
     // workspace.  Layers reserve what their kernels need when they are constructed, so the buffer has
     // its final size and address before the first forward -- and before any graph capture.  A block
     // that has been outgrown is kept until the context goes, for graphs captured with its address.
+    // Growing allocates and fills: an error while the context's stream is being captured (the constructors'
+    // reservations are the growth path; a capture must find the buffer at its final size).
     void reserveWorkspace(std::size_t bytes)
     {
         if (bytes <= workspaceBytes()) return;
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        const hipError_t asked = hipStreamIsCapturing(stream, &capturing);
+        if (asked != hipSuccess) (void) hipGetLastError();
+        PX_CHECK(asked == hipSuccess && capturing == hipStreamCaptureStatusNone,
+                 "the context's workspace cannot grow while its stream is being captured: construct every layer "
+                 "(or call reserveWorkspace) before the capture");
+        // at least doubled, so that the retired blocks add up to less than the live one
+        const std::size_t floats = std::max((bytes + sizeof(float) - 1) / sizeof(float), 2 * workspace_.size());
         if (!workspace_.empty()) retiredWorkspaces_.push_back(std::move(workspace_));
-        workspace_ = FloatVector((bytes + sizeof(float) - 1) / sizeof(float));
+        workspace_ = FloatVector(floats, 0.0f, stream);
     }
 
     void* workspace() noexcept { return workspace_.empty() ? nullptr : workspace_.data(); }

@@ -14,6 +14,7 @@
 #include "hip/ShortcutLayer.h"
 #include "hip/BatchNormLayer.h"
 #include "hip/ConvLayer.h"
+#include "hip/YoloLayerCommon.h"
 #include "hip/YoloLayer.h"
 
 namespace px {

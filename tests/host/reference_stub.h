@@ -47,6 +47,7 @@ public:
     void copy(const PxHipVectorT& rhs);
     void copy(const PxCpuVectorT<T>& rhs);
     void copyHost(const T* host, std::size_t n);
+    void copyToHost(T* host, std::size_t n) const;       // the first n elements (cudaMemcpy device to host)
     std::vector<T> asVector() const;
 };
 using PxHipVector = PxHipVectorT<float>;
@@ -67,11 +68,32 @@ public:
 };
 using Detections = std::vector<Detection>;
 
+template<Device D> class Layer;
+
+// include/Model.h:101-127: per-device state of a model (cuBLAS / cuDNN contexts for Device::CUDA)
 template<Device D>
-class Model
+class DeviceExtras
+{
+};
+
+// The engine keeps the CUDA specialisation right here, under USE_CUDA (include/Model.h:105-127); the lean HIP
+// bindings put theirs in the same place.
+#ifdef PX_HIP_LEAN_BINDINGS
+}   // px
+#include "hip_lean/ModelExtras.h"
+namespace px {
+#endif
+
+template<Device D>
+class Model : public DeviceExtras<D>
 {
 public:
     using V = PxHipVector;
+    void update();
+    bool gradRescaling() const noexcept;
+    float gradThreshold() const noexcept;
+    bool gradClipping() const noexcept;
+    float gradClipValue() const noexcept;
     int width() const noexcept;
     int height() const noexcept;
     int updateBatch() const noexcept;
@@ -84,6 +106,11 @@ public:
     float adamEpsilon() const noexcept;
     int updateCount() const noexcept;
     std::size_t seen() const noexcept;
+
+private:
+    void updateLR();
+    std::vector<std::shared_ptr<Layer<D>>> layers_;
+    std::size_t optimizerStep_ = 0;
 };
 
 template<Device D>
@@ -235,6 +262,8 @@ public:
     void addDetects(Detections& detections, int width, int height, float threshold) override;
 private:
     void setup();
+    void uploadTruths();        // added by include/hip/YoloLayer.h
+    void collectCost();         // added by include/hip/YoloLayer.h
     void resetStats();
     void writeStats();
     std::vector<int> mask_, anchors_;

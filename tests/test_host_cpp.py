@@ -59,3 +59,74 @@ def test_reference_side_bindings_compile_against_the_engine_interface():
     text = open(src).read()
     for name in names:
         assert '#include "hip/%s"' % name in text, "%s is not compiled by the check" % name
+
+
+def test_lean_reference_side_bindings_compile_against_the_engine_interface():
+    """docs/reference_patch/include/hip_lean/*.h -- the variants that ship the lean step (first-writer shortcuts,
+    the norm of a delta from its last writer, all heads in one pass, one optimiser step for all layers)."""
+    src = os.path.join(ROOT, "tests", "host", "patch_check_lean.cpp")
+    proc = subprocess.run(["g++", "-std=c++20", "-fsyntax-only", "-Wall", "-Wextra", "-Wno-unused-parameter",
+                           "-I" + os.path.join(ROOT, "include"),
+                           "-I" + os.path.join(ROOT, "docs", "reference_patch", "include"),
+                           "-I" + os.path.join(ROOT, "tests", "host"), src],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr
+    assert "warning" not in proc.stderr, proc.stderr
+    text = open(src).read()
+    for name in sorted(os.listdir(os.path.join(ROOT, "docs", "reference_patch", "include", "hip_lean"))):
+        assert '#include "hip_lean/%s"' % name in text, name
+
+
+REFERENCE = "/root/reference"
+
+
+@pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE, "include")), reason="the reference tree is not here")
+def test_binding_headers_and_stub_name_only_members_the_engine_has():
+    """The bindings are compiled against a stand-in for the engine's headers; this keeps the stand-in and the
+    bindings honest against the engine itself: every data member (trailing underscore) and every method reached
+    through this-> that a binding header names must occur in the engine's header of that layer, in its CUDA
+    counterpart, in include/Layer.h or include/Model.h -- or be declared by the binding's own
+    ...Extras<Device::HIP> class.  Likewise every member the stand-in declares."""
+    import re
+
+    def engine(*names):
+        text = ""
+        for n in names:
+            path = os.path.join(REFERENCE, "include", n)
+            if os.path.exists(path):
+                text += open(path).read()
+        return text
+
+    def identifiers(text):
+        return set(re.findall(r"\b[A-Za-z]\w*\b", text))
+
+    base = engine("Layer.h", "Model.h", "PxTensor.h", "Detection.h", "Activation.h")
+    patch_root = os.path.join(ROOT, "docs", "reference_patch", "include")
+    own = set()       # declared by the bindings themselves (the Device::HIP extras and the two YOLO helpers)
+    for folder in ("hip", "hip_lean"):
+        for name in os.listdir(os.path.join(patch_root, folder)):
+            text = open(os.path.join(patch_root, folder, name)).read()
+            for body in re.findall(r"class \w*Extras<Device::HIP>\s*\{(.*?)\n\};", text, flags=re.S):
+                own |= set(re.findall(r"\b\w+_\b", body))
+    own |= {"uploadTruths", "collectCost"}
+    checked = 0
+    for folder in ("hip", "hip_lean"):
+        for name in sorted(os.listdir(os.path.join(patch_root, folder))):
+            layer = {"YoloLayerCommon.h": "YoloLayer.h", "ModelExtras.h": "Model.h"}.get(name, name)
+            known = identifiers(base + engine(layer, os.path.join("cuda", layer)))
+            text = re.sub(r"//[^\n]*", "", open(os.path.join(patch_root, folder, name)).read())
+            members = set(re.findall(r"\b[a-z]\w*_\b", text)) - {"px_hip_status_"}
+            methods = set(re.findall(r"this->(\w+)\(", text)) | set(re.findall(r"\bnet\.(\w+)\(", text))
+            for m in sorted(members | methods):
+                if m in own or m in ("deferHead", "normGroupsFor", "noteNormGroups", "takeNormGroups", "overwritten",
+                                     "registerParameters", "updateAll"):
+                    continue
+                assert m in known, "%s/%s names `%s`, which the engine's %s does not have" % (folder, name, m, layer)
+                checked += 1
+    assert checked > 60
+    stub = re.sub(r"//[^\n]*", "", open(os.path.join(ROOT, "tests", "host", "reference_stub.h")).read())
+    headers = [n for n in os.listdir(os.path.join(REFERENCE, "include")) if n.endswith(".h")]
+    headers += [os.path.join("cuda", n) for n in os.listdir(os.path.join(REFERENCE, "include", "cuda")) if n.endswith(".h")]
+    everything = identifiers(engine(*headers))
+    for m in sorted(set(re.findall(r"\b[a-z]\w*_\b", stub))):
+        assert m in everything, "the stand-in declares `%s`, which no header of the engine has" % m
