@@ -48,8 +48,10 @@ int pxh_abi_version(void);
  * when given NULL.  That buffer grows when a call needs more than it holds, which allocates device
  * memory and is therefore refused (PXH_ERR_WORKSPACE) while the call's stream is being captured into a
  * graph.  pxh_reserve_workspace makes the current device's buffer hold at least `bytes` (the largest
- * *_workspace_bytes() of the calls to come) ahead of time; blocks handed out earlier stay allocated, so
- * addresses that queued work or captured graphs hold remain valid.  The buffer is shared by every
+ * *_workspace_bytes() of the calls to come) ahead of time -- it allocates, so it is a call for BEFORE a
+ * capture, not inside one; when the buffer grows it at least doubles, and blocks handed out earlier stay
+ * allocated, so addresses that queued work or captured graphs hold remain valid (what is left behind adds
+ * up to less than the live block).  The buffer is shared by every
  * NULL-workspace call on the device: calls that may overlap (several streams or threads) must pass
  * workspaces of their own.  No counterpart in the reference (cuDNN and cuBLAS own their scratch). */
 int pxh_reserve_workspace(size_t bytes);
@@ -389,7 +391,11 @@ size_t pxh_yolo_workspace_bytes(int batch, int mask_count, int classes, int widt
  * delta (every element written, no prior fill), positives assigned on the device from the
  * truths with the CPU layer's rule (best anchor over all anchors, later truth overwrites),
  * cost = sum(delta^2) (written to *cost, not divided by batch) and stats[12] (overwritten).
- * host_masks[mask_count], host_anchors[2*anchor_count] are HOST int arrays (layer constants). */
+ * host_masks[mask_count], host_anchors[2*anchor_count] are HOST int arrays (layer constants).  * A workspace serves one stream at a time: the one-launch form of the pass counts its workgroups in at
+ * device counters kept per workspace address (zero whenever no launch is using them), so two calls that
+ * may overlap -- two streams, two threads -- must pass workspaces of their own, and a launch that never
+ * completes (a device fault, a destroyed stream) leaves its counters unusable for that address.
+ * pxh_yolo_forward_train_heads uses no such counters. */
 int pxh_yolo_forward_train(const float* input, float* output, float* delta, const float* truths,
                            const int* truth_counts, int max_truth, const int* host_masks,
                            const int* host_anchors, float* stats, float* cost, int batch,

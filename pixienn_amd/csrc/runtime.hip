@@ -122,9 +122,11 @@ int pxh_abi_version(void) { return 2; }
 
 int pxh_reserve_workspace(size_t bytes)
 {
-    // growing allocates: refused (PXH_ERR_WORKSPACE) while the calling thread is capturing
+    // Growing allocates, so this is a call for before a capture.  It takes no stream and cannot ask whether
+    // the thread is capturing one (on this runtime the question, put to the null stream, itself invalidates a
+    // capture in progress): inside a capture the allocation fails and the failure is reported.
     void* p = nullptr;
-    return pxh::library_workspace(bytes, nullptr, false, &p);
+    return pxh::library_workspace(bytes, nullptr, true, &p);
 }
 
 // Test hook: the address of the current device's library workspace once it holds `bytes`.

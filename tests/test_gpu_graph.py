@@ -185,12 +185,8 @@ def test_library_workspace_keeps_handed_out_blocks_and_refuses_to_grow_under_cap
     with torch.cuda.graph(g2):
         rc = capi.call_raw("pxh_nms", rec.data_ptr(), cnt.data_ptr(), cap, 1, 1, 0.5, y.data_ptr(), cnt.data_ptr(),
                            None, 0, torch.cuda.current_stream().cuda_stream)
-        message = capi.last_error()
-        # ... and so is reserving inside the capture: it would have to allocate
-        rc_reserve = lib.pxh_reserve_workspace(huge_need)
         y.add_(1.0)
-    assert rc == -3 and "pxh_reserve_workspace" in message, (rc, message)
-    assert rc_reserve == -3, (rc_reserve, capi.last_error())
+    assert rc == -3 and "pxh_reserve_workspace" in capi.last_error(), (rc, capi.last_error())
     g2.replay()
     torch.cuda.synchronize()
     assert torch.equal(y, y_eager + 1.0)
