@@ -281,12 +281,14 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
 
     def forward(_, first_writer=False, fills_together=False, heads_apart=False):
         n = 0
-        cleared = [t["d"] for i, t in enumerate(T) if not absorbed(i) and not (first_writer and i in overwritten)]
+        # (a head's delta is not cleared either: the training pass writes every element of it)
+        cleared = [t["d"] for i, t in enumerate(T) if not absorbed(i) and layers[i]["type"] != "yolo"
+                   and not (first_writer and i in overwritten)]
         if fills_together:      # the deltas of all layers cleared at the start of the pass, in a few launches
             ops.fill_multi(cleared, 0.0)
         n += len(cleared)
         for i, (l, t) in enumerate(zip(layers, T)):
-            if not fills_together and not absorbed(i) and not (first_writer and i in overwritten):
+            if not fills_together and not absorbed(i) and l["type"] != "yolo" and not (first_writer and i in overwritten):
                 ops.fill(t["d"], 0.0)
             kind = l["type"]
             if kind == "conv" and l["bn"]:

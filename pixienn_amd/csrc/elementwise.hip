@@ -950,7 +950,8 @@ int launch_mix(size_t n, const float* const* in, float* const* out, hipStream_t 
     MixOp<R, W> op{};
     for (int i = 0; i < R; ++i) op.in[i] = in[i];
     for (int i = 0; i < W; ++i) op.out[i] = out[i];
-    return launch_stream("pxh_debug_stream_mix", n, true, 4 * (R + W), op, s);
+    // launched as the library launches an operation of that many streams (two vectors per lane for 4 + 4)
+    return launch_stream("pxh_debug_stream_mix", n, true, 4 * (R + W), op, s, kStreamingBytes, R + W >= 8);
 }
 
 }  // namespace
@@ -1355,7 +1356,7 @@ int pxh_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch,
     op.c2 = 1.0f - powf(beta2, static_cast<float>(t));
     op.lr = lr; op.eps = eps; op.apply_decay = apply_decay;
     return launch_stream("pxh_adam_update", n, aligned16(w) && aligned16(d) && aligned16(m) && aligned16(v), 32, op,
-                         as_stream(stream));
+                         as_stream(stream), kStreamingBytes, true);
 }
 
 int pxh_adam_update_multi(int count, float* const* w, float* const* d, float* const* m, float* const* v, const size_t* n,

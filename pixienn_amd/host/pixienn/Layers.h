@@ -884,7 +884,8 @@ public:
 
     void forward(const V& input) override
     {
-        Layer::forward(input);
+        // no zero-fill of delta_ (Layer::forward): the training pass writes every element of it
+        cost_ = 0.0f;
         checkInput(input, "YoloLayer");
         const auto& c = context();
         const int masks = static_cast<int>(mask_.size());
