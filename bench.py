@@ -658,10 +658,19 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
                                                                 1e30, 1e30), 10, rotate=rot)
         add("bn_bwd_clipped(leaky)", "%dx%dx%d^2" % (N, c, s), (16 if one_launch else 20) * e, ms_c,
             "rescale + clip decided in the backward's own first pass; plain backward %.4f ms" % ms_b)
+        if (c, s) in ((64, 304), (256, 76)):
+            # ... and when the norm is beyond the threshold (every call rescales; the clamp is far away): the sums
+            # of the first pass still serve, multiplied by the factor; the one-launch form rewrites dx once more
+            ms_r = timer.time(lambda i: ops.bn_act_backward_clipped(d[i], x[i], mean, var, scale, bias, su, bu, "leaky",
+                                                                    1e-6, 1e30), 10, rotate=rot)
+            add("bn_bwd_clipped(rescaling)", "%dx%dx%d^2" % (N, c, s), ((16 if one_launch else 20) + (8 if one_launch else 0)) * e,
+                ms_r, "the delta is rescaled on every call; as two calls this costs a 12 B/elem rescale_clip + the backward")
         if one_launch:
             # both conventions in the row: the bytes this launch moves (frac above) and the 12 / 20 B per
             # element that the three-launch form moves, which is the figure the per-kernel bar was written for
-            for row, per_elem, ms in ((rows[-3], 12, ms_f), (rows[-2], 20, ms_b)):
+            fwd_row = [r for r in rows if r["kernel"] == "bn_train_fwd(leaky)"][-1]
+            bwd_row = [r for r in rows if r["kernel"] == "bn_bwd(leaky)"][-1]
+            for row, per_elem, ms in ((fwd_row, 12, ms_f), (bwd_row, 20, ms_b)):
                 row["three_launch_bytes_MB"] = round(per_elem * e / 1e6, 1)
                 row["frac_of_peak_at_three_launch_bytes"] = round(per_elem * e / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 3)
         bn_ms[(c, s)] = (ms_f, ms_b, count)

@@ -92,6 +92,51 @@ def test_bn_training_largest_shape(ops, oracle):
     assert float((dx * xhat).sum(dim=(0, 2, 3)).abs().max()) <= 2e-5 * norm, "dx must be orthogonal to x_hat"
 
 
+@pytest.mark.parametrize("shape", [(16, 32, 608), (16, 256, 76), (16, 1024, 19)])
+def test_bn_backward_clipped_at_training_shapes(ops, shape):
+    """The rescale + clip folded into the backward at configs[4] shapes -- three launches with 11 552 norm partials,
+    the one-launch form with part of the slice in LDS, the scalar one-launch form at 1024 channels -- against the
+    two-call sequence it replaces (pxh_rescale_clip, then pxh_bn_act_backward; each held to the checker elsewhere):
+    to the bit when nothing changes, within 1e-5 when the delta is rescaled or clamped."""
+    import torch
+    N, C, S = shape
+    x = device_normal((N, C, S, S), 21) * 1.3 + 0.2
+    scale, bias, rmean, rvar = (gpu(a) for a in wl.bn_params(2101, C))
+    mean = torch.zeros(C, device="cuda"); var = torch.zeros(C, device="cuda")
+    y = torch.empty_like(x)
+    ops.bn_train_act_forward(x, y, mean, var, rmean, rvar, scale, bias, "leaky")
+    del y
+    delta = device_normal((N, C, S, S), 22)
+    spiky = delta.clone()
+    spiky[:, 0] *= 20.0
+    norm = float(torch.linalg.vector_norm(delta.double()))
+    spiky_norm = float(torch.linalg.vector_norm(spiky.double()))
+    peak = float(delta.abs().max())
+    cases = [("nothing changes", delta, 2.0 * norm, 2.0 * peak), ("rescale only", delta, 0.37 * norm, 0.0),
+             ("rescale and clamp", delta, 0.5 * norm, 0.3),
+             ("clamp in one channel only", spiky, 2.0 * spiky_norm, 1.5 * peak)]
+    for name, d0, threshold, clip in cases:
+        want = d0.clone(); su_w = torch.zeros(C, device="cuda"); bu_w = torch.zeros(C, device="cuda")
+        norm_w = torch.zeros(1, device="cuda")
+        ops.rescale_clip(want, threshold, clip, norm_out=norm_w)
+        size = float(want.double().pow(2).mean().sqrt())
+        ops.bn_act_backward(want, x, mean, var, scale, bias, su_w, bu_w, "leaky")
+        got = d0.clone(); su = torch.zeros(C, device="cuda"); bu = torch.zeros(C, device="cuda")
+        norm_g = torch.zeros(1, device="cuda")
+        ops.bn_act_backward_clipped(got, x, mean, var, scale, bias, su, bu, "leaky", threshold, clip, norm_out=norm_g)
+        what = "%s %s" % (shape, name)
+        assert_close(host(norm_g), host(norm_w), 1e-6, 1e-30, what + " norm")
+        if name == "nothing changes":
+            assert torch.equal(got, want) and torch.equal(su, su_w) and torch.equal(bu, bu_w), what
+        else:
+            sums = float(np.sqrt(N * S * S)) * size
+            assert_close(host(su), host(su_w), 1e-5, sums, what + " scale updates")
+            assert_close(host(bu), host(bu_w), 1e-5, sums, what + " bias updates")
+            worst = float(((got - want).abs() / want.abs().clamp_min(0.1 * size)).max())
+            assert worst <= 1e-5, (what, worst)
+        del want, got
+
+
 def test_maxpool_largest_shape(ops, oracle):
     """16 x 64 x 304^2: whole tensor against the checker and against an independent routine."""
     import torch
