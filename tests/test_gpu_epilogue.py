@@ -146,7 +146,10 @@ TRAIN_SHAPES = [(4, 8, 52 * 52), (3, 16, 361), (16, 5, 169), (2, 3, 4096 + 512),
                 # scalar and 128-bit; then the same channel counts with slices that do not fit
                 (3, 96, 361), (2, 100, 1444), (16, 128, 1444), (4, 96, 2047), (4, 96, 5001), (16, 97, 76 * 76),
                 # the large single-launch form (part of the slice in LDS), above and below 128 channels
-                (8, 192, 4800), (9, 100, 4096 + 8)]
+                (8, 192, 4800), (9, 100, 4096 + 8),
+                # scalar slices with 512 and 1024 channels: the single-launch path with workgroups of half the size
+                # (forward from 512 channels, backward from 1024), a few values per thread and close to its sixteen
+                (2, 512, 361), (5, 1024, 361), (15, 1030, 529)]
 
 
 @pytest.mark.parametrize("act", ["leaky", "mish", "linear", "swish", "logistic"])
