@@ -1151,13 +1151,17 @@ __device__ __forceinline__ void resident_bwd_channel(const ResidentBwdArgs& a, c
     Pack<V> d[R];
     float fa = 0.0f, fb = 0.0f;
     [[maybe_unused]] float fq = 0.0f, peak = 0.0f;
-    // Two shapes of the same two passes.  The large form (part of the slice in LDS) is bound by its
-    // loads and takes them in groups with no branch in between; the small form does more arithmetic
-    // per byte than it waits, and is fastest when a step past the end of the slice is skipped outright.
-    // The large form: no branch around the loads (see the forward kernel), lanes past the end read the
-    // first vector; kGroup steps at a time, their loads go out together, then each is used as it arrives.
-    constexpr int kGroup = 4;
-    static_assert(L == 0 || (R % kGroup == 0 && L % kGroup == 0), "steps come in whole groups");
+    // Two shapes of the first pass.  Grouped: no branch around the loads (see the forward kernel), lanes
+    // past the end read the first vector; kGroup steps at a time, their loads go out together, then each
+    // is used as it arrives.  The large form (part of the slice in LDS) is bound by its loads and takes
+    // them so in groups of four; the scalar form in groups of eight (behind a branch a lane waits for
+    // each step's loads before it asks for the next: six trips to memory one after the other at
+    // 16 x 256 x 19^2, 10.4 us against 8.8).  The 128-bit form without an LDS part is held to 64
+    // registers, where a group of two already spills (18.3 against 16.4 us at 16 x 256 x 38^2): it skips a step
+    // past the end of the slice outright, as every form does in the second pass, which finds x in the cache.
+    constexpr int kGroup = L > 0 ? 4 : 8;
+    constexpr bool kGrouped = L > 0 || V == 1;
+    static_assert(!kGrouped || (R % kGroup == 0 && L % kGroup == 0), "steps come in whole groups");
     // `lane` is the thread index; the second pass takes it through an empty asm statement, so that
     // its addresses are formed again there instead of being held in registers (48 of them) from the first
     [[maybe_unused]] uint32_t lane = threadIdx.x;
@@ -1177,7 +1181,7 @@ __device__ __forceinline__ void resident_bwd_channel(const ResidentBwdArgs& a, c
         if constexpr (ACT != PXH_LINEAR) t = t * act_grad<ACT>(pre);
         return t;
     };
-    if constexpr (L > 0) {
+    if constexpr (kGrouped) {
         // delta * f'(pre) in dv, and the step's share of the sums
         const auto take = [&](int r, Pack<V>& dv, const Pack<V>& xv, const Pack<V>& pv) {
             const bool valid = element(r) < a.g.per_channel;
@@ -1253,14 +1257,6 @@ __device__ __forceinline__ void resident_bwd_channel(const ResidentBwdArgs& a, c
                 }
                 if (r < R) d[r < R ? r : 0] = dv;
                 else *resident_lds_slot<V, R>(resident_lds, r) = dv;
-            }
-            // the scalar form with the norm's two extra sums: the steps in two halves, so that half of
-            // their loads are in flight at a time and the lane stays within its 64 registers
-            if constexpr (MODE == kFirst && V == 1) {
-                if (r == (R + L) / 2) {
-                    asm volatile("" : "+v"(fa), "+v"(fb), "+v"(fq), "+v"(peak));
-                    __builtin_amdgcn_sched_barrier(0);
-                }
             }
         }
     }
