@@ -112,6 +112,30 @@ int pxh_bn_train_act_forward(const float* x, float* y, float* pre_activation, fl
                              int batch, int channels, int spatial, int activation,
                              void* workspace, size_t workspace_bytes, void* stream);
 
+/* A convolution's epilogue with the ShortcutLayer that follows it in the same pass, for a shortcut with
+ * a linear activation over tensors of one shape (every residual block of the shipped YOLOv3 graphs):
+ *   y = alpha * act(pre) + beta * from      (two products and one sum, each rounded)
+ * i.e. what pxh_shortcut_forward(in = the epilogue's result, from, out = y, alpha, beta, PXH_LINEAR) would
+ * leave, without the epilogue's result ever reaching memory: the shortcut's pass (12 bytes per element)
+ * becomes one more stream read by the epilogue (4).  Everything else -- statistics, rolling averages,
+ * x_saved, x_norm, pre_activation (the CONVOLUTION's pre-activation) -- as in the call without the
+ * shortcut.  `from` may be y itself (read before it is written, element by element) but no other output.
+ * The layer's own output is not materialised: only for a layer whose output nothing but the shortcut
+ * reads (a route or a second shortcut that names the convolution needs the two separate calls), and
+ * the layer's backward must not need its output (pxh_bn_act_backward recomputes from x).  In the
+ * backward pass the convolution's delta is alpha times the shortcut's.
+ * Replaces include/cuda/ConvLayer.h:284-307 followed by include/cuda/ShortcutLayer.h:23-37. */
+int pxh_bn_train_act_shortcut_forward(const float* x, float* y, float* pre_activation, float* x_saved,
+                                      float* x_norm, float* mean, float* var, float* rolling_mean,
+                                      float* rolling_var, const float* scale, const float* bias,
+                                      const float* from, float alpha, float beta, int batch, int channels,
+                                      int spatial, int activation, void* workspace, size_t workspace_bytes,
+                                      void* stream);
+/* The same for inference, on constants folded by pxh_bn_fold (pxh_bn_folded_act_forward + shortcut). */
+int pxh_bn_folded_act_shortcut_forward(const float* x, float* y, float* pre_activation, const void* folded,
+                                       const float* from, float alpha, float beta, int batch, int channels,
+                                       int spatial, int activation, void* stream);
+
 /* pxh_bn_train_act_forward for callers that cannot allocate device memory and have no workspace
  * to pass (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc): same
  * arguments without the workspace, same kernels, same results.  The partial sums and per-channel

@@ -105,7 +105,20 @@ struct EpilogueArgs {
     FastDiv by_spatial;
     FastDiv by_channels;
     uint32_t total;
+    // the shortcut that follows the layer, taken into the same pass (else null): what is stored in y is
+    // res_alpha * act(pre) + res_beta * residual, the two products and the sum each rounded
+    const float* residual;
+    float res_alpha, res_beta;
 };
+
+// The linear shortcut on top of an activation's result (cuda/ShortcutLayer.h:23-37 with a linear
+// activation: alpha * input + beta * from).
+__device__ __forceinline__ float with_residual(float y, float from, float alpha, float beta)
+{
+    const float pa = alpha * y;
+    const float pb = beta * from;
+    return pa + pb;
+}
 
 template<bool BN>
 __device__ __forceinline__ FoldCoef fetch_coef(const EpilogueArgs& a, uint32_t c)
@@ -134,18 +147,23 @@ __device__ __forceinline__ float pre_value(float x, const FoldCoef& k, float& xn
 // One 128-bit vector per lane over the flat tensor.  A lane finds its plane with one
 // multiply-high division and loads that channel's folded constants (a 32-byte, cache-resident
 // broadcast); the rare vector that straddles two planes loads the next channel's as well.
-template<int ACT, bool BN, bool NT>
-__global__ __launch_bounds__(kBlock) void epilogue_fwd_kernel(EpilogueArgs a)
+template<int ACT, bool BN, bool NT, bool RES>
+__device__ __forceinline__ void epilogue_fwd_body(const EpilogueArgs& a)
 {
     const uint32_t e = (blockIdx.x * static_cast<uint32_t>(kBlock) + threadIdx.x) * 4;
     if (e >= a.total) return;
     const bool full = e + 3 < a.total;
     Pack<4> xin;
+    [[maybe_unused]] Pack<4> rin;
     if (full) {
         xin = ld<4, NT>(a.x, e);
+        if constexpr (RES) rin = ld<4, NT>(a.residual, e);
     } else {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) xin.v[k] = (e + k < a.total) ? a.x[e + k] : 0.0f;
+        for (int k = 0; k < 4; ++k) {
+            xin.v[k] = (e + k < a.total) ? a.x[e + k] : 0.0f;
+            if constexpr (RES) rin.v[k] = (e + k < a.total) ? a.residual[e + k] : 0.0f;
+        }
     }
     const uint32_t hw = a.by_spatial.d;
     uint32_t plane, r, q, c;
@@ -194,6 +212,10 @@ __global__ __launch_bounds__(kBlock) void epilogue_fwd_kernel(EpilogueArgs a)
             ++rr;
         }
     }
+    if constexpr (RES) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) yo.v[j] = with_residual(yo.v[j], rin.v[j], a.res_alpha, a.res_beta);
+    }
     if (full) {
         if (a.x_saved) st<4, NT>(a.x_saved, e, xin);
         if (BN && a.x_norm) st<4, NT>(a.x_norm, e, no);
@@ -207,6 +229,19 @@ __global__ __launch_bounds__(kBlock) void epilogue_fwd_kernel(EpilogueArgs a)
             a.y[e + j] = yo.v[j];
         }
     }
+}
+
+template<int ACT, bool BN, bool NT>
+__global__ __launch_bounds__(kBlock) void epilogue_fwd_kernel(EpilogueArgs a)
+{
+    epilogue_fwd_body<ACT, BN, NT, false>(a);
+}
+
+// The same pass with the shortcut that follows the layer: one more stream read, no tensor in between.
+template<int ACT, bool BN, bool NT>
+__global__ __launch_bounds__(kBlock) void epilogue_shortcut_fwd_kernel(EpilogueArgs a)
+{
+    epilogue_fwd_body<ACT, BN, NT, true>(a);
 }
 
 // Pointers that are not 16-byte aligned: one element per lane.
@@ -225,7 +260,9 @@ __global__ __launch_bounds__(kBlock) void epilogue_fwd_scalar_kernel(EpilogueArg
     if (a.x_saved) a.x_saved[e] = x;
     if (BN && a.x_norm) a.x_norm[e] = xn;
     if (a.pre) a.pre[e] = pre;
-    a.y[e] = act_apply<ACT>(pre);
+    float y = act_apply<ACT>(pre);
+    if (a.residual) y = with_residual(y, a.residual[e], a.res_alpha, a.res_beta);
+    a.y[e] = y;
 }
 
 int check_shape(const char* who, int batch, int channels, int spatial, uint32_t* total)
@@ -247,14 +284,17 @@ int launch_epilogue_fwd(const char* who, EpilogueArgs a, int activation, hipStre
 {
     // the walk across a plane boundary handles any plane size, including single elements
     const bool vec = aligned16(a.x) && aligned16(a.y) && aligned16(a.pre) && aligned16(a.x_saved) &&
-                     aligned16(a.x_norm);
-    // bytes this launch moves: x in, y out, plus each materialised extra output
-    const size_t streams = 2 + (a.pre ? 1 : 0) + (a.x_saved ? 1 : 0) + (a.x_norm ? 1 : 0);
+                     aligned16(a.x_norm) && aligned16(a.residual);
+    // bytes this launch moves: x in, y out, plus each materialised extra output and the shortcut's source
+    const size_t streams = 2 + (a.pre ? 1 : 0) + (a.x_saved ? 1 : 0) + (a.x_norm ? 1 : 0) + (a.residual ? 1 : 0);
     const bool nt = static_cast<size_t>(a.total) * 4 * streams >= kStreamingBytes;
     const bool known = dispatch_activation(activation, [&]<int ACT>() {
         if (vec) {
             const dim3 grid(grid_for(a.total, static_cast<size_t>(kBlock) * 4));
-            if (nt) hipLaunchKernelGGL((epilogue_fwd_kernel<ACT, BN, true>), grid, dim3(kBlock), 0, stream, a);
+            if (a.residual) {
+                if (nt) hipLaunchKernelGGL((epilogue_shortcut_fwd_kernel<ACT, BN, true>), grid, dim3(kBlock), 0, stream, a);
+                else hipLaunchKernelGGL((epilogue_shortcut_fwd_kernel<ACT, BN, false>), grid, dim3(kBlock), 0, stream, a);
+            } else if (nt) hipLaunchKernelGGL((epilogue_fwd_kernel<ACT, BN, true>), grid, dim3(kBlock), 0, stream, a);
             else hipLaunchKernelGGL((epilogue_fwd_kernel<ACT, BN, false>), grid, dim3(kBlock), 0, stream, a);
         } else {
             hipLaunchKernelGGL((epilogue_fwd_scalar_kernel<ACT, BN>), dim3(grid_for(a.total, kBlock)),
@@ -950,6 +990,9 @@ struct ResidentFwdArgs {
     const float* scale;
     const float* bias;
     ResidentGeom g;
+    // the shortcut that follows the layer (else null), as in EpilogueArgs
+    const float* residual;
+    float res_alpha, res_beta;
 };
 
 // A thread keeps R vectors in registers and L more in LDS (dynamic, L * kResidentThreads vectors:
@@ -961,8 +1004,8 @@ __device__ __forceinline__ Pack<V>* resident_lds_slot(float* lds, int r)
 }
 
 // V = 4 needs spatial % 4 == 0 and 16-byte aligned tensors.  R + L vectors per thread at most.
-template<int ACT, int V, int R, int L, int T = kResidentThreads>
-__global__ __launch_bounds__(T) void bn_resident_fwd_kernel(ResidentFwdArgs a)
+template<int ACT, int V, int R, int L, int T = kResidentThreads, bool RES = false>
+__global__ __launch_bounds__(T, L == 0 && V * R <= 32 ? 8 : 4) void bn_resident_fwd_kernel(ResidentFwdArgs a)
 {
     static_assert(L == 0 || T == kResidentThreads, "the LDS part is laid out for the full workgroup");
     extern __shared__ __align__(16) float resident_lds[];
@@ -1024,8 +1067,7 @@ __global__ __launch_bounds__(T) void bn_resident_fwd_kernel(ResidentFwdArgs a)
     }
     __syncthreads();
     const FoldCoef k = shared_coef;
-#pragma unroll
-    for (int r = 0; r < R + L; ++r) {
+    const auto apply = [&](int r, [[maybe_unused]] const Pack<V>& from) {
         const uint32_t e = (r * T + threadIdx.x) * V;
         if (e < a.g.per_channel) {
             const size_t where = a.g.at(c, e);
@@ -1036,12 +1078,32 @@ __global__ __launch_bounds__(T) void bn_resident_fwd_kernel(ResidentFwdArgs a)
                 xn.v[q] = normalize(t.v[q], k);
                 pre.v[q] = affine(xn.v[q], k);
                 out.v[q] = act_apply<ACT>(pre.v[q]);
+                if constexpr (RES) out.v[q] = with_residual(out.v[q], from.v[q], a.res_alpha, a.res_beta);
             }
             if (a.x_saved) st<V, true>(a.x_saved, where, t);
             if (a.x_norm) st<V, true>(a.x_norm, where, xn);
             if (a.pre) st<V, true>(a.pre, where, pre);
             st<V, true>(a.y, where, out);
         }
+    };
+    if constexpr (RES) {
+        // the shortcut's source four steps at a time, no branch around its loads (see above)
+        constexpr int kGroup = 4;
+        static_assert((R + L) % kGroup == 0, "steps come in whole groups");
+#pragma unroll
+        for (int first = 0; first < R + L; first += kGroup) {
+            Pack<V> from[kGroup];
+#pragma unroll
+            for (int i = 0; i < kGroup; ++i) {
+                const uint32_t e = element(first + i);
+                from[i] = ld<V, true>(a.residual, a.g.at(c, e < a.g.per_channel ? e : 0u));
+            }
+#pragma unroll
+            for (int i = 0; i < kGroup; ++i) apply(first + i, from[i]);
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R + L; ++r) apply(r, Pack<V>{});
     }
 }
 
@@ -1491,13 +1553,19 @@ int launch_stats(const float* x, float* mean, float* var, float* rolling_mean, f
     return check_launch("bn_stats_finish");
 }
 
+// The linear shortcut taken into a forward pass (from == nullptr: none).
+struct Residual {
+    const float* from = nullptr;
+    float alpha = 1.0f, beta = 1.0f;
+};
+
 // BN training forward + activation.  `get_workspace(need, &ws)` is asked for the `need` bytes of the
 // three-launch form only when the shape does not take the one-launch form, which uses none.
 template<typename GetWorkspace>
 int bn_train_forward(const char* who, const float* x, float* y, float* pre_activation, float* x_saved, float* x_norm,
                      float* mean, float* var, float* rolling_mean, float* rolling_var, const float* scale,
                      const float* bias, int batch, int channels, int spatial, int activation,
-                     GetWorkspace&& get_workspace, void* stream)
+                     GetWorkspace&& get_workspace, void* stream, const Residual& res = Residual{})
 {
     if (!x || !y || !mean || !var || !rolling_mean || !rolling_var || !scale || !bias)
         return fail_invalid("%s: null pointer", who);
@@ -1508,28 +1576,39 @@ int bn_train_forward(const char* who, const float* x, float* y, float* pre_activ
     hipStream_t s = as_stream(stream);
     {
         const bool vec = spatial % 4 == 0 && aligned16(x) && aligned16(y) && aligned16(pre_activation) &&
-                         aligned16(x_saved) && aligned16(x_norm);
+                         aligned16(x_saved) && aligned16(x_norm) && aligned16(res.from);
         const int per_thread = resident_vectors(batch, channels, spatial, vec);
         if (per_thread) {
             const ResidentFwdArgs r{ x, y, pre_activation, x_saved, x_norm, mean, var, rolling_mean, rolling_var,
-                                     scale, bias, resident_geom(batch, channels, spatial) };
-            const bool narrow = resident_narrow(batch, channels, spatial, vec, false);
+                                     scale, bias, resident_geom(batch, channels, spatial), res.from, res.alpha, res.beta };
+            // (with the shortcut's source on top, sixteen values per lane no longer fit the registers of four
+            // workgroups per compute unit: that form keeps the full workgroups)
+            const bool narrow = !res.from && resident_narrow(batch, channels, spatial, vec, false);
             const dim3 grid(channels), block(narrow ? kResidentNarrowThreads : kResidentThreads);
             int large_lds_rc = PXH_OK;
-            const bool known = dispatch_activation(activation, [&]<int ACT>() {
-                if (narrow) {
-                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 1, kResidentNarrowVectors, 0, kResidentNarrowThreads>),
-                                       grid, block, 0, s, r);
-                } else if (per_thread > kResidentVectors) {
-                    auto kernel = bn_resident_fwd_kernel<ACT, 4, kResidentLargeRegs, kResidentLargeLds>;
+            const auto launch = [&]<int ACT, bool RES>() {
+                constexpr int kT = kResidentThreads;
+                if constexpr (!RES) {
+                    if (narrow) {
+                        hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 1, kResidentNarrowVectors, 0, kResidentNarrowThreads>),
+                                           grid, block, 0, s, r);
+                        return;
+                    }
+                }
+                if (per_thread > kResidentVectors) {
+                    auto kernel = bn_resident_fwd_kernel<ACT, 4, kResidentLargeRegs, kResidentLargeLds, kT, RES>;
                     large_lds_rc = allow_large_lds(reinterpret_cast<const void*>(kernel));
                     if (large_lds_rc == PXH_OK)
                         hipLaunchKernelGGL(kernel, grid, block, kResidentLargeLdsBytes, s, r);
                 } else if (vec) {
-                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 4, kResidentVectors, 0>), grid, block, 0, s, r);
+                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 4, kResidentVectors, 0, kT, RES>), grid, block, 0, s, r);
                 } else {
-                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 1, kResidentVectors, 0>), grid, block, 0, s, r);
+                    hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 1, kResidentVectors, 0, kT, RES>), grid, block, 0, s, r);
                 }
+            };
+            const bool known = dispatch_activation(activation, [&]<int ACT>() {
+                if (res.from) launch.template operator()<ACT, true>();
+                else launch.template operator()<ACT, false>();
             });
             if (!known) return fail_invalid("%s: unknown activation %d", who, activation);
             if (large_lds_rc) return large_lds_rc;
@@ -1546,6 +1625,7 @@ int bn_train_forward(const char* who, const float* x, float* y, float* pre_activ
     a.x = x; a.y = y; a.pre = pre_activation; a.x_saved = x_saved; a.x_norm = x_norm;
     a.table = table;
     a.by_spatial = FastDiv(spatial); a.by_channels = FastDiv(channels);
+    a.residual = res.from; a.res_alpha = res.alpha; a.res_beta = res.beta;
     return launch_epilogue_fwd<true>(who, a, activation, s);
 }
 
@@ -1650,6 +1730,41 @@ int pxh_bn_train_act_forward(const float* x, float* y, float* pre_activation, fl
         "pxh_bn_train_act_forward", x, y, pre_activation, x_saved, x_norm, mean, var, rolling_mean, rolling_var,
         scale, bias, batch, channels, spatial, activation,
         [&](size_t need, void** ws) { return resolve_workspace(workspace, workspace_bytes_given, need, ws, as_stream(stream)); }, stream);
+}
+
+int pxh_bn_train_act_shortcut_forward(const float* x, float* y, float* pre_activation, float* x_saved, float* x_norm,
+                                      float* mean, float* var, float* rolling_mean, float* rolling_var,
+                                      const float* scale, const float* bias, const float* from, float alpha, float beta,
+                                      int batch, int channels, int spatial, int activation, void* workspace,
+                                      size_t workspace_bytes_given, void* stream)
+{
+    const char* who = "pxh_bn_train_act_shortcut_forward";
+    if (!from) return fail_invalid("%s: null pointer (from)", who);
+    if (from == x_saved || from == x_norm || from == pre_activation)
+        return fail_invalid("%s: from must not alias an output other than y", who);
+    return bn_train_forward(
+        who, x, y, pre_activation, x_saved, x_norm, mean, var, rolling_mean, rolling_var, scale, bias, batch, channels,
+        spatial, activation,
+        [&](size_t need, void** ws) { return resolve_workspace(workspace, workspace_bytes_given, need, ws, as_stream(stream)); },
+        stream, Residual{ from, alpha, beta });
+}
+
+int pxh_bn_folded_act_shortcut_forward(const float* x, float* y, float* pre_activation, const void* folded,
+                                       const float* from, float alpha, float beta, int batch, int channels,
+                                       int spatial, int activation, void* stream)
+{
+    const char* who = "pxh_bn_folded_act_shortcut_forward";
+    if (!x || !y || !folded || !from) return fail_invalid("%s: null pointer", who);
+    if (!aligned16(folded)) return fail_invalid("%s: folded must be 16-byte aligned", who);
+    if (from == pre_activation) return fail_invalid("%s: from must not alias an output other than y", who);
+    EpilogueArgs a{};
+    int rc = check_shape(who, batch, channels, spatial, &a.total);
+    if (rc) return rc;
+    a.x = x; a.y = y; a.pre = pre_activation;
+    a.table = static_cast<const FoldCoef*>(folded);
+    a.by_spatial = FastDiv(spatial); a.by_channels = FastDiv(channels);
+    a.residual = from; a.res_alpha = alpha; a.res_beta = beta;
+    return launch_epilogue_fwd<true>(who, a, activation, as_stream(stream));
 }
 
 int pxh_bn_train_act_forward_static(const float* x, float* y, float* pre_activation, float* x_saved, float* x_norm,

@@ -103,6 +103,25 @@ def bn_stats(x, mean, var, workspace=None):
 
 
 # ---------------------------------------------------------------- epilogue backward
+def bn_train_act_shortcut_forward(x, y, mean, var, rolling_mean, rolling_var, scale, bias, activation, from_, alpha=1.0,
+                                  beta=1.0, pre_activation=None, x_saved=None, x_norm=None, workspace=None):
+    """bn_train_act_forward with the linear shortcut that follows the layer: y = alpha*act(pre) + beta*from_."""
+    _chk_all(x, y, mean, var, rolling_mean, rolling_var, scale, bias, from_, pre_activation, x_saved, x_norm)
+    n, c, s = _nchw(x)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("pxh_bn_train_act_shortcut_forward", ptr(x), ptr(y), ptr(pre_activation), ptr(x_saved), ptr(x_norm), ptr(mean),
+         ptr(var), ptr(rolling_mean), ptr(rolling_var), ptr(scale), ptr(bias), ptr(from_), float(alpha), float(beta),
+         n, c, s, act_id(activation), ptr(workspace), wb, _stream())
+
+
+def bn_folded_act_shortcut_forward(x, y, folded, activation, from_, alpha=1.0, beta=1.0, pre_activation=None):
+    """bn_folded_act_forward with the linear shortcut that follows the layer."""
+    _chk_all(x, y, from_, pre_activation)
+    n, c, s = _nchw(x)
+    call("pxh_bn_folded_act_shortcut_forward", ptr(x), ptr(y), ptr(pre_activation), ptr(folded), ptr(from_),
+         float(alpha), float(beta), n, c, s, act_id(activation), _stream())
+
+
 def bn_act_backward(delta, x, mean, var, scale, bias, scale_updates, bias_updates, activation,
                     pre_activation=None, mean_delta=None, var_delta=None, workspace=None):
     _chk_all(delta, x, mean, var, scale, bias, scale_updates, bias_updates, pre_activation, mean_delta, var_delta)
