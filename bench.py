@@ -274,12 +274,25 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
         if l["type"] == "shortcut":
             overwritten.update((i - 1, l["frm"]))
 
+    # convolutions whose output only the shortcut behind them reads (every residual block of YOLOv3): the
+    # shortcut can ride on the convolution's epilogue (pxh_bn_train_act_shortcut_forward), and in the backward
+    # pass the convolution works on the shortcut's delta itself (alpha = 1: the two are the same values)
+    read_elsewhere = set()
+    for i, l in enumerate(layers):
+        if l["type"] == "shortcut":
+            read_elsewhere.add(l["frm"])
+        elif l["type"] == "route":
+            read_elsewhere.update(l["sources"])
+    rides = {i - 1: i for i, l in enumerate(layers)
+             if l["type"] == "shortcut" and layers[i - 1]["type"] == "conv" and layers[i - 1]["bn"]
+             and (i - 1) not in read_elsewhere}
+
     head_table = ops.yolo_head_table([dict(input=T[i - 1]["y"], output=T[i]["y"], delta=T[i]["d"], masks=l["mask"],
                                            width=l["s"], height=l["s"], stats=T[i]["stats"], cost=T[i]["cost"],
                                            ignore_thresh=0.7, truth_thresh=1.0)
                                       for i, l in enumerate(layers) if l["type"] == "yolo"])
 
-    def forward(_, first_writer=False, fills_together=False, heads_apart=False):
+    def forward(_, first_writer=False, fills_together=False, heads_apart=False, shortcut_rides=False):
         n = 0
         # (a head's delta is not cleared either: the training pass writes every element of it)
         cleared = [t["d"] for i, t in enumerate(T) if not absorbed(i) and layers[i]["type"] != "yolo"
@@ -291,7 +304,13 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
             if not fills_together and not absorbed(i) and l["type"] != "yolo" and not (first_writer and i in overwritten):
                 ops.fill(t["d"], 0.0)
             kind = l["type"]
-            if kind == "conv" and l["bn"]:
+            if shortcut_rides and kind == "conv" and i in rides:
+                sc = rides[i]
+                ops.bn_train_act_shortcut_forward(t["x"], T[sc]["y"], t["mean"], t["var"], t["rmean"], t["rvar"],
+                                                  t["scale"], t["bias"], "leaky", T[layers[sc]["frm"]]["y"])
+            elif shortcut_rides and kind == "shortcut" and i - 1 in rides:
+                n -= 1
+            elif kind == "conv" and l["bn"]:
                 ops.bn_train_act_forward(t["x"], t["y"], t["mean"], t["var"], t["rmean"], t["rvar"], t["scale"],
                                          t["bias"], "leaky")
             elif kind == "conv":
@@ -324,11 +343,23 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     groups = {i - 1: ops.norm_groups_like(T[i - 1]["d"]) for i, l in enumerate(layers)
               if l["type"] in ("shortcut", "yolo")}
 
-    def backward(_, first_writer=False, norm_from_writer=False, two_calls=False):
+    def backward(_, first_writer=False, norm_from_writer=False, two_calls=False, shortcut_rides=False):
         n = 0
         for i in reversed(range(len(layers))):
             l, t = layers[i], T[i]
             kind = l["type"]
+            if shortcut_rides and kind == "shortcut" and i - 1 in rides:
+                # the shortcut's own rescale + clip, its delta to the `from` layer (first writer), and
+                # nothing to the convolution in front, which takes this delta as its own
+                ops.rescale_clip(t["d"], 100.0, 10.0)
+                ops.shortcut_backward_first(t["d"], T[l["frm"]]["d"], None, "linear")
+                n += 2
+                continue
+            if shortcut_rides and kind == "conv" and i in rides:
+                ops.bn_act_backward_clipped(T[rides[i]]["d"], t["x"], t["mean"], t["var"], t["scale"], t["bias"],
+                                            t["su"], t["bu"], "leaky", 100.0, 10.0)
+                n += 1
+                continue
             # a convolution's rescale + clip rides on its epilogue's backward (pxh_*_backward_clipped) unless
             # the kernel that wrote its delta last left the norm behind; `two_calls`: as two calls, for comparison
             fused = kind == "conv" and not two_calls and not (norm_from_writer and i in groups)
@@ -410,13 +441,20 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     out["backward_norm_from_writer_ms"] = round(timer.time(lambda i: backward(i, False, True), 3, warm=1), 3)
     out["backward_first_writer_norm_from_writer_ms"] = round(timer.time(lambda i: backward(i, True, True), 3, warm=1), 3)
     out["deltas_with_norm_from_writer"] = len(groups)
-    # the leanest step: first-writer shortcuts, no dead pass in update(), and whichever of the two backward
-    # forms is faster here (since the rescale + clip rides on the convolutions' own backward, leaving the
-    # norm with the writer no longer pays for them)
-    lean_backward = min(("backward_first_writer_ms", "backward_first_writer_norm_from_writer_ms"), key=lambda k: out[k])
+    # the shortcut of a residual block on the epilogue of the convolution in front of it (first-writer forms
+    # everywhere else): no pass of its own forward, and backward the convolution takes the shortcut's delta
+    out["forward_shortcut_in_epilogue_ms"] = round(timer.time(lambda i: forward(i, True, True, shortcut_rides=True), 3, warm=1), 3)
+    out["backward_shortcut_in_epilogue_ms"] = round(timer.time(lambda i: backward(i, True, shortcut_rides=True), 3, warm=1), 3)
+    out["shortcuts_in_epilogue"] = len(rides)
+    # the leanest step: no dead pass in update(), and whichever of the lean forward and backward forms is
+    # faster here (since the rescale + clip rides on the convolutions' own backward, leaving the norm with
+    # the writer no longer pays for them)
+    lean_forward = min(("forward_first_writer_ms", "forward_shortcut_in_epilogue_ms"), key=lambda k: out[k])
+    lean_backward = min(("backward_first_writer_ms", "backward_first_writer_norm_from_writer_ms",
+                         "backward_shortcut_in_epilogue_ms"), key=lambda k: out[k])
+    out["leanest_forward"] = lean_forward
     out["leanest_backward"] = lean_backward
-    out["leanest_total_ms"] = round(out["forward_first_writer_ms"] + out[lean_backward] +
-                                    out["update_without_delta_pass_ms"], 3)
+    out["leanest_total_ms"] = round(out[lean_forward] + out[lean_backward] + out["update_without_delta_pass_ms"], 3)
     out["elements_per_tensor_kind"] = int(sum(N * l["c"] * l["s"] * l["s"] for l in layers))
     del T, w, g, m, v
     torch.cuda.empty_cache()
@@ -652,6 +690,13 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
         add("bn_train_fwd(leaky)", "%dx%dx%d^2" % (N, c, s), (8 if one_launch else 12) * e, ms_f,
             "one launch: x read once, 8B per elem (three launches move 12)" if one_launch
             else "stats 4B + apply 8B per elem; x kept")
+        if (c, s) in [(sc, ss) for sc, ss, _ in wl.YOLOV3_SHORTCUT_SHAPES]:
+            # the residual block's shortcut in the same pass: one more stream read (the block's input, here `d`),
+            # against this row + the shortcut's own 12 B/elem pass
+            ms_s = timer.time(lambda i: ops.bn_train_act_shortcut_forward(x[i], y[i], mean, var, rmean, rvar, scale,
+                                                                          bias, "leaky", d[i]), 10, rotate=rot)
+            add("bn_train_fwd+shortcut(leaky)", "%dx%dx%d^2" % (N, c, s), (12 if one_launch else 16) * e, ms_s,
+                "y = act(bn(x)) + from in the layer's own pass; the layer alone %.4f ms, then a shortcut of 12B/elem" % ms_f)
         ms_b = timer.time(lambda i: ops.bn_act_backward(d[i], x[i], mean, var, scale, bias, su, bu, "leaky"),
                           10, rotate=rot)
         add("bn_bwd(leaky)", "%dx%dx%d^2" % (N, c, s), (16 if one_launch else 20) * e, ms_b,

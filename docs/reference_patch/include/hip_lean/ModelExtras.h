@@ -1,12 +1,13 @@
 // include/hip_lean/ModelExtras.h -- DeviceExtras<Device::HIP>, the model-wide state of the lean forms (the
 // engine's DeviceExtras<Device::CUDA>, include/Model.h:101-127, holds the cuBLAS and cuDNN contexts in the same
-// place).  Four things that a layer cannot know by itself:
+// place).  Five things that a layer cannot know by itself:
 //   * which deltas are OVERWRITTEN by the first backward that reaches them (a residual block's shortcut is the
 //     first to write the delta of the layer in front of it and of its `from` layer): Layer::forward need not
 //     clear those, and the shortcut writes instead of adding (pxh_shortcut_backward_first);
 //   * where the kernel that wrote a delta last left the delta's norm and peak (pxh_shortcut_backward_norm,
 //     pxh_axpy_norm): the rescale + clip that opens that layer's backward then reads 8 bytes per 256 values
 //     instead of the tensor (pxh_rescale_clip_from_groups);
+//   * which shortcuts ride on the epilogue of the convolution in front of them (pxh_bn_train_act_shortcut_forward);
 //   * the YOLO heads that wait for the end of the forward pass to run as one pass
 //     (pxh_yolo_forward_train_heads);
 //   * every layer's parameter tensors, as tables kept on the device: the update hooks and the optimiser step
@@ -48,6 +49,28 @@ public:
         notes_.erase(it);
         return groups;
     }
+
+    // ---- shortcuts that ride on the epilogue of the convolution in front of them (marked once, when the graph
+    // is built, where nothing but the shortcut reads that convolution's output, the shortcut is linear over
+    // tensors of one shape and its alpha is 1): the convolution writes the shortcut's output and works on the
+    // shortcut's delta; the convolution's own delta is marked overwritten, it is never used
+    struct Rider {
+        PxHipVector* output;
+        PxHipVector* delta;
+        const PxHipVector* from;
+        float alpha, beta;
+    };
+    void carry(const void* conv, const void* shortcut, const Rider& rider) const
+    {
+        riders_[conv] = rider;
+        riding_.insert(shortcut);
+    }
+    const Rider* riderOf(const void* conv) const
+    {
+        const auto it = riders_.find(conv);
+        return it == riders_.end() ? nullptr : &it->second;
+    }
+    bool rides(const void* shortcut) const { return riding_.count(shortcut) != 0; }
 
     // ---- YOLO heads waiting for the end of the forward pass
     struct WaitingHead {
@@ -120,6 +143,8 @@ private:
     mutable std::set<const float*> overwritten_;
     mutable std::map<const void*, PxHipVector> groups_;
     mutable std::map<const float*, const float*> notes_;
+    mutable std::map<const void*, Rider> riders_;
+    mutable std::set<const void*> riding_;
     mutable std::vector<WaitingHead> waiting_;
     mutable std::vector<float*> tensors_[4];
     mutable std::vector<std::size_t> sizes_;

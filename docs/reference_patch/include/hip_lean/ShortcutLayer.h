@@ -2,7 +2,9 @@
 // the FIRST writer of the two deltas it reaches (the layer in front of it and its `from` layer: in a residual
 // block nothing else has written them when the shortcut's backward runs) and as the LAST writer of the first
 // of them: it overwrites instead of adding into cleared tensors, and leaves that delta's norm and peak behind.
-// Whoever builds the graph marks the two deltas (DeviceExtras<HIP>::markOverwritten) when that holds.
+// Whoever builds the graph marks the two deltas (DeviceExtras<HIP>::markOverwritten) when that holds -- or lets
+// the shortcut ride on the convolution in front of it (DeviceExtras<HIP>::carry), which then writes this layer's
+// output and takes this layer's delta: forward has nothing left to do here, backward only the `from` layer's share.
 #pragma once
 
 #include "Layer.h"
@@ -14,6 +16,7 @@ template<>
 inline void ShortcutLayer<Device::HIP>::forward(const V& input)
 {
     Layer<Device::HIP>::forward(input);
+    if (this->model().rides(this)) return;      // the convolution in front has written output_ (hip_lean/ConvLayer.h)
     const bool sameShape = from_->outWidth() == this->outWidth() && from_->outHeight() == this->outHeight() &&
                            from_->outChannels() == this->outChannels();
     float* pre = preActivation_.empty() ? nullptr : preActivation_.data();
@@ -38,6 +41,16 @@ inline void ShortcutLayer<Device::HIP>::backward(const V& input, V* grad)
     const bool sameShape = from_->outWidth() == this->outWidth() && from_->outHeight() == this->outHeight() &&
                            from_->outChannels() == this->outChannels();
     const float* pre = preActivation_.empty() ? nullptr : preActivation_.data();
+    if (net.rides(this)) {
+        // the `from` layer's share only: the convolution in front works on delta_ itself
+        if (net.overwritten(from_->delta().data()))
+            PX_HIP_CHECK(pxh_shortcut_backward_first(this->delta_.data(), nullptr, from_->delta().data(), nullptr,
+                                                     this->delta_.size(), alpha_, beta_, activation_->type(), nullptr));
+        else
+            PX_HIP_CHECK(pxh_shortcut_backward(this->delta_.data(), nullptr, from_->delta().data(), nullptr,
+                                               this->delta_.size(), alpha_, beta_, activation_->type(), nullptr));
+        return;
+    }
     if (sameShape && grad != nullptr) {
         const bool first = net.overwritten(grad->data()) && net.overwritten(from_->delta().data());
         PxHipVector& groups = net.normGroupsFor(this, grad->size());

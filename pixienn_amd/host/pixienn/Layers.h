@@ -83,6 +83,29 @@ public:
         }
     }
 
+    // The ShortcutLayer behind this layer, when nothing else reads this layer's output and the shortcut
+    // is linear over tensors of one shape (every residual block of the shipped YOLOv3 graphs): its sum
+    // rides on this layer's epilogue (ShortcutLayer::rideOn).  Forward, this layer writes the SHORTCUT's
+    // output (its own is never materialised); backward, it works on the shortcut's delta as its own
+    // (alpha = 1: the two hold the same values).
+    struct Rider {
+        V* output = nullptr;
+        V* delta = nullptr;
+        const V* from = nullptr;
+        float alpha = 1.0f, beta = 1.0f;
+    };
+    void carry(const Rider& rider)
+    {
+        PX_CHECK(batchNorm_, "a shortcut rides on a batch-normalised convolution only");
+        PX_CHECK(rider.output && rider.from && rider.output->size() == output_.size() &&
+                 rider.from->size() == output_.size(), "ConvLayer: the shortcut's tensors do not match the layer's");
+        PX_CHECK(!training() || (rider.delta && rider.alpha == 1.0f),
+                 "ConvLayer: in training a shortcut rides only with alpha = 1 (the layer takes the shortcut's delta)");
+        rider_ = rider;
+        setFirstConsumerOverwrites(true);       // this layer's own delta is not used: nothing to clear
+    }
+    bool carriesShortcut() const noexcept { return rider_.output != nullptr; }
+
     void setConvolution(Convolve fwd, ConvolveBackward bwd)
     {
         convolve_ = std::move(fwd);
@@ -108,6 +131,23 @@ public:
         }
         x_ = x;
         const int spatial = outHeight() * outWidth();
+        if (rider_.output) {
+            if (training()) {
+                PX_HIP_CHECK(pxh_bn_train_act_shortcut_forward(x, rider_.output->data(), nullptr, nullptr, nullptr,
+                                                               mean_.data(), var_.data(), rollingMean_.data(),
+                                                               rollingVar_.data(), scales_.data(), biases_.data(),
+                                                               rider_.from->data(), rider_.alpha, rider_.beta, batch(),
+                                                               filters_, spatial, activation_, context().workspace(),
+                                                               context().workspaceBytes(), stream()));
+                foldedValid_ = false;
+            } else {
+                fold();
+                PX_HIP_CHECK(pxh_bn_folded_act_shortcut_forward(x, rider_.output->data(), nullptr, folded_.data(),
+                                                                rider_.from->data(), rider_.alpha, rider_.beta, batch(),
+                                                                filters_, spatial, activation_, stream()));
+            }
+            return;
+        }
         if (!batchNorm_) {
             PX_HIP_CHECK(pxh_bias_act_forward(x, output_.data(), nullptr, biases_.data(), batch(), filters_, spatial,
                                               activation_, stream()));
@@ -119,11 +159,7 @@ public:
                                                   stream()));
             foldedValid_ = false;       // the rolling statistics moved
         } else {
-            if (!foldedValid_) {
-                PX_HIP_CHECK(pxh_bn_fold(rollingMean_.data(), rollingVar_.data(), scales_.data(), biases_.data(),
-                                         filters_, folded_.data(), stream()));
-                foldedValid_ = true;
-            }
+            fold();
             PX_HIP_CHECK(pxh_bn_folded_act_forward(x, output_.data(), nullptr, folded_.data(), batch(), filters_,
                                                    spatial, activation_, stream()));
         }
@@ -139,18 +175,21 @@ public:
     {
         PX_CHECK(training() && x_ != nullptr, "ConvLayer: backward without a training forward");
         const float threshold = rescaleThreshold(), clip = clipValue();
-        const bool fused = (threshold > 0.0f || clip > 0.0f) && !context().hasNormGroups(delta_.data());
-        if (!fused) Layer::backward(input, grad);
+        // with a shortcut riding on the layer, its delta is the shortcut's (already through the shortcut's own
+        // helpers, which the layer's repeat without changing a value, as they would on the copy)
+        V& d = rider_.delta ? *rider_.delta : delta_;
+        const bool fused = (threshold > 0.0f || clip > 0.0f) && (rider_.delta || !context().hasNormGroups(d.data()));
+        if (!fused && !rider_.delta) Layer::backward(input, grad);
         const int spatial = outHeight() * outWidth();
         if (batchNorm_) {
             if (fused)
-                PX_HIP_CHECK(pxh_bn_act_backward_clipped(delta_.data(), x_, nullptr, mean_.data(), var_.data(),
+                PX_HIP_CHECK(pxh_bn_act_backward_clipped(d.data(), x_, nullptr, mean_.data(), var_.data(),
                                                          scales_.data(), biases_.data(), scaleUpdates_.data(),
                                                          biasUpdates_.data(), nullptr, nullptr, batch(), filters_,
                                                          spatial, activation_, threshold, clip, nullptr,
                                                          context().workspace(), context().workspaceBytes(), stream()));
             else
-                PX_HIP_CHECK(pxh_bn_act_backward(delta_.data(), x_, nullptr, mean_.data(), var_.data(),
+                PX_HIP_CHECK(pxh_bn_act_backward(d.data(), x_, nullptr, mean_.data(), var_.data(),
                                                  scales_.data(), biases_.data(), scaleUpdates_.data(),
                                                  biasUpdates_.data(), nullptr, nullptr, batch(), filters_, spatial,
                                                  activation_, context().workspace(), context().workspaceBytes(),
@@ -160,19 +199,19 @@ public:
             preActivation(spatial);
             const float* pre = pre_.empty() ? nullptr : pre_.data();
             if (fused)
-                PX_HIP_CHECK(pxh_bias_act_backward_clipped(delta_.data(), pre, biasUpdates_.data(), batch(), filters_,
+                PX_HIP_CHECK(pxh_bias_act_backward_clipped(d.data(), pre, biasUpdates_.data(), batch(), filters_,
                                                            spatial, activation_, threshold, clip, nullptr,
                                                            context().workspace(), context().workspaceBytes(),
                                                            stream()));
             else
-                PX_HIP_CHECK(pxh_bias_act_backward(delta_.data(), pre, biasUpdates_.data(), batch(), filters_, spatial,
+                PX_HIP_CHECK(pxh_bias_act_backward(d.data(), pre, biasUpdates_.data(), batch(), filters_, spatial,
                                                    activation_, context().workspace(), context().workspaceBytes(),
                                                    stream()));
         }
         if (convolveBackward_) {
-            convolveBackward_(input, delta_, grad);
+            convolveBackward_(input, d, grad);
         } else if (grad) {
-            PX_HIP_CHECK(pxh_axpy(delta_.size(), 1.0f, delta_.data(), grad->data(), stream()));
+            PX_HIP_CHECK(pxh_axpy(d.size(), 1.0f, d.data(), grad->data(), stream()));
         }
     }
 
@@ -315,8 +354,18 @@ private:
                                           PXH_LINEAR, stream()));
     }
 
+    // the inference constants, folded again only after the parameters changed
+    void fold()
+    {
+        if (foldedValid_) return;
+        PX_HIP_CHECK(pxh_bn_fold(rollingMean_.data(), rollingVar_.data(), scales_.data(), biases_.data(), filters_,
+                                 folded_.data(), stream()));
+        foldedValid_ = true;
+    }
+
     int activation_ = PXH_LOGISTIC, filters_ = 1;
     bool batchNorm_ = false, foldedValid_ = false;
+    Rider rider_;
     const float* x_ = nullptr;      // conv result of the last forward (borrowed)
     V biases_, scales_, rollingMean_, rollingVar_, mean_, var_, folded_;
     V biasUpdates_, scaleUpdates_, biasM_, biasV_, scaleM_, scaleV_;
@@ -592,9 +641,24 @@ public:
         if (leavesNorm_) normGroups_ = normGroupsFor(output_.size());
     }
 
+    // This shortcut's sum rides on the epilogue of the convolution in front of it
+    // (pxh_bn_train_act_shortcut_forward): for whoever builds the network, when nothing but this shortcut
+    // reads that convolution's output.  forward() then finds its output written, and backward() leaves the
+    // convolution's delta alone: the convolution works on this layer's.
+    void rideOn(ConvLayer& conv)
+    {
+        PX_CHECK(sameShape_ && activation_ == PXH_LINEAR, "a shortcut rides only with a linear activation over one shape");
+        PX_CHECK(!leavesNorm_, "a riding shortcut writes no delta of the layer in front: nothing to leave a norm of");
+        PX_CHECK(conv.batch() == batch() && conv.outChannels() == outChannels() && conv.outHeight() == outHeight() &&
+                 conv.outWidth() == outWidth(), "shortcut: the convolution in front has another shape");
+        conv.carry(ConvLayer::Rider{ &output_, training() ? &delta_ : nullptr, &from_->output(), alpha_, beta_ });
+        riding_ = true;
+    }
+
     void forward(const V& input) override
     {
         Layer::forward(input);
+        if (riding_) return;        // the convolution in front has written output_
         checkInput(input, "ShortcutLayer");
         float* pre = preActivation_.empty() ? nullptr : preActivation_.data();
         if (sameShape_) {
@@ -615,6 +679,16 @@ public:
     {
         Layer::backward(input, grad);
         const float* pre = preActivation_.empty() ? nullptr : preActivation_.data();
+        if (riding_) {
+            // the `from` layer's share only; the convolution in front takes delta_ itself
+            if (firstWriter_)
+                PX_HIP_CHECK(pxh_shortcut_backward_first(delta_.data(), nullptr, from_->delta().data(), nullptr,
+                                                         delta_.size(), alpha_, beta_, activation_, stream()));
+            else
+                PX_HIP_CHECK(pxh_shortcut_backward(delta_.data(), nullptr, from_->delta().data(), nullptr, delta_.size(),
+                                                   alpha_, beta_, activation_, stream()));
+            return;
+        }
         if (leavesNorm_ && grad) {
             PX_HIP_CHECK(pxh_shortcut_backward_norm(delta_.data(), pre, from_->delta().data(), grad->data(),
                                                     delta_.size(), alpha_, beta_, activation_, firstWriter_ ? 1 : 0,
@@ -646,7 +720,7 @@ private:
     Layer::Ptr from_;
     int activation_ = PXH_LINEAR;
     float alpha_ = 1.0f, beta_ = 1.0f;
-    bool sameShape_ = true, firstWriter_ = false, leavesNorm_ = false;
+    bool sameShape_ = true, firstWriter_ = false, leavesNorm_ = false, riding_ = false;
     V preActivation_, normGroups_;
 };
 

@@ -982,6 +982,107 @@ void leavesNormShortcutChecks()
     }
 }
 
+// A residual block whose shortcut rides on the epilogue of the convolution in front of it: that
+// convolution writes the shortcut's output (its own is never formed) and takes the shortcut's delta as its
+// own.  Output, every gradient behind it and every update buffer are those of the two layers one after the
+// other, bit for bit -- helpers off, below the threshold, rescaled, clamped; training and inference.
+void ridingShortcutChecks()
+{
+    struct Block {
+        Context ctx;
+        std::shared_ptr<ConvLayer> a, b, c;
+        std::shared_ptr<ShortcutLayer> add;
+        Block(bool riding, bool firstWriter, bool training, float threshold, float clip)
+        {
+            ctx.training = training;
+            const Properties conv{ { "batch", N }, { "channels", C }, { "height", S }, { "width", S }, { "filters", C },
+                                   { "batch_normalize", true }, { "activation", std::string("leaky") } };
+            a = std::make_shared<ConvLayer>(ctx, conv);
+            b = std::make_shared<ConvLayer>(ctx, conv);
+            c = std::make_shared<ConvLayer>(ctx, conv);
+            add = std::make_shared<ShortcutLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S },
+                                                                   { "width", S }, { "first_writer", firstWriter },
+                                                                   { "beta", 0.75f } }, a);
+            if (firstWriter) c->setFirstConsumerOverwrites(true);
+            if (riding) add->rideOn(*c);
+            int seed = 730;
+            for (auto* l: { a.get(), b.get(), c.get() }) {
+                l->copyScales(normals(seed++, C));
+                l->copyBiases(normals(seed++, C));
+                l->copyRollingMean(normals(seed++, C));
+                Host var = normals(seed++, C);
+                for (float& v: var) v = 0.5f + v * v;
+                l->copyRollingVariance(var);
+            }
+            for (Layer* l: { static_cast<Layer*>(a.get()), static_cast<Layer*>(b.get()), static_cast<Layer*>(c.get()),
+                             static_cast<Layer*>(add.get()) }) {
+                l->setGradientRescaling(threshold > 0.0f, threshold);
+                l->setGradientClipping(clip > 0.0f, clip);
+            }
+        }
+        void forward(const FloatVector& input)
+        {
+            a->forward(input);
+            b->forward(a->output());
+            c->forward(b->output());
+            add->forward(c->output());
+        }
+        void step(const FloatVector& input, const Host& outDelta)
+        {
+            forward(input);
+            add->delta().copyHost(outDelta);
+            add->backward(c->output(), &c->delta());
+            c->backward(b->output(), &b->delta());
+            b->backward(a->output(), &a->delta());
+            a->backward(input, nullptr);
+        }
+    };
+    const FloatVector input(normals(721, size_t(N) * C * S * S));
+    const Host outDelta = normals(722, size_t(N) * C * S * S);
+    double norm = 0.0;
+    for (float v: outDelta) norm += double(v) * v;
+    norm = std::sqrt(norm);
+    {
+        Block plain(false, false, false, 0.0f, 0.0f), riding(true, false, false, 0.0f, 0.0f);
+        plain.forward(input);
+        riding.forward(input);
+        report("riding shortcut: output at inference", riding.add->output().asVector() == plain.add->output().asVector());
+        report("riding shortcut: the convolution says so", riding.c->carriesShortcut() && !plain.c->carriesShortcut());
+    }
+    struct Case { const char* name; float threshold, clip; };
+    const Case cases[] = { { "helpers off", 0.0f, 0.0f }, { "below the threshold", float(4.0 * norm), 0.0f },
+                           { "rescaled", float(0.5 * norm), 0.0f }, { "rescaled and clamped", float(0.5 * norm), 0.25f } };
+    for (const bool firstWriter: { false, true }) {
+        for (const Case& k: cases) {
+            Block plain(false, firstWriter, true, k.threshold, k.clip), riding(true, firstWriter, true, k.threshold, k.clip);
+            for (int round = 0; round < 2; ++round) {
+                plain.step(input, outDelta);
+                riding.step(input, outDelta);
+                const std::string tag = std::string(" (") + k.name + (firstWriter ? ", first writer" : "") + ", step " +
+                                        std::to_string(round + 1) + ")";
+                report("riding shortcut: output" + tag, riding.add->output().asVector() == plain.add->output().asVector());
+                report("riding shortcut: delta behind the convolution" + tag,
+                       riding.b->delta().asVector() == plain.b->delta().asVector());
+                report("riding shortcut: the convolution's updates" + tag,
+                       riding.c->scaleUpdates().asVector() == plain.c->scaleUpdates().asVector() &&
+                       riding.c->biasUpdates().asVector() == plain.c->biasUpdates().asVector());
+                report("riding shortcut: delta and updates of the from layer" + tag,
+                       riding.a->delta().asVector() == plain.a->delta().asVector() &&
+                       riding.a->scaleUpdates().asVector() == plain.a->scaleUpdates().asVector());
+            }
+        }
+    }
+    expectThrows("a shortcut with an activation of its own does not ride", [] {
+        Context ctx;
+        const Properties conv{ { "batch", N }, { "channels", C }, { "height", S }, { "width", S }, { "filters", C },
+                               { "batch_normalize", true } };
+        auto a = std::make_shared<ConvLayer>(ctx, conv);
+        ShortcutLayer add(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S }, { "width", S },
+                                           { "activation", std::string("leaky") } }, a);
+        add.rideOn(*a);
+    }, "linear");
+}
+
 // The small network with the shortcut and the head leaving the norms of the deltas they write last
 // (conv2's and conv6's): every delta and every update buffer as without, bit for bit.
 void leavesNormNetChecks()
@@ -1201,6 +1302,7 @@ int main(int argc, char** argv)
             weightsFileChecks();
             firstWriterShortcutChecks();
             leavesNormShortcutChecks();
+            ridingShortcutChecks();
             leavesNormNetChecks();
             deferredHeadsChecks();
             capturedSequenceChecks();

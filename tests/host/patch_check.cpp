@@ -13,6 +13,7 @@
 #include "hip/RouteLayer.h"
 #include "hip/ShortcutLayer.h"
 #include "hip/BatchNormLayer.h"
+#include "hip/ConvLayerCommon.h"
 #include "hip/ConvLayer.h"
 #include "hip/YoloLayerCommon.h"
 #include "hip/YoloLayer.h"

@@ -112,14 +112,15 @@ def test_binding_headers_and_stub_name_only_members_the_engine_has():
     checked = 0
     for folder in ("hip", "hip_lean"):
         for name in sorted(os.listdir(os.path.join(patch_root, folder))):
-            layer = {"YoloLayerCommon.h": "YoloLayer.h", "ModelExtras.h": "Model.h"}.get(name, name)
+            layer = {"YoloLayerCommon.h": "YoloLayer.h", "ConvLayerCommon.h": "ConvLayer.h",
+                     "ModelExtras.h": "Model.h"}.get(name, name)
             known = identifiers(base + engine(layer, os.path.join("cuda", layer)))
             text = re.sub(r"//[^\n]*", "", open(os.path.join(patch_root, folder, name)).read())
             members = set(re.findall(r"\b[a-z]\w*_\b", text)) - {"px_hip_status_"}
             methods = set(re.findall(r"this->(\w+)\(", text)) | set(re.findall(r"\bnet\.(\w+)\(", text))
             for m in sorted(members | methods):
                 if m in own or m in ("deferHead", "normGroupsFor", "noteNormGroups", "takeNormGroups", "overwritten",
-                                     "registerParameters", "updateAll"):
+                                     "registerParameters", "updateAll", "rides", "riderOf"):
                     continue
                 assert m in known, "%s/%s names `%s`, which the engine's %s does not have" % (folder, name, m, layer)
                 checked += 1
