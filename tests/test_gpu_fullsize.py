@@ -137,6 +137,34 @@ def test_bn_backward_clipped_at_training_shapes(ops, shape):
         del want, got
 
 
+@pytest.mark.parametrize("shape", [(16, 64, 304), (16, 256, 76), (16, 512, 38), (16, 1024, 19)])
+def test_epilogue_with_shortcut_at_training_shapes(ops, shape):
+    """A residual block's shortcut taken into the epilogue of the convolution in front of it, at the shapes of
+    YOLOv3's blocks at batch 16 -- three launches, the one-launch form with part of the slice in LDS, the 128-bit
+    and the scalar one-launch forms -- against the two calls it replaces (each held to the checker elsewhere)."""
+    import torch
+    N, C, S = shape
+    x = device_normal((N, C, S, S), 31) * 1.3 + 0.2
+    frm = device_normal((N, C, S, S), 32)
+    scale, bias, rmean, rvar = (gpu(a) for a in wl.bn_params(3101, C))
+    m0, v0, m1, v1 = (torch.zeros(C, device="cuda") for _ in range(4))
+    rm0, rv0, rm1, rv1 = rmean.clone(), rvar.clone(), rmean.clone(), rvar.clone()
+    y = torch.empty_like(x); want = torch.empty_like(x)
+    ops.bn_train_act_forward(x, y, m0, v0, rm0, rv0, scale, bias, "leaky")
+    ops.shortcut_forward(y, frm, want, "linear")
+    del y
+    got = torch.empty_like(x)
+    ops.bn_train_act_shortcut_forward(x, got, m1, v1, rm1, rv1, scale, bias, "leaky", frm)
+    if S % 2 == 0 or C < 512:
+        assert torch.equal(got, want) and torch.equal(m1, m0) and torch.equal(v1, v0) and torch.equal(rm1, rm0), shape
+    else:
+        # 1024 scalar slices: alone, the layer adds its statistics up with workgroups of half the size
+        assert_close(host(m1), host(m0), 2e-6, 1.0, "mean")
+        assert_close(host(v1), host(v0), 2e-6, 1.0, "var")
+        worst = float(((got - want).abs() / (want.abs() + frm.abs()).clamp_min(1.0)).max())
+        assert worst <= 2e-6, (shape, worst)
+
+
 def test_maxpool_largest_shape(ops, oracle):
     """16 x 64 x 304^2: whole tensor against the checker and against an independent routine."""
     import torch
