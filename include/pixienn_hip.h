@@ -136,6 +136,19 @@ int pxh_bn_folded_act_shortcut_forward(const float* x, float* y, float* pre_acti
                                        const float* from, float alpha, float beta, int batch, int channels,
                                        int spatial, int activation, void* stream);
 
+/* A convolution's inference epilogue with the MaxPoolLayer that follows it in the same pass, for the
+ * 2 x 2 window at stride 2 over planes of even height and width (five of the six pools of YOLOv3-tiny):
+ *   pooled[n][c][i][j] = max over the window of act(bn(x)), compared in the pool's own order
+ * i.e. what pxh_bn_folded_act_forward followed by pxh_maxpool_forward (kernel 2, stride 2, padding 1)
+ * leaves in the pool's output, to the bit, without the layer's output reaching memory and without the
+ * indexes, which only a backward pass reads: 5 bytes per element of x instead of 8 + 6.
+ *   y       nullable: the layer's own output, for a layer that something else reads as well (a route);
+ *   pooled  batch x channels x height/2 x width/2.
+ * PXH_ERR_UNSUPPORTED for an odd height or width, or for tensors off a 16-byte boundary: take the two calls.
+ * Replaces include/cuda/ConvLayer.h:284-307 (inference) followed by include/cuda/MaxPoolLayer.h:23-37. */
+int pxh_bn_folded_act_maxpool_forward(const float* x, float* y, float* pooled, const void* folded, int batch,
+                                      int channels, int height, int width, int activation, void* stream);
+
 /* pxh_bn_train_act_forward for callers that cannot allocate device memory and have no workspace
  * to pass (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc): same
  * arguments without the workspace, same kernels, same results.  The partial sums and per-channel

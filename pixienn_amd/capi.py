@@ -30,6 +30,7 @@ SIGNATURES = {
     "pxh_bn_train_act_forward_static": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, P],
     "pxh_bn_train_act_shortcut_forward": [P, P, P, P, P, P, P, P, P, P, P, P, F, F, I, I, I, I, P, Z, P],
     "pxh_bn_folded_act_shortcut_forward": [P, P, P, P, P, F, F, I, I, I, I, P],
+    "pxh_bn_folded_act_maxpool_forward": [P, P, P, P, I, I, I, I, I, P],
     "pxh_bn_stats": [P, P, P, I, I, I, P, Z, P],
     "pxh_bn_act_backward": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, P, Z, P],
     "pxh_bias_act_backward": [P, P, P, I, I, I, I, P, Z, P],

@@ -265,6 +265,61 @@ __global__ __launch_bounds__(kBlock) void epilogue_fwd_scalar_kernel(EpilogueArg
     a.y[e] = y;
 }
 
+// ---- the inference epilogue with the 2 x 2, stride 2 max-pool that follows the layer ----
+// A lane takes VX consecutive outputs of one output row: 2 * VX inputs of each of two input rows (one
+// plane, so one channel's constants), applies the epilogue to them and keeps the largest of each window,
+// compared in the order the pool's own kernel compares them.  The layer's own output is written only when
+// something else reads it.
+struct EpiloguePoolArgs {
+    const float* x;
+    float* y;             // nullable: the layer's own output
+    float* pooled;
+    const FoldCoef* table;
+    uint32_t units;       // lanes with work
+    uint32_t iw, ow;
+    FastDiv by_owv;       // ow / VX
+    FastDiv by_oh;
+    FastDiv by_channels;
+};
+
+template<int ACT, int VX, bool NT>
+__global__ __launch_bounds__(kBlock) void epilogue_pool2_fwd_kernel(EpiloguePoolArgs a)
+{
+    const uint32_t t = blockIdx.x * static_cast<uint32_t>(kBlock) + threadIdx.x;
+    if (t >= a.units) return;
+    uint32_t rows, oxv, plane, oy, q, c;
+    a.by_owv.divmod(t, rows, oxv);
+    a.by_oh.divmod(rows, plane, oy);
+    a.by_channels.divmod(plane, q, c);
+    const uint32_t ih = a.by_oh.d * 2;
+    const uint32_t in0 = (plane * ih + 2 * oy) * a.iw + 2 * oxv * VX;      // < 2^31 checked by the host
+    const Pack<2 * VX> r0 = ld<2 * VX, NT>(a.x, in0);
+    const Pack<2 * VX> r1 = ld<2 * VX, NT>(a.x, in0 + a.iw);
+    const FoldCoef k = a.table[c];
+    Pack<2 * VX> y0, y1;
+    float pre[2 * VX], xn;
+#pragma unroll
+    for (int j = 0; j < 2 * VX; ++j) pre[j] = pre_value<true>(r0.v[j], k, xn);
+    act_apply_n<ACT>(pre, y0.v);
+#pragma unroll
+    for (int j = 0; j < 2 * VX; ++j) pre[j] = pre_value<true>(r1.v[j], k, xn);
+    act_apply_n<ACT>(pre, y1.v);
+    if (a.y) {
+        st<2 * VX, NT>(a.y, in0, y0);
+        st<2 * VX, NT>(a.y, in0 + a.iw, y1);
+    }
+    Pack<VX> best;
+#pragma unroll
+    for (int j = 0; j < VX; ++j) {
+        float b = y0.v[2 * j];
+        if (y0.v[2 * j + 1] > b) b = y0.v[2 * j + 1];
+        if (y1.v[2 * j] > b) b = y1.v[2 * j];
+        if (y1.v[2 * j + 1] > b) b = y1.v[2 * j + 1];
+        best.v[j] = b;
+    }
+    st<VX, NT>(a.pooled, (plane * a.by_oh.d + oy) * a.ow + oxv * VX, best);
+}
+
 int check_shape(const char* who, int batch, int channels, int spatial, uint32_t* total)
 {
     if (batch <= 0 || channels <= 0 || spatial <= 0)
@@ -1765,6 +1820,48 @@ int pxh_bn_folded_act_shortcut_forward(const float* x, float* y, float* pre_acti
     a.by_spatial = FastDiv(spatial); a.by_channels = FastDiv(channels);
     a.residual = from; a.res_alpha = alpha; a.res_beta = beta;
     return launch_epilogue_fwd<true>(who, a, activation, as_stream(stream));
+}
+
+int pxh_bn_folded_act_maxpool_forward(const float* x, float* y, float* pooled, const void* folded, int batch,
+                                      int channels, int height, int width, int activation, void* stream)
+{
+    const char* who = "pxh_bn_folded_act_maxpool_forward";
+    if (!x || !pooled || !folded) return fail_invalid("%s: null pointer", who);
+    if (!aligned16(folded)) return fail_invalid("%s: folded must be 16-byte aligned", who);
+    if (height <= 0 || width <= 0) return fail_invalid("%s: height and width must be positive", who);
+    if (pooled == x || pooled == y) return fail_invalid("%s: the pooled output must be a tensor of its own", who);
+    uint32_t total;
+    int rc = check_shape(who, batch, channels, height * width, &total);
+    if (rc) return rc;
+    if (height % 2 || width % 2 || !aligned16(x) || !aligned16(y) || !aligned16(pooled)) {
+        set_error("%s: windows that do not tile the plane (%d x %d) or tensors off a 16-byte boundary take the two "
+                  "calls (pxh_bn_folded_act_forward, pxh_maxpool_forward)", who, height, width);
+        return PXH_ERR_UNSUPPORTED;
+    }
+    const uint32_t oh = height / 2, ow = width / 2;
+    EpiloguePoolArgs a{};
+    a.x = x; a.y = y; a.pooled = pooled;
+    a.table = static_cast<const FoldCoef*>(folded);
+    a.iw = width; a.ow = ow;
+    a.by_oh = FastDiv(oh); a.by_channels = FastDiv(channels);
+    const uint32_t outputs = total / 4;
+    // x in, the pooled quarter out, the layer's own output when asked for
+    const bool nt = static_cast<size_t>(total) * (y ? 9 : 5) >= kStreamingBytes;
+    hipStream_t s = as_stream(stream);
+    const auto launch = [&]<int ACT, int VX>() {
+        a.units = outputs / VX;
+        a.by_owv = FastDiv(ow / VX);
+        const dim3 grid(grid_for(a.units, kBlock));
+        if (nt) hipLaunchKernelGGL((epilogue_pool2_fwd_kernel<ACT, VX, true>), grid, dim3(kBlock), 0, s, a);
+        else hipLaunchKernelGGL((epilogue_pool2_fwd_kernel<ACT, VX, false>), grid, dim3(kBlock), 0, s, a);
+    };
+    const bool known = dispatch_activation(activation, [&]<int ACT>() {
+        if (width % 8 == 0) launch.template operator()<ACT, 4>();
+        else if (width % 4 == 0) launch.template operator()<ACT, 2>();
+        else launch.template operator()<ACT, 1>();
+    });
+    if (!known) return fail_invalid("%s: unknown activation %d", who, activation);
+    return check_launch(who);
 }
 
 int pxh_bn_train_act_forward_static(const float* x, float* y, float* pre_activation, float* x_saved, float* x_norm,

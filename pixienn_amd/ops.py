@@ -122,6 +122,14 @@ def bn_folded_act_shortcut_forward(x, y, folded, activation, from_, alpha=1.0, b
          float(alpha), float(beta), n, c, s, act_id(activation), _stream())
 
 
+def bn_folded_act_maxpool_forward(x, pooled, folded, activation, y=None):
+    """bn_folded_act_forward with the 2x2 / 2 max-pool that follows the layer; x is [N, C, H, W]."""
+    _chk_all(x, pooled, y)
+    n, c, h, w = x.shape
+    call("pxh_bn_folded_act_maxpool_forward", ptr(x), ptr(y), ptr(pooled), ptr(folded), n, c, h, w, act_id(activation),
+         _stream())
+
+
 def bn_act_backward(delta, x, mean, var, scale, bias, scale_updates, bias_updates, activation,
                     pre_activation=None, mean_delta=None, var_delta=None, workspace=None):
     _chk_all(delta, x, mean, var, scale, bias, scale_updates, bias_updates, pre_activation, mean_delta, var_delta)
