@@ -522,6 +522,30 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
             ms = timer.time(lambda i: ops.maxpool_backward(deltas[i], idxs[i], xs[i], 2, 2, 1), 20, rotate=rot)
             add("maxpool_bwd", "%dx%dx%d^2" % (N, c, s), 8 * e_out + 8 * e_in, ms, "full-grad RMW: 8B/out + 8B/in")
             del xs, outs, idxs, deltas
+        # ---- the inference epilogue with the 2x2 / 2 pool behind it in one pass (YOLOv3-tiny, batch 64: the
+        # headline sweep's own shapes that a pool follows), against the two calls one after the other
+        scale_t, bias_t, rmean_t, rvar_t = (torch.from_numpy(a_).to(dev) for a_ in wl.bn_params(2900, 1024))
+        for c, s in ((16, 416), (32, 208), (64, 104), (128, 52), (256, 26)):
+            n64 = 64
+            e_in = n64 * c * s * s
+            rot = rotation_for(5 * e_in)
+            xs = [randn(n64, c, s, s) for _ in range(rot)]
+            ys = [torch.empty((n64, c, s, s), device=dev) for _ in range(min(rot, 3))]
+            outs = [torch.empty((n64, c, s // 2, s // 2), device=dev) for _ in range(rot)]
+            idxs = [torch.empty((n64, c, s // 2, s // 2), device=dev, dtype=torch.int32) for _ in range(min(rot, 3))]
+            folded = ops.bn_fold(rmean_t[:c].contiguous(), rvar_t[:c].contiguous(), scale_t[:c].contiguous(),
+                                 bias_t[:c].contiguous())
+            ms = timer.time(lambda i: ops.bn_folded_act_maxpool_forward(xs[i], outs[i], folded, "leaky"), 20, rotate=rot)
+
+            def two(i):
+                ops.bn_folded_act_forward(xs[i], ys[i % len(ys)], folded, "leaky")
+                ops.maxpool_forward(ys[i % len(ys)], outs[i], idxs[i % len(idxs)], 2, 2, 1)
+
+            ms_two = timer.time(two, 20, rotate=rot)
+            add("epilogue+maxpool(leaky, inference)", "%dx%dx%d^2" % (n64, c, s), 5 * e_in, ms,
+                "4B/in + 1B/in out; the two calls (8B + 6B per input element) %.4f ms" % ms_two)
+            rows[-1]["two_calls_ms"] = round(ms_two, 4)
+            del xs, ys, outs, idxs
         # ---- upsample x2 forward + backward
         for c, s in wl.YOLOV3_UPSAMPLE_SHAPES:
             e_in = N * c * s * s
@@ -902,12 +926,50 @@ def measure_config0(torch, ops, wl, timer, with_cpu=True):
             elif kind == "yolo":
                 ops.yolo_activate(T[i - 1]["y"], t["y"], 1, 3, 80, l["s"] * l["s"])
 
+    # the five 2 x 2 / 2 pools on the epilogue of the convolution in front of them
+    # (pxh_bn_folded_act_maxpool_forward): the convolution's own output is written only where a route reads it
+    routed = {src for l in layers if l["type"] == "route" for src in l["sources"]}
+    pooled_by = {i: i + 1 for i, l in enumerate(layers[:-1])
+                 if l["type"] == "conv" and l["bn"] and layers[i + 1]["type"] == "maxpool" and layers[i + 1]["stride"] == 2}
+
+    def forward_pools_ride(_):
+        for i, (l, t) in enumerate(zip(layers, T)):
+            kind = l["type"]
+            if i in pooled_by:
+                ops.bn_folded_act_maxpool_forward(t["x"], T[pooled_by[i]]["y"], t["folded"], l["act"],
+                                                  y=t["y"] if i in routed else None)
+            elif kind == "maxpool" and i - 1 in pooled_by:
+                continue
+            elif kind == "conv" and l["bn"]:
+                ops.bn_folded_act_forward(t["x"], t["y"], t["folded"], l["act"])
+            elif kind == "conv":
+                ops.bias_act_forward(t["x"], t["y"], t["bias"], l["act"])
+            elif kind == "maxpool":
+                ops.maxpool_forward(T[i - 1]["y"], t["y"], t["idx"], 2, l["stride"], 1)
+            elif kind == "upsample":
+                ops.upsample_forward(T[i - 1]["y"], t["y"], 2, 1.0)
+            elif kind == "route":
+                offset = 0
+                for src in l["sources"]:
+                    ops.route_forward(T[src]["y"], t["y"], offset)
+                    offset += layers[src]["c"] * l["s"] * l["s"]
+            elif kind == "yolo":
+                ops.yolo_activate(T[i - 1]["y"], t["y"], 1, 3, 80, l["s"] * l["s"])
+
     out = dict(workload="YOLOv3-tiny inference forward, batch 1, 416x416: non-conv layers in model order "
                         "(13 conv epilogues, 6 max-pools, 1 upsample, 2 routes, 2 head decodes; 27 launches)")
     out["gpu_graph_ms"] = round(timer.time(forward, 5, warm=2), 4)
     timer.use_graphs, saved = False, timer.use_graphs
     out["gpu_eager_ms"] = round(timer.time(forward, 5, warm=2), 4)
     timer.use_graphs = saved
+    # the same outputs with the pools riding: 22 launches
+    plain_pools = {p: T[p]["y"].clone() for p in pooled_by.values()}
+    for p in pooled_by.values():
+        T[p]["y"].fill_(-1.0)
+    out["gpu_graph_pools_ride_ms"] = round(timer.time(forward_pools_ride, 5, warm=2), 4)
+    out["pools_riding"] = len(pooled_by)
+    out["pools_ride_same_outputs"] = all(bool(torch.equal(T[p]["y"], plain_pools[p])) for p in pooled_by.values())
+    del plain_pools
     elems = sum(int(t["y"].numel()) for t in T)
     out["elements_written"] = elems
     if with_cpu:
@@ -1160,6 +1222,7 @@ def final_line(steps, warmup, value, ms_per_step, bytes_step, launches_per_step,
         "noconv_ms_per_batch_yolov3_608_leanest": mo.get("leanest_total_ms"),
         "noconv_layer_kernels_sum_ms_yolov3_608": None if layer_kernels_sum_ms is None else round(layer_kernels_sum_ms, 3),
         "config0_gpu_ms": c0.get("gpu_graph_ms"),
+        "config0_gpu_ms_pools_on_the_epilogue": c0.get("gpu_graph_pools_ride_ms"),
         "config0_cpu_ms": c0.get("cpu_ms"),
         "value_folding_every_call": round(value_raw, 1),
         "value_as_one_hip_graph": round(value_graph, 1),

@@ -1,4 +1,4 @@
-// include/hip_lean/ConvLayer.h -- ConvLayer<Device::HIP> with two things the plain bodies cannot know:
+// include/hip_lean/ConvLayer.h -- ConvLayer<Device::HIP> with three things the plain bodies cannot know:
 //   * setup() hands the layer's parameter tensors to the model, so that Model<HIP>::update (Model.h here) steps
 //     the tensors of all layers together: the layer's own update() is then never called;
 //   * a ShortcutLayer that RIDES on this layer (DeviceExtras<HIP>::carry, for a residual block: nothing but the
@@ -7,6 +7,9 @@
 //     per element become 4 more read here, this layer's own output_ is never formed), and backward works on the
 //     shortcut's delta as this layer's own (alpha = 1: the two hold the same values; the shortcut's helpers have
 //     been over it, and this layer's repeat without changing a value, as they would on the copy).
+//   * a MaxPoolLayer that rides on this layer at inference (DeviceExtras<HIP>::carryPool): the epilogue writes the
+//     pool's output in its own pass (pxh_bn_folded_act_maxpool_forward), and this layer's own only when a route
+//     reads it as well.
 // Everything else as in include/hip/ConvLayer.h.
 #pragma once
 
@@ -56,10 +59,17 @@ inline void ConvLayer<Device::HIP>::forward(const V& input)
                                      folded_.data(), nullptr));
             foldedReady_ = true;
         }
+        const auto* pool = this->model().poolOf(this);
         if (rider)
             PX_HIP_CHECK(pxh_bn_folded_act_shortcut_forward(this->output_.data(), rider->output->data(), nullptr,
                                                             folded_.data(), rider->from->data(), rider->alpha,
                                                             rider->beta, this->batch(), filters_, spatial, act, nullptr));
+        else if (pool)
+            // in place on the GEMM result when the layer's output is kept, else that tensor is only read
+            PX_HIP_CHECK(pxh_bn_folded_act_maxpool_forward(this->output_.data(),
+                                                           pool->keepOutput ? this->output_.data() : nullptr,
+                                                           pool->pooled->data(), folded_.data(), this->batch(), filters_,
+                                                           this->outHeight(), this->outWidth(), act, nullptr));
         else
             PX_HIP_CHECK(pxh_bn_folded_act_forward(this->output_.data(), this->output_.data(), nullptr, folded_.data(),
                                                    this->batch(), filters_, spatial, act, nullptr));

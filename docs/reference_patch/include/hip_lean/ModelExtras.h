@@ -1,6 +1,6 @@
 // include/hip_lean/ModelExtras.h -- DeviceExtras<Device::HIP>, the model-wide state of the lean forms (the
 // engine's DeviceExtras<Device::CUDA>, include/Model.h:101-127, holds the cuBLAS and cuDNN contexts in the same
-// place).  Five things that a layer cannot know by itself:
+// place).  Six things that a layer cannot know by itself:
 //   * which deltas are OVERWRITTEN by the first backward that reaches them (a residual block's shortcut is the
 //     first to write the delta of the layer in front of it and of its `from` layer): Layer::forward need not
 //     clear those, and the shortcut writes instead of adding (pxh_shortcut_backward_first);
@@ -8,6 +8,7 @@
 //     pxh_axpy_norm): the rescale + clip that opens that layer's backward then reads 8 bytes per 256 values
 //     instead of the tensor (pxh_rescale_clip_from_groups);
 //   * which shortcuts ride on the epilogue of the convolution in front of them (pxh_bn_train_act_shortcut_forward);
+//   * which max-pools do, at inference (pxh_bn_folded_act_maxpool_forward);
 //   * the YOLO heads that wait for the end of the forward pass to run as one pass
 //     (pxh_yolo_forward_train_heads);
 //   * every layer's parameter tensors, as tables kept on the device: the update hooks and the optimiser step
@@ -70,7 +71,25 @@ public:
         const auto it = riders_.find(conv);
         return it == riders_.end() ? nullptr : &it->second;
     }
-    bool rides(const void* shortcut) const { return riding_.count(shortcut) != 0; }
+    bool rides(const void* layer) const { return riding_.count(layer) != 0; }
+
+    // ---- max-pools that ride on the epilogue of the convolution in front of them, at inference (the 2 x 2 window
+    // at stride 2 over planes of even size): the convolution writes the pool's output; its own only when
+    // something else reads it as well (`keepOutput`: a route names the convolution)
+    struct PoolRider {
+        PxHipVector* pooled;
+        bool keepOutput;
+    };
+    void carryPool(const void* conv, const void* pool, const PoolRider& rider) const
+    {
+        poolRiders_[conv] = rider;
+        riding_.insert(pool);
+    }
+    const PoolRider* poolOf(const void* conv) const
+    {
+        const auto it = poolRiders_.find(conv);
+        return it == poolRiders_.end() ? nullptr : &it->second;
+    }
 
     // ---- YOLO heads waiting for the end of the forward pass
     struct WaitingHead {
@@ -144,6 +163,7 @@ private:
     mutable std::map<const void*, PxHipVector> groups_;
     mutable std::map<const float*, const float*> notes_;
     mutable std::map<const void*, Rider> riders_;
+    mutable std::map<const void*, PoolRider> poolRiders_;
     mutable std::set<const void*> riding_;
     mutable std::vector<WaitingHead> waiting_;
     mutable std::vector<float*> tensors_[4];

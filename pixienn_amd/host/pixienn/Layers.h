@@ -106,6 +106,19 @@ public:
     }
     bool carriesShortcut() const noexcept { return rider_.output != nullptr; }
 
+    // The 2 x 2, stride 2 MaxPoolLayer behind this layer, at inference (MaxPoolLayer::rideOn): the epilogue
+    // writes the pool's output in its own pass (pxh_bn_folded_act_maxpool_forward).  `keepOutput`: something
+    // else reads this layer's output too (a route), so it is written as well; else it is never formed.
+    void carryPool(V* pooled, bool keepOutput)
+    {
+        PX_CHECK(!training() && batchNorm_, "a max-pool rides on a batch-normalised convolution at inference only");
+        PX_CHECK(outHeight() % 2 == 0 && outWidth() % 2 == 0, "a max-pool rides only where its windows tile the plane");
+        PX_CHECK(pooled && pooled->size() * 4 == output_.size(), "ConvLayer: the pool's output does not match the layer's");
+        pooled_ = pooled;
+        keepOutput_ = keepOutput;
+    }
+    bool carriesPool() const noexcept { return pooled_ != nullptr; }
+
     void setConvolution(Convolve fwd, ConvolveBackward bwd)
     {
         convolve_ = std::move(fwd);
@@ -146,6 +159,13 @@ public:
                                                                 rider_.from->data(), rider_.alpha, rider_.beta, batch(),
                                                                 filters_, spatial, activation_, stream()));
             }
+            return;
+        }
+        if (pooled_) {
+            fold();
+            PX_HIP_CHECK(pxh_bn_folded_act_maxpool_forward(x, keepOutput_ ? output_.data() : nullptr, pooled_->data(),
+                                                           folded_.data(), batch(), filters_, outHeight(), outWidth(),
+                                                           activation_, stream()));
             return;
         }
         if (!batchNorm_) {
@@ -366,6 +386,8 @@ private:
     int activation_ = PXH_LOGISTIC, filters_ = 1;
     bool batchNorm_ = false, foldedValid_ = false;
     Rider rider_;
+    V* pooled_ = nullptr;           // the riding pool's output
+    bool keepOutput_ = false;
     const float* x_ = nullptr;      // conv result of the last forward (borrowed)
     V biases_, scales_, rollingMean_, rollingVar_, mean_, var_, folded_;
     V biasUpdates_, scaleUpdates_, biasM_, biasV_, scaleM_, scaleV_;
@@ -520,9 +542,23 @@ public:
         if (training()) indexes_ = IntVector(output_.size());
     }
 
+    // At inference this pool rides on the epilogue of the convolution in front of it
+    // (pxh_bn_folded_act_maxpool_forward): for whoever builds the network, for the 2 x 2 window at stride 2
+    // over planes of even size.  `convOutputIsRead`: something else reads the convolution's output as well.
+    // forward() then finds its output written (and keeps no indexes: nothing reads them at inference).
+    void rideOn(ConvLayer& conv, bool convOutputIsRead)
+    {
+        PX_CHECK(kernel_ == 2 && stride_ == 2 && padding_ <= 1, "only the 2 x 2 pool at stride 2 rides");
+        PX_CHECK(conv.batch() == batch() && conv.outChannels() == channels() && conv.outHeight() == height() &&
+                 conv.outWidth() == width(), "maxpool: the convolution in front has another shape");
+        conv.carryPool(&output_, convOutputIsRead);
+        riding_ = true;
+    }
+
     void forward(const V& input) override
     {
         Layer::forward(input);
+        if (riding_) return;        // the convolution in front has written output_
         checkInput(input, "MaxPoolLayer");
         if (indexes_.empty()) indexes_ = IntVector(output_.size());
         PX_HIP_CHECK(pxh_maxpool_forward(input.data(), output_.data(), indexes_.data(), batch(), channels(),
@@ -543,6 +579,7 @@ public:
 
 private:
     int kernel_ = 1, stride_ = 1, padding_ = 0;
+    bool riding_ = false;
     IntVector indexes_;
 };
 

@@ -1083,6 +1083,60 @@ void ridingShortcutChecks()
     }, "linear");
 }
 
+// At inference a 2 x 2 / 2 max-pool rides on the epilogue of the convolution in front of it: the pool's output
+// is that of the two layers one after the other, bit for bit; the convolution's own output is written only
+// when something else reads it.
+void ridingPoolChecks()
+{
+    struct Pair {
+        Context ctx;
+        std::shared_ptr<ConvLayer> conv;
+        std::shared_ptr<MaxPoolLayer> pool;
+        Pair(bool riding, bool keep)
+        {
+            ctx.training = false;
+            conv = std::make_shared<ConvLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S },
+                                                                { "width", S }, { "filters", C },
+                                                                { "batch_normalize", true },
+                                                                { "activation", std::string("leaky") } });
+            pool = std::make_shared<MaxPoolLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S },
+                                                                   { "width", S }, { "kernel", 2 }, { "stride", 2 } });
+            conv->copyScales(normals(741, C));
+            conv->copyBiases(normals(742, C));
+            conv->copyRollingMean(normals(743, C));
+            Host var = normals(744, C);
+            for (float& v: var) v = 0.5f + v * v;
+            conv->copyRollingVariance(var);
+            if (riding) pool->rideOn(*conv, keep);
+        }
+        void forward(const FloatVector& input)
+        {
+            conv->forward(input);
+            pool->forward(conv->output());
+        }
+    };
+    const FloatVector input(normals(745, size_t(N) * C * S * S));
+    Pair plain(false, false), riding(true, false), keeping(true, true);
+    plain.forward(input);
+    riding.forward(input);
+    keeping.forward(input);
+    report("riding pool: the convolution says so", riding.conv->carriesPool() && !plain.conv->carriesPool());
+    report("riding pool: the pool's output", riding.pool->output().asVector() == plain.pool->output().asVector());
+    report("riding pool: the pool's output, the convolution's kept",
+           keeping.pool->output().asVector() == plain.pool->output().asVector());
+    report("riding pool: the convolution's output when kept",
+           keeping.conv->output().asVector() == plain.conv->output().asVector());
+    expectThrows("a pool does not ride in training", [] {
+        Context ctx;
+        ctx.training = true;
+        ConvLayer conv(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S }, { "width", S }, { "filters", C },
+                                        { "batch_normalize", true } });
+        MaxPoolLayer pool(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S }, { "width", S },
+                                           { "kernel", 2 }, { "stride", 2 } });
+        pool.rideOn(conv, false);
+    }, "inference");
+}
+
 // The small network with the shortcut and the head leaving the norms of the deltas they write last
 // (conv2's and conv6's): every delta and every update buffer as without, bit for bit.
 void leavesNormNetChecks()
@@ -1303,6 +1357,7 @@ int main(int argc, char** argv)
             firstWriterShortcutChecks();
             leavesNormShortcutChecks();
             ridingShortcutChecks();
+            ridingPoolChecks();
             leavesNormNetChecks();
             deferredHeadsChecks();
             capturedSequenceChecks();

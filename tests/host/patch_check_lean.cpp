@@ -10,7 +10,7 @@
 #include "hip_lean/Layer.h"
 #include "hip_lean/Model.h"
 #include "hip/Adam.h"
-#include "hip/MaxPoolLayer.h"
+#include "hip_lean/MaxPoolLayer.h"
 #include "hip/UpsampleLayer.h"
 #include "hip/RouteLayer.h"
 #include "hip_lean/ShortcutLayer.h"

@@ -120,7 +120,7 @@ def test_binding_headers_and_stub_name_only_members_the_engine_has():
             methods = set(re.findall(r"this->(\w+)\(", text)) | set(re.findall(r"\bnet\.(\w+)\(", text))
             for m in sorted(members | methods):
                 if m in own or m in ("deferHead", "normGroupsFor", "noteNormGroups", "takeNormGroups", "overwritten",
-                                     "registerParameters", "updateAll", "rides", "riderOf"):
+                                     "registerParameters", "updateAll", "rides", "riderOf", "poolOf"):
                     continue
                 assert m in known, "%s/%s names `%s`, which the engine's %s does not have" % (folder, name, m, layer)
                 checked += 1
