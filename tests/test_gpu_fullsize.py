@@ -272,6 +272,31 @@ def test_yolo_largest_head(ops, oracle):
     assert again[2] == cost and np.array_equal(again[3], stats), "cost and statistics must not depend on timing"
 
 
+def test_yolo_three_heads_at_full_batch_in_one_pass(ops, oracle):
+    """64 x 255 x {19, 38, 76}^2 through pxh_yolo_forward_train_heads: every head against the checker run head by
+    head on the same logits and truths; every truth claims exactly one slot on the head that holds its best
+    anchor; each head's cost is the checksum of its delta."""
+    from test_gpu_yolo_adam import compare_head, oracle_head
+    from test_gpu_yolo_heads import run_heads
+    N, K = 64, 80
+    sizes = [19, 38, 76]
+    masks = [wl.YOLOV3_MASKS[s] for s in sizes]
+    xs = [wl.normal(5000 + W, (N, 3 * (K + 5), W, W), std=2.0) for W in sizes]
+    truths, counts = wl.yolo_truths(5100, N)
+    kw = dict(ignore_thresh=0.7, truth_thresh=1.0, coord_scale=1.0, object_scale=2.0, noobject_scale=0.1,
+              class_scale=1.0)
+    got = run_heads(ops, xs, truths, counts, sizes, K, masks, wl.YOLOV3_ANCHORS, 608, [kw] * 3)
+    positives = 0
+    for x, W, mask, g in zip(xs, sizes, masks, got):
+        want = oracle_head(oracle, x, truths, counts, W, W, K, mask, wl.YOLOV3_ANCHORS, 608, **kw)
+        # the CPU layer's statistics are running fp32 sums over up to 1.1 M slots (see test_yolo_largest_head)
+        compare_head(g, want, "head %d of three at batch 64" % W, 3, kw, sum_rtol=2e-3)
+        positives += want[3][6]
+        checksum = float(np.square(g[1].astype(np.float64)).sum())
+        assert abs(g[2] - checksum) <= 1e-5 * checksum, (W, g[2], checksum)
+    assert positives == counts.sum()
+
+
 def test_yolo_one_launch_sums_do_not_depend_on_arrival_order(ops, oracle):
     """64 x 255 x 19^2 in the one-launch form, where whichever head workgroup finishes last adds up the
     sums of all of them: cost, statistics and every delta are bit-identical from run to run, for each
