@@ -782,6 +782,9 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
     rows[-1]["vs_same_mix"] = round(mix_ms / ms_adam, 3)
     add("copy_same_mix(4 read + 4 written)", "%d floats per stream" % P, 32 * P, mix_ms,
         "no arithmetic: the ceiling of Adam's traffic mix; a 1+1 copy of these bytes runs at 6.5 TB/s")
+    ms_adamw = timer.time(lambda i: ops.adam_update(w, d, m, v, 16, 7, 1e-3, 0.9, 0.999, 1e-8, 5e-4, 2), 10)
+    add("adam_update(decoupled decay)", "%d params" % P, 32 * P, ms_adamw,
+        "32B/param; the decay as the baseline's configuration words it; not in ms/batch (the reference's form is)")
 
     # ---- SGD with momentum over the same buffer (the optimiser of the shipped presets)
     ms_sgd = timer.time(lambda i: ops.sgd_update(w, d, 16, 1e-3, 0.9, 5e-4, True), 10)

@@ -519,7 +519,12 @@ int pxh_adam(int n, float* x, const float* m, const float* v, float beta1, float
 /* Whole Adam<CUDA>::update in one pass, same per-element operation order:
  *   d *= 1/batch; if apply_decay d += -decay*w; m = b1*m + (1-b1)*d; v = b2*v + (1-b2)*d*d;
  *   w += lr * (m/(1-b1^t)) / (sqrt(v/(1-b2^t)) + eps);  d = 0.
- * (L2 decay folded into the update before the moments, as the reference does; not decoupled.) */
+ * (apply_decay == 1: L2 decay folded into the update before the moments, as the reference does.)
+ * apply_decay == 2 is the decoupled form, which the reference does not have: the moments are formed from
+ * the plain update and the weight also shrinks by lr * decay of its old value,
+ *   w = (w + lr * (m/(1-b1^t)) / (sqrt(v/(1-b2^t)) + eps)) + (-(lr * decay)) * w,
+ * each operation rounded to fp32.  Other values of apply_decay are rejected.  The many-tensor forms
+ * below take the reference's form only. */
 int pxh_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch, int t, float lr,
                     float beta1, float beta2, float eps, float decay, int apply_decay, void* stream);
 

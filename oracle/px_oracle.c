@@ -934,19 +934,25 @@ int pxo_yolo_build_targets(const pxo_yolo_cfg* g, const float* truths, int count
 /* One fp32 rounding per BLAS call of the reference sequence, in its order:
  * scale the update by 1/batch; fold L2 decay into it (weights only); decay
  * both moments; add the update / its square; bias-corrected step ADDED to the
- * weights (updates are negative gradients); clear the update buffer. */
+ * weights (updates are negative gradients); clear the update buffer.
+ * apply_decay: 0 no decay; 1 the reference's L2 term, folded into the update before
+ * the moments; 2 decoupled decay, w += step - (lr * decay) * w with the moments formed
+ * from the plain update.  The reference has no such form (parity unpinned by the
+ * reference): it is the textbook AdamW recurrence in the reference's sign convention,
+ * held against that recurrence in fp64 and against its closed form at t = 1. */
 void pxo_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch, int t, float lr,
                      float beta1, float beta2, float eps, float decay, int apply_decay)
 {
     const float inv_batch = 1.0f / (float) batch;
     const float neg_decay = -decay;
+    const float neg_lr_decay = -(lr * decay);
     const float a1 = 1.0f - beta1;
     const float a2 = 1.0f - beta2;
     const float c1 = 1.0f - powf(beta1, (float) t);
     const float c2 = 1.0f - powf(beta2, (float) t);
     for (size_t i = 0; i < n; ++i) {
         float g = d[i] * inv_batch;
-        if (apply_decay) {
+        if (apply_decay == 1) {
             float l2 = neg_decay * w[i];
             g = g + l2;
         }
@@ -960,7 +966,12 @@ void pxo_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch
         float mhat = mi / c1;
         float vhat = vi / c2;
         float step = lr * mhat / (sqrtf(vhat) + eps);
-        w[i] = w[i] + step;
+        float wi = w[i] + step;
+        if (apply_decay == 2) {
+            float shrink = neg_lr_decay * w[i];
+            wi = wi + shrink;
+        }
+        w[i] = wi;
         m[i] = mi;
         v[i] = vi;
         d[i] = 0.0f;

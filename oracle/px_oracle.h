@@ -135,7 +135,9 @@ void pxo_route_forward(const float* layer_output, float* route_output, int batch
 void pxo_route_backward(const float* route_delta, float* layer_delta, int batch, int layer_outputs,
                         int route_outputs, int offset);
 
-/* ---- Adam: include/cuda/Adam.h:49-90 + src/Adam.cu:26-37 ---- */
+/* ---- Adam: include/cuda/Adam.h:49-90 + src/Adam.cu:26-37.  apply_decay: 0 none, 1 the reference's L2 term
+ * (folded into the update before the moments), 2 decoupled (no counterpart in the reference; pinned by the
+ * fp64 AdamW recurrence and its closed form at t = 1). ---- */
 void pxo_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch, int t, float lr,
                      float beta1, float beta2, float eps, float decay, int apply_decay);
 

@@ -599,7 +599,8 @@ struct AdamUpdateOp {
     float* m;
     float* v;
     float inv_batch, neg_decay, beta1, beta2, a1, a2, c1, c2, lr, eps;
-    int apply_decay;
+    float neg_lr_decay;     // -(lr * decay), for the decoupled form only
+    int apply_decay;        // 0: none; 1: folded into the update before the moments (the reference); 2: decoupled
     template<int V> struct Regs { Pack<V> w, d, m, v; };
     template<int V, bool NT> __device__ void load(size_t e, Regs<V>& r) const
     {
@@ -614,7 +615,7 @@ struct AdamUpdateOp {
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             float g = r.d.v[k] * inv_batch;
-            if (apply_decay) {
+            if (apply_decay == 1) {
                 const float l2 = neg_decay * r.w.v[k];
                 g = g + l2;
             }
@@ -628,7 +629,13 @@ struct AdamUpdateOp {
             const float mhat = mi / c1;
             const float vhat = vi / c2;
             const float step = lr * mhat / (sqrtf(vhat) + eps);
-            ow.v[k] = r.w.v[k] + step;
+            float wi = r.w.v[k] + step;
+            if (apply_decay == 2) {
+                // decoupled: the weight shrinks by lr * decay of its old value, outside the moments
+                const float shrink = neg_lr_decay * r.w.v[k];
+                wi = wi + shrink;
+            }
+            ow.v[k] = wi;
             om.v[k] = mi;
             ov.v[k] = vi;
             od.v[k] = 0.0f;
@@ -1346,10 +1353,13 @@ int pxh_adam_update(size_t n, float* w, float* d, float* m, float* v, int batch,
     if ((!w || !d || !m || !v) && n) return fail_invalid("pxh_adam_update: null pointer");
     if (batch <= 0) return fail_invalid("pxh_adam_update: batch must be positive");
     if (t < 1) return fail_invalid("pxh_adam_update: t must be at least 1 (the update count is pre-incremented)");
+    if (apply_decay < 0 || apply_decay > 2)
+        return fail_invalid("pxh_adam_update: apply_decay is 0 (none), 1 (folded into the update) or 2 (decoupled)");
     AdamUpdateOp op;
     op.w = w; op.d = d; op.m = m; op.v = v;
     op.inv_batch = 1.0f / static_cast<float>(batch);
     op.neg_decay = -decay;
+    op.neg_lr_decay = -(lr * decay);
     op.beta1 = beta1; op.beta2 = beta2;
     op.a1 = 1.0f - beta1; op.a2 = 1.0f - beta2;
     op.c1 = 1.0f - powf(beta1, static_cast<float>(t));

@@ -410,9 +410,10 @@ def adam(x, m, v, beta1, beta2, rate, eps, t):
 
 
 def adam_update(w, d, m, v, batch, t, lr, beta1=0.9, beta2=0.999, eps=1e-8, decay=0.0, apply_decay=False):
+    """apply_decay: False / 0 none, True / 1 the reference's L2 term, 2 decoupled decay."""
     _chk_all(w, d, m, v)
     call("pxh_adam_update", w.numel(), ptr(w), ptr(d), ptr(m), ptr(v), int(batch), int(t), float(lr), float(beta1),
-         float(beta2), float(eps), float(decay), int(bool(apply_decay)), _stream())
+         float(beta2), float(eps), float(decay), int(apply_decay), _stream())
 
 
 def _pointer_table(tensors):

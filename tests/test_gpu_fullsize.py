@@ -324,8 +324,10 @@ def test_yolo_one_launch_sums_do_not_depend_on_arrival_order(ops, oracle):
         lib.pxh_debug_yolo_tuning(0, 0, 0)
 
 
-def test_adam_full_parameter_buffer(ops, oracle):
-    """61.9 M parameters, 10 steps: the first, a middle and the last million against the checker."""
+@pytest.mark.parametrize("decay_form", [1, 2])
+def test_adam_full_parameter_buffer(ops, oracle, decay_form):
+    """61.9 M parameters, 10 steps: the first, a middle and the last million against the checker, with the
+    reference's L2 term (1) and with the decoupled decay the baseline's configuration names (2)."""
     import torch
     P = wl.YOLOV3_PARAMS
     w = device_normal((P,), 27, 0.02); g = device_normal((P,), 28, 1e-3)
@@ -337,10 +339,10 @@ def test_adam_full_parameter_buffer(ops, oracle):
     hm = [np.zeros(b - a, F) for a, b in spans]; hv = [np.zeros(b - a, F) for a, b in spans]
     for t in range(1, 11):
         d.copy_(g)
-        ops.adam_update(w, d, m, v, 16, t, 1e-3, 0.9, 0.999, 1e-8, 5e-4, True)
+        ops.adam_update(w, d, m, v, 16, t, 1e-3, 0.9, 0.999, 1e-8, 5e-4, decay_form)
         for k in range(len(spans)):
             hd = hg[k].copy()
-            oracle.adam_update(hw[k], hd, hm[k], hv[k], 16, t, 1e-3, 0.9, 0.999, 1e-8, 5e-4, True)
+            oracle.adam_update(hw[k], hd, hm[k], hv[k], 16, t, 1e-3, 0.9, 0.999, 1e-8, 5e-4, decay_form)
     assert float(d.abs().max()) == 0.0, "the update buffer must be zero after a step"
     for k, (a, b) in enumerate(spans):
         assert_close(host(w[a:b]), hw[k], 1e-6, 1e-3, "weights of span %d" % k)

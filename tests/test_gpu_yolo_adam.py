@@ -289,6 +289,28 @@ def test_adam_update_10_steps_matches_oracle(ops, oracle, n):
     assert np.max(np.abs(w - w0)) > 1e-4
 
 
+@pytest.mark.parametrize("n", [5, 4096, 1000003])
+def test_adam_update_with_decoupled_decay_matches_oracle(ops, oracle, n):
+    """apply_decay = 2, the decoupled weight decay the baseline's training configuration names (the reference
+    folds an L2 term into the update instead): 10 steps against the CPU checker, <= 1e-6."""
+    from pixienn_amd import capi
+    w0 = wl.normal(3200, n, std=0.02)
+    w, m, v = w0.copy(), np.zeros(n, F), np.zeros(n, F)
+    gw, gm, gv = gpu(w0), gpu(m), gpu(v)
+    for t in range(1, 11):
+        g = wl.normal(3200 + t, n, std=1e-3)
+        oracle.adam_update(w, g.copy(), m, v, 16, t, ADAM["lr"], ADAM["beta1"], ADAM["beta2"], ADAM["eps"], ADAM["decay"], 2)
+        gd = gpu(g)
+        ops.adam_update(gw, gd, gm, gv, 16, t, apply_decay=2, **ADAM)
+        assert not host(gd).any(), "the update buffer is cleared"
+    assert_close(host(gw), w, 1e-6, 1e-3, "weights after 10 decoupled steps")
+    assert_close(host(gm), m, 1e-6, 1e-7, "first moment")
+    assert_close(host(gv), v, 1e-6, 1e-14, "second moment")
+    rc = capi.call_raw("pxh_adam_update", n, gw.data_ptr(), gd.data_ptr(), gm.data_ptr(), gv.data_ptr(), 16, 1, 1e-3, 0.9,
+                       0.999, 1e-8, 5e-4, 3, None)
+    assert rc == -1 and "apply_decay" in capi.last_error()
+
+
 def test_adam_without_decay_and_batch1(ops, oracle):
     n = 10001
     w0 = wl.normal(3100, n, std=0.02); g = wl.normal(3101, n, std=1e-3)

@@ -548,6 +548,36 @@ def test_adam_10_steps_vs_fp64_l2(oracle):
     assert np.max(np.abs(w - w64)) < 1e-6
 
 
+def test_adam_decoupled_decay_closed_form_and_fp64_recurrence(oracle):
+    """apply_decay = 2 (no counterpart in the reference): from zero moments at t = 1 the weight is
+    w0 + lr*g/(|g|+eps) - lr*decay*w0; ten steps against the AdamW recurrence carried in fp64, which the
+    L2 form (apply_decay = 1) measurably is not."""
+    rng = np.random.default_rng(53)
+    n = 2048
+    lr, b1, b2, eps, decay, batch = 1e-3, 0.9, 0.999, 1e-8, 5e-4, 16
+    w0 = (0.02 * rng.standard_normal(n)).astype(F)
+    g0 = (1e-3 * rng.standard_normal(n)).astype(F)
+    w, d, m, v = w0.copy(), g0.copy(), np.zeros(n, F), np.zeros(n, F)
+    oracle.adam_update(w, d, m, v, 1, 1, lr, b1, b2, eps, 0.5, 2)          # a decay large enough to see
+    g = g0.astype(np.float64)
+    want = w0 + lr * g / (np.abs(g) + eps) - lr * 0.5 * w0.astype(np.float64)
+    assert np.max(np.abs(w - want) / np.maximum(np.abs(want), 1e-3)) < 1e-5
+    assert np.allclose(m, 0.1 * g, rtol=1e-6) and np.all(d == 0)           # the moments do not see the decay
+    w = w0.copy(); m = np.zeros(n, F); v = np.zeros(n, F)
+    l2 = w0.copy(); m2 = np.zeros(n, F); v2 = np.zeros(n, F)
+    w64 = w.astype(np.float64); m64 = np.zeros(n); v64 = np.zeros(n)
+    for t in range(1, 11):
+        g = (1e-3 * rng.standard_normal(n)).astype(F)
+        oracle.adam_update(w, g.copy(), m, v, batch, t, lr, b1, b2, eps, decay, 2)
+        oracle.adam_update(l2, g.copy(), m2, v2, batch, t, lr, b1, b2, eps, decay, 1)
+        g64 = g.astype(np.float64) / batch
+        m64 = b1 * m64 + (1 - b1) * g64
+        v64 = b2 * v64 + (1 - b2) * g64 * g64
+        w64 = w64 + lr * (m64 / (1 - b1 ** t)) / (np.sqrt(v64 / (1 - b2 ** t)) + eps) - lr * decay * w64
+    assert np.max(np.abs(w - w64) / np.maximum(np.abs(w64), 1e-2)) < 1e-6
+    assert np.max(np.abs(l2 - w64) / np.maximum(np.abs(w64), 1e-2)) > 1e-3
+
+
 def test_sgd_closed_form_and_fp64_recurrence(oracle):
     """The reference holds no numeric test of ConvLayer::update: one step against its closed form,
     ten steps against the same recurrence carried in fp64."""
