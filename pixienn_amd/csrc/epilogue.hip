@@ -984,6 +984,36 @@ __device__ __forceinline__ void resident_sum2(double& a, double& b, double (*slo
     b = tb;
 }
 
+// The same for a workgroup of half the size whose thread t stands in for threads t and t + T of a workgroup
+// of 2 T threads (sums a of the first, b of the second): the additions of resident_sum2<2 * T>, in its order.
+template<int T>
+__device__ __forceinline__ void resident_sum2_twin(double& a1, double& a2, double b1, double b2,
+                                                   double (*slots)[2 * T / kWave])
+{
+    a1 = wave_sum(a1);
+    a2 = wave_sum(a2);
+    b1 = wave_sum(b1);
+    b2 = wave_sum(b2);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) {
+        slots[0][wave] = a1;
+        slots[1][wave] = a2;
+        slots[0][wave + T / kWave] = b1;
+        slots[1][wave + T / kWave] = b2;
+    }
+    __syncthreads();
+    double ta = 0.0, tb = 0.0;
+#pragma unroll
+    for (int w = 0; w < 2 * T / kWave; ++w) {
+        ta += slots[0][w];
+        tb += slots[1][w];
+    }
+    a1 = ta;
+    a2 = tb;
+}
+
 // The same for three sums and a maximum (the first pass of a clipped backward).
 template<int T>
 __device__ __forceinline__ void resident_sum3_max(double& a, double& b, double& q, float& top,
@@ -1069,7 +1099,12 @@ __global__ __launch_bounds__(T, L == 0 && V * R <= 32 ? 8 : 4) void bn_resident_
 {
     static_assert(L == 0 || T == kResidentThreads, "the LDS part is laid out for the full workgroup");
     extern __shared__ __align__(16) float resident_lds[];
-    __shared__ double slots[2][T / kWave];
+    // The 128-bit form with workgroups of half the size adds a channel up exactly as the full workgroups do,
+    // so that a layer gives the same statistics to the bit with and without a shortcut riding on it: thread t
+    // keeps the sums of the full form's threads t (even steps) and t + T (odd steps) apart.
+    constexpr bool kTwin = V == 4 && T < kResidentThreads;
+    static_assert(!kTwin || 2 * T == kResidentThreads, "half the size");
+    __shared__ double slots[2][(kTwin ? 2 : 1) * T / kWave];
     __shared__ FoldCoef shared_coef;
     const uint32_t c = blockIdx.x;
     const float shift = a.x[static_cast<size_t>(c) * a.g.spatial];
@@ -1077,6 +1112,7 @@ __global__ __launch_bounds__(T, L == 0 && V * R <= 32 ? 8 : 4) void bn_resident_
     const float rm_in = a.rolling_mean[c], rv_in = a.rolling_var[c], scale_in = a.scale[c], bias_in = a.bias[c];
     Pack<V> v[R];
     float a1 = 0.0f, a2 = 0.0f;
+    [[maybe_unused]] float b1 = 0.0f, b2 = 0.0f;
     // Every tensor here is touched once and goes past the caches (non-temporal: with the whole slice
     // of every channel asked for at once, cached reads run at two thirds of the rate; the backward
     // kernel keeps x cached, which it reads twice).
@@ -1090,11 +1126,17 @@ __global__ __launch_bounds__(T, L == 0 && V * R <= 32 ? 8 : 4) void bn_resident_
     };
     const auto add = [&](int r, const Pack<V>& t) {
         const bool valid = element(r) < a.g.per_channel;
+        const bool second = kTwin && (r & 1);
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             const float d = t.v[k] - shift;
-            a1 += valid ? d : 0.0f;
-            a2 += valid ? d * d : 0.0f;
+            if (second) {
+                b1 += valid ? d : 0.0f;
+                b2 += valid ? d * d : 0.0f;
+            } else {
+                a1 += valid ? d : 0.0f;
+                a2 += valid ? d * d : 0.0f;
+            }
         }
     };
     // the LDS part first, all of it at once: its registers are free again before the register part
@@ -1116,7 +1158,9 @@ __global__ __launch_bounds__(T, L == 0 && V * R <= 32 ? 8 : 4) void bn_resident_
     // The shortcut's source does not wait for the statistics: its first steps are asked for now, behind the
     // slice's own loads, and arrive while the sums are formed -- all of them where a lane holds few values
     // (16 x 1024 x 19^2: 19.9 us against 25.6 us with every step's load behind the reduction).
-    constexpr int kAhead = !RES ? 0 : V * (R + L) <= 8 ? R + L : L > 0 ? kResidualAhead : 0;
+    // (the half-size workgroups of the 128-bit form have 128 registers: eight of twelve steps, four of sixteen)
+    constexpr int kAhead = !RES ? 0 : V * (R + L) <= 8 ? R + L : L > 0 ? kResidualAhead
+                                : T < kResidentThreads ? (R <= 12 ? 8 : 4) : 0;
     [[maybe_unused]] Pack<V> ahead[kAhead > 0 ? kAhead : 1];
     if constexpr (RES) {
 #pragma unroll
@@ -1128,7 +1172,8 @@ __global__ __launch_bounds__(T, L == 0 && V * R <= 32 ? 8 : 4) void bn_resident_
 #pragma unroll
     for (int r = R - 1; r >= 0; --r) add(r, v[r]);
     double s1 = static_cast<double>(a1), s2 = static_cast<double>(a2);
-    resident_sum2<T>(s1, s2, slots);
+    if constexpr (kTwin) resident_sum2_twin<T>(s1, s2, static_cast<double>(b1), static_cast<double>(b2), slots);
+    else resident_sum2<T>(s1, s2, slots);
     if (threadIdx.x == 0) {
         const ChannelStats st = channel_stats(s1, s2, shift, static_cast<double>(a.g.per_channel), rm_in, rv_in);
         a.mean[c] = st.mean;
@@ -1668,6 +1713,22 @@ int bn_train_forward(const char* who, const float* x, float* y, float* pre_activ
                     if (narrow) {
                         hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 1, kResidentNarrowVectors, 0, kResidentNarrowThreads>),
                                            grid, block, 0, s, r);
+                        return;
+                    }
+                }
+                if constexpr (RES) {
+                    // The 128-bit form with the shortcut's source on top of eight vectors of the slice spills at
+                    // 64 registers: half-size workgroups with twice the vectors per lane and twice the registers
+                    // keep the same two workgroups per compute unit (16 x 512 x 38^2: 26.2 against 30.9 us).
+                    if (vec && per_thread <= kResidentVectors) {
+                        const size_t vectors = (static_cast<size_t>(batch) * spatial + 3) / 4;
+                        const dim3 half(kResidentNarrowThreads);
+                        if (vectors <= 12u * kResidentNarrowThreads)
+                            hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 4, 12, 0, kResidentNarrowThreads, true>), grid,
+                                               half, 0, s, r);
+                        else
+                            hipLaunchKernelGGL((bn_resident_fwd_kernel<ACT, 4, 16, 0, kResidentNarrowThreads, true>), grid,
+                                               half, 0, s, r);
                         return;
                     }
                 }

@@ -26,7 +26,8 @@ def ops():
 
 @pytest.mark.parametrize("act", ["leaky", "mish", "linear", "logistic"])
 def test_training_epilogue_with_shortcut_is_the_two_calls_to_the_bit(ops, act):
-    for si, (N, C, HW) in enumerate(TRAIN_SHAPES):
+    # (+ a 128-bit slice of 7000 vectors: the half-size workgroups with sixteen vectors per lane)
+    for si, (N, C, HW) in enumerate(TRAIN_SHAPES + [(4, 96, 7000)]):
         x, scale, bias, rmean, rvar = bn_case(3000 + si, N, C, HW, spread=1.5)
         frm = wl.normal(3050 + si, x.shape)
         alpha, beta = FACTORS[si % 2]
