@@ -344,7 +344,8 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     groups = {i - 1: ops.norm_groups_like(T[i - 1]["d"]) for i, l in enumerate(layers)
               if l["type"] in ("shortcut", "yolo")}
 
-    def backward(_, first_writer=False, norm_from_writer=False, two_calls=False, shortcut_rides=False):
+    def backward(_, first_writer=False, norm_from_writer=False, two_calls=False, shortcut_rides=False,
+                 shortcut_clipped=False):
         n = 0
         for i in reversed(range(len(layers))):
             l, t = layers[i], T[i]
@@ -352,9 +353,19 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
             if shortcut_rides and kind == "shortcut" and i - 1 in rides:
                 # the shortcut's own rescale + clip, its delta to the `from` layer (first writer), and
                 # nothing to the convolution in front, which takes this delta as its own
+                if shortcut_clipped:        # ... as one call that reads the delta once
+                    ops.shortcut_backward_clipped(t["d"], T[l["frm"]]["d"], None, "linear", first=True, threshold=100.0,
+                                                  clip=10.0)
+                    n += 1
+                    continue
                 ops.rescale_clip(t["d"], 100.0, 10.0)
                 ops.shortcut_backward_first(t["d"], T[l["frm"]]["d"], None, "linear")
                 n += 2
+                continue
+            if shortcut_clipped and kind == "shortcut" and first_writer and not norm_from_writer:
+                ops.shortcut_backward_clipped(t["d"], T[l["frm"]]["d"], T[i - 1]["d"], "linear", first=True,
+                                              threshold=100.0, clip=10.0)
+                n += 1
                 continue
             if shortcut_rides and kind == "conv" and i in rides:
                 ops.bn_act_backward_clipped(T[rides[i]]["d"], t["x"], t["mean"], t["var"], t["scale"], t["bias"],
@@ -436,7 +447,11 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     out["forward_heads_one_call_each_ms"] = round(timer.time(lambda i: forward(i, heads_apart=True), 3, warm=1), 3)
     out["forward_fills_together_ms"] = round(timer.time(lambda i: forward(i, False, True), 3, warm=1), 3)
     out["forward_first_writer_ms"] = round(timer.time(lambda i: forward(i, True, True), 3, warm=1), 3)
-    out["backward_first_writer_ms"] = round(timer.time(lambda i: backward(i, True), 3, warm=1), 3)
+    # (a first-writer shortcut's targets are plain functions of its delta: the rescale + clip that opens its backward
+    # and the backward itself run as one call that reads the delta once, pxh_shortcut_backward_clipped;
+    # `..._shortcut_helpers_apart_ms`: as the two calls, for comparison)
+    out["backward_first_writer_ms"] = round(timer.time(lambda i: backward(i, True, shortcut_clipped=True), 3, warm=1), 3)
+    out["backward_first_writer_shortcut_helpers_apart_ms"] = round(timer.time(lambda i: backward(i, True), 3, warm=1), 3)
     # the 23 shortcuts and 3 heads leave the norm and peak of the delta they write last: 26 deltas are not
     # read for their norm ("leaves_norm" of the C++ layer interface); same values to the bit
     out["backward_norm_from_writer_ms"] = round(timer.time(lambda i: backward(i, False, True), 3, warm=1), 3)
@@ -445,7 +460,10 @@ def measure_model_order(torch, ops, wl, timer, N=16, plain_only=False):
     # the shortcut of a residual block on the epilogue of the convolution in front of it (first-writer forms
     # everywhere else): no pass of its own forward, and backward the convolution takes the shortcut's delta
     out["forward_shortcut_in_epilogue_ms"] = round(timer.time(lambda i: forward(i, True, True, shortcut_rides=True), 3, warm=1), 3)
-    out["backward_shortcut_in_epilogue_ms"] = round(timer.time(lambda i: backward(i, True, shortcut_rides=True), 3, warm=1), 3)
+    out["backward_shortcut_in_epilogue_ms"] = round(timer.time(
+        lambda i: backward(i, True, shortcut_rides=True, shortcut_clipped=True), 3, warm=1), 3)
+    out["backward_shortcut_in_epilogue_shortcut_helpers_apart_ms"] = round(timer.time(
+        lambda i: backward(i, True, shortcut_rides=True), 3, warm=1), 3)
     out["shortcuts_in_epilogue"] = len(rides)
     # the leanest step: no dead pass in update(), and whichever of the lean forward and backward forms is
     # faster here (since the rescale + clip rides on the convolutions' own backward, leaving the norm with
@@ -576,6 +594,17 @@ def measure_extras(torch, ops, wl, timer, capi, cpu=None, only_heads=False):
             ms_n = timer.time(lambda i: ops.shortcut_backward_norm(o[i], a[i], b[i], groups[i], "linear"), 20, rotate=rot)
             add("shortcut_bwd+norm", "%dx%dx%d^2" % (N, c, s), 20 * e, ms_n, "20B/elem + 8B per 256 values of grad")
             del groups
+            # a first writer with Layer::backward's rescale + clip in front, as one call (the delta read once when
+            # nothing changes: thresholds far away) and as the two calls it stands for
+            ms_c = timer.time(lambda i: ops.shortcut_backward_clipped(o[i], a[i], b[i], "linear", first=True,
+                                                                      threshold=1e9, clip=1e9), 20, rotate=rot)
+            def two_calls(i):
+                ops.rescale_clip(o[i], 1e9, 1e9)
+                ops.shortcut_backward_first(o[i], a[i], b[i], "linear")
+            ms_2 = timer.time(two_calls, 20, rotate=rot)
+            add("shortcut_bwd_first+clip", "%dx%dx%d^2" % (N, c, s), 12 * e, ms_c,
+                "rescale + clip of the delta, then the first writer's backward: 12B/elem; as two calls (16B/elem) %.4f ms"
+                % ms_2)
             shortcut_ms[(c, s)] = (ms_f, ms_b, count)
             del a, b, o
         # ---- the delta zero-fill of Layer::forward (include/Layer.h:377-383): write-only, 4 B per element

@@ -42,6 +42,7 @@ public:
         return g;
     }
     void noteNormGroups(const float* delta, const float* groups) const { notes_[delta] = groups; }
+    bool hasNormGroups(const float* delta) const { return notes_.count(delta) != 0; }
     const float* takeNormGroups(const float* delta) const
     {
         const auto it = notes_.find(delta);

@@ -36,11 +36,23 @@ inline void ShortcutLayer<Device::HIP>::forward(const V& input)
 template<>
 inline void ShortcutLayer<Device::HIP>::backward(const V& input, V* grad)
 {
-    Layer<Device::HIP>::backward(input, grad);
     const auto& net = this->model();
     const bool sameShape = from_->outWidth() == this->outWidth() && from_->outHeight() == this->outHeight() &&
                            from_->outChannels() == this->outChannels();
     const float* pre = preActivation_.empty() ? nullptr : preActivation_.data();
+    // A riding shortcut that is the first to write its `from` layer's delta: the rescale + clip of delta_ that opens
+    // every layer's backward and the shortcut's own backward as ONE call, which reads delta_ once when nothing has
+    // to change (pxh_shortcut_backward_clipped: the values of the two calls to the bit).
+    const float threshold = this->gradientRescaling_ ? this->gradientThreshold_ : 0.0f;
+    const float clip = this->gradientClipping_ ? this->gradientClipValue_ : 0.0f;
+    if (net.rides(this) && net.overwritten(from_->delta().data()) && (threshold > 0.0f || clip > 0.0f) &&
+        !net.hasNormGroups(this->delta_.data())) {
+        PX_HIP_CHECK(pxh_shortcut_backward_clipped(this->delta_.data(), nullptr, from_->delta().data(), nullptr,
+                                                   this->delta_.size(), alpha_, beta_, activation_->type(), 1, threshold,
+                                                   clip, nullptr, nullptr, 0, nullptr));
+        return;
+    }
+    Layer<Device::HIP>::backward(input, grad);
     if (net.rides(this)) {
         // the `from` layer's share only: the convolution in front works on delta_ itself
         if (net.overwritten(from_->delta().data()))

@@ -509,6 +509,23 @@ int pxh_rescale_clip_from_groups(float* x, size_t n, float threshold, float clip
                                  const void* groups, void* workspace, size_t workspace_bytes,
                                  void* stream);
 
+/* A ShortcutLayer's whole backward: Layer::backward's rescale + clip of its delta (include/Layer.h:385-397,
+ * 474-499), then the shortcut's own backward (include/ShortcutLayer.h:98-111) --
+ *   pxh_rescale_clip(delta, n, threshold, clip, norm_out, ...), then
+ *   first ? pxh_shortcut_backward_first(delta, ...) : pxh_shortcut_backward(delta, ...)
+ * with the values of that sequence to the bit.  For a first writer (first != 0) with a linear activation
+ * over 16-byte aligned tensors of a multiple of four values -- every shortcut of the shipped YOLOv3 graph
+ * once its targets are known to be written here first -- the two run as two launches that read the
+ * delta once when nothing has to change (the common case: the pass that adds up the norm writes both
+ * targets as well, the second launch forms the verdict and leaves; otherwise it rewrites the delta and
+ * both targets from it): 8 or 12 bytes per element where the sequence moves 12 or 16.  Every other case
+ * runs the sequence itself.  delta must not alias from_delta or grad; grad is nullable.
+ * workspace: pxh_rescale_workspace_bytes() bytes or NULL. */
+int pxh_shortcut_backward_clipped(float* delta, const float* pre_activation, float* from_delta,
+                                  float* grad, size_t n, float alpha, float beta, int activation,
+                                  int first, float threshold, float clip, float* norm_out,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------
  * Adam.  include/Adam.cuh:21, include/cuda/Adam.h:49-90.
  * ---------------------------------------------------------------------- */

@@ -66,6 +66,7 @@ SIGNATURES = {
     "pxh_axpy_norm": [Z, F, P, P, P, P],
     "pxh_shortcut_backward_norm": [P, P, P, P, Z, F, F, I, I, P, P],
     "pxh_rescale_clip_from_groups": [P, Z, F, F, P, P, P, Z, P],
+    "pxh_shortcut_backward_clipped": [P, P, P, P, Z, F, F, I, I, F, F, P, P, Z, P],
     "pxh_yolo_detections": [P, I, P, I, P, I, I, I, I, I, I, I, I, F, P, I, P, P],
     "pxh_yolo_detections_append": [P, I, P, I, P, I, I, I, I, I, I, I, I, F, U, P, I, P, P],
     "pxh_nms": [P, P, I, I, I, F, P, P, P, Z, P],

@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstring>
 #include <new>
+#include <type_traits>
 #include <vector>
 
 namespace pxh {
@@ -341,8 +342,15 @@ __device__ __forceinline__ double chains_to_partial(double chain)
     return chain;
 }
 
-template<int V, bool NT>
-__device__ __forceinline__ void sumsq_walk(const float* x, size_t n_vec, uint32_t block, uint32_t blocks, double2* out)
+// What a walk over a tensor hands every vector it holds to, besides its own work: nothing, or the kernel
+// that would read the tensor next (so that the tensor is read once for both).
+struct NoSink {
+    template<int V, bool NT> __device__ __forceinline__ void take(size_t, const Pack<V>&) const {}
+};
+
+template<int V, bool NT, typename Sink = NoSink>
+__device__ __forceinline__ void sumsq_walk(const float* x, size_t n_vec, uint32_t block, uint32_t blocks, double2* out,
+                                           const Sink& sink = Sink{})
 {
     const size_t per_step = static_cast<size_t>(kBlock) * V * kNormLoads;
     if constexpr (V == 4) {
@@ -374,6 +382,13 @@ __device__ __forceinline__ void sumsq_walk(const float* x, size_t n_vec, uint32_
             for (int u = 0; u < kNormLoads; ++u) {
                 peak = fmaxf(peak, peak_of(v[u]));
                 chain[u] += static_cast<double>(wave_sum_by_rows(square_sum(v[u])));
+            }
+            if constexpr (!std::is_same_v<Sink, NoSink>) {
+#pragma unroll
+                for (int u = 0; u < kNormLoads; ++u) {
+                    const size_t e = base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V;
+                    if (e < n_vec) sink.template take<V, NT>(e, v[u]);
+                }
             }
         }
         peak = wave_max(peak);
@@ -492,10 +507,10 @@ __device__ __forceinline__ RescalePlan rescale_plan(const double2* partial, int 
 
 // x = clamp(factor * x); leaves without touching the tensor when there is nothing to do.  The grid
 // is the reduction's capped one and strides over the tensor.
-template<int V, bool NT>
+template<int V, bool NT, typename Sink = NoSink>
 __device__ __forceinline__ void rescale_walk(float* x, size_t n_vec, const double2* partial, int partials,
                                              uint32_t block, uint32_t blocks, float threshold, float clip,
-                                             float* norm_out)
+                                             float* norm_out, const Sink& sink = Sink{})
 {
     const RescalePlan plan = rescale_plan(partial, partials, threshold, clip);
     if (norm_out && block == 0 && threadIdx.x == 0) *norm_out = plan.norm;
@@ -517,6 +532,7 @@ __device__ __forceinline__ void rescale_walk(float* x, size_t n_vec, const doubl
             for (int u = 0; u < kNormLoads; ++u) {
                 rewrite(v[u]);
                 st<V, NT>(x, base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V, v[u]);
+                sink.template take<V, NT>(base + (static_cast<size_t>(u) * kBlock + threadIdx.x) * V, v[u]);
             }
         } else {
 #pragma unroll
@@ -526,6 +542,7 @@ __device__ __forceinline__ void rescale_walk(float* x, size_t n_vec, const doubl
                     v[u] = ld<V, NT>(x, e);
                     rewrite(v[u]);
                     st<V, NT>(x, e, v[u]);
+                    sink.template take<V, NT>(e, v[u]);
                 }
             }
         }
@@ -538,6 +555,43 @@ __global__ __launch_bounds__(kBlock) void rescale_clip_kernel(float* x, size_t n
                                                               float* norm_out)
 {
     rescale_walk<V, NT>(x, n_vec, partial, partials, blockIdx.x, gridDim.x, threshold, clip, norm_out);
+}
+
+// ---- Layer::backward's rescale + clip of a shortcut's delta with the shortcut's backward in the same passes ----
+// A shortcut that is the first to write its two targets in the backward pass (ShortcutBackwardOp<LINEAR, true>)
+// leaves in them plain functions of its delta.  The pass that adds up the delta's norm therefore also writes
+// them, as if nothing had to change; the second launch forms the plan, leaves at once when that was right, and
+// otherwise rewrites the delta and both targets from it: the values of pxh_rescale_clip followed by
+// pxh_shortcut_backward_first either way, with the delta read once where it had been read twice.
+struct ShortcutFirstSink {
+    float* from_delta;
+    float* grad;   // nullable
+    float alpha, beta;
+    template<int V, bool NT> __device__ __forceinline__ void take(size_t e, const Pack<V>& d) const
+    {
+        Pack<V> f, g;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            f.v[k] = beta * d.v[k];
+            g.v[k] = alpha * d.v[k];
+        }
+        st<V, NT>(from_delta, e, f);
+        if (grad) st<V, NT>(grad, e, g);
+    }
+};
+
+template<bool NT, typename Sink>
+__global__ __launch_bounds__(kBlock) void sumsq_sink_kernel(const float* x, size_t n_vec, double2* partial, Sink sink)
+{
+    sumsq_walk<4, NT, Sink>(x, n_vec, blockIdx.x, gridDim.x, partial + blockIdx.x, sink);
+}
+
+template<bool NT, typename Sink>
+__global__ __launch_bounds__(kBlock) void rescale_clip_sink_kernel(float* x, size_t n_vec, const double2* partial,
+                                                                   int partials, float threshold, float clip,
+                                                                   float* norm_out, Sink sink)
+{
+    rescale_walk<4, NT, Sink>(x, n_vec, partial, partials, blockIdx.x, gridDim.x, threshold, clip, norm_out, sink);
 }
 
 // The same two passes over up to kRescaleTensors tensors per launch (the update hooks of a model run
@@ -1284,6 +1338,56 @@ int pxh_rescale_clip_from_groups(float* x, size_t n, float threshold, float clip
     if (!groups && n) return fail_invalid("pxh_rescale_clip_from_groups: null group buffer");
     return rescale_clip("pxh_rescale_clip_from_groups", x, n, threshold, clip, norm_out,
                         static_cast<const float2*>(groups), workspace, workspace_bytes, stream);
+}
+
+int pxh_shortcut_backward_clipped(float* delta, const float* pre_activation, float* from_delta, float* grad, size_t n,
+                                  float alpha, float beta, int activation, int first, float threshold, float clip,
+                                  float* norm_out, void* workspace, size_t workspace_bytes, void* stream)
+{
+    const char* who = "pxh_shortcut_backward_clipped";
+    if ((!delta || !from_delta) && n) return fail_invalid("%s: null pointer", who);
+    if (activation != PXH_LINEAR && !pre_activation && n)
+        return fail_invalid("%s: pre_activation is required for a non-linear activation", who);
+    if (first && from_delta == grad && n)
+        return fail_invalid("%s: from_delta and grad must be distinct when both are overwritten", who);
+    if ((delta == from_delta || delta == grad) && n) return fail_invalid("%s: delta must be a tensor of its own", who);
+    if (activation < PXH_LEAKY || activation > PXH_TANH) return fail_invalid("%s: unknown activation %d", who, activation);
+    if (n == 0) return PXH_OK;
+    const bool helpers = threshold > 0.0f || clip > 0.0f || norm_out != nullptr;
+    const bool fused = helpers && first && activation == PXH_LINEAR && has_groups(delta, n) && aligned16(from_delta) &&
+                       aligned16(grad);
+    if (!fused) {
+        // the two calls one after the other: the accumulating form (what it adds to cannot be taken back), a
+        // non-linear shortcut (its backward rewrites the delta), tensors without a 128-bit walk
+        int rc = helpers ? rescale_clip(who, delta, n, threshold, clip, norm_out, nullptr, workspace, workspace_bytes, stream)
+                         : PXH_OK;
+        if (rc) return rc;
+        return first ? pxh_shortcut_backward_first(delta, pre_activation, from_delta, grad, n, alpha, beta, activation, stream)
+                     : pxh_shortcut_backward(delta, pre_activation, from_delta, grad, n, alpha, beta, activation, stream);
+    }
+    void* ws = nullptr;
+    int rc = resolve_workspace(workspace, workspace_bytes, pxh_rescale_workspace_bytes(), &ws, as_stream(stream));
+    if (rc) return rc;
+    double2* partial = static_cast<double2*>(ws);
+    hipStream_t s = as_stream(stream);
+    const bool nt = n * (grad ? 12 : 8) >= kStreamingBytes;
+    // the workgroups and the walk of pxh_rescale_clip's own passes: the same partial sums, the same norm
+    const size_t per_step = static_cast<size_t>(kBlock) * 4 * kNormLoads;
+    const size_t want = (n + per_step - 1) / per_step;
+    const int blocks = static_cast<int>(want < static_cast<size_t>(kNormBlocks) ? want : kNormBlocks);
+    const ShortcutFirstSink sink{ from_delta, grad, alpha, beta };
+    if (nt) hipLaunchKernelGGL((sumsq_sink_kernel<true, ShortcutFirstSink>), dim3(blocks), dim3(kBlock), 0, s, delta, n,
+                               partial, sink);
+    else hipLaunchKernelGGL((sumsq_sink_kernel<false, ShortcutFirstSink>), dim3(blocks), dim3(kBlock), 0, s, delta, n,
+                            partial, sink);
+    rc = check_launch(who);
+    if (rc) return rc;
+    const dim3 grid(threshold > 0.0f || clip > 0.0f ? static_cast<unsigned>(blocks) : 1u);
+    if (nt) hipLaunchKernelGGL((rescale_clip_sink_kernel<true, ShortcutFirstSink>), grid, dim3(kBlock), 0, s, delta, n,
+                               partial, blocks, threshold, clip, norm_out, sink);
+    else hipLaunchKernelGGL((rescale_clip_sink_kernel<false, ShortcutFirstSink>), grid, dim3(kBlock), 0, s, delta, n,
+                            partial, blocks, threshold, clip, norm_out, sink);
+    return check_launch(who);
 }
 
 size_t pxh_rescale_multi_workspace_bytes(void)

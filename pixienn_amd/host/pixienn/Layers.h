@@ -714,8 +714,23 @@ public:
 
     void backward(const V& input, V* grad) override
     {
-        Layer::backward(input, grad);
         const float* pre = preActivation_.empty() ? nullptr : preActivation_.data();
+        // A first writer's targets are plain functions of its delta: Layer::backward's rescale + clip and the
+        // layer's own backward run as one call that reads the delta once when nothing has to change
+        // (pxh_shortcut_backward_clipped; the values of the two calls to the bit).  Not where the norm of the
+        // delta is already known from its writer, nor where this layer has to leave one behind.
+        const float threshold = rescaleThreshold(), clip = clipValue();
+        const bool fused = firstWriter_ && sameShape_ && (threshold > 0.0f || clip > 0.0f) && !leavesNorm_ &&
+                           (riding_ || grad != nullptr) && !context().hasNormGroups(delta_.data());
+        if (fused) {
+            context().reserveWorkspace(pxh_rescale_workspace_bytes());
+            PX_HIP_CHECK(pxh_shortcut_backward_clipped(delta_.data(), pre, from_->delta().data(),
+                                                       riding_ ? nullptr : grad->data(), delta_.size(), alpha_, beta_,
+                                                       activation_, 1, threshold, clip, nullptr, context().workspace(),
+                                                       context().workspaceBytes(), stream()));
+            return;
+        }
+        Layer::backward(input, grad);
         if (riding_) {
             // the `from` layer's share only; the convolution in front takes delta_ itself
             if (firstWriter_)

@@ -332,6 +332,16 @@ def shortcut_backward_first(delta, from_delta, grad=None, activation="linear", a
          float(alpha), float(beta), act_id(activation), _stream())
 
 
+def shortcut_backward_clipped(delta, from_delta, grad=None, activation="linear", alpha=1.0, beta=1.0,
+                              pre_activation=None, first=True, threshold=0.0, clip=0.0, norm_out=None, workspace=None):
+    """rescale_clip(delta, threshold, clip, norm_out), then the shortcut's backward (first writer or accumulating)."""
+    _chk_all(delta, from_delta, grad, pre_activation, norm_out, workspace)
+    wb = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("pxh_shortcut_backward_clipped", ptr(delta), ptr(pre_activation), ptr(from_delta), ptr(grad), delta.numel(),
+         float(alpha), float(beta), act_id(activation), int(bool(first)), float(threshold), float(clip), ptr(norm_out),
+         ptr(workspace), wb, _stream())
+
+
 # ---------------------------------------------------------------- YOLO head
 def yolo_activate(inp, out, batch, masks, classes, area):
     _chk_all(inp, out)

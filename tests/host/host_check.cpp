@@ -868,7 +868,7 @@ void firstWriterShortcutChecks()
         Context ctx;
         std::shared_ptr<ConvLayer> a, b, c;
         std::shared_ptr<ShortcutLayer> add;
-        explicit Block(bool firstWriter)
+        Block(bool firstWriter, float threshold, float clip)
         {
             ctx.training = true;
             const Properties conv{ { "batch", N }, { "channels", C }, { "height", S }, { "width", S }, { "filters", C },
@@ -879,6 +879,11 @@ void firstWriterShortcutChecks()
             add = std::make_shared<ShortcutLayer>(ctx, Properties{ { "batch", N }, { "channels", C }, { "height", S },
                                                                    { "width", S }, { "first_writer", firstWriter } }, a);
             if (firstWriter) c->setFirstConsumerOverwrites(true);
+            for (Layer* l: { static_cast<Layer*>(a.get()), static_cast<Layer*>(b.get()), static_cast<Layer*>(c.get()),
+                             static_cast<Layer*>(add.get()) }) {
+                l->setGradientRescaling(threshold > 0.0f, threshold);
+                l->setGradientClipping(clip > 0.0f, clip);
+            }
         }
         void step(const FloatVector& input, const Host& outDelta)
         {
@@ -893,24 +898,36 @@ void firstWriterShortcutChecks()
             a->backward(input, nullptr);
         }
     };
-    Block plain(false), first(true);
-    report("the shortcut marks its from layer", first.a->firstConsumerOverwrites() && !plain.a->firstConsumerOverwrites() &&
-                                                !first.b->firstConsumerOverwrites());
     const FloatVector input(normals(701, size_t(N) * C * S * S));
-    for (int round = 0; round < 2; ++round) {
-        const Host outDelta = normals(702 + round, size_t(N) * C * S * S);
-        // stale values where the fill used to be: they must not survive
-        first.a->delta().fill(std::nanf(""));
-        first.c->delta().fill(std::nanf(""));
-        plain.step(input, outDelta);
-        first.step(input, outDelta);
-        const std::string tag = " (step " + std::to_string(round + 1) + ")";
-        expectClose("first-writer block: delta of the layer in front" + tag, first.c->delta().asVector(),
-                    plain.c->delta().asVector(), 0.0, 1.0);
-        expectClose("first-writer block: delta of the from layer" + tag, first.a->delta().asVector(),
-                    plain.a->delta().asVector(), 0.0, 1.0);
-        expectClose("first-writer block: scale updates of the from layer" + tag, first.a->scaleUpdates().asVector(),
-                    plain.a->scaleUpdates().asVector(), 0.0, 1.0);
+    double norm = 0.0;
+    for (float v: normals(702, size_t(N) * C * S * S)) norm += double(v) * v;
+    norm = std::sqrt(norm);
+    // with the layers' gradient helpers on, the first writer's rescale + clip and its backward are one call
+    // that reads the delta once (pxh_shortcut_backward_clipped): the same values again
+    struct Case { const char* name; float threshold, clip; };
+    const Case cases[] = { { "helpers off", 0.0f, 0.0f }, { "below the threshold", float(4.0 * norm), 0.0f },
+                           { "rescaled", float(0.5 * norm), 0.0f }, { "rescaled and clamped", float(0.5 * norm), 0.25f } };
+    for (const Case& k: cases) {
+        Block plain(false, k.threshold, k.clip), first(true, k.threshold, k.clip);
+        report("the shortcut marks its from layer", first.a->firstConsumerOverwrites() &&
+                                                    !plain.a->firstConsumerOverwrites() && !first.b->firstConsumerOverwrites());
+        for (int round = 0; round < 2; ++round) {
+            const Host outDelta = normals(702 + round, size_t(N) * C * S * S);
+            // stale values where the fill used to be: they must not survive
+            first.a->delta().fill(std::nanf(""));
+            first.c->delta().fill(std::nanf(""));
+            plain.step(input, outDelta);
+            first.step(input, outDelta);
+            const std::string tag = std::string(" (") + k.name + ", step " + std::to_string(round + 1) + ")";
+            expectClose("first-writer block: delta of the layer in front" + tag, first.c->delta().asVector(),
+                        plain.c->delta().asVector(), 0.0, 1.0);
+            expectClose("first-writer block: delta of the from layer" + tag, first.a->delta().asVector(),
+                        plain.a->delta().asVector(), 0.0, 1.0);
+            expectClose("first-writer block: the shortcut's own delta" + tag, first.add->delta().asVector(),
+                        plain.add->delta().asVector(), 0.0, 1.0);
+            expectClose("first-writer block: scale updates of the from layer" + tag, first.a->scaleUpdates().asVector(),
+                        plain.a->scaleUpdates().asVector(), 0.0, 1.0);
+        }
     }
 }
 

@@ -119,7 +119,7 @@ def test_binding_headers_and_stub_name_only_members_the_engine_has():
             members = set(re.findall(r"\b[a-z]\w*_\b", text)) - {"px_hip_status_"}
             methods = set(re.findall(r"this->(\w+)\(", text)) | set(re.findall(r"\bnet\.(\w+)\(", text))
             for m in sorted(members | methods):
-                if m in own or m in ("deferHead", "normGroupsFor", "noteNormGroups", "takeNormGroups", "overwritten",
+                if m in own or m in ("deferHead", "normGroupsFor", "noteNormGroups", "takeNormGroups", "hasNormGroups", "overwritten",
                                      "registerParameters", "updateAll", "rides", "riderOf", "poolOf"):
                     continue
                 assert m in known, "%s/%s names `%s`, which the engine's %s does not have" % (folder, name, m, layer)
